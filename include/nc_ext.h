@@ -1,0 +1,78 @@
+/*
+ * nc_ext.h - additive entry points beside the libnc-compatible ABI of
+ * nc_api.h.  The reference API already carries fused ops of this kind
+ * (nc_fused_layer_norm libnc.h:394, nc_geglu libnc.h:254, nc_apply
+ * libnc.h:634); these follow the same ownership rules (NCTensor* arguments are
+ * consumed, the result is owned by the caller) and take part in nc_backward().
+ * libnc_hip.so implements them as single fused HIP kernels; libnc_ref.so (the
+ * CPU checker) implements them as direct scalar loops.
+ */
+#ifndef NC_EXT_H
+#define NC_EXT_H
+
+#include "nc_api.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* activations for nc_linear() */
+#define NC_ACT_NONE 0
+#define NC_ACT_GELU 1 /* tanh form: 0.5x(1+tanh(0.7978845608(x+0.044715x^3))) */
+#define NC_ACT_RELU 2
+
+/* y = act(w * x + bias).  w (m,k), x (k,n), bias (m) or NULL -> (m,n).
+   Replaces the nc_matmul + nc_add + nc_gelu triple of nncp.c:930-943 and
+   the matmul + bias pairs at nncp.c:659-661, 970-972, 1002-1004. */
+NCTensor *nc_linear(NCTensor *w, NCTensor *x, NCTensor *bias, int act);
+
+/* Relative-position causal attention over memory + current segment, all
+   heads and streams in one call.  Replaces nncp.c:722-800 and the
+   split_head/concat_head copies (nncp.c:554-579).
+     q      (H*dk, B, T)            queries, head h owns rows h*dk..h*dk+dk-1
+     kv     (H*dk + H*dv, B, T)     keys (first H*dk rows) and values, current
+     kv_mem (H*dk + H*dv, B, M)     the same for the memory, or NULL (M = 0)
+     w_r    (dk, d_pos, H) or NULL  relative-position vectors
+     b_r    (K, H) or NULL          relative-position scalar bias, K = M+T
+   With key j in [0,K), query i in [0,T), distance delta = i + M - j:
+     S[j,i] = (k_j.q_i + w_r[:, max(d_pos-1-delta,0), h].q_i
+               + b_r_scale * b_r[K-1-delta, h]) / sqrt(dk)
+              for 0 <= delta < attn_len, else -inf
+     out[:, i] = sum_j v_j softmax_j(S[:, i])
+   Result (H*dv, B, T).  Gradients flow to q, kv, kv_mem, w_r and b_r. */
+NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv_mem,
+                              NCTensor *w_r, NCTensor *b_r, int n_head,
+                              int d_key, int attn_len, float b_r_scale);
+
+/* Integer CDF for the arithmetic coder (anchor: nc_soft_max_int libnc.h:384).
+   logits (V, n) f32 -> (V, n) NC_TYPE_U16 with, per column,
+     cdf[0] = 0, cdf[i+1] - cdf[i] >= 1, implicit cdf[V] = 65536.
+   Pure function of the logits, bit-identical between the two libraries:
+     m = max_i x_i ;  e_i = nc_exp_det(max(x_i - m, -30)) ;
+     q_i = (uint32)(e_i * 2^24) ;  Q_i = sum_{j<i} q_j (exact integers) ;
+     cdf[i] = floor(Q_i * (65536 - V) / Q_V) + i.                          */
+NCTensor *nc_soft_max_cdf16(NCTensor *logits);
+
+/* cdf (V, n) U16, targets (m, n) U16 -> (m, n) U16 symbols: the largest s
+   with cdf[s, col] <= target (cumulative-frequency search of a decoder). */
+NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets);
+
+/* The deterministic exponential used by nc_soft_max_cdf16, for x <= 0:
+   n = rint(x*log2e); r = x - n*ln2 (two fmaf steps); degree-6 polynomial in
+   fmaf form; result scaled by 2^n through the exponent field.  Only IEEE
+   single-precision operations that round identically on x86 and gfx950. */
+float nc_exp_det(float x);
+
+/* When non-zero, every nc_matmul / nc_linear on device tensors rounds both
+   operands to bf16 (round-to-nearest-even) as it loads them and accumulates in
+   fp32 on the bf16 MFMA units; parameters and activations stay fp32 in memory.
+   Returns the previous setting.  libnc_ref.so emulates the same rounding. */
+int nc_set_matmul_bf16(NCContext *m, int enable);
+
+/* Number of kernel launches issued so far (0 in libnc_ref.so). */
+int64_t nc_get_launch_count(NCContext *m);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NC_EXT_H */

@@ -1,0 +1,56 @@
+"""Shared fixtures.  `ref` is the CPU checker (oracle/libnc_ref.so); `hip` is
+the product library on the GPU.  Only tests may load the checker."""
+import importlib.util
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+REF_LIB = os.path.join(ROOT, "oracle", "libnc_ref.so")
+
+
+def load_pkg():
+    """The package directory name holds a hyphen, so it is loaded by path."""
+    name = "nncp_metal_amd"
+    if name in sys.modules:
+        return sys.modules[name]
+    spec = importlib.util.spec_from_file_location(
+        name, os.path.join(ROOT, "nncp-metal_amd", "__init__.py"),
+        submodule_search_locations=[os.path.join(ROOT, "nncp-metal_amd")])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def pkg():
+    return load_pkg()
+
+
+@pytest.fixture()
+def ref(pkg):
+    if not os.path.exists(REF_LIB):
+        pytest.fail("oracle/libnc_ref.so missing: run `make -C oracle`")
+    nc = pkg.binding.NC(REF_LIB, use_device=False, nb_threads=4)
+    yield nc
+    nc.close()
+
+
+@pytest.fixture()
+def hip(pkg):
+    nc = pkg.binding.NC(pkg.binding.HIP_LIB, use_device=True)
+    yield nc
+    nc.close()
+
+
+@pytest.fixture()
+def rng():
+    return np.random.default_rng(1234)

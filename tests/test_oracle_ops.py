@@ -1,0 +1,159 @@
+"""Pins the CPU checker (oracle/libnc_ref.so): every op the Transformer path
+uses is compared with an independent float64 numpy restatement (forward) and
+with central finite differences of that restatement (backward)."""
+import numpy as np
+import pytest
+
+import cases
+import nputil as U
+
+
+@pytest.mark.parametrize("name", [c.name for c in cases.CASES])
+def test_op_forward_backward(ref, rng, name):
+    case = cases.BY_NAME[name]
+    arrays = case.inputs(rng)
+    expect = case.ref(*[a.astype(np.float64) for a in arrays])
+    weight = rng.standard_normal(np.shape(expect))
+    out, grads = case.run(ref, arrays, weight)
+    assert out.shape == np.shape(expect)
+    np.testing.assert_allclose(out, expect, rtol=2e-5, atol=2e-6)
+    fd = U.fd_grad(lambda *xs: float((case.ref(*xs) * weight).sum()), arrays)
+    for g, f in zip(grads, fd):
+        assert g.shape == f.shape
+        np.testing.assert_allclose(g, f, rtol=3e-3, atol=3e-4)
+
+
+def test_softmax_closed_forms(ref, rng):
+    x = rng.standard_normal((4, 9)).astype(np.float32) * 3
+    p = ref.numpy(ref.nc_soft_max(ref.tensor(x)), free=True)
+    np.testing.assert_allclose(p.sum(axis=-1), 1.0, rtol=1e-6)
+    p2 = ref.numpy(ref.nc_soft_max(ref.tensor(x + 5.0)), free=True)
+    np.testing.assert_allclose(p, p2, rtol=1e-5)
+    big = np.array([[1000.0, 0.0, -1000.0]], dtype=np.float32)
+    p3 = ref.numpy(ref.nc_soft_max(ref.tensor(big)), free=True)
+    np.testing.assert_array_equal(p3, [[1.0, 0.0, 0.0]])
+
+
+def test_layer_norm_closed_forms(ref, rng):
+    x = rng.standard_normal((5, 64)).astype(np.float32) * 4 + 2
+    y = ref.numpy(ref.nc_layer_norm(ref.tensor(x), 1e-5), free=True)
+    np.testing.assert_allclose(y.mean(axis=-1), 0, atol=1e-6)
+    np.testing.assert_allclose(y.var(axis=-1), 1, rtol=1e-4)
+    y2 = ref.numpy(ref.nc_layer_norm(ref.tensor(3 * x + 7), 1e-5), free=True)
+    np.testing.assert_allclose(y, y2, atol=1e-5)
+    r = ref.numpy(ref.nc_rms_norm(ref.tensor(x), 1e-5), free=True)
+    np.testing.assert_allclose((r ** 2).mean(axis=-1), 1, rtol=1e-4)
+
+
+def test_attention_special_cases(ref, rng):
+    """w_r = b_r = 0 reduces to textbook causal attention with memory;
+    q = 0 reduces to the softmax of the bias profile."""
+    H, dk, dv, B, T, M = 2, 4, 4, 2, 6, 4
+    K = M + T
+    q = rng.standard_normal((T, B, H * dk)).astype(np.float32)
+    kv = rng.standard_normal((T, B, H * (dk + dv))).astype(np.float32)
+    kvm = rng.standard_normal((M, B, H * (dk + dv))).astype(np.float32)
+    y = ref.numpy(ref.nc_relpos_attention(ref.tensor(q), ref.tensor(kv), ref.tensor(kvm),
+                                          None, None, H, dk, K, 1.0), free=True)
+    allkv = np.concatenate([kvm, kv], 0).astype(np.float64)
+    for b in range(B):
+        for h in range(H):
+            k = allkv[:, b, h * dk:(h + 1) * dk]
+            v = allkv[:, b, H * dk + h * dv:H * dk + (h + 1) * dv]
+            s = q[:, b, h * dk:(h + 1) * dk].astype(np.float64) @ k.T / np.sqrt(dk)
+            causal = np.arange(K)[None, :] <= np.arange(T)[:, None] + M
+            s = np.where(causal, s, -np.inf)
+            np.testing.assert_allclose(y[:, b, h * dv:(h + 1) * dv], U.softmax(s) @ v,
+                                       rtol=1e-5, atol=1e-6)
+    b_r = rng.standard_normal((H, K)).astype(np.float32)
+    y0 = ref.numpy(ref.nc_relpos_attention(ref.tensor(np.zeros_like(q)), ref.tensor(kv),
+                                           ref.tensor(kvm), None, ref.tensor(b_r), H, dk, K, 2.0),
+                   free=True)
+    for h in range(H):
+        for i in range(T):
+            # key j sees bias row K-1-(i+M-j)
+            prof = np.array([2.0 * b_r[h, K - 1 - (i + M - j)] / np.sqrt(dk) if j <= i + M
+                             else -np.inf for j in range(K)])
+            a = U.softmax(prof[None])[0]
+            v = allkv[:, 0, H * dk + h * dv:H * dk + (h + 1) * dv]
+            np.testing.assert_allclose(y0[i, 0, h * dv:(h + 1) * dv], a @ v, rtol=1e-5, atol=1e-6)
+
+
+def test_rel_shift_places_distance_zero_on_last_row(ref):
+    """nncp.c:784 with the mask of nncp.c:355-363: after the shift, row j of
+    query column i must hold the entry of distance (i+M)-j, i.e. source row
+    j+T-1-i; distance 0 (source row K-1) lands on key j = i+M."""
+    T, M = 4, 3
+    K = T + M
+    rd = np.arange(K, dtype=np.float32)[None, :].repeat(T, 0)  # value = source row p
+    y = ref.numpy(ref.nc_rel_shift(ref.tensor(rd), -(T - 1), 1), free=True)
+    for i in range(T):
+        for j in range(K):
+            p = j + T - 1 - i
+            assert y[i, j] == (p if p < K else 0)
+        assert y[i, i + M] == K - 1
+
+
+def test_backward_sums_tied_parameter(ref, rng):
+    """A tensor used twice (tied w_r/b_r, nncp.c:742-760) is reported once with
+    the summed gradient."""
+    w = rng.standard_normal((3, 3)).astype(np.float32)
+    x = rng.standard_normal((2, 3)).astype(np.float32)
+    h, p = ref.param(w)
+    y = ref.nc_matmul(ref.dup(h.value), ref.nc_matmul(ref.dup(h.value), ref.tensor(x)))
+    loss = ref.nc_sum(y)
+    g = ref.backward(loss)[p]
+    fd = U.fd_grad(lambda w_: float((x @ w_ @ w_).sum()), [w])[0]
+    np.testing.assert_allclose(g, fd, rtol=2e-3, atol=1e-4)
+
+
+def test_views_and_copies(ref, rng):
+    """nc_slice_alias shares storage; nc_tensor_copy through it mutates the
+    parent (nncp.c:650-657); nc_tensor_copy_slice shifts memory (nncp.c:1212)."""
+    x = rng.standard_normal((6, 2, 3)).astype(np.float32)  # libnc (3,2,6)
+    t = ref.tensor(x)
+    src = rng.standard_normal((1, 2, 3)).astype(np.float32)
+    a = ref.nc_slice_alias(t, 2, 4, 5)
+    s = ref.tensor(src)
+    ref.nc_tensor_copy(a, s)
+    ref.free(a, s)
+    x[4:5] = src
+    np.testing.assert_array_equal(ref.numpy(t), x)
+    ref.nc_tensor_copy_slice(t, t, 2, 0, 4, 2)  # overlapping shift left by 2
+    x[0:4] = x[2:6].copy()
+    np.testing.assert_array_equal(ref.numpy(t), x)
+    ref.nc_tensor_set_zero(t)
+    assert not ref.numpy(t).any()
+    ref.free(t)
+
+
+def test_optimisers_closed_form(ref, pkg):
+    """One scalar parameter, known gradients: RMSProp as BASELINE states it
+    and Adam(beta1=0) with bias correction."""
+    B = pkg.binding
+    import ctypes as C
+    for algo in (B.SGD_OPT_RMSPROP, B.SGD_OPT_ADAM, B.SGD_OPT_BASIC):
+        nc = B.NC(ref.lib._name, use_device=False)
+        h, p = nc.param(np.array([1.0, -2.0], dtype=np.float32))
+        sp = B.SGDOptParams(algo=algo, beta1=0.0, beta2=0.99, eps=1e-8, gradient_clip=0.0, lr=3e-4)
+        opt = nc.nc_sgd_opt_init(nc.ctx, C.byref(sp))
+        nc.nc_sgd_opt_set_all(C.byref(nc.plist), opt)
+        w = np.array([1.0, -2.0])
+        v = np.zeros(2)
+        for t in range(1, 4):
+            g = np.array([0.5 * t, -0.25])
+            nc.sgd_opt_update_var(p, nc.tensor(g.astype(np.float32)), None)
+            nc.nc_sgd_opt_set_lr(opt, 3e-4)
+            nc.nc_sgd_opt_update(opt)
+            if algo == B.SGD_OPT_RMSPROP:
+                v = 0.99 * v + 0.01 * g * g
+                w = w - 3e-4 * g / (np.sqrt(v) + 1e-8)
+            elif algo == B.SGD_OPT_ADAM:
+                v = 0.99 * v + 0.01 * g * g
+                w = w - 3e-4 * g / (np.sqrt(v / (1 - 0.99 ** t)) + 1e-8)
+            else:
+                w = w - 3e-4 * g
+            np.testing.assert_allclose(nc.numpy(h.value), w, rtol=1e-6)
+        nc.nc_sgd_opt_set_all(C.byref(nc.plist), None)
+        nc.nc_sgd_opt_end(opt)
+        nc.close()
