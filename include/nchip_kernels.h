@@ -1,0 +1,133 @@
+/*
+ * nchip_kernels.h - the thin C ABI over the hand-written gfx950 kernels of
+ * libnc_hip.so.  Plain device pointers and sizes, no C++ or torch types; every
+ * entry point enqueues on `stream` (a hipStream_t passed as void*) and returns
+ * 0, or a negative value after printing the reason when the arguments do not
+ * fit what the kernel assumes.  Matrices are column-major as in libnc
+ * (libnc.h:106-115): element (i, j) of an m x n matrix with leading dimension
+ * ld lives at base[i + j*ld].  The libnc-level ops of nc_api.h / nc_ext.h are
+ * thin wrappers over these.
+ */
+#ifndef NCHIP_KERNELS_H
+#define NCHIP_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NCHIP_ACT_NONE 0
+#define NCHIP_ACT_GELU 1
+#define NCHIP_ACT_RELU 2
+
+/* C = act(alpha * op(A) * op(B) + beta * C + bias), batched.
+   Replaces nc_matmul / nc_matmul_add (libnc.h:365-373, call sites
+   nncp.c:659-1004).  op(A) is m x k: A is (m,k) when ta == 0, (k,m) when
+   ta == 1; likewise B is (k,n) or (n,k).  bias (m) may be NULL.  When `pre`
+   is not NULL the value before the activation is stored there too (same
+   layout as C).  precision 0: fp32 MFMA; 1: operands rounded to bf16
+   (nearest-even) on load, fp32 accumulation on the bf16 MFMA units.
+   ksplit > 1 splits the reduction over that many workgroups whose partial
+   tiles are summed in a fixed order by a second kernel; it needs
+   `workspace` of at least batch*ksplit*m*n floats.  Every output element is a
+   sequential MFMA accumulation chain over k = 0..K-1 that does not depend on
+   m, n or the tile shape. */
+int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+               const float *A, int64_t lda, int64_t stride_a,
+               const float *B, int64_t ldb, int64_t stride_b,
+               float beta, float *C, int64_t ldc, int64_t stride_c, int batch,
+               const float *bias, int act, float *pre, int precision,
+               int ksplit, float *workspace);
+
+/* Same with two-level batching: batch index z addresses
+   A + (z / batch_in)*sa_out + (z % batch_in)*sa_in (likewise B and C).  Lets
+   per-(stream, head) products read the (features, streams, time) activations
+   in place, without the split_head / concat_head copies of nncp.c:554-579. */
+int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                const float *A, int64_t lda, int64_t sa_out, int64_t sa_in,
+                const float *B, int64_t ldb, int64_t sb_out, int64_t sb_in,
+                float beta, float *C, int64_t ldc, int64_t sc_out, int64_t sc_in,
+                int batch, int batch_in,
+                const float *bias, int act, float *pre, int precision,
+                int ksplit, float *workspace);
+
+/* Chooses ksplit for nchip_gemm from the shape alone (never from data). */
+int nchip_gemm_pick_ksplit(int m, int n, int k, int batch);
+
+/* Relative-position causal attention, forward (nncp.c:722-800 fused).
+   Layouts as in nc_relpos_attention (nc_ext.h): q (H*dk, B, T) with leading
+   dimension ldq per token column, kv/kvm (H*dk+H*dv, B, T|M) with ldkv,
+   w_r (dk, d_pos, H) or NULL, b_r (K, H) or NULL, out (H*dv, B, T) with ldo.
+   probs (K, T, H, B) receives the attention probabilities (kept for the
+   backward pass); rel (d_pos, T, H, B) is scratch for w_r^T q (unused when
+   w_r is NULL).  precision as in nchip_gemm. */
+int nchip_relpos_attn_fwd(void *stream, const float *q, int64_t ldq,
+                          const float *kv, const float *kvm, int64_t ldkv,
+                          const float *w_r, const float *b_r,
+                          float *out, int64_t ldo, float *probs, float *rel,
+                          int H, int dk, int dv, int B, int T, int M, int d_pos,
+                          int attn_len, float b_r_scale, int precision);
+
+/* Backward of the above from the saved probs.  dq, dkv, dkvm are fully
+   overwritten; dw_r (dk, d_pos, H) and db_r (K, H) are overwritten with the
+   sums over streams, reduced in a fixed order (no atomics).  scratch needs
+   nchip_relpos_attn_bwd_scratch() floats. */
+size_t nchip_relpos_attn_bwd_scratch(int H, int dk, int B, int T, int M, int d_pos);
+int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
+                          const float *kv, const float *kvm, int64_t ldkv,
+                          const float *w_r, const float *probs,
+                          const float *dout, int64_t ldo,
+                          float *dq, float *dkv, float *dkvm, float *dw_r, float *db_r,
+                          int H, int dk, int dv, int B, int T, int M, int d_pos,
+                          int attn_len, float b_r_scale, int precision, float *scratch);
+
+/* LayerNorm / RMSNorm over axis 0 of (d, n) with optional affine
+   (nncp.c:279-288; libnc.h:389-395).  xhat (d, n) and rstd (n) are saved for
+   the backward.  w/b may be NULL (then y == xhat may alias). */
+int nchip_norm_fwd(void *stream, const float *x, const float *w, const float *b,
+                   float *y, float *xhat, float *rstd, int d, int64_t n,
+                   float eps, int avg);
+/* dx (d,n); dw, db (d) overwritten (may be NULL when w is NULL).  partial
+   needs nchip_norm_bwd_partial_rows(n) * 2 * d floats. */
+int nchip_norm_bwd_partial_rows(int64_t n);
+int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float *rstd,
+                   const float *w, float *dx, float *dw, float *db, float *partial,
+                   int d, int64_t n, int avg);
+
+/* softmax over axis 0 of (v, n) and its backward dx = y*(g - sum(g*y))
+   (libnc.h:382; nncp.c:796, 1008). */
+int nchip_softmax_fwd(void *stream, const float *x, float *y, int v, int64_t n);
+int nchip_softmax_bwd(void *stream, const float *y, const float *g, float *dx, int v, int64_t n);
+
+/* y[c] = log p[idx[c], c]; fused gradient dlogits = g[c]*(onehot - p)
+   (libnc.h:385-388; nncp.c:1170). */
+int nchip_indexed_log(void *stream, const float *p, const int32_t *idx, float *y, int v, int64_t n);
+int nchip_nll_bwd(void *stream, const float *p, const int32_t *idx, const float *g,
+                  float *dlogits, int v, int64_t n, int fused);
+
+/* embedding gather y[:, c] = w[:, idx[c]] and its deterministic scatter-add
+   backward (libnc.h:374-377; nncp.c:625): dw (d, v) overwritten; columns that
+   share an index are summed in increasing c. */
+int nchip_get_col(void *stream, const float *w, const int32_t *idx, float *y, int d, int v, int64_t n);
+int nchip_add_col(void *stream, const float *g, const int32_t *idx, float *dw, int d, int v, int64_t n);
+
+/* fused optimiser step over one parameter (libnc.h:540-572 semantics as
+   defined in nc_api.h): algo 0 SGD, 1 Adam (bias corrections c1, c2 passed
+   in), 16 RMSProp. */
+int nchip_opt_update(void *stream, int algo, float *w, float *m, float *v, const float *g,
+                     int64_t n, float lr, float beta1, float beta2, float eps, float clip,
+                     float c1, float c2);
+
+/* logits (v, n) f32 -> cdf (v, n) u16 as specified in nc_ext.h
+   (nc_soft_max_cdf16); bit-identical to the CPU checker. */
+int nchip_softmax_cdf16(void *stream, const float *logits, uint16_t *cdf, int v, int64_t n);
+/* sym[i, c] = largest s with cdf[s, c] <= target[i, c]; targets (m, n). */
+int nchip_cdf_lookup(void *stream, const uint16_t *cdf, const uint16_t *target,
+                     uint16_t *sym, int v, int64_t m, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NCHIP_KERNELS_H */

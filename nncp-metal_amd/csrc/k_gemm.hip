@@ -1,0 +1,421 @@
+// GEMM for gfx950 (MI355X): column-major C = act(alpha*op(A)*op(B) + beta*C + bias).
+//
+// One workgroup of 256 threads (4 wavefronts of 64 lanes, arranged 2x2) owns a
+// BM x BN tile of C.  A and B tiles of depth BK = 16 are staged through LDS
+// (double buffered, k-major rows so a wavefront reads 32 consecutive floats),
+// and every wavefront accumulates its (BM/2) x (BN/2) part with
+// v_mfma_f32_32x32x2_f32.  The MFMA is issued as D[n][m] = sum_k B[k][n]*A[k][m]
+// so that the 32 lanes of a half-wavefront hold 32 consecutive m of one column:
+// the epilogue stores are 128-byte coalesced in column-major C.
+//
+// Each C element is one sequential chain of MFMA accumulations over
+// k = 0, 2, 4, ... ; the chain does not depend on the tile shape, on m/n or on
+// the number of columns, so a column computed alone equals the same column
+// computed inside a larger matrix (needed for bit-exact decode).
+//
+// precision 1 rounds both operands to bf16 (nearest-even) while they are
+// written to LDS and feeds v_mfma_f32_32x32x16_bf16 (fp32 accumulate).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include "../../include/nchip_kernels.h"
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef short shortx8 __attribute__((ext_vector_type(8)));
+
+namespace {
+
+constexpr int BK = 16;
+constexpr int PAD = 4;   // keeps 16-byte alignment of LDS rows, staggers banks
+constexpr int NXCD = 8;
+
+struct GemmArgs {
+    const float *A, *B;
+    float *C;
+    const float *bias;
+    float *pre;
+    float *ws;
+    int64_t lda, ldb, ldc, sa, sb, sc;   // outer batch strides
+    int64_t sa_in, sb_in, sc_in;         // inner batch strides
+    int batch_in;                        // batch index z -> (z / batch_in, z % batch_in)
+    int M, N, K, batch, ksplit, kchunk;
+    float alpha, beta;
+    int act;
+    int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ float gelu_tanh(float x)
+{
+    const float c0 = 0.7978845608f, c1 = 0.044715f;
+    return 0.5f * x * (1.0f + tanhf(c0 * (x + c1 * x * x * x)));
+}
+
+__device__ __forceinline__ float apply_act(float v, int act)
+{
+    if (act == NCHIP_ACT_GELU) return gelu_tanh(v);
+    if (act == NCHIP_ACT_RELU) return v > 0.0f ? v : 0.0f;
+    return v;
+}
+
+__device__ __forceinline__ unsigned short f32_to_bf16(float f)
+{
+    unsigned int u = __float_as_uint(f);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+
+// Loads a BT x BK tile (BT = BM or BN) of an operand into registers.
+// MAJOR = 1: the tile's long axis (m or n) is contiguous in memory
+//            (A with ta = 0, B with tb = 1);  element (i, k) at p[i + k*ld].
+// MAJOR = 0: k is contiguous (A with ta = 1, B with tb = 0); (i, k) at p[k + i*ld].
+template <int BT, int MAJOR>
+struct TileLoader {
+    static constexpr int NV = BT * BK / 4 / 256; // float4 per thread
+    floatx4 r[NV];
+
+    __device__ __forceinline__ void load(const float *p, int64_t ld, int i0, int k0,
+                                         int imax, int kmax, bool fast, int t)
+    {
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            int idx = t + v * 256;
+            int i, k;
+            if (MAJOR) { i = (idx % (BT / 4)) * 4; k = idx / (BT / 4); }
+            else       { i = idx % BT;             k = (idx / BT) * 4; }
+            if (fast) {
+                const float *src = MAJOR ? p + (int64_t)(k0 + k) * ld + (i0 + i)
+                                         : p + (int64_t)(i0 + i) * ld + (k0 + k);
+                r[v] = *reinterpret_cast<const floatx4 *>(src);
+            } else {
+                floatx4 tmp;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    int ii = MAJOR ? i + e : i, kk = MAJOR ? k : k + e;
+                    float val = 0.0f;
+                    if (i0 + ii < imax && k0 + kk < kmax)
+                        val = MAJOR ? p[(int64_t)(k0 + kk) * ld + (i0 + ii)]
+                                    : p[(int64_t)(i0 + ii) * ld + (k0 + kk)];
+                    tmp[e] = val;
+                }
+                r[v] = tmp;
+            }
+        }
+    }
+
+    // fp32 LDS tile: rows are k, BT + PAD floats each
+    __device__ __forceinline__ void store_f32(float *lds, int t) const
+    {
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            int idx = t + v * 256;
+            if (MAJOR) {
+                int i = (idx % (BT / 4)) * 4, k = idx / (BT / 4);
+                *reinterpret_cast<floatx4 *>(lds + k * (BT + PAD) + i) = r[v];
+            } else {
+                int i = idx % BT, k = (idx / BT) * 4;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    lds[(k + e) * (BT + PAD) + i] = r[v][e];
+            }
+        }
+    }
+
+    // bf16 LDS tile: rows are i (m or n), BK + 8 halves each, k contiguous so a
+    // lane can fetch its 8 consecutive k for v_mfma_f32_32x32x16_bf16 in one read
+    __device__ __forceinline__ void store_bf16(unsigned short *lds, int t) const
+    {
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            int idx = t + v * 256;
+            if (MAJOR) {
+                int i = (idx % (BT / 4)) * 4, k = idx / (BT / 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    lds[(i + e) * (BK + 8) + k] = f32_to_bf16(r[v][e]);
+            } else {
+                int i = idx % BT, k = (idx / BT) * 4;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    lds[i * (BK + 8) + k + e] = f32_to_bf16(r[v][e]);
+            }
+        }
+    }
+};
+
+template <int BM, int BN, int TA, int TB, int BF16>
+__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g)
+{
+    constexpr int TM = BM / 64, TN = BN / 64; // 32x32 MFMA tiles per wavefront
+    constexpr int LDS_A = BF16 ? BM * (BK + 8) / 2 : BK * (BM + PAD); // in floats
+    constexpr int LDS_B = BF16 ? BN * (BK + 8) / 2 : BK * (BN + PAD);
+    __shared__ __attribute__((aligned(16))) float smem[2 * (LDS_A + LDS_B)];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave & 1, wn = wave >> 1;
+
+    // XCD-aware tile order: the hardware deals consecutive workgroup ids round
+    // robin over the 8 XCDs; give each XCD a contiguous run of tiles so tiles
+    // that share an A/B panel also share an L2.
+    int ntiles = g.tiles_m * g.tiles_n;
+    int bid = blockIdx.x;
+    if (ntiles % NXCD == 0)
+        bid = (bid % NXCD) * (ntiles / NXCD) + bid / NXCD;
+    const int tile_m = bid % g.tiles_m, tile_n = bid / g.tiles_m;
+    const int bz = blockIdx.y;
+    const int b = bz / g.ksplit, kz = bz % g.ksplit;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int kbeg = kz * g.kchunk;
+    const int kend = min(g.K, kbeg + g.kchunk);
+
+    const int b_out = b / g.batch_in, b_in = b % g.batch_in;
+    const float *A = g.A + (int64_t)b_out * g.sa + (int64_t)b_in * g.sa_in;
+    const float *B = g.B + (int64_t)b_out * g.sb + (int64_t)b_in * g.sb_in;
+
+    // fast (vector, unguarded) loads need whole tiles and 16-byte alignment
+    const bool a_full = (m0 + BM <= g.M) && (g.lda % 4 == 0) && (((uintptr_t)A & 15) == 0);
+    const bool b_full = (n0 + BN <= g.N) && (g.ldb % 4 == 0) && (((uintptr_t)B & 15) == 0);
+
+    TileLoader<BM, TA ? 0 : 1> la;
+    TileLoader<BN, TB ? 1 : 0> lb;
+
+    floatx16 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.0f;
+
+    int nk = (kend - kbeg + BK - 1) / BK;
+    if (nk > 0) {
+        bool kf = (kbeg + BK <= kend);
+        la.load(A, g.lda, m0, kbeg, g.M, kend, a_full && kf, t);
+        lb.load(B, g.ldb, n0, kbeg, g.N, kend, b_full && kf, t);
+    }
+    for (int it = 0; it < nk; it++) {
+        float *sa = smem + (it & 1) * (LDS_A + LDS_B);
+        float *sb = sa + LDS_A;
+        if (BF16) {
+            la.store_bf16(reinterpret_cast<unsigned short *>(sa), t);
+            lb.store_bf16(reinterpret_cast<unsigned short *>(sb), t);
+        } else {
+            la.store_f32(sa, t);
+            lb.store_f32(sb, t);
+        }
+        __syncthreads();
+        if (it + 1 < nk) {
+            int k0 = kbeg + (it + 1) * BK;
+            bool kf = (k0 + BK <= kend);
+            la.load(A, g.lda, m0, k0, g.M, kend, a_full && kf, t);
+            lb.load(B, g.ldb, n0, k0, g.N, kend, b_full && kf, t);
+        }
+        if (BF16) {
+            // one 32x32x16 MFMA per tile pair covers the whole BK = 16
+            const unsigned short *ha = reinterpret_cast<const unsigned short *>(sa);
+            const unsigned short *hb = reinterpret_cast<const unsigned short *>(sb);
+            shortx8 fa[TM], fb[TN];
+#pragma unroll
+            for (int j = 0; j < TM; j++)
+                fa[j] = *reinterpret_cast<const shortx8 *>(
+                    ha + (wm * (BM / 2) + j * 32 + (lane & 31)) * (BK + 8) + (lane >> 5) * 8);
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+                fb[i] = *reinterpret_cast<const shortx8 *>(
+                    hb + (wn * (BN / 2) + i * 32 + (lane & 31)) * (BK + 8) + (lane >> 5) * 8);
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+#pragma unroll
+                for (int j = 0; j < TM; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(__attribute__((ext_vector_type(8))) __bf16, fb[i]),
+                        __builtin_bit_cast(__attribute__((ext_vector_type(8))) __bf16, fa[j]),
+                        acc[i][j], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < BK / 2; ks++) {
+                int kk = ks * 2 + (lane >> 5);
+                float fa[TM], fb[TN];
+#pragma unroll
+                for (int j = 0; j < TM; j++)
+                    fa[j] = sa[kk * (BM + PAD) + wm * (BM / 2) + j * 32 + (lane & 31)];
+#pragma unroll
+                for (int i = 0; i < TN; i++)
+                    fb[i] = sb[kk * (BN + PAD) + wn * (BN / 2) + i * 32 + (lane & 31)];
+#pragma unroll
+                for (int i = 0; i < TN; i++)
+#pragma unroll
+                    for (int j = 0; j < TM; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[i], fa[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        // the next iteration writes the other buffer; one barrier per tile is
+        // enough because a buffer is rewritten only two iterations later
+    }
+
+    // epilogue.  acc[i][j][r] is C[m][n] with
+    //   m = m0 + wm*BM/2 + j*32 + lane%32
+    //   n = n0 + wn*BN/2 + i*32 + (r/4)*8 + (lane/32)*4 + r%4
+    const int mm_base = m0 + wm * (BM / 2) + (lane & 31);
+    const int nn_base = n0 + wn * (BN / 2) + (lane >> 5) * 4;
+    if (g.ksplit > 1) {
+        float *ws = g.ws + ((int64_t)(kz * g.batch + b)) * g.M * g.N;
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int j = 0; j < TM; j++) {
+                int m = mm_base + j * 32;
+                if (m >= g.M) continue;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    int n = nn_base + i * 32 + (r >> 2) * 8 + (r & 3);
+                    if (n < g.N)
+                        ws[(int64_t)n * g.M + m] = acc[i][j][r];
+                }
+            }
+        return;
+    }
+    const int64_t coff = (int64_t)b_out * g.sc + (int64_t)b_in * g.sc_in;
+    float *C = g.C + coff;
+    float *P = g.pre ? g.pre + coff : nullptr;
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++) {
+            int m = mm_base + j * 32;
+            if (m >= g.M) continue;
+            float bv = g.bias ? g.bias[m] : 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                int n = nn_base + i * 32 + (r >> 2) * 8 + (r & 3);
+                if (n >= g.N) continue;
+                int64_t off = (int64_t)n * g.ldc + m;
+                float v = g.alpha * acc[i][j][r];
+                if (g.beta != 0.0f) v += g.beta * C[off];
+                v += bv;
+                if (P) P[off] = v;
+                C[off] = apply_act(v, g.act);
+            }
+        }
+}
+
+// sums the ksplit partial tiles in increasing k order, then the same epilogue
+__global__ __launch_bounds__(256) void gemm_splitk_reduce(GemmArgs g)
+{
+    int64_t total = (int64_t)g.M * g.N;
+    int b = blockIdx.y;
+    const int64_t coff = (int64_t)(b / g.batch_in) * g.sc + (int64_t)(b % g.batch_in) * g.sc_in;
+    float *C = g.C + coff;
+    float *P = g.pre ? g.pre + coff : nullptr;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+        int m = (int)(e % g.M);
+        int64_t n = e / g.M;
+        float s = 0.0f;
+        for (int kz = 0; kz < g.ksplit; kz++)
+            s += g.ws[((int64_t)(kz * g.batch + b)) * total + e];
+        int64_t off = n * g.ldc + m;
+        float v = g.alpha * s;
+        if (g.beta != 0.0f) v += g.beta * C[off];
+        if (g.bias) v += g.bias[m];
+        if (P) P[off] = v;
+        C[off] = apply_act(v, g.act);
+    }
+}
+
+template <int BM, int BN, int BF16>
+void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g)
+{
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(256);
+    if (!ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, 0, 0, BF16>), grid, block, 0, st, g);
+    else if (ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, 1, 0, BF16>), grid, block, 0, st, g);
+    else if (!ta && tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, 0, 1, BF16>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_kernel<BM, BN, 1, 1, BF16>), grid, block, 0, st, g);
+}
+
+} // namespace
+
+extern "C" int nchip_gemm_pick_ksplit(int m, int n, int k, int batch)
+{
+    // Aim at >= 512 workgroups (2 per CU on 256 CUs) when the output is small
+    // and the reduction long (the weight-gradient GEMMs: k = tokens).
+    int64_t tiles = (int64_t)((m + 63) / 64) * ((n + 63) / 64) * batch;
+    if (tiles >= 256 || k < 1024)
+        return 1;
+    int s = (int)((512 + tiles - 1) / tiles);
+    int smax = k / 256;
+    if (s > smax) s = smax;
+    if (s > 16) s = 16;
+    return s < 1 ? 1 : s;
+}
+
+extern "C" int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                           const float *A, int64_t lda, int64_t sa_out, int64_t sa_in,
+                           const float *B, int64_t ldb, int64_t sb_out, int64_t sb_in,
+                           float beta, float *C, int64_t ldc, int64_t sc_out, int64_t sc_in,
+                           int batch, int batch_in,
+                           const float *bias, int act, float *pre, int precision,
+                           int ksplit, float *workspace)
+{
+    if (m <= 0 || n <= 0 || batch <= 0)
+        return 0;
+    if (k < 0 || !A || !B || !C || lda < (ta ? k : m) || ldb < (tb ? n : k) || ldc < m || batch_in < 1) {
+        fprintf(stderr, "nchip_gemm: bad arguments (m=%d n=%d k=%d lda=%ld ldb=%ld ldc=%ld)\n",
+                m, n, k, (long)lda, (long)ldb, (long)ldc);
+        return -1;
+    }
+    if (ksplit < 1) ksplit = 1;
+    if (ksplit > 1 && !workspace) {
+        fprintf(stderr, "nchip_gemm: ksplit=%d needs a workspace\n", ksplit);
+        return -1;
+    }
+    if ((int64_t)batch * ksplit > 65535) {
+        fprintf(stderr, "nchip_gemm: batch*ksplit=%ld exceeds the grid limit\n", (long)batch * ksplit);
+        return -1;
+    }
+    GemmArgs g;
+    g.A = A; g.B = B; g.C = C; g.bias = bias; g.pre = pre; g.ws = workspace;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.sa = sa_out; g.sb = sb_out; g.sc = sc_out;
+    g.sa_in = sa_in; g.sb_in = sb_in; g.sc_in = sc_in; g.batch_in = batch_in;
+    g.M = m; g.N = n; g.K = k; g.batch = batch; g.ksplit = ksplit;
+    g.kchunk = ((k + ksplit - 1) / ksplit + BK - 1) / BK * BK;
+    if (g.kchunk < BK) g.kchunk = BK;
+    g.alpha = alpha; g.beta = beta; g.act = act;
+    hipStream_t st = (hipStream_t)stream;
+    // tile choice from the shape only: large tiles when they still fill the chip
+    int64_t t128 = (int64_t)((m + 127) / 128) * ((n + 127) / 128) * batch * ksplit;
+    bool big = (t128 >= 256) && m >= 128 && n >= 128;
+    if (precision == 1) {
+        if (big) launch_tile<128, 128, 1>(st, ta, tb, g);
+        else launch_tile<64, 64, 1>(st, ta, tb, g);
+    } else {
+        if (big) launch_tile<128, 128, 0>(st, ta, tb, g);
+        else launch_tile<64, 64, 0>(st, ta, tb, g);
+    }
+    if (ksplit > 1) {
+        int64_t total = (int64_t)m * n;
+        int nb = (int)((total + 255) / 256);
+        if (nb > 2048) nb = 2048;
+        hipLaunchKernelGGL(gemm_splitk_reduce, dim3(nb, batch), dim3(256), 0, st, g);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        fprintf(stderr, "nchip_gemm: launch failed: %s\n", hipGetErrorString(e));
+        return -2;
+    }
+    return 0;
+}
+
+extern "C" int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                          const float *A, int64_t lda, int64_t stride_a,
+                          const float *B, int64_t ldb, int64_t stride_b,
+                          float beta, float *C, int64_t ldc, int64_t stride_c, int batch,
+                          const float *bias, int act, float *pre, int precision,
+                          int ksplit, float *workspace)
+{
+    return nchip_gemm2(stream, ta, tb, m, n, k, alpha, A, lda, stride_a, 0, B, ldb, stride_b, 0,
+                       beta, C, ldc, stride_c, 0, batch, 1, bias, act, pre, precision, ksplit,
+                       workspace);
+}

@@ -1,0 +1,75 @@
+// Launchers of the small data-movement / element-wise kernels used by the
+// libnc front end (k_elementwise.hip).  All enqueue on `st` and return nothing;
+// argument checking is done by the callers in nc_ops.cpp.
+#ifndef K_INTERNAL_H
+#define K_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define K_MAX_DIMS 8
+
+// n-d descriptor: iterate over dims[], reading with stride sa/sb (0 = broadcast)
+struct NdDesc {
+    int nd;
+    int64_t dims[K_MAX_DIMS];
+    int64_t sa[K_MAX_DIMS];
+    int64_t sb[K_MAX_DIMS];
+};
+
+enum KBinOp { KB_ADD = 0, KB_MUL = 1 };
+enum KUnOp { KU_SIGMOID = 0, KU_TANH, KU_RELU, KU_GELU };
+
+extern "C" {
+// dst (strides d.sb) = src (strides d.sa); esize in {1,2,4}
+void k_copy_nd(hipStream_t st, const void *src, void *dst, const NdDesc *d, int esize);
+// i32/i8/u16 -> f32 style conversions are not needed on the device path
+void k_fill_f32(hipStream_t st, float *p, float v, int64_t n);
+void k_fill_bytes(hipStream_t st, void *p, int v, int64_t nbytes);
+// y[i] = a[i] op b[i % nb]   (b's shape is a prefix of a's)
+void k_binary_prefix(hipStream_t st, int op, const float *a, const float *b, float *y,
+                     int64_t n, int64_t nb);
+// general broadcast: y contiguous over d.dims, a strides d.sa, b strides d.sb
+void k_binary_nd(hipStream_t st, int op, const float *a, const float *b, float *y,
+                 const NdDesc *d, int64_t n);
+// y = mask[i % nm] (xor inv) ? c : x ;  backward: (mask ? 0 : g)
+void k_masked_fill(hipStream_t st, const float *x, const int8_t *mask, float *y,
+                   int64_t n, int64_t nm, float c, int inv);
+void k_unary_fwd(hipStream_t st, int op, const float *x, float *y, int64_t n);
+void k_unary_bwd(hipStream_t st, int op, const float *x, const float *g, float *dx, int64_t n);
+// gated_swish: y = g*x*sigmoid(beta x); bwd writes dg, dx
+void k_gated_swish_fwd(hipStream_t st, const float *g, const float *x, float *y, int64_t n, float beta);
+void k_gated_swish_bwd(hipStream_t st, const float *g, const float *x, const float *gy,
+                       float *dg, float *dx, int64_t n, float beta);
+void k_lerp_fwd(hipStream_t st, const float *a, const float *b, const float *t, float *y, int64_t n);
+void k_lerp_bwd(hipStream_t st, const float *a, const float *b, const float *t, const float *g,
+                float *da, float *db, float *dt, int64_t n);
+void k_lstm_clamped_fwd(hipStream_t st, const float *cp, const float *in, const float *fg,
+                        const float *ig, float *y, int64_t n);
+void k_lstm_clamped_bwd(hipStream_t st, const float *cp, const float *in, const float *fg,
+                        const float *ig, const float *g, float *dcp, float *din, float *dfg,
+                        float *dig, int64_t n);
+// y = a * b * ... helpers for backward of mul: t = g * other[i % nb]
+// (k_binary_prefix with KB_MUL covers it)
+
+// out[i] = sum_o x[i + o*inner], o < outer, fixed order; tmp: nsplit*inner floats
+int k_reduce_trailing_nsplit(int64_t inner, int64_t outer);
+void k_reduce_trailing(hipStream_t st, const float *x, const float *y0, float *out, float *tmp,
+                       int64_t inner, int64_t outer);
+// out[0] = sum of all n elements (fixed tree); tmp: 1024 floats
+void k_reduce_all(hipStream_t st, const float *x, float *out, float *tmp, int64_t n);
+// general un-broadcast: out (numel nout, dims d.dims with strides d.sb over the
+// REDUCED iteration) -- slow fallback, one thread per output element
+void k_unbroadcast_nd(hipStream_t st, const float *g, float *out, const NdDesc *keep,
+                      const NdDesc *red, int64_t nout, int64_t nred);
+// y[j,i,o] = x[j - (pos + i*mult), i, o] or 0  (adjoint: + instead of -)
+void k_rel_shift(hipStream_t st, const float *x, float *y, int64_t n0, int64_t n1,
+                 int64_t outer, int64_t pos, int64_t mult, int adjoint);
+// axis-0 pad/trim as in nc_pad; adjoint = backward (x gets the gradient)
+void k_pad(hipStream_t st, const float *x, float *y, int64_t n_in, int64_t cols,
+           int64_t left, int lop, int64_t right, int rop);
+void k_pad_bwd(hipStream_t st, const float *gy, float *gx, int64_t n_in, int64_t cols,
+               int64_t left, int lop, int64_t right, int rop);
+}
+
+#endif

@@ -1,0 +1,320 @@
+// Bandwidth-bound column kernels: LayerNorm/RMSNorm, softmax, log-likelihood,
+// embedding gather / scatter-add, optimiser step.  One 64-lane wavefront owns
+// one column (libnc axis 0) and reduces with xor-shuffles, so every lane ends
+// with the same, order-fixed sum; cross-column reductions (dw, db of the norm
+// affine, embedding gradient) are two-stage or sequential and use no atomics.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include "../../include/nchip_kernels.h"
+
+namespace {
+
+constexpr int TPB = 256;
+constexpr int WPB = TPB / 64; // wavefronts (columns) per block
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+__global__ __launch_bounds__(TPB) void norm_fwd_kernel(const float *x, const float *w, const float *b,
+                                                       float *y, float *xhat, float *rstd,
+                                                       int d, int64_t n, float eps, int avg)
+{
+    int lane = threadIdx.x & 63;
+    int64_t c = (int64_t)blockIdx.x * WPB + (threadIdx.x >> 6);
+    if (c >= n) return;
+    const float *xc = x + c * d;
+    float s = 0.0f;
+    for (int i = lane; i < d; i += 64) s += xc[i];
+    float mean = avg ? wave_sum(s) / (float)d : 0.0f;
+    float v = 0.0f;
+    for (int i = lane; i < d; i += 64) { float t = xc[i] - mean; v += t * t; }
+    float r = 1.0f / sqrtf(wave_sum(v) / (float)d + eps);
+    if (lane == 0) rstd[c] = r;
+    for (int i = lane; i < d; i += 64) {
+        float h = (xc[i] - mean) * r;
+        if (xhat) xhat[c * d + i] = h;
+        y[c * d + i] = w ? h * w[i] + b[i] : h;
+    }
+}
+
+// dx = rstd * (gh - mean(gh) - xhat * mean(gh * xhat)),  gh = g * w
+__global__ __launch_bounds__(TPB) void norm_bwd_dx_kernel(const float *g, const float *xhat,
+                                                          const float *rstd, const float *w,
+                                                          float *dx, int d, int64_t n, int avg)
+{
+    int lane = threadIdx.x & 63;
+    int64_t c = (int64_t)blockIdx.x * WPB + (threadIdx.x >> 6);
+    if (c >= n) return;
+    const float *gc = g + c * d, *hc = xhat + c * d;
+    float s1 = 0.0f, s2 = 0.0f;
+    for (int i = lane; i < d; i += 64) {
+        float gh = w ? gc[i] * w[i] : gc[i];
+        s1 += gh;
+        s2 += gh * hc[i];
+    }
+    s1 = avg ? wave_sum(s1) / (float)d : 0.0f;
+    s2 = wave_sum(s2) / (float)d;
+    float r = rstd[c];
+    for (int i = lane; i < d; i += 64) {
+        float gh = w ? gc[i] * w[i] : gc[i];
+        dx[c * d + i] = r * (gh - s1 - hc[i] * s2);
+    }
+}
+
+// partial[s][0][i] = sum_c g*xhat, partial[s][1][i] = sum_c g over slice s of the columns
+__global__ __launch_bounds__(TPB) void norm_bwd_wb_stage1(const float *g, const float *xhat,
+                                                          float *partial, int d, int64_t n, int rows)
+{
+    int i = blockIdx.x * TPB + threadIdx.x;
+    int s = blockIdx.y;
+    if (i >= d) return;
+    int64_t per = (n + rows - 1) / rows, c0 = s * per, c1 = c0 + per < n ? c0 + per : n;
+    float aw = 0.0f, ab = 0.0f;
+    for (int64_t c = c0; c < c1; c++) {
+        float gv = g[c * d + i];
+        aw += gv * xhat[c * d + i];
+        ab += gv;
+    }
+    partial[((int64_t)s * 2) * d + i] = aw;
+    partial[((int64_t)s * 2 + 1) * d + i] = ab;
+}
+
+__global__ void norm_bwd_wb_stage2(const float *partial, float *dw, float *db, int d, int rows)
+{
+    int i = blockIdx.x * TPB + threadIdx.x;
+    if (i >= d) return;
+    float aw = 0.0f, ab = 0.0f;
+    for (int s = 0; s < rows; s++) {
+        aw += partial[((int64_t)s * 2) * d + i];
+        ab += partial[((int64_t)s * 2 + 1) * d + i];
+    }
+    if (dw) dw[i] = aw;
+    if (db) db[i] = ab;
+}
+
+__global__ __launch_bounds__(TPB) void softmax_fwd_kernel(const float *x, float *y, int v, int64_t n)
+{
+    int lane = threadIdx.x & 63;
+    int64_t c = (int64_t)blockIdx.x * WPB + (threadIdx.x >> 6);
+    if (c >= n) return;
+    const float *xc = x + c * v;
+    float *yc = y + c * v;
+    float mx = -INFINITY;
+    for (int i = lane; i < v; i += 64) mx = fmaxf(mx, xc[i]);
+    mx = wave_max(mx);
+    float s = 0.0f;
+    for (int i = lane; i < v; i += 64) {
+        float e = expf(xc[i] - mx);
+        yc[i] = e;
+        s += e;
+    }
+    float inv = 1.0f / wave_sum(s);
+    for (int i = lane; i < v; i += 64) yc[i] *= inv;
+}
+
+__global__ __launch_bounds__(TPB) void softmax_bwd_kernel(const float *y, const float *g, float *dx,
+                                                          int v, int64_t n)
+{
+    int lane = threadIdx.x & 63;
+    int64_t c = (int64_t)blockIdx.x * WPB + (threadIdx.x >> 6);
+    if (c >= n) return;
+    const float *yc = y + c * v, *gc = g + c * v;
+    float s = 0.0f;
+    for (int i = lane; i < v; i += 64) s += gc[i] * yc[i];
+    s = wave_sum(s);
+    for (int i = lane; i < v; i += 64) dx[c * v + i] = yc[i] * (gc[i] - s);
+}
+
+__global__ void indexed_log_kernel(const float *p, const int32_t *idx, float *y, int v, int64_t n)
+{
+    int64_t c = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (c < n) y[c] = logf(p[c * v + idx[c]]);
+}
+
+__global__ void nll_bwd_kernel(const float *p, const int32_t *idx, const float *g, float *dl,
+                               int v, int64_t total, int fused)
+{
+    for (int64_t e = (int64_t)blockIdx.x * TPB + threadIdx.x; e < total; e += (int64_t)gridDim.x * TPB) {
+        int64_t c = e / v;
+        int i = (int)(e % v);
+        float gc = g[c];
+        float r;
+        if (fused) r = gc * ((i == idx[c] ? 1.0f : 0.0f) - p[e]);
+        else r = (i == idx[c]) ? gc / p[e] : 0.0f;
+        dl[e] = r;
+    }
+}
+
+__global__ void get_col_kernel(const float *w, const int32_t *idx, float *y, int d, int64_t total)
+{
+    for (int64_t e = (int64_t)blockIdx.x * TPB + threadIdx.x; e < total; e += (int64_t)gridDim.x * TPB) {
+        int64_t c = e / d;
+        int i = (int)(e % d);
+        y[e] = w[(int64_t)idx[c] * d + i];
+    }
+}
+
+// one block per vocabulary entry; the token loop is sequential so that columns
+// sharing a symbol are added in increasing token order
+__global__ __launch_bounds__(TPB) void add_col_kernel(const float *g, const int32_t *idx, float *dw,
+                                                      int d, int64_t n)
+{
+    int sym = blockIdx.x;
+    for (int i0 = 0; i0 < d; i0 += TPB) {
+        int i = i0 + threadIdx.x;
+        float acc = 0.0f;
+        for (int64_t c = 0; c < n; c++)
+            if (idx[c] == sym && i < d)
+                acc += g[c * d + i];
+        if (i < d) dw[(int64_t)sym * d + i] = acc;
+    }
+}
+
+__global__ void opt_update_kernel(int algo, float *w, float *m, float *v, const float *g, int64_t n,
+                                  float lr, float b1, float b2, float eps, float clip, float c1, float c2)
+{
+    for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (int64_t)gridDim.x * TPB) {
+        float gi = g[i];
+        if (algo == 0) {
+            w[i] -= lr * gi;
+        } else if (algo == 1) {
+            if (clip != 0.0f) gi = fminf(fmaxf(gi, -clip), clip);
+            float mi = b1 * m[i] + (1.0f - b1) * gi;
+            float vi = b2 * v[i] + (1.0f - b2) * gi * gi;
+            m[i] = mi;
+            v[i] = vi;
+            w[i] -= lr * (mi * c1) / (sqrtf(vi * c2) + eps);
+        } else {
+            float vi = b2 * v[i] + (1.0f - b2) * gi * gi;
+            v[i] = vi;
+            w[i] -= lr * gi / (sqrtf(vi) + eps);
+        }
+    }
+}
+
+inline int grid_for(int64_t n, int cap = 8192)
+{
+    int64_t b = (n + TPB - 1) / TPB;
+    return (int)(b > cap ? cap : (b < 1 ? 1 : b));
+}
+
+inline int check(const char *what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        fprintf(stderr, "%s: launch failed: %s\n", what, hipGetErrorString(e));
+        return -2;
+    }
+    return 0;
+}
+
+} // namespace
+
+extern "C" {
+
+int nchip_norm_fwd(void *stream, const float *x, const float *w, const float *b, float *y,
+                   float *xhat, float *rstd, int d, int64_t n, float eps, int avg)
+{
+    if (n <= 0 || d <= 0) return 0;
+    if ((w == nullptr) != (b == nullptr)) { fprintf(stderr, "nchip_norm_fwd: w and b go together\n"); return -1; }
+    hipLaunchKernelGGL(norm_fwd_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, (hipStream_t)stream,
+                       x, w, b, y, xhat, rstd, d, n, eps, avg);
+    return check("nchip_norm_fwd");
+}
+
+int nchip_norm_bwd_partial_rows(int64_t n)
+{
+    int64_t r = n / 16;
+    if (r > 128) r = 128;
+    if (r < 1) r = 1;
+    return (int)r;
+}
+
+int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float *rstd, const float *w,
+                   float *dx, float *dw, float *db, float *partial, int d, int64_t n, int avg)
+{
+    if (n <= 0 || d <= 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    if (dx)
+        hipLaunchKernelGGL(norm_bwd_dx_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, st,
+                           g, xhat, rstd, w, dx, d, n, avg);
+    if (dw || db) {
+        if (!partial) { fprintf(stderr, "nchip_norm_bwd: partial buffer missing\n"); return -1; }
+        int rows = nchip_norm_bwd_partial_rows(n);
+        hipLaunchKernelGGL(norm_bwd_wb_stage1, dim3((d + TPB - 1) / TPB, rows), dim3(TPB), 0, st,
+                           g, xhat, partial, d, n, rows);
+        hipLaunchKernelGGL(norm_bwd_wb_stage2, dim3((d + TPB - 1) / TPB), dim3(TPB), 0, st,
+                           (const float *)partial, dw, db, d, rows);
+    }
+    return check("nchip_norm_bwd");
+}
+
+int nchip_softmax_fwd(void *stream, const float *x, float *y, int v, int64_t n)
+{
+    if (n <= 0 || v <= 0) return 0;
+    hipLaunchKernelGGL(softmax_fwd_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, (hipStream_t)stream, x, y, v, n);
+    return check("nchip_softmax_fwd");
+}
+
+int nchip_softmax_bwd(void *stream, const float *y, const float *g, float *dx, int v, int64_t n)
+{
+    if (n <= 0 || v <= 0) return 0;
+    hipLaunchKernelGGL(softmax_bwd_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, (hipStream_t)stream, y, g, dx, v, n);
+    return check("nchip_softmax_bwd");
+}
+
+int nchip_indexed_log(void *stream, const float *p, const int32_t *idx, float *y, int v, int64_t n)
+{
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(indexed_log_kernel, dim3(grid_for(n, 1 << 20)), dim3(TPB), 0, (hipStream_t)stream, p, idx, y, v, n);
+    return check("nchip_indexed_log");
+}
+
+int nchip_nll_bwd(void *stream, const float *p, const int32_t *idx, const float *g, float *dl,
+                  int v, int64_t n, int fused)
+{
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(nll_bwd_kernel, dim3(grid_for(n * v)), dim3(TPB), 0, (hipStream_t)stream, p, idx, g, dl, v, n * v, fused);
+    return check("nchip_nll_bwd");
+}
+
+int nchip_get_col(void *stream, const float *w, const int32_t *idx, float *y, int d, int v, int64_t n)
+{
+    (void)v;
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(get_col_kernel, dim3(grid_for(n * d)), dim3(TPB), 0, (hipStream_t)stream, w, idx, y, d, n * d);
+    return check("nchip_get_col");
+}
+
+int nchip_add_col(void *stream, const float *g, const int32_t *idx, float *dw, int d, int v, int64_t n)
+{
+    if (v <= 0 || d <= 0) return 0;
+    hipLaunchKernelGGL(add_col_kernel, dim3(v), dim3(TPB), 0, (hipStream_t)stream, g, idx, dw, d, n);
+    return check("nchip_add_col");
+}
+
+int nchip_opt_update(void *stream, int algo, float *w, float *m, float *v, const float *g, int64_t n,
+                     float lr, float beta1, float beta2, float eps, float clip, float c1, float c2)
+{
+    if (n <= 0) return 0;
+    if (algo != 0 && algo != 1 && algo != 16) { fprintf(stderr, "nchip_opt_update: unknown algo %d\n", algo); return -1; }
+    hipLaunchKernelGGL(opt_update_kernel, dim3(grid_for(n)), dim3(TPB), 0, (hipStream_t)stream,
+                       algo, w, m, v, g, n, lr, beta1, beta2, eps, clip, c1, c2);
+    return check("nchip_opt_update");
+}
+
+} // extern "C"

@@ -1,0 +1,126 @@
+// Internal structures of libnc_hip: the libnc-compatible front end over the
+// gfx950 kernels.  Host tensors exist only for staging (token ids, masks,
+// probabilities copied back for the coder); every compute op requires device
+// tensors and aborts otherwise - there is no CPU compute path in this library.
+#ifndef NC_HIP_INTERNAL_H
+#define NC_HIP_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <unordered_map>
+#include <vector>
+#include "../../include/nc_api.h"
+#include "../../include/nc_ext.h"
+#include "../../include/nchip_kernels.h"
+#include "k_internal.h"
+
+#define NC_MAX_SAVED 6
+#define NC_SHAPE_ARGS 5
+
+struct Shape {
+    int nd = 0;
+    size_t d[NC_N_DIMS_MAX] = { 0 };
+};
+
+// size-class caching allocator; a freed block is reusable at once because all
+// work is ordered on one stream
+struct Pool {
+    bool device = false;
+    std::unordered_map<size_t, std::vector<void *>> free_lists;
+    std::vector<void *> all;
+    int64_t bytes = 0;
+    static size_t round_size(size_t n);
+    void *get(size_t n, size_t *cap);
+    void put(void *p, size_t cap);
+    void release_all();
+};
+
+struct NCDevice {
+    NCContext *ctx;
+    bool is_hip;
+};
+
+struct NCContext {
+    int nb_threads;
+    NCDevice cpu, hip;
+    bool hip_ready;
+    hipStream_t stream;
+    Pool dev_pool, host_pool;
+    int matmul_bf16;
+    int64_t launches;
+    int64_t node_seq;
+    int epoch;
+};
+
+struct NCTensorBuffer {
+    int ref;
+    NCDevice *dev;
+    void *ptr;
+    size_t cap;
+};
+
+struct NCTensor {
+    int ref;
+    NCDevice *dev;
+    NCTensorBuffer *buf;
+    size_t off; // in elements
+    NCTypeEnum type;
+    int n_dims;
+    size_t dims[NC_N_DIMS_MAX];
+    size_t strides[NC_N_DIMS_MAX]; // in elements
+    NCNode *node;
+};
+
+enum NCOp {
+    OP_PARAM, OP_ADD, OP_MUL, OP_MASKED_FILL, OP_UNARY, OP_GATED_SWISH, OP_LSTM_CLAMPED,
+    OP_LERP, OP_RESHAPE, OP_REPEAT, OP_REDUCE_SUM, OP_SUM, OP_SLICE, OP_CONCAT, OP_PAD,
+    OP_PERMUTE, OP_MATMUL, OP_GET_COL, OP_SOFT_MAX, OP_INDEXED_LOG, OP_NORM, OP_REL_SHIFT,
+    OP_CONCAT_NODE, OP_ATTN, OP_LINEAR,
+};
+
+struct NCNode {
+    int ref = 1;
+    int op = 0;
+    int n_args = 0;
+    std::vector<NCNode *> parents;
+    NCTensor *saved[NC_MAX_SAVED] = { nullptr };
+    Shape arg_shape[NC_SHAPE_ARGS];
+    int ia[8] = { 0 };
+    float fa[4] = { 0 };
+    std::vector<size_t> sizes;
+    void *opaque = nullptr;
+    NCContext *ctx = nullptr;
+    // backward-walk state
+    NCTensor *grad = nullptr;
+    int pending = 0;
+    int mark = 0;
+};
+
+// nc_core.cpp
+[[noreturn]] void nc_fatal(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+void hip_check(hipError_t e, const char *what);
+size_t nc_type_size(NCTypeEnum t);
+size_t nc_numel(const NCTensor *x);
+bool nc_is_contig(const NCTensor *x);
+NCTensor *nc_alloc(NCDevice *d, NCTypeEnum t, int nd, const size_t *dims, bool zero);
+NCTensor *nc_alloc_like(const NCTensor *x);
+NCTensor *nc_view(const NCTensor *x);
+NCTensor *nc_contig(NCTensor *x);                  // consumes
+void nc_copy_any(NCTensor *dst, const NCTensor *src); // strided, same device
+void *nc_data(const NCTensor *x);
+static inline float *nc_f32(const NCTensor *x) { return (float *)nc_data(x); }
+void need_dev(const NCTensor *x, const char *op);
+NCContext *nc_ctx(const NCTensor *x);
+static inline hipStream_t nc_stream(const NCTensor *x) { return x->dev->ctx->stream; }
+float *nc_tmp_f32(NCContext *m, size_t n, size_t *cap); // pool scratch; give back with nc_tmp_free
+void nc_tmp_free(NCContext *m, void *p, size_t cap);
+NCTensor *nc_reshape_view(NCTensor *x, int nd, const size_t *dims); // consumes, no graph
+
+// nc_autodiff.cpp
+NCNode *nc_new_node(NCContext *m, int op, int n_args, NCTensor **args);
+NCTensor *nc_finish(NCTensor *y, NCNode *n, NCTensor **args, int n_args);
+void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga); // nc_ops.cpp
+
+#endif

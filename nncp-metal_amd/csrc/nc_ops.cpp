@@ -1,0 +1,1097 @@
+// libnc_hip ops: shape logic, graph recording and the per-op backward, all
+// dispatching to the gfx950 kernels (k_*.hip).  The op list is the one
+// trf_eval / trf_eval_gradient issue (nncp.c:581-1193) plus the fused entry
+// points of nc_ext.h.  Device tensors only: a host tensor reaching a compute op
+// aborts (see need_dev).
+#include <math.h>
+#include "nc_hip_internal.h"
+
+#define LAUNCHED(x) (nc_ctx(x)->launches++)
+
+static NCTensor *new_f32(const NCTensor *like, int nd, const size_t *dims)
+{
+    return nc_alloc(like->dev, NC_TYPE_F32, nd, dims, false);
+}
+
+static void need_f32(const NCTensor *x, const char *op)
+{
+    need_dev(x, op);
+    if (x->type != NC_TYPE_F32) nc_fatal("%s: f32 tensor expected (type %d)", op, (int)x->type);
+}
+
+static void same_numel(const NCTensor *a, const NCTensor *b, const char *op)
+{
+    if (nc_numel(a) != nc_numel(b)) nc_fatal("%s: operands must have the same shape", op);
+}
+
+// ---- broadcasting -----------------------------------------------------------
+struct BPlan {
+    int nd;
+    size_t dims[NC_N_DIMS_MAX], n;
+    NdDesc desc;
+};
+
+static void bplan(BPlan *bp, int na, const size_t *da, int nb, const size_t *db, const char *op)
+{
+    size_t sa = 1, sb = 1;
+    bp->nd = na > nb ? na : nb;
+    bp->n = 1;
+    bp->desc.nd = bp->nd;
+    for (int i = 0; i < bp->nd; i++) {
+        size_t a = i < na ? da[i] : 1, b = i < nb ? db[i] : 1;
+        if (a != b && a != 1 && b != 1)
+            nc_fatal("%s: incompatible shapes on axis %d (%zu vs %zu)", op, i, a, b);
+        bp->dims[i] = a > b ? a : b;
+        bp->desc.dims[i] = (int64_t)bp->dims[i];
+        bp->desc.sa[i] = a == 1 ? 0 : (int64_t)sa;
+        bp->desc.sb[i] = b == 1 ? 0 : (int64_t)sb;
+        sa *= a; sb *= b;
+        bp->n *= bp->dims[i];
+    }
+    if (bp->nd == 0) { bp->desc.nd = 1; bp->desc.dims[0] = 1; bp->desc.sa[0] = bp->desc.sb[0] = 0; }
+}
+
+// b's dims equal the leading dims of the result (trailing 1s allowed)
+static bool is_prefix(const BPlan *bp, int nb, const size_t *db)
+{
+    for (int i = 0; i < nb; i++)
+        if (db[i] != bp->dims[i]) {
+            for (int j = i; j < nb; j++)
+                if (db[j] != 1) return false;
+            break;
+        }
+    return true;
+}
+
+// a op b with broadcasting; operands borrowed and contiguous
+static NCTensor *dev_binary(int op, const NCTensor *a, const NCTensor *b)
+{
+    BPlan bp;
+    bplan(&bp, a->n_dims, a->dims, b->n_dims, b->dims, op == KB_ADD ? "add" : "mul");
+    NCTensor *y = new_f32(a, bp.nd, bp.dims);
+    if (bp.n == 0) return y;
+    if (nc_numel(a) == bp.n && is_prefix(&bp, b->n_dims, b->dims))
+        k_binary_prefix(nc_stream(a), op, nc_f32(a), nc_f32(b), nc_f32(y), (int64_t)bp.n, (int64_t)nc_numel(b));
+    else if (nc_numel(b) == bp.n && is_prefix(&bp, a->n_dims, a->dims))
+        k_binary_prefix(nc_stream(a), op, nc_f32(b), nc_f32(a), nc_f32(y), (int64_t)bp.n, (int64_t)nc_numel(a));
+    else
+        k_binary_nd(nc_stream(a), op, nc_f32(a), nc_f32(b), nc_f32(y), &bp.desc, (int64_t)bp.n);
+    LAUNCHED(a);
+    return y;
+}
+
+// sums g (consumed) down to `target` (each target dim equals g's or is 1/missing)
+static NCTensor *dev_unbroadcast(NCTensor *g, const Shape &target)
+{
+    size_t nt = 1;
+    for (int i = 0; i < target.nd; i++) nt *= target.d[i];
+    if (nt == nc_numel(g)) return nc_reshape_view(g, target.nd, target.d);
+    NCContext *m = nc_ctx(g);
+    g = nc_contig(g);
+    NCTensor *y = nc_alloc(g->dev, NC_TYPE_F32, target.nd, target.d, false);
+    // trailing reduction: target dims are a prefix of g's
+    bool prefix = true;
+    for (int i = 0; i < target.nd && prefix; i++)
+        if (target.d[i] != g->dims[i]) {
+            for (int j = i; j < target.nd; j++)
+                if (target.d[j] != 1) prefix = false;
+            break;
+        }
+    size_t cap;
+    if (nt == 1) {
+        float *tmp = nc_tmp_f32(m, 1024, &cap);
+        k_reduce_all(m->stream, nc_f32(g), nc_f32(y), tmp, (int64_t)nc_numel(g));
+        nc_tmp_free(m, tmp, cap);
+    } else if (prefix) {
+        int64_t inner = (int64_t)nt, outer = (int64_t)(nc_numel(g) / nt);
+        float *tmp = nc_tmp_f32(m, (size_t)k_reduce_trailing_nsplit(inner, outer) * inner, &cap);
+        k_reduce_trailing(m->stream, nc_f32(g), nullptr, nc_f32(y), tmp, inner, outer);
+        nc_tmp_free(m, tmp, cap);
+    } else {
+        // general case: one thread per kept element loops over the reduced axes
+        NdDesc keep, red;
+        keep.nd = red.nd = 0;
+        int64_t stride = 1, nred = 1;
+        for (int i = 0; i < g->n_dims; i++) {
+            size_t td = i < target.nd ? target.d[i] : 1;
+            if (td == g->dims[i]) {
+                keep.dims[keep.nd] = (int64_t)g->dims[i]; keep.sa[keep.nd] = stride; keep.sb[keep.nd] = 0; keep.nd++;
+            } else {
+                red.dims[red.nd] = (int64_t)g->dims[i]; red.sa[red.nd] = stride; red.sb[red.nd] = 0; red.nd++;
+                nred *= (int64_t)g->dims[i];
+            }
+            stride *= (int64_t)g->dims[i];
+        }
+        if (keep.nd == 0) { keep.nd = 1; keep.dims[0] = 1; keep.sa[0] = keep.sb[0] = 0; }
+        if (red.nd == 0) { red.nd = 1; red.dims[0] = 1; red.sa[0] = red.sb[0] = 0; }
+        k_unbroadcast_nd(m->stream, nc_f32(g), nc_f32(y), &keep, &red, (int64_t)nt, nred);
+    }
+    m->launches++;
+    nc_free_tensor(g);
+    return y;
+}
+
+static NCTensor *binary_op(NCTensor *a, NCTensor *b, int kop, int op)
+{
+    a = nc_contig(a); b = nc_contig(b);
+    need_f32(a, "binary op"); need_f32(b, "binary op");
+    NCTensor *y = dev_binary(kop, a, b);
+    NCTensor *args[2] = { a, b };
+    NCNode *n = nc_new_node(nc_ctx(a), op, 2, args);
+    if (op == OP_MUL && (a->node || b->node)) {
+        n->saved[0] = nc_view(a);
+        n->saved[1] = nc_view(b);
+    }
+    y = nc_finish(y, n, args, 2);
+    nc_free_tensor(a); nc_free_tensor(b);
+    return y;
+}
+
+extern "C" NCTensor *nc_add(NCTensor *x1, NCTensor *x2) { return binary_op(x1, x2, KB_ADD, OP_ADD); } // libnc.h:232
+extern "C" NCTensor *nc_mul(NCTensor *x1, NCTensor *x2) { return binary_op(x1, x2, KB_MUL, OP_MUL); } // libnc.h:235
+
+// libnc.h:231: storage stays fp32 in this library (the bf16 variant rounds
+// inside the matmul), so only identity conversions exist
+extern "C" NCTensor *nc_convert(NCTensor *x, NCTypeEnum new_type)
+{
+    if (x->type == new_type) return x;
+    nc_fatal("nc_convert %d -> %d: only fp32 storage is supported; for bf16 matrix math use "
+             "nc_set_matmul_bf16() or NCHIP_MATMUL_BF16=1", (int)x->type, (int)new_type);
+}
+
+// libnc.h:242-244; the mask (K,T) or (K,1) is a prefix of x (K,T,H,B)
+extern "C" NCTensor *nc_masked_fill(NCTensor *x, NCTensor *mask, float c, BOOL mask_inv)
+{
+    x = nc_contig(x); mask = nc_contig(mask);
+    need_f32(x, "nc_masked_fill"); need_dev(mask, "nc_masked_fill");
+    if (mask->type != NC_TYPE_I8) nc_fatal("nc_masked_fill: i8 mask expected");
+    BPlan bp;
+    bplan(&bp, x->n_dims, x->dims, mask->n_dims, mask->dims, "masked_fill");
+    if (bp.n != nc_numel(x) || !is_prefix(&bp, mask->n_dims, mask->dims))
+        nc_fatal("nc_masked_fill: the mask must match the leading axes of x");
+    NCTensor *y = nc_alloc_like(x);
+    k_masked_fill(nc_stream(x), nc_f32(x), (const int8_t *)nc_data(mask), nc_f32(y),
+                  (int64_t)bp.n, (int64_t)nc_numel(mask), c, mask_inv != 0);
+    LAUNCHED(x);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_MASKED_FILL, 1, args);
+    n->saved[0] = nc_view(mask);
+    n->ia[0] = mask_inv != 0;
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x); nc_free_tensor(mask);
+    return y;
+}
+
+static NCTensor *unary_op(NCTensor *x, int kop)
+{
+    x = nc_contig(x);
+    need_f32(x, "activation");
+    NCTensor *y = nc_alloc_like(x);
+    k_unary_fwd(nc_stream(x), kop, nc_f32(x), nc_f32(y), (int64_t)nc_numel(x));
+    LAUNCHED(x);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_UNARY, 1, args);
+    n->ia[0] = kop;
+    if (x->node) n->saved[0] = nc_view(x);
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
+extern "C" NCTensor *nc_sigmoid(NCTensor *x) { return unary_op(x, KU_SIGMOID); } // libnc.h:245
+extern "C" NCTensor *nc_tanh(NCTensor *x) { return unary_op(x, KU_TANH); }       // libnc.h:246
+extern "C" NCTensor *nc_relu(NCTensor *x) { return unary_op(x, KU_RELU); }       // libnc.h:247
+extern "C" NCTensor *nc_gelu(NCTensor *x) { return unary_op(x, KU_GELU); }       // libnc.h:252 (tanh form)
+
+extern "C" NCTensor *nc_gated_swish(NCTensor *g, NCTensor *x, float beta) // libnc.h:249-251
+{
+    g = nc_contig(g); x = nc_contig(x);
+    need_f32(g, "nc_gated_swish"); need_f32(x, "nc_gated_swish");
+    same_numel(g, x, "nc_gated_swish");
+    NCTensor *y = nc_alloc_like(x);
+    k_gated_swish_fwd(nc_stream(x), nc_f32(g), nc_f32(x), nc_f32(y), (int64_t)nc_numel(x), beta);
+    LAUNCHED(x);
+    NCTensor *args[2] = { g, x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_GATED_SWISH, 2, args);
+    n->saved[0] = nc_view(g); n->saved[1] = nc_view(x);
+    n->fa[0] = beta;
+    y = nc_finish(y, n, args, 2);
+    nc_free_tensor(g); nc_free_tensor(x);
+    return y;
+}
+
+extern "C" NCTensor *nc_lstm_clamped(NCTensor *cp, NCTensor *in, NCTensor *fg, NCTensor *ig) // libnc.h:261-263
+{
+    NCTensor *args[4] = { nc_contig(cp), nc_contig(in), nc_contig(fg), nc_contig(ig) };
+    for (int i = 0; i < 4; i++) { need_f32(args[i], "nc_lstm_clamped"); same_numel(args[0], args[i], "nc_lstm_clamped"); }
+    NCTensor *y = nc_alloc_like(args[0]);
+    k_lstm_clamped_fwd(nc_stream(y), nc_f32(args[0]), nc_f32(args[1]), nc_f32(args[2]), nc_f32(args[3]),
+                       nc_f32(y), (int64_t)nc_numel(y));
+    LAUNCHED(y);
+    NCNode *n = nc_new_node(nc_ctx(y), OP_LSTM_CLAMPED, 4, args);
+    for (int i = 0; i < 4; i++) n->saved[i] = nc_view(args[i]);
+    y = nc_finish(y, n, args, 4);
+    for (int i = 0; i < 4; i++) nc_free_tensor(args[i]);
+    return y;
+}
+
+extern "C" NCTensor *nc_lerp(NCTensor *a, NCTensor *b, NCTensor *t) // libnc.h:272-273
+{
+    NCTensor *args[3] = { nc_contig(a), nc_contig(b), nc_contig(t) };
+    for (int i = 0; i < 3; i++) { need_f32(args[i], "nc_lerp"); same_numel(args[0], args[i], "nc_lerp"); }
+    NCTensor *y = nc_alloc_like(args[0]);
+    k_lerp_fwd(nc_stream(y), nc_f32(args[0]), nc_f32(args[1]), nc_f32(args[2]), nc_f32(y), (int64_t)nc_numel(y));
+    LAUNCHED(y);
+    NCNode *n = nc_new_node(nc_ctx(y), OP_LERP, 3, args);
+    for (int i = 0; i < 3; i++) n->saved[i] = nc_view(args[i]);
+    y = nc_finish(y, n, args, 3);
+    for (int i = 0; i < 3; i++) nc_free_tensor(args[i]);
+    return y;
+}
+
+// ---- shape ops --------------------------------------------------------------
+static NCTensor *reshape_nd(NCTensor *x, int nd, const size_t *dims)
+{
+    x = nc_contig(x);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_RESHAPE, 1, args);
+    NCTensor *y = nc_reshape_view(nc_dup_tensor(x), nd, dims);
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
+extern "C" NCTensor *nc_reshape_1d(NCTensor *x, size_t n0) { size_t d[1] = { n0 }; return reshape_nd(x, 1, d); }
+extern "C" NCTensor *nc_reshape_2d(NCTensor *x, size_t n0, size_t n1) { size_t d[2] = { n0, n1 }; return reshape_nd(x, 2, d); }
+extern "C" NCTensor *nc_reshape_3d(NCTensor *x, size_t n0, size_t n1, size_t n2) { size_t d[3] = { n0, n1, n2 }; return reshape_nd(x, 3, d); }
+extern "C" NCTensor *nc_reshape_4d(NCTensor *x, size_t n0, size_t n1, size_t n2, size_t n3) { size_t d[4] = { n0, n1, n2, n3 }; return reshape_nd(x, 4, d); }
+
+// libnc.h:289-292: duplicate along new trailing axes (stride-0 source copy)
+static NCTensor *repeat_raw(const NCTensor *x, int nr, const size_t *rd)
+{
+    size_t dims[NC_N_DIMS_MAX];
+    if (x->n_dims + nr > NC_N_DIMS_MAX) nc_fatal("repeat: too many axes");
+    memcpy(dims, x->dims, sizeof(size_t) * x->n_dims);
+    for (int i = 0; i < nr; i++) dims[x->n_dims + i] = rd[i];
+    NCTensor *y = nc_alloc(x->dev, x->type, x->n_dims + nr, dims, false);
+    NCTensor *v = nc_view(x);
+    v->n_dims = x->n_dims + nr;
+    for (int i = 0; i < nr; i++) { v->dims[x->n_dims + i] = rd[i]; v->strides[x->n_dims + i] = 0; }
+    nc_copy_any(y, v);
+    nc_free_tensor(v);
+    return y;
+}
+
+static NCTensor *repeat_nd(NCTensor *x, int nr, const size_t *rd)
+{
+    x = nc_contig(x);
+    need_dev(x, "nc_repeat");
+    NCTensor *y = repeat_raw(x, nr, rd);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_REPEAT, 1, args);
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
+extern "C" NCTensor *nc_repeat_1d(NCTensor *x, size_t n0) { size_t d[1] = { n0 }; return repeat_nd(x, 1, d); }
+extern "C" NCTensor *nc_repeat_2d(NCTensor *x, size_t n0, size_t n1) { size_t d[2] = { n0, n1 }; return repeat_nd(x, 2, d); }
+
+// libnc.h:293-295: y0 + sum over the axes >= n_dims
+extern "C" NCTensor *nc_reduce_sum(NCTensor *y0, NCTensor *x, int n_dims)
+{
+    x = nc_contig(x);
+    need_f32(x, "nc_reduce_sum");
+    if (y0) { y0 = nc_contig(y0); need_f32(y0, "nc_reduce_sum"); }
+    NCContext *m = nc_ctx(x);
+    int64_t inner = 1;
+    for (int i = 0; i < n_dims; i++) inner *= (int64_t)x->dims[i];
+    int64_t outer = (int64_t)nc_numel(x) / inner;
+    if (y0 && (int64_t)nc_numel(y0) != inner) nc_fatal("nc_reduce_sum: y0 shape mismatch");
+    NCTensor *y = new_f32(x, n_dims, x->dims);
+    size_t cap;
+    float *tmp = nc_tmp_f32(m, (size_t)k_reduce_trailing_nsplit(inner, outer) * inner, &cap);
+    k_reduce_trailing(m->stream, nc_f32(x), y0 ? nc_f32(y0) : nullptr, nc_f32(y), tmp, inner, outer);
+    nc_tmp_free(m, tmp, cap);
+    m->launches += 2;
+    NCTensor *args[2] = { y0, x };
+    NCNode *n = nc_new_node(m, OP_REDUCE_SUM, 2, args);
+    y = nc_finish(y, n, args, 2);
+    nc_free_tensor(y0); nc_free_tensor(x);
+    return y;
+}
+
+extern "C" NCTensor *nc_sum(NCTensor *x) // libnc.h:298-299
+{
+    x = nc_contig(x);
+    need_f32(x, "nc_sum");
+    NCContext *m = nc_ctx(x);
+    NCTensor *y = nc_alloc(x->dev, NC_TYPE_F32, 0, nullptr, false);
+    size_t cap;
+    float *tmp = nc_tmp_f32(m, 1024, &cap);
+    k_reduce_all(m->stream, nc_f32(x), nc_f32(y), tmp, (int64_t)nc_numel(x));
+    nc_tmp_free(m, tmp, cap);
+    m->launches += 2;
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(m, OP_SUM, 1, args);
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
+// libnc.h:306-307: alias sharing storage, no graph; writing through it with
+// nc_tensor_copy mutates the parent (nncp.c:650-657, 697-702)
+extern "C" NCTensor *nc_slice_alias(const NCTensor *x, int axis, size_t start, size_t end)
+{
+    if (axis < 0 || axis >= x->n_dims || end > x->dims[axis] || start > end)
+        nc_fatal("nc_slice_alias: range [%zu,%zu) outside axis %d", start, end, axis);
+    NCTensor *y = nc_view(x);
+    y->off += start * x->strides[axis];
+    y->dims[axis] = end - start;
+    return y;
+}
+
+extern "C" NCTensor *nc_slice(NCTensor *x, int axis, size_t start, size_t end) // libnc.h:308
+{
+    NCTensor *v = nc_slice_alias(x, axis, start, end);
+    NCTensor *y = nc_alloc(x->dev, x->type, v->n_dims, v->dims, false);
+    nc_copy_any(y, v);
+    nc_free_tensor(v);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_SLICE, 1, args);
+    n->ia[0] = axis; n->ia[1] = (int)start;
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
+extern "C" NCTensor *nc_concat(NCTensor **inputs, int n_inputs, int axis) // libnc.h:310-311
+{
+    int nd = inputs[0]->n_dims;
+    size_t dims[NC_N_DIMS_MAX], total = 0, pos = 0;
+    if (axis < 0 || axis >= nd) nc_fatal("nc_concat: axis %d out of range", axis);
+    memcpy(dims, inputs[0]->dims, sizeof(size_t) * nd);
+    for (int i = 0; i < n_inputs; i++) {
+        if (inputs[i]->n_dims != nd) nc_fatal("nc_concat: rank mismatch");
+        for (int a = 0; a < nd; a++)
+            if (a != axis && inputs[i]->dims[a] != dims[a]) nc_fatal("nc_concat: shape mismatch on axis %d", a);
+        total += inputs[i]->dims[axis];
+    }
+    dims[axis] = total;
+    NCTensor *y = nc_alloc(inputs[0]->dev, inputs[0]->type, nd, dims, false);
+    NCNode *n = nc_new_node(nc_ctx(y), OP_CONCAT, n_inputs, nullptr);
+    n->ia[0] = axis;
+    for (int i = 0; i < n_inputs; i++) {
+        NCTensor *v = nc_slice_alias(y, axis, pos, pos + inputs[i]->dims[axis]);
+        nc_copy_any(v, inputs[i]);
+        nc_free_tensor(v);
+        n->sizes.push_back(inputs[i]->dims[axis]);
+        n->parents[i] = nc_dup_node(inputs[i]->node);
+        pos += inputs[i]->dims[axis];
+    }
+    y = nc_finish(y, n, inputs, n_inputs);
+    for (int i = 0; i < n_inputs; i++) nc_free_tensor(inputs[i]);
+    return y;
+}
+
+extern "C" NCTensor *nc_vconcat(NCTensor **inputs, int n) { return nc_concat(inputs, n, 0); } // libnc.h:315
+extern "C" NCTensor *nc_hconcat(NCTensor **inputs, int n) { return nc_concat(inputs, n, 1); } // libnc.h:317
+
+extern "C" void nc_split(NCTensor **tab_y, NCTensor *x, int n_outputs, const size_t *tab_size, int axis) // libnc.h:318-320
+{
+    size_t pos = 0;
+    for (int i = 0; i < n_outputs; i++) {
+        size_t sz = tab_size ? tab_size[i] : x->dims[axis] / n_outputs;
+        tab_y[i] = nc_slice(nc_dup_tensor(x), axis, pos, pos + sz);
+        pos += sz;
+    }
+    nc_free_tensor(x);
+}
+
+// libnc.h:325-335 (nncp.c:777 left-pads w_r^T q from d_pos to K rows)
+extern "C" NCTensor *nc_pad(NCTensor *x, ssize_t left_len, NCPadEnum left_op, ssize_t right_len, NCPadEnum right_op)
+{
+    x = nc_contig(x);
+    need_f32(x, "nc_pad");
+    size_t dims[NC_N_DIMS_MAX];
+    memcpy(dims, x->dims, sizeof(size_t) * x->n_dims);
+    ssize_t n_out = (ssize_t)dims[0] + left_len + right_len;
+    if (x->n_dims < 1 || n_out <= 0) nc_fatal("nc_pad: empty result");
+    dims[0] = (size_t)n_out;
+    NCTensor *y = new_f32(x, x->n_dims, dims);
+    k_pad(nc_stream(x), nc_f32(x), nc_f32(y), (int64_t)x->dims[0], (int64_t)(nc_numel(x) / x->dims[0]),
+          left_len, left_op, right_len, right_op);
+    LAUNCHED(x);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_PAD, 1, args);
+    n->ia[0] = (int)left_len; n->ia[1] = left_op; n->ia[2] = (int)right_len; n->ia[3] = right_op;
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
+// libnc.h:353-360: result axis i is x axis axis[i], made contiguous
+static NCTensor *permute_raw(const NCTensor *x, int nd, const int *axis)
+{
+    if (nd != x->n_dims) nc_fatal("nc_permute: rank mismatch");
+    NCTensor *v = nc_view(x);
+    for (int i = 0; i < nd; i++) { v->dims[i] = x->dims[axis[i]]; v->strides[i] = x->strides[axis[i]]; }
+    NCTensor *y = nc_alloc(x->dev, x->type, nd, v->dims, false);
+    nc_copy_any(y, v);
+    nc_free_tensor(v);
+    return y;
+}
+
+extern "C" NCTensor *nc_permute(NCTensor *x, int n_dims, const int *axis)
+{
+    x = nc_contig(x);
+    need_dev(x, "nc_permute");
+    NCTensor *y = permute_raw(x, n_dims, axis);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_PERMUTE, 1, args);
+    for (int i = 0; i < n_dims; i++) n->ia[i] = axis[i];
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
+extern "C" NCTensor *nc_permute_4d(NCTensor *x, int a0, int a1, int a2, int a3)
+{
+    int axis[4] = { a0, a1, a2, a3 };
+    return nc_permute(x, 4, axis);
+}
+
+// libnc.h:396-397 (see k_rel_shift): y[j,i] = x[j - (pos + i*mult), i]
+extern "C" NCTensor *nc_rel_shift(NCTensor *x, ssize_t pos, ssize_t mult)
+{
+    x = nc_contig(x);
+    need_f32(x, "nc_rel_shift");
+    if (x->n_dims < 2) nc_fatal("nc_rel_shift: at least 2 axes expected");
+    NCTensor *y = nc_alloc_like(x);
+    k_rel_shift(nc_stream(x), nc_f32(x), nc_f32(y), (int64_t)x->dims[0], (int64_t)x->dims[1],
+                (int64_t)(nc_numel(x) / (x->dims[0] * x->dims[1])), pos, mult, 0);
+    LAUNCHED(x);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_REL_SHIFT, 1, args);
+    n->ia[0] = (int)pos; n->ia[1] = (int)mult;
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
+extern "C" NCTensor *nc_cmul(NCTensor *x1, NCTensor *x2, BOOL is_conj, BOOL is_planar)
+{
+    (void)x1; (void)x2; (void)is_conj; (void)is_planar;
+    nc_fatal("nc_cmul (rotary position embedding, nncp.c:764-770) is not supported");
+}
+
+// ---- matmul -----------------------------------------------------------------
+struct MMShape {
+    size_t m, n, k, batch;
+    bool flat;
+};
+
+static MMShape mm_shape(const NCTensor *a, const NCTensor *b, bool ta, bool tb)
+{
+    MMShape s;
+    if (a->n_dims < 2 || b->n_dims < 2) nc_fatal("nc_matmul: operands need at least 2 axes");
+    s.m = ta ? a->dims[1] : a->dims[0];
+    s.k = ta ? a->dims[0] : a->dims[1];
+    s.batch = 1;
+    s.flat = false;
+    size_t kb;
+    if (a->n_dims == 2 && b->n_dims > 2 && !tb) {
+        s.flat = true;
+        kb = b->dims[0];
+        s.n = nc_numel(b) / kb;
+    } else {
+        if (a->n_dims != b->n_dims) nc_fatal("nc_matmul: rank mismatch (%d vs %d)", a->n_dims, b->n_dims);
+        for (int i = 2; i < a->n_dims; i++) {
+            if (a->dims[i] != b->dims[i]) nc_fatal("nc_matmul: batch axis %d mismatch", i);
+            s.batch *= a->dims[i];
+        }
+        kb = tb ? b->dims[1] : b->dims[0];
+        s.n = tb ? b->dims[0] : b->dims[1];
+    }
+    if (s.k != kb) nc_fatal("nc_matmul: inner dimension mismatch (%zu vs %zu)", s.k, kb);
+    return s;
+}
+
+// C (contiguous m x n per batch) = alpha op(A) op(B) + beta C [+ bias, act]
+static void dev_gemm(NCContext *m, bool ta, bool tb, size_t M, size_t N, size_t K, float alpha,
+                     const NCTensor *a, const NCTensor *b, float beta, NCTensor *c, size_t batch,
+                     const float *bias, int act, float *pre)
+{
+    int ks = nchip_gemm_pick_ksplit((int)M, (int)N, (int)K, (int)batch);
+    size_t cap = 0;
+    float *ws = nullptr;
+    if (ks > 1) ws = nc_tmp_f32(m, batch * ks * M * N, &cap);
+    int rc = nchip_gemm(m->stream, ta, tb, (int)M, (int)N, (int)K, alpha,
+                        nc_f32(a), (int64_t)(ta ? K : M), (int64_t)(M * K),
+                        nc_f32(b), (int64_t)(tb ? N : K), (int64_t)(K * N),
+                        beta, nc_f32(c), (int64_t)M, (int64_t)(M * N), (int)batch,
+                        bias, act, pre, m->matmul_bf16, ks, ws);
+    if (ws) nc_tmp_free(m, ws, cap);
+    if (rc) nc_fatal("gemm failed (m=%zu n=%zu k=%zu)", M, N, K);
+    m->launches += ks > 1 ? 2 : 1;
+}
+
+// libnc.h:365-373
+extern "C" NCTensor *nc_matmul_add(NCTensor *a, NCTensor *b, NCTensor *c, BOOL ta, BOOL tb, float alpha)
+{
+    a = nc_contig(a); b = nc_contig(b);
+    need_f32(a, "nc_matmul"); need_f32(b, "nc_matmul");
+    NCContext *m = nc_ctx(a);
+    MMShape s = mm_shape(a, b, ta != 0, tb != 0);
+    size_t dims[NC_N_DIMS_MAX];
+    memcpy(dims, b->dims, sizeof(size_t) * b->n_dims);
+    dims[0] = s.m;
+    if (!s.flat) dims[1] = s.n;
+    NCTensor *y = new_f32(a, b->n_dims, dims);
+    if (c) {
+        c = nc_contig(c);
+        need_f32(c, "nc_matmul_add");
+        if (nc_numel(c) != nc_numel(y)) nc_fatal("nc_matmul_add: addend shape mismatch");
+        hip_check(hipMemcpyAsync(nc_data(y), nc_data(c), nc_numel(y) * sizeof(float),
+                                 hipMemcpyDeviceToDevice, m->stream), "hipMemcpyAsync");
+    }
+    dev_gemm(m, ta != 0, tb != 0, s.m, s.n, s.k, alpha, a, b, c ? 1.0f : 0.0f, y, s.batch, nullptr, 0, nullptr);
+    NCTensor *args[3] = { a, b, c };
+    NCNode *n = nc_new_node(m, OP_MATMUL, 3, args);
+    if (a->node || b->node || (c && c->node)) {
+        n->saved[0] = nc_view(a);
+        n->saved[1] = nc_view(b);
+    }
+    n->ia[0] = ta != 0; n->ia[1] = tb != 0; n->ia[2] = s.flat;
+    n->fa[0] = alpha;
+    y = nc_finish(y, n, args, 3);
+    nc_free_tensor(a); nc_free_tensor(b); nc_free_tensor(c);
+    return y;
+}
+
+extern "C" NCTensor *nc_matmul(NCTensor *w, NCTensor *x) { return nc_matmul_add(w, x, nullptr, 0, 0, 1.0f); }
+
+// gradients of alpha op(A) op(B): the four transposition cases
+static void matmul_bw(NCNode *nd, NCTensor *g, NCTensor **ga, int ia, int ib)
+{
+    NCTensor *a = nd->saved[0], *b = nd->saved[1];
+    if (!a || !b) nc_fatal("matmul backward: arguments were not saved");
+    NCContext *m = nc_ctx(g);
+    bool ta = nd->ia[0], tb = nd->ia[1];
+    float alpha = nd->fa[0];
+    MMShape s = mm_shape(a, b, ta, tb);
+    if (nd->parents[ia]) {
+        NCTensor *da = nc_alloc_like(a);
+        if (!ta) dev_gemm(m, false, !tb, s.m, s.k, s.n, alpha, g, b, 0.0f, da, s.batch, nullptr, 0, nullptr);
+        else     dev_gemm(m, tb, true, s.k, s.m, s.n, alpha, b, g, 0.0f, da, s.batch, nullptr, 0, nullptr);
+        ga[ia] = da;
+    }
+    if (nd->parents[ib]) {
+        NCTensor *db = nc_alloc_like(b);
+        if (!tb) dev_gemm(m, !ta, false, s.k, s.n, s.m, alpha, a, g, 0.0f, db, s.batch, nullptr, 0, nullptr);
+        else     dev_gemm(m, true, ta, s.n, s.k, s.m, alpha, g, a, 0.0f, db, s.batch, nullptr, 0, nullptr);
+        ga[ib] = db;
+    }
+}
+
+// y = act(w x + bias) in one GEMM with a fused epilogue (nc_ext.h)
+extern "C" NCTensor *nc_linear(NCTensor *w, NCTensor *x, NCTensor *bias, int act)
+{
+    w = nc_contig(w); x = nc_contig(x);
+    need_f32(w, "nc_linear"); need_f32(x, "nc_linear");
+    NCContext *m = nc_ctx(w);
+    if (w->n_dims != 2) nc_fatal("nc_linear: w must be (m, k)");
+    MMShape s = mm_shape(w, x, false, false);
+    if (bias) {
+        bias = nc_contig(bias);
+        need_f32(bias, "nc_linear");
+        if (nc_numel(bias) != s.m) nc_fatal("nc_linear: bias must have m = %zu elements", s.m);
+    }
+    size_t dims[NC_N_DIMS_MAX];
+    memcpy(dims, x->dims, sizeof(size_t) * x->n_dims);
+    dims[0] = s.m;
+    NCTensor *y = new_f32(w, x->n_dims, dims);
+    bool graph = w->node || x->node || (bias && bias->node);
+    NCTensor *pre = (act != NC_ACT_NONE && graph) ? nc_alloc_like(y) : nullptr;
+    dev_gemm(m, false, false, s.m, s.n, s.k, 1.0f, w, x, 0.0f, y, 1, bias ? nc_f32(bias) : nullptr, act,
+             pre ? nc_f32(pre) : nullptr);
+    NCTensor *args[3] = { w, x, bias };
+    NCNode *n = nc_new_node(m, OP_LINEAR, 3, args);
+    if (graph) {
+        n->saved[0] = nc_view(w);
+        n->saved[1] = nc_view(x);
+        n->saved[2] = pre;
+        pre = nullptr;
+    }
+    n->ia[0] = 0; n->ia[1] = 0; n->ia[2] = 1; n->ia[3] = act;
+    n->fa[0] = 1.0f;
+    y = nc_finish(y, n, args, 3);
+    nc_free_tensor(pre);
+    nc_free_tensor(w); nc_free_tensor(x); nc_free_tensor(bias);
+    return y;
+}
+
+// ---- embedding, softmax, loss, norms ----------------------------------------
+extern "C" NCTensor *nc_get_col(NCTensor *w, NCTensor *x) // libnc.h:374-375
+{
+    w = nc_contig(w); x = nc_contig(x);
+    need_f32(w, "nc_get_col"); need_dev(x, "nc_get_col");
+    if (x->type != NC_TYPE_I32 || w->n_dims != 2) nc_fatal("nc_get_col: (D,V) f32 matrix and i32 indices expected");
+    size_t dims[2] = { w->dims[0], nc_numel(x) };
+    NCTensor *y = new_f32(w, 2, dims);
+    if (nchip_get_col(nc_stream(w), nc_f32(w), (const int32_t *)nc_data(x), nc_f32(y), (int)dims[0],
+                      (int)w->dims[1], (int64_t)dims[1]))
+        nc_fatal("nc_get_col failed");
+    LAUNCHED(w);
+    NCTensor *args[1] = { w };
+    NCNode *n = nc_new_node(nc_ctx(w), OP_GET_COL, 1, args);
+    n->saved[0] = nc_view(x);
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(w); nc_free_tensor(x);
+    return y;
+}
+
+extern "C" NCTensor *nc_soft_max(NCTensor *x) // libnc.h:382
+{
+    x = nc_contig(x);
+    need_f32(x, "nc_soft_max");
+    NCTensor *y = nc_alloc_like(x);
+    size_t v = x->n_dims ? x->dims[0] : 1;
+    if (nchip_softmax_fwd(nc_stream(x), nc_f32(x), nc_f32(y), (int)v, (int64_t)(nc_numel(x) / v)))
+        nc_fatal("nc_soft_max failed");
+    LAUNCHED(x);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_SOFT_MAX, 1, args);
+    if (x->node) n->saved[0] = nc_view(y);
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
+// libnc.h:385-388; straight after nc_soft_max the gradient goes to the logits
+// as g*(onehot - p)
+extern "C" NCTensor *nc_indexed_log(NCTensor *x, NCTensor *eout)
+{
+    x = nc_contig(x); eout = nc_contig(eout);
+    need_f32(x, "nc_indexed_log"); need_dev(eout, "nc_indexed_log");
+    if (eout->type != NC_TYPE_I32) nc_fatal("nc_indexed_log: i32 indices expected");
+    size_t v = x->dims[0], cols = nc_numel(x) / v;
+    if (nc_numel(eout) != cols) nc_fatal("nc_indexed_log: %zu indices for %zu columns", nc_numel(eout), cols);
+    NCTensor *y = new_f32(x, x->n_dims - 1, x->dims + 1);
+    if (nchip_indexed_log(nc_stream(x), nc_f32(x), (const int32_t *)nc_data(eout), nc_f32(y), (int)v, (int64_t)cols))
+        nc_fatal("nc_indexed_log failed");
+    LAUNCHED(x);
+    NCTensor *args[1] = { x };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_INDEXED_LOG, 1, args);
+    if (x->node) {
+        n->saved[0] = nc_view(x);
+        n->saved[1] = nc_view(eout);
+        if (x->node->op == OP_SOFT_MAX && x->node->parents[0]) {
+            nc_free_node(n->parents[0]);
+            n->parents[0] = nc_dup_node(x->node->parents[0]);
+            n->ia[0] = 1;
+        }
+    }
+    y = nc_finish(y, n, args, 1);
+    nc_free_tensor(x); nc_free_tensor(eout);
+    return y;
+}
+
+// libnc.h:389-395
+static NCTensor *norm_op(NCTensor *x, NCTensor *w, NCTensor *b, float eps, int avg)
+{
+    x = nc_contig(x);
+    need_f32(x, "layer norm");
+    if (w) { w = nc_contig(w); b = nc_contig(b); need_f32(w, "layer norm"); need_f32(b, "layer norm"); }
+    size_t d = x->dims[0], cols = nc_numel(x) / d;
+    if (w && (nc_numel(w) != d || nc_numel(b) != d)) nc_fatal("layer norm: affine parameters must have %zu elements", d);
+    NCTensor *y = nc_alloc_like(x);
+    NCTensor *xhat = w ? nc_alloc_like(x) : nc_dup_tensor(y);
+    NCTensor *rstd = nc_alloc(x->dev, NC_TYPE_F32, 1, &cols, false);
+    if (nchip_norm_fwd(nc_stream(x), nc_f32(x), w ? nc_f32(w) : nullptr, b ? nc_f32(b) : nullptr, nc_f32(y),
+                       nc_f32(xhat), nc_f32(rstd), (int)d, (int64_t)cols, eps, avg))
+        nc_fatal("layer norm failed");
+    LAUNCHED(x);
+    NCTensor *args[3] = { x, w, b };
+    NCNode *n = nc_new_node(nc_ctx(x), OP_NORM, 3, args);
+    if (x->node || (w && (w->node || b->node))) {
+        n->saved[0] = nc_view(xhat);
+        n->saved[1] = nc_view(rstd);
+        if (w) n->saved[2] = nc_view(w);
+    }
+    n->ia[0] = avg;
+    y = nc_finish(y, n, args, 3);
+    nc_free_tensor(xhat); nc_free_tensor(rstd);
+    nc_free_tensor(x); nc_free_tensor(w); nc_free_tensor(b);
+    return y;
+}
+
+extern "C" NCTensor *nc_layer_norm(NCTensor *x, float eps) { return norm_op(x, nullptr, nullptr, eps, 1); }
+extern "C" NCTensor *nc_rms_norm(NCTensor *x, float eps) { return norm_op(x, nullptr, nullptr, eps, 0); }
+
+extern "C" NCTensor *nc_fused_layer_norm(NCTensor *x, NCTensor *w, NCTensor *b, float eps, BOOL avg_flag)
+{
+    if ((w == nullptr) != (b == nullptr)) nc_fatal("nc_fused_layer_norm: w and b go together");
+    return norm_op(x, w, b, eps, avg_flag != 0);
+}
+
+// ---- fused attention (nc_ext.h) ---------------------------------------------
+struct AttnDims {
+    int H, dk, dv, B, T, M, K, d_pos;
+};
+
+static AttnDims attn_dims(const NCTensor *q, const NCTensor *kv, const NCTensor *kvm,
+                          const NCTensor *w_r, const NCTensor *b_r, int n_head, int d_key)
+{
+    AttnDims a;
+    if (q->n_dims != 3 || kv->n_dims != 3) nc_fatal("nc_relpos_attention: q and kv must be (features, B, T)");
+    a.H = n_head; a.dk = d_key;
+    a.B = (int)q->dims[1]; a.T = (int)q->dims[2];
+    a.M = kvm ? (int)kvm->dims[2] : 0;
+    a.K = a.M + a.T;
+    if ((int)q->dims[0] != n_head * d_key || kv->dims[1] != q->dims[1] || kv->dims[2] != q->dims[2])
+        nc_fatal("nc_relpos_attention: q/kv shape mismatch");
+    if (kv->dims[0] <= q->dims[0] || (kv->dims[0] - q->dims[0]) % n_head)
+        nc_fatal("nc_relpos_attention: kv must hold H*dk key rows then H*dv value rows");
+    a.dv = (int)(kv->dims[0] - q->dims[0]) / n_head;
+    if (kvm && (kvm->n_dims != 3 || kvm->dims[0] != kv->dims[0] || kvm->dims[1] != kv->dims[1]))
+        nc_fatal("nc_relpos_attention: kv_mem shape mismatch");
+    a.d_pos = 1;
+    if (w_r) {
+        if (w_r->n_dims != 3 || (int)w_r->dims[0] != d_key || (int)w_r->dims[2] != n_head)
+            nc_fatal("nc_relpos_attention: w_r must be (dk, d_pos, H)");
+        a.d_pos = (int)w_r->dims[1];
+        if (a.d_pos > a.K) nc_fatal("nc_relpos_attention: d_pos > K is not supported");
+    }
+    if (b_r && (b_r->n_dims != 2 || (int)b_r->dims[0] != a.K || (int)b_r->dims[1] != n_head))
+        nc_fatal("nc_relpos_attention: b_r must be (K, H)");
+    return a;
+}
+
+extern "C" NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv_mem, NCTensor *w_r,
+                                         NCTensor *b_r, int n_head, int d_key, int attn_len,
+                                         float b_r_scale)
+{
+    NCTensor *all[5] = { nc_contig(q), nc_contig(kv), kv_mem ? nc_contig(kv_mem) : nullptr,
+                         w_r ? nc_contig(w_r) : nullptr, b_r ? nc_contig(b_r) : nullptr };
+    for (int i = 0; i < 5; i++)
+        if (all[i]) need_f32(all[i], "nc_relpos_attention");
+    NCContext *m = nc_ctx(all[0]);
+    AttnDims a = attn_dims(all[0], all[1], all[2], all[3], all[4], n_head, d_key);
+    size_t od[3] = { (size_t)a.H * a.dv, (size_t)a.B, (size_t)a.T };
+    size_t pd[4] = { (size_t)a.K, (size_t)a.T, (size_t)a.H, (size_t)a.B };
+    NCTensor *y = new_f32(all[0], 3, od);
+    NCTensor *probs = new_f32(all[0], 4, pd);
+    size_t cap = 0;
+    float *rel = all[3] ? nc_tmp_f32(m, (size_t)a.d_pos * a.T * a.H * a.B, &cap) : nullptr;
+    int rc = nchip_relpos_attn_fwd(m->stream, nc_f32(all[0]), (int64_t)all[0]->dims[0],
+                                   nc_f32(all[1]), all[2] ? nc_f32(all[2]) : nullptr, (int64_t)all[1]->dims[0],
+                                   all[3] ? nc_f32(all[3]) : nullptr, all[4] ? nc_f32(all[4]) : nullptr,
+                                   nc_f32(y), (int64_t)od[0], nc_f32(probs), rel,
+                                   a.H, a.dk, a.dv, a.B, a.T, a.M, a.d_pos, attn_len, b_r_scale,
+                                   m->matmul_bf16);
+    if (rel) nc_tmp_free(m, rel, cap);
+    if (rc) nc_fatal("nc_relpos_attention: kernel rejected the shapes");
+    m->launches += 6;
+    NCNode *n = nc_new_node(m, OP_ATTN, 5, all);
+    bool graph = false;
+    for (int i = 0; i < 5; i++)
+        if (all[i] && all[i]->node) graph = true;
+    if (graph) {
+        for (int i = 0; i < 4; i++)
+            if (all[i]) n->saved[i] = nc_view(all[i]);
+        n->saved[4] = probs;
+        probs = nullptr;
+    }
+    n->ia[0] = n_head; n->ia[1] = d_key; n->ia[2] = attn_len;
+    n->ia[3] = all[3] != nullptr; n->ia[4] = all[4] != nullptr;
+    n->fa[0] = b_r_scale;
+    y = nc_finish(y, n, all, 5);
+    nc_free_tensor(probs);
+    for (int i = 0; i < 5; i++) nc_free_tensor(all[i]);
+    return y;
+}
+
+static void attn_bw(NCNode *nd, NCTensor *g, NCTensor **ga)
+{
+    NCTensor *q = nd->saved[0], *kv = nd->saved[1], *kvm = nd->saved[2], *w_r = nd->saved[3];
+    NCTensor *probs = nd->saved[4];
+    NCContext *m = nc_ctx(g);
+    AttnDims a = attn_dims(q, kv, kvm, w_r, nullptr, nd->ia[0], nd->ia[1]);
+    NCTensor *gc = nc_contig(nc_dup_tensor(g));
+    NCTensor *dq = nc_alloc_like(q), *dkv = nc_alloc_like(kv);
+    NCTensor *dkvm = kvm ? nc_alloc_like(kvm) : nullptr;
+    NCTensor *dwr = w_r ? nc_alloc_like(w_r) : nullptr;
+    size_t bd[2] = { (size_t)a.K, (size_t)a.H };
+    NCTensor *dbr = nd->ia[4] ? new_f32(q, 2, bd) : nullptr;
+    size_t cap;
+    float *scratch = nc_tmp_f32(m, nchip_relpos_attn_bwd_scratch(a.H, a.dk, a.B, a.T, a.M, a.d_pos), &cap);
+    int rc = nchip_relpos_attn_bwd(m->stream, nc_f32(q), (int64_t)q->dims[0], nc_f32(kv),
+                                   kvm ? nc_f32(kvm) : nullptr, (int64_t)kv->dims[0],
+                                   w_r ? nc_f32(w_r) : nullptr, nc_f32(probs), nc_f32(gc),
+                                   (int64_t)gc->dims[0], nc_f32(dq), nc_f32(dkv),
+                                   dkvm ? nc_f32(dkvm) : nullptr, dwr ? nc_f32(dwr) : nullptr,
+                                   dbr ? nc_f32(dbr) : nullptr, a.H, a.dk, a.dv, a.B, a.T, a.M, a.d_pos,
+                                   nd->ia[2], nd->fa[0], m->matmul_bf16, scratch);
+    nc_tmp_free(m, scratch, cap);
+    if (rc) nc_fatal("nc_relpos_attention backward failed");
+    m->launches += 14;
+    nc_free_tensor(gc);
+    NCTensor *out[5] = { dq, dkv, dkvm, dwr, dbr };
+    for (int i = 0; i < 5; i++) {
+        if (out[i] && nd->parents[i]) ga[i] = out[i];
+        else nc_free_tensor(out[i]);
+    }
+}
+
+// ---- integer CDF path (nc_ext.h) --------------------------------------------
+extern "C" NCTensor *nc_soft_max_cdf16(NCTensor *logits)
+{
+    logits = nc_contig(logits);
+    need_f32(logits, "nc_soft_max_cdf16");
+    size_t v = logits->dims[0];
+    NCTensor *y = nc_alloc(logits->dev, NC_TYPE_U16, logits->n_dims, logits->dims, false);
+    if (nchip_softmax_cdf16(nc_stream(logits), nc_f32(logits), (uint16_t *)nc_data(y), (int)v,
+                            (int64_t)(nc_numel(logits) / v)))
+        nc_fatal("nc_soft_max_cdf16 failed");
+    LAUNCHED(logits);
+    nc_free_tensor(logits);
+    return y;
+}
+
+extern "C" NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets)
+{
+    cdf = nc_contig(cdf); targets = nc_contig(targets);
+    need_dev(cdf, "nc_cdf_lookup"); need_dev(targets, "nc_cdf_lookup");
+    if (cdf->type != NC_TYPE_U16 || targets->type != NC_TYPE_U16) nc_fatal("nc_cdf_lookup: u16 tensors expected");
+    size_t v = cdf->dims[0], cols = nc_numel(cdf) / v, mm = targets->dims[0];
+    if (nc_numel(targets) != mm * cols) nc_fatal("nc_cdf_lookup: targets must be (m, n) for a (V, n) cdf");
+    NCTensor *y = nc_alloc_like(targets);
+    if (nchip_cdf_lookup(nc_stream(cdf), (const uint16_t *)nc_data(cdf), (const uint16_t *)nc_data(targets),
+                         (uint16_t *)nc_data(y), (int)v, (int64_t)mm, (int64_t)cols))
+        nc_fatal("nc_cdf_lookup failed");
+    LAUNCHED(cdf);
+    nc_free_tensor(cdf); nc_free_tensor(targets);
+    return y;
+}
+
+// same arithmetic as the device exponential of k_cdf.hip, for host callers
+extern "C" float nc_exp_det(float x)
+{
+    const float log2e = 0x1.715476p+0f, ln2_hi = 0x1.63p-1f, ln2_lo = -0x1.bd0106p-13f;
+    float n = rintf(x * log2e);
+    float r = fmaf(-n, ln2_hi, x);
+    r = fmaf(-n, ln2_lo, r);
+    float p = 0x1.6c16c2p-10f;
+    p = fmaf(p, r, 0x1.111112p-7f);
+    p = fmaf(p, r, 0x1.555556p-5f);
+    p = fmaf(p, r, 0x1.555556p-3f);
+    p = fmaf(p, r, 0.5f);
+    p = fmaf(p, r, 1.0f);
+    p = fmaf(p, r, 1.0f);
+    union { float f; uint32_t u; } v = { p };
+    v.u += (uint32_t)((int32_t)n * (1 << 23));
+    return v.f;
+}
+
+// ---- backward dispatch --------------------------------------------------------
+void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
+{
+    NCContext *m = nc_ctx(g);
+    hipStream_t st = m->stream;
+    g = nc_contig(nc_dup_tensor(g));
+    int64_t cnt = (int64_t)nc_numel(g);
+    switch (nd->op) {
+    case OP_ADD:
+        for (int w = 0; w < 2; w++)
+            if (nd->parents[w]) ga[w] = dev_unbroadcast(nc_dup_tensor(g), nd->arg_shape[w]);
+        break;
+    case OP_MUL:
+        for (int w = 0; w < 2; w++)
+            if (nd->parents[w]) ga[w] = dev_unbroadcast(dev_binary(KB_MUL, g, nd->saved[1 - w]), nd->arg_shape[w]);
+        break;
+    case OP_MASKED_FILL: {
+        NCTensor *mask = nd->saved[0], *t = nc_alloc_like(g);
+        // (mask ? 0 : g) is masked_fill of g with c = 0
+        k_masked_fill(st, nc_f32(g), (const int8_t *)nc_data(mask), nc_f32(t), cnt, (int64_t)nc_numel(mask), 0.0f, nd->ia[0]);
+        m->launches++;
+        ga[0] = t;
+        break;
+    }
+    case OP_UNARY: {
+        NCTensor *t = nc_alloc_like(g);
+        k_unary_bwd(st, nd->ia[0], nc_f32(nd->saved[0]), nc_f32(g), nc_f32(t), cnt);
+        m->launches++;
+        ga[0] = t;
+        break;
+    }
+    case OP_GATED_SWISH: {
+        NCTensor *dg = nc_alloc_like(g), *dx = nc_alloc_like(g);
+        k_gated_swish_bwd(st, nc_f32(nd->saved[0]), nc_f32(nd->saved[1]), nc_f32(g), nc_f32(dg), nc_f32(dx), cnt, nd->fa[0]);
+        m->launches++;
+        if (nd->parents[0]) ga[0] = dg; else nc_free_tensor(dg);
+        if (nd->parents[1]) ga[1] = dx; else nc_free_tensor(dx);
+        break;
+    }
+    case OP_LSTM_CLAMPED: {
+        NCTensor *t[4];
+        for (int i = 0; i < 4; i++) t[i] = nc_alloc_like(g);
+        k_lstm_clamped_bwd(st, nc_f32(nd->saved[0]), nc_f32(nd->saved[1]), nc_f32(nd->saved[2]), nc_f32(nd->saved[3]),
+                           nc_f32(g), nc_f32(t[0]), nc_f32(t[1]), nc_f32(t[2]), nc_f32(t[3]), cnt);
+        m->launches++;
+        for (int i = 0; i < 4; i++)
+            if (nd->parents[i]) ga[i] = t[i]; else nc_free_tensor(t[i]);
+        break;
+    }
+    case OP_LERP: {
+        NCTensor *t[3];
+        for (int i = 0; i < 3; i++) t[i] = nc_alloc_like(g);
+        k_lerp_bwd(st, nc_f32(nd->saved[0]), nc_f32(nd->saved[1]), nc_f32(nd->saved[2]), nc_f32(g),
+                   nc_f32(t[0]), nc_f32(t[1]), nc_f32(t[2]), cnt);
+        m->launches++;
+        for (int i = 0; i < 3; i++)
+            if (nd->parents[i]) ga[i] = t[i]; else nc_free_tensor(t[i]);
+        break;
+    }
+    case OP_RESHAPE:
+        ga[0] = nc_reshape_view(nc_dup_tensor(g), nd->arg_shape[0].nd, nd->arg_shape[0].d);
+        break;
+    case OP_REPEAT:
+        ga[0] = dev_unbroadcast(nc_dup_tensor(g), nd->arg_shape[0]);
+        break;
+    case OP_REDUCE_SUM:
+        if (nd->parents[0]) ga[0] = nc_dup_tensor(g);
+        if (nd->parents[1])
+            ga[1] = repeat_raw(g, nd->arg_shape[1].nd - g->n_dims, nd->arg_shape[1].d + g->n_dims);
+        break;
+    case OP_SUM: {
+        // broadcast the scalar gradient: 0-stride source copy
+        NCTensor *t = nc_alloc(g->dev, NC_TYPE_F32, nd->arg_shape[0].nd, nd->arg_shape[0].d, false);
+        NCTensor *v = nc_view(g);
+        v->n_dims = t->n_dims;
+        for (int i = 0; i < t->n_dims; i++) { v->dims[i] = t->dims[i]; v->strides[i] = 0; }
+        nc_copy_any(t, v);
+        nc_free_tensor(v);
+        ga[0] = t;
+        break;
+    }
+    case OP_SLICE: {
+        NCTensor *t = nc_alloc(g->dev, g->type, nd->arg_shape[0].nd, nd->arg_shape[0].d, true);
+        NCTensor *v = nc_slice_alias(t, nd->ia[0], (size_t)nd->ia[1], (size_t)nd->ia[1] + g->dims[nd->ia[0]]);
+        nc_copy_any(v, g);
+        nc_free_tensor(v);
+        ga[0] = t;
+        break;
+    }
+    case OP_CONCAT: case OP_CONCAT_NODE: {
+        size_t pos = 0;
+        for (int i = 0; i < nd->n_args; i++) {
+            if (nd->parents[i]) {
+                NCTensor *v = nc_slice_alias(g, nd->ia[0], pos, pos + nd->sizes[i]);
+                ga[i] = nc_alloc(g->dev, g->type, v->n_dims, v->dims, false);
+                nc_copy_any(ga[i], v);
+                nc_free_tensor(v);
+            }
+            pos += nd->sizes[i];
+        }
+        break;
+    }
+    case OP_PAD: {
+        NCTensor *t = nc_alloc(g->dev, NC_TYPE_F32, nd->arg_shape[0].nd, nd->arg_shape[0].d, false);
+        int64_t n_in = (int64_t)nd->arg_shape[0].d[0];
+        k_pad_bwd(st, nc_f32(g), nc_f32(t), n_in, (int64_t)nc_numel(t) / n_in, nd->ia[0], nd->ia[1], nd->ia[2], nd->ia[3]);
+        m->launches++;
+        ga[0] = t;
+        break;
+    }
+    case OP_PERMUTE: {
+        int inv[NC_N_DIMS_MAX];
+        for (int i = 0; i < g->n_dims; i++) inv[nd->ia[i]] = i;
+        ga[0] = permute_raw(g, g->n_dims, inv);
+        break;
+    }
+    case OP_REL_SHIFT: {
+        NCTensor *t = nc_alloc_like(g);
+        k_rel_shift(st, nc_f32(g), nc_f32(t), (int64_t)g->dims[0], (int64_t)g->dims[1],
+                    cnt / (int64_t)(g->dims[0] * g->dims[1]), nd->ia[0], nd->ia[1], 1);
+        m->launches++;
+        ga[0] = t;
+        break;
+    }
+    case OP_MATMUL:
+        matmul_bw(nd, g, ga, 0, 1);
+        if (nd->parents[2]) ga[2] = nc_dup_tensor(g);
+        break;
+    case OP_LINEAR: {
+        NCTensor *gz = nc_dup_tensor(g);
+        if (nd->ia[3] != NC_ACT_NONE) {
+            NCTensor *t = nc_alloc_like(g);
+            k_unary_bwd(st, nd->ia[3] == NC_ACT_GELU ? KU_GELU : KU_RELU, nc_f32(nd->saved[2]), nc_f32(g), nc_f32(t), cnt);
+            m->launches++;
+            nc_free_tensor(gz);
+            gz = t;
+        }
+        matmul_bw(nd, gz, ga, 0, 1);
+        if (nd->parents[2]) {
+            Shape bs;
+            bs.nd = 1; bs.d[0] = nd->saved[0]->dims[0];
+            ga[2] = dev_unbroadcast(nc_dup_tensor(gz), bs);
+        }
+        nc_free_tensor(gz);
+        break;
+    }
+    case OP_GET_COL: {
+        NCTensor *idx = nd->saved[0];
+        NCTensor *t = nc_alloc(g->dev, NC_TYPE_F32, nd->arg_shape[0].nd, nd->arg_shape[0].d, false);
+        if (nchip_add_col(st, nc_f32(g), (const int32_t *)nc_data(idx), nc_f32(t), (int)t->dims[0], (int)t->dims[1],
+                          (int64_t)nc_numel(idx)))
+            nc_fatal("get_col backward failed");
+        m->launches++;
+        ga[0] = t;
+        break;
+    }
+    case OP_SOFT_MAX: {
+        NCTensor *y = nd->saved[0], *t = nc_alloc_like(g);
+        int v = (int)y->dims[0];
+        if (nchip_softmax_bwd(st, nc_f32(y), nc_f32(g), nc_f32(t), v, cnt / v)) nc_fatal("softmax backward failed");
+        m->launches++;
+        ga[0] = t;
+        break;
+    }
+    case OP_INDEXED_LOG: {
+        NCTensor *p = nd->saved[0], *idx = nd->saved[1];
+        NCTensor *t = nc_alloc_like(p);
+        int v = (int)p->dims[0];
+        if (nchip_nll_bwd(st, nc_f32(p), (const int32_t *)nc_data(idx), nc_f32(g), nc_f32(t), v,
+                          (int64_t)nc_numel(p) / v, nd->ia[0]))
+            nc_fatal("indexed_log backward failed");
+        m->launches++;
+        ga[0] = t;
+        break;
+    }
+    case OP_NORM: {
+        NCTensor *xhat = nd->saved[0], *rstd = nd->saved[1], *w = nd->saved[2];
+        int d = (int)xhat->dims[0];
+        int64_t cols = (int64_t)nc_numel(xhat) / d;
+        NCTensor *dx = nd->parents[0] ? nc_alloc_like(xhat) : nullptr;
+        size_t dd = (size_t)d, cap = 0;
+        NCTensor *dw = (w && nd->parents[1]) ? nc_alloc(g->dev, NC_TYPE_F32, 1, &dd, false) : nullptr;
+        NCTensor *db = (w && nd->parents[2]) ? nc_alloc(g->dev, NC_TYPE_F32, 1, &dd, false) : nullptr;
+        float *partial = (dw || db) ? nc_tmp_f32(m, (size_t)nchip_norm_bwd_partial_rows(cols) * 2 * d, &cap) : nullptr;
+        if (nchip_norm_bwd(st, nc_f32(g), nc_f32(xhat), nc_f32(rstd), w ? nc_f32(w) : nullptr,
+                           dx ? nc_f32(dx) : nullptr, dw ? nc_f32(dw) : nullptr, db ? nc_f32(db) : nullptr,
+                           partial, d, cols, nd->ia[0]))
+            nc_fatal("layer norm backward failed");
+        if (partial) nc_tmp_free(m, partial, cap);
+        m->launches += 3;
+        ga[0] = dx; ga[1] = dw; ga[2] = db;
+        break;
+    }
+    case OP_ATTN:
+        attn_bw(nd, g, ga);
+        break;
+    default:
+        nc_fatal("backward: op %d not handled", nd->op);
+    }
+    nc_free_tensor(g);
+}

@@ -1,0 +1,190 @@
+"""GPU parity: every op of the libnc ABI on the MI355X (libnc_hip.so) against
+the CPU checker on the same seeded inputs, forward and backward.  Float
+results must agree within 1e-5 of the largest reference magnitude (the fp32
+bar); integer results bit-exactly."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import cases
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+
+
+def relerr(a, b):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return float(np.abs(a - b).max() / (np.abs(b).max() + 1e-30))
+
+
+@pytest.mark.parametrize("name", [c.name for c in cases.CASES])
+def test_op_matches_checker(hip, ref, rng, name):
+    case = cases.BY_NAME[name]
+    arrays = case.inputs(rng)
+    expect = case.ref(*[a.astype(np.float64) for a in arrays])
+    weight = rng.standard_normal(np.shape(expect))
+    out_r, grads_r = case.run(ref, arrays, weight)
+    out_h, grads_h = case.run(hip, arrays, weight)
+    assert out_h.shape == out_r.shape
+    assert relerr(out_h, out_r) <= TOL, name
+    for gh, gr in zip(grads_h, grads_r):
+        assert gh.shape == gr.shape
+        assert relerr(gh, gr) <= 5 * TOL, name
+
+
+GEMM_SHAPES = [(130, 70, 33, 1), (128, 128, 64, 1), (64, 64, 4096, 1), (512, 384, 512, 1),
+               (96, 40, 72, 5), (1, 1, 1, 1), (257, 129, 1030, 1), (256, 2048, 128, 1)]
+
+
+@pytest.mark.parametrize("ta", [0, 1])
+@pytest.mark.parametrize("tb", [0, 1])
+@pytest.mark.parametrize("shape", GEMM_SHAPES)
+def test_gemm_vs_checker(hip, ref, rng, ta, tb, shape):
+    m, n, k, batch = shape
+    bsh = (batch,) if batch > 1 else ()
+    a = rng.standard_normal(bsh + ((m, k) if ta else (k, m))).astype(np.float32)
+    b = rng.standard_normal(bsh + ((k, n) if tb else (n, k))).astype(np.float32)
+    outs = []
+    for nc in (hip, ref):
+        y = nc.nc_matmul_add(nc.tensor(a), nc.tensor(b), None, ta, tb, 1.0)
+        outs.append(nc.numpy(y, free=True))
+    assert relerr(outs[0], outs[1]) <= TOL
+
+
+def test_gemm_columns_do_not_depend_on_batch_width(hip, rng):
+    """A column computed alone is bit-identical to the same column computed in
+    a wide matrix (what lets a decoder replay an encoder's step)."""
+    w = rng.standard_normal((512, 512)).astype(np.float32)
+    x = rng.standard_normal((2048, 512)).astype(np.float32)
+    full = hip.numpy(hip.nc_matmul(hip.tensor(w), hip.tensor(x)), free=True)
+    part = hip.numpy(hip.nc_matmul(hip.tensor(w), hip.tensor(x[64:96])), free=True)
+    assert np.array_equal(full[64:96], part)
+    again = hip.numpy(hip.nc_matmul(hip.tensor(w), hip.tensor(x)), free=True)
+    assert np.array_equal(full, again)
+
+
+def test_gemm_bf16_variant(hip, ref, rng):
+    w = rng.standard_normal((256, 320)).astype(np.float32)
+    x = rng.standard_normal((200, 256)).astype(np.float32)
+    outs = []
+    for nc in (hip, ref):
+        nc.nc_set_matmul_bf16(nc.ctx, 1)
+        outs.append(nc.numpy(nc.nc_matmul(nc.tensor(w), nc.tensor(x)), free=True))
+        nc.nc_set_matmul_bf16(nc.ctx, 0)
+    # same rounded operands, fp32 accumulation in a different order
+    assert relerr(outs[0], outs[1]) <= 1e-5
+    exact = x.astype(np.float64) @ w.astype(np.float64)
+    assert relerr(outs[0], exact) <= 2e-2
+
+
+@pytest.mark.parametrize("cfg", [dict(H=2, dk=64, dv=64, B=2, T=64, M=64, d_pos=128, attn_len=128),
+                                 dict(H=4, dk=32, dv=32, B=3, T=20, M=20, d_pos=40, attn_len=40),
+                                 dict(H=2, dk=32, dv=32, B=2, T=32, M=32, d_pos=32, attn_len=48)])
+def test_relpos_attention_model_shapes(hip, ref, rng, cfg):
+    H, dk, dv, B, T, M, d_pos = (cfg[k] for k in ("H", "dk", "dv", "B", "T", "M", "d_pos"))
+    K = M + T
+    shapes = [(T, B, H * dk), (T, B, H * (dk + dv)), (M, B, H * (dk + dv)), (H, d_pos, dk), (H, K)]
+    arrays = [(rng.standard_normal(s) * 0.5).astype(np.float32) for s in shapes]
+    weight = rng.standard_normal((T, B, H * dv)).astype(np.float32)
+    res = []
+    for nc in (hip, ref):
+        hs = [nc.param(a, "p%d" % i) for i, a in enumerate(arrays)]
+        y = nc.nc_relpos_attention(*[nc.dup(h.value) for h, _ in hs], H, dk, cfg["attn_len"], 2.5)
+        out = nc.numpy(y)
+        loss = nc.nc_sum(nc.nc_mul(y, nc.tensor(weight)))
+        g = nc.backward(loss)
+        nc.free(loss)
+        res.append((out, [g[p] for _, p in hs]))
+    assert relerr(res[0][0], res[1][0]) <= TOL
+    for gh, gr in zip(res[0][1], res[1][1]):
+        assert relerr(gh, gr) <= 5 * TOL
+
+
+def _adversarial_logits(rng, V, n):
+    x = rng.standard_normal((n, V)).astype(np.float32) * 3
+    x[0] = 0.0                       # all equal
+    x[1] = -50.0; x[1, V // 3] = 40  # one dominant symbol
+    x[2] = np.linspace(-200, 200, V, dtype=np.float32)
+    x[3] *= 1e-3
+    x[4] += -np.log(np.arange(1, V + 1, dtype=np.float32))[rng.permutation(V)]
+    return x
+
+
+@pytest.mark.parametrize("V,n", [(256, 64), (16384, 16), (2, 8), (1000, 33), (65535, 6)])
+def test_cdf16_bit_exact(hip, ref, rng, V, n):
+    x = _adversarial_logits(rng, V, max(n, 5))
+    c_h = hip.numpy(hip.nc_soft_max_cdf16(hip.tensor(x)), free=True)
+    c_r = ref.numpy(ref.nc_soft_max_cdf16(ref.tensor(x)), free=True)
+    assert np.array_equal(c_h, c_r)
+    c = c_h.astype(np.int64)
+    assert (c[:, 0] == 0).all()
+    freq = np.diff(np.concatenate([c, np.full((c.shape[0], 1), 65536)], axis=1), axis=1)
+    assert (freq >= 1).all() and (freq.sum(axis=1) == 65536).all()
+
+
+def test_cdf_lookup_bit_exact(hip, ref, rng):
+    V, n, m = 16384, 4, 50000
+    x = _adversarial_logits(rng, V, 5)[:n]
+    t = rng.integers(0, 65536, size=(n, m)).astype(np.uint16)
+    res = []
+    for nc in (hip, ref):
+        cdf = nc.nc_soft_max_cdf16(nc.tensor(x))
+        res.append(nc.numpy(nc.nc_cdf_lookup(cdf, nc.tensor(t)), free=True))
+    assert np.array_equal(res[0], res[1])
+
+
+@pytest.mark.parametrize("algo", [16, 1, 0])
+def test_optimiser_step(hip, ref, rng, pkg, algo):
+    B = pkg.binding
+    w0 = rng.standard_normal((300, 70)).astype(np.float32)
+    res = []
+    for lib, dev in ((hip.lib._name, True), (ref.lib._name, False)):
+        nc = B.NC(lib, use_device=dev)
+        h, p = nc.param(w0)
+        sp = B.SGDOptParams(algo=algo, beta1=0.0, beta2=0.99, eps=1e-8, gradient_clip=0.1, lr=3e-4)
+        opt = nc.nc_sgd_opt_init(nc.ctx, C.byref(sp))
+        nc.nc_sgd_opt_set_all(C.byref(nc.plist), opt)
+        r2 = np.random.default_rng(7)
+        for _ in range(3):
+            g = r2.standard_normal(w0.shape).astype(np.float32)
+            nc.sgd_opt_update_var(p, nc.tensor(g), None)
+            nc.sgd_opt_update_var(p, nc.tensor(0.5 * g), None)  # tied use: accumulates
+            nc.nc_sgd_opt_update(opt)
+        res.append(nc.numpy(h.value))
+        nc.nc_sgd_opt_set_all(C.byref(nc.plist), None)
+        nc.nc_sgd_opt_end(opt)
+        nc.close()
+    assert relerr(res[0], res[1]) <= 1e-6
+
+
+def test_views_and_copies_on_device(hip, rng):
+    x = rng.standard_normal((6, 2, 3)).astype(np.float32)
+    t = hip.tensor(x)
+    src = rng.standard_normal((1, 2, 3)).astype(np.float32)
+    a = hip.nc_slice_alias(t, 2, 4, 5)
+    s = hip.tensor(src)
+    hip.nc_tensor_copy(a, s)
+    hip.free(a, s)
+    x[4:5] = src
+    assert np.array_equal(hip.numpy(t), x)
+    hip.nc_tensor_copy_slice(t, t, 2, 0, 4, 2)
+    x[0:4] = x[2:6].copy()
+    assert np.array_equal(hip.numpy(t), x)
+    hip.nc_tensor_set_zero(t)
+    assert not hip.numpy(t).any()
+    hip.free(t)
+
+
+def test_host_tensor_compute_is_refused(pkg):
+    """No CPU fallback: the product library aborts on host-tensor compute."""
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r); from conftest import load_pkg; import numpy as np;"
+            "B = load_pkg().binding; nc = B.NC(B.HIP_LIB, use_device=True);"
+            "a = nc.tensor(np.ones((2, 2), np.float32), device=nc.cpu);"
+            "nc.nc_add(a, nc.dup(a))") % (__file__.rsplit("/", 1)[0],)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+    assert r.returncode != 0 and "GPU only" in r.stderr
