@@ -719,7 +719,7 @@ extern "C" void nc_sgd_opt_update(NCSGDOptState *s)
         NCTensor *w = *vs->param->pval;
         need_dev(w, "nc_sgd_opt_update");
         // with beta1 == 0 the first moment equals the gradient; m is not stored
-        float *mp = vs->m ? nc_f32(vs->m) : nc_f32(vs->v);
+        float *mp = vs->m ? nc_f32(vs->m) : (vs->v ? nc_f32(vs->v) : nullptr);
         if (nchip_opt_update(s->ctx->stream, (int)p->algo, nc_f32(w), mp, vs->v ? nc_f32(vs->v) : nullptr,
                              nc_f32(vs->g), (int64_t)vs->n, p->lr * vs->param->lr_mult,
                              vs->m ? b1 : 0.0f, b2, p->u.adam.eps, p->u.adam.gradient_clip, c1, c2))
