@@ -1,0 +1,149 @@
+/*
+ * nncp_host.h - host side of the train+code step, above the libnc ABI.
+ *
+ * A C mirror of the part of nncp.c that drives libnc for the Transformer-XL
+ * model: the NNCPModelClass entry points of the `trf` model (nncp.c:49-69,
+ * 1544-1562) with the same names, argument meaning and ownership rules, the
+ * block loop of process_block (nncp.c:2968-3147), the symbol coder of
+ * cp_utils.c:299-349 and the binary range coder of arith.c.  It links against
+ * any library exporting nc_api.h (+ nc_ext.h when cfg.fused is set), so the
+ * same code runs on libnc_hip.so (product) and on the CPU checker (tests).
+ */
+#ifndef NNCP_HOST_H
+#define NNCP_HOST_H
+
+#include "nc_api.h"
+#include "nc_ext.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- binary range coder, bit-compatible with arith.c ----------------------- */
+#define NNCP_PROB_BITS 15 /* arith.h:27 */
+
+typedef struct { /* arith.h:32-43, in-memory output */
+    uint32_t range, low;
+    uint8_t current_byte;
+    uint32_t n_bytes;
+    uint8_t *buf;
+    size_t buf_size, idx;
+    int overflow;
+} NNCPPutBit;
+
+typedef struct { /* arith.h:50-61, in-memory input, zero padded past the end */
+    const uint8_t *buf;
+    size_t buf_len, idx;
+    uint32_t low, range;
+} NNCPGetBit;
+
+void nncp_put_bit_init(NNCPPutBit *s, uint8_t *buf, size_t buf_size);  /* arith.c:43 */
+void nncp_put_bit(NNCPPutBit *s, int prob0, int bit);                  /* arith.c:122 */
+size_t nncp_put_bit_flush(NNCPPutBit *s);        /* arith.c:164; returns bytes written */
+void nncp_get_bit_init(NNCPGetBit *s, const uint8_t *buf, size_t len); /* arith.c:233 */
+int nncp_get_bit(NNCPGetBit *s, int prob0);                            /* arith.c:259 */
+
+/* ---- symbol coders ------------------------------------------------------------ */
+/* float probabilities, balanced binary decomposition (cp_utils.c:299-349) */
+void nncp_write_sym(NNCPPutBit *pb, const float *prob, int n_symb, int sym);
+int nncp_read_sym(NNCPGetBit *gb, const float *prob, int n_symb);
+/* same decomposition driven by a 16-bit integer CDF (cdf[0] = 0, implicit
+   cdf[n_symb] = 65536): prob0 = ((cdf[mid]-cdf[lo]) << 15) / (cdf[hi]-cdf[lo])
+   clamped to [1, 32767]; O(log n_symb) integer work per symbol */
+void nncp_write_sym_cdf(NNCPPutBit *pb, const uint16_t *cdf, int n_symb, int sym);
+int nncp_read_sym_cdf(NNCPGetBit *gb, const uint16_t *cdf, int n_symb);
+
+/* piece-wise linear schedule with optional power decay (cp_utils.c:380-410) */
+typedef struct {
+    int n_steps;
+    float val[9];
+    int64_t pos[8];
+    float decay_power;
+} NNCPInterp;
+float nncp_interp(const NNCPInterp *p, int64_t pos);
+
+/* ---- Transformer-XL model ------------------------------------------------------ */
+#define NNCP_LN_POST (1 << 0)    /* nncp.c:74-78 */
+#define NNCP_LN_PRE (1 << 1)
+#define NNCP_LN_FINAL (1 << 2)
+#define NNCP_LN_COEF (1 << 3)
+#define NNCP_LN_RMSNORM (1 << 4)
+#define NNCP_FF_RELU 0           /* nncp.c:82-87 */
+#define NNCP_FF_GELU 1
+#define NNCP_FF_GEGLU 2
+#define NNCP_FF_GATED_SILU 3
+#define NNCP_N_LAYER_MAX 32
+
+typedef struct { /* TransformerModelParams + the NNCPModelParams fields it needs */
+    int n_layer, d_model, n_head, d_key, d_value, d_inner, d_pos, mem_len;
+    int attn_len[NNCP_N_LAYER_MAX];
+    int use_bias, use_w_r, tied_w_r, tied_b_r, query_bias, ln_flags, ff_act;
+    float init_range, embed_mult;
+    SGDOptParams sgd_opt;
+    int batch_size, seg_len, n_symbols;
+    uint32_t seed;
+    int use_device; /* nncp --cuda: compute on the accelerator device */
+    int fused;      /* 1: trf_eval uses nc_linear / nc_relpos_attention /
+                       nc_fused_layer_norm (full-segment evaluation only) */
+    int nb_threads;
+} NNCPConfig;
+
+typedef struct NNCPModel NNCPModel;
+
+void nncp_config_default(NNCPConfig *cfg);           /* nncp.c:2471-2513 */
+NNCPModel *nncp_model_new(const NNCPConfig *cfg);    /* nncp_init + trf_init, nncp.c:2762, 304 */
+void nncp_model_free(NNCPModel *s);                  /* nncp_end + trf_end, nncp.c:2802, 522 */
+const NNCPConfig *nncp_model_config(NNCPModel *s);
+NCContext *nncp_model_context(NNCPModel *s);
+NCDevice *nncp_model_device(NNCPModel *s);
+NCDevice *nncp_model_cpu_device(NNCPModel *s);
+/* address of the parameter tensor registered under `name` ("w_q_0", "embed",
+   ...: the names of trf_init), or NULL */
+NCTensor **nncp_model_param(NNCPModel *s, const char *name);
+int nncp_model_param_count(NNCPModel *s);
+const char *nncp_model_param_name(NNCPModel *s, int index);
+int64_t nncp_model_train_step(NNCPModel *s);
+
+/* the `trf` model class (nncp.c:1544-1562); input/expected are (B, T) i32
+   host tensors, borrowed; trf_eval returns an owned (V, B, T|1) tensor */
+NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input); /* nncp.c:581 */
+void trf_eval_end(NNCPModel *s);                                           /* nncp.c:1032 */
+float trf_eval_gradient(NNCPModel *s, const NCTensor *expected_output);    /* nncp.c:1099 */
+void trf_reset(NNCPModel *s);                                              /* nncp.c:1195 */
+void trf_update(NNCPModel *s);                                             /* nncp.c:1224 */
+void trf_set_lr(NNCPModel *s, float lr);                                   /* nncp.c:1243 */
+/* logits of the last trf_eval (V, B, T|1), borrowed; used by the CDF path */
+NCTensor *trf_last_logits(NNCPModel *s);
+
+/* ---- block loop (process_block, nncp.c:2968-3147) ------------------------------ */
+#define NNCP_MODE_SEQ_EVAL 0   /* one trf_eval per timestep: decodable, as nncp c/d */
+#define NNCP_MODE_SEGMENT 1    /* one trf_eval per segment (nncp --encode_only); the
+                                  decoder replays the same segment evaluation T times */
+#define NNCP_CODER_FLOAT 0     /* write_sym on float probabilities */
+#define NNCP_CODER_CDF16 2     /* nc_soft_max_cdf16 + integer symbol coder */
+
+typedef struct {
+    int64_t n_symbols, n_steps;
+    double loss_bits;   /* -sum log2 p[target] over the trained symbols */
+    double t_eval, t_code, t_grad, t_update; /* seconds, host wall clock */
+} NNCPStats;
+
+/* Codes block_len symbols (values < n_symbols) as one block: B contiguous
+   sub-streams, training after every full segment, the tail without training.
+   is_decode = 0: reads block_buf, writes through pb.  is_decode = 1: reads
+   through gb, fills block_buf.  lr: learning-rate schedule. */
+void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *block_buf,
+                        int block_len, int is_decode, int mode, const NNCPInterp *lr,
+                        NNCPStats *st);
+
+/* convenience: whole buffer as one block, in memory; returns the number of
+   bytes written (compress) */
+size_t nncp_compress(NNCPModel *s, const uint16_t *syms, int n, uint8_t *out, size_t cap,
+                     int mode, const NNCPInterp *lr, NNCPStats *st);
+void nncp_decompress(NNCPModel *s, const uint8_t *in, size_t len, uint16_t *syms, int n,
+                     int mode, const NNCPInterp *lr, NNCPStats *st);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NNCP_HOST_H */

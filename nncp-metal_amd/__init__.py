@@ -3,3 +3,4 @@ the libnc C ABI.  The compute lives in csrc/libnc_hip.so (HIP, gfx950); this
 package holds the ctypes binding and the host-side mirror of the reference's
 model interface."""
 from . import binding  # noqa: F401
+from . import host  # noqa: F401,E402

@@ -1,0 +1,239 @@
+"""ctypes binding of the host side (include/nncp_host.h): the Transformer-XL
+model class of nncp.c, the block loop and the coders, linked against
+csrc/libnc_hip.so in host/libnncp_host_hip.so."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import binding as B
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+HOST_HIP_LIB = os.path.join(HERE, "host", "libnncp_host_hip.so")
+
+MODE_SEQ_EVAL, MODE_SEGMENT = 0, 1
+CODER_FLOAT, CODER_CDF16 = 0, 2
+LN_POST, LN_PRE, LN_FINAL, LN_COEF, LN_RMSNORM = 1, 2, 4, 8, 16
+FF_RELU, FF_GELU, FF_GEGLU, FF_GATED_SILU = 0, 1, 2, 3
+
+
+class NNCPConfig(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("n_layer", "d_model", "n_head", "d_key", "d_value",
+                                       "d_inner", "d_pos", "mem_len")] + \
+               [("attn_len", C.c_int * 32)] + \
+               [(n, C.c_int) for n in ("use_bias", "use_w_r", "tied_w_r", "tied_b_r", "query_bias",
+                                       "ln_flags", "ff_act")] + \
+               [("init_range", C.c_float), ("embed_mult", C.c_float), ("sgd_opt", B.SGDOptParams)] + \
+               [(n, C.c_int) for n in ("batch_size", "seg_len", "n_symbols")] + \
+               [("seed", C.c_uint32), ("use_device", C.c_int), ("fused", C.c_int), ("nb_threads", C.c_int)]
+
+
+class NNCPInterp(C.Structure):
+    _fields_ = [("n_steps", C.c_int), ("val", C.c_float * 9), ("pos", C.c_int64 * 8),
+                ("decay_power", C.c_float)]
+
+
+class NNCPStats(C.Structure):
+    _fields_ = [("n_symbols", C.c_int64), ("n_steps", C.c_int64), ("loss_bits", C.c_double),
+                ("t_eval", C.c_double), ("t_code", C.c_double), ("t_grad", C.c_double),
+                ("t_update", C.c_double)]
+
+
+class NNCPPutBit(C.Structure):
+    _fields_ = [("range", C.c_uint32), ("low", C.c_uint32), ("current_byte", C.c_uint8),
+                ("n_bytes", C.c_uint32), ("buf", C.c_void_p), ("buf_size", C.c_size_t),
+                ("idx", C.c_size_t), ("overflow", C.c_int)]
+
+
+class NNCPGetBit(C.Structure):
+    _fields_ = [("buf", C.c_void_p), ("buf_len", C.c_size_t), ("idx", C.c_size_t),
+                ("low", C.c_uint32), ("range", C.c_uint32)]
+
+
+def constant_lr(lr):
+    p = NNCPInterp()
+    p.n_steps = 0
+    p.val[0] = lr
+    return p
+
+
+def make_config(**kw):
+    """nncp's default profile (nncp.c:2471-2513) with overrides; d_key/d_value
+    follow d_model / n_head and attn_len defaults to mem_len + seg_len."""
+    cfg = NNCPConfig()
+    opt = kw.pop("sgd_opt", None)
+    attn = kw.pop("attn_len", None)
+    base = dict(n_layer=4, d_model=256, n_head=8, d_inner=512, d_pos=32, mem_len=32, use_bias=1,
+                use_w_r=1, tied_w_r=1, tied_b_r=1, query_bias=0, ln_flags=LN_POST, ff_act=FF_GELU,
+                init_range=1.0, embed_mult=1.0, batch_size=16, seg_len=32, n_symbols=256, seed=123,
+                use_device=1, fused=0, nb_threads=1)
+    base.update(kw)
+    base.setdefault("d_key", base["d_model"] // base["n_head"])
+    base.setdefault("d_value", base["d_key"])
+    for k, v in base.items():
+        setattr(cfg, k, v)
+    for i in range(base["n_layer"]):
+        cfg.attn_len[i] = (attn[i] if attn else base["mem_len"] + base["seg_len"])
+    cfg.sgd_opt = opt if opt is not None else B.SGDOptParams(
+        algo=B.SGD_OPT_ADAM, beta1=0.0, beta2=0.9999, eps=1e-8, gradient_clip=0.1, lr=3e-4)
+    return cfg
+
+
+_P = C.c_void_p
+
+
+class Host:
+    """Loaded host library; its libnc functions come from the libnc it links."""
+
+    def __init__(self, libpath=HOST_HIP_LIB, nc_libpath=B.HIP_LIB):
+        for p in (libpath, nc_libpath):
+            if not os.path.exists(p):
+                raise RuntimeError("%s is missing: run __graft_entry__.build() first" % p)
+        # the libnc dependency is found through the rpath recorded at link time
+        self.lib = C.CDLL(libpath, mode=C.RTLD_LOCAL)
+        L = self.lib
+        L.nncp_model_new.restype = _P
+        L.nncp_model_new.argtypes = [C.POINTER(NNCPConfig)]
+        L.nncp_model_free.argtypes = [_P]
+        for n in ("nncp_model_context", "nncp_model_device", "nncp_model_cpu_device"):
+            getattr(L, n).restype = _P
+            getattr(L, n).argtypes = [_P]
+        L.nncp_model_param.restype = C.POINTER(_P)
+        L.nncp_model_param.argtypes = [_P, C.c_char_p]
+        L.nncp_model_param_count.argtypes = [_P]
+        L.nncp_model_param_name.restype = C.c_char_p
+        L.nncp_model_param_name.argtypes = [_P, C.c_int]
+        L.nncp_model_train_step.restype = C.c_int64
+        L.nncp_model_train_step.argtypes = [_P]
+        L.trf_eval.restype = _P
+        L.trf_eval.argtypes = [_P, C.c_int, _P]
+        L.trf_eval_end.argtypes = [_P]
+        L.trf_eval_gradient.restype = C.c_float
+        L.trf_eval_gradient.argtypes = [_P, _P]
+        L.trf_reset.argtypes = [_P]
+        L.trf_update.argtypes = [_P]
+        L.trf_set_lr.argtypes = [_P, C.c_float]
+        L.trf_last_logits.restype = _P
+        L.trf_last_logits.argtypes = [_P]
+        L.nncp_compress.restype = C.c_size_t
+        L.nncp_compress.argtypes = [_P, _P, C.c_int, _P, C.c_size_t, C.c_int,
+                                    C.POINTER(NNCPInterp), C.POINTER(NNCPStats)]
+        L.nncp_decompress.argtypes = [_P, _P, C.c_size_t, _P, C.c_int, C.c_int,
+                                      C.POINTER(NNCPInterp), C.POINTER(NNCPStats)]
+        L.nncp_put_bit_init.argtypes = [C.POINTER(NNCPPutBit), _P, C.c_size_t]
+        L.nncp_put_bit.argtypes = [C.POINTER(NNCPPutBit), C.c_int, C.c_int]
+        L.nncp_put_bit_flush.restype = C.c_size_t
+        L.nncp_put_bit_flush.argtypes = [C.POINTER(NNCPPutBit)]
+        L.nncp_get_bit_init.argtypes = [C.POINTER(NNCPGetBit), _P, C.c_size_t]
+        L.nncp_get_bit.argtypes = [C.POINTER(NNCPGetBit), C.c_int]
+        L.nncp_write_sym.argtypes = [C.POINTER(NNCPPutBit), _P, C.c_int, C.c_int]
+        L.nncp_read_sym.argtypes = [C.POINTER(NNCPGetBit), _P, C.c_int]
+        L.nncp_write_sym_cdf.argtypes = [C.POINTER(NNCPPutBit), _P, C.c_int, C.c_int]
+        L.nncp_read_sym_cdf.argtypes = [C.POINTER(NNCPGetBit), _P, C.c_int]
+        L.nncp_interp.restype = C.c_float
+        L.nncp_interp.argtypes = [C.POINTER(NNCPInterp), C.c_int64]
+        # the libnc symbols the host library resolved (same handle namespace)
+        self.ncl = C.CDLL(nc_libpath, mode=C.RTLD_LOCAL)
+        for name, (res, args) in B._PROTOS.items():
+            f = getattr(self.ncl, name)
+            f.restype, f.argtypes = res, args
+
+
+class Model:
+    """One NNCPModel plus helpers to move numpy data in and out."""
+
+    def __init__(self, host, cfg):
+        self.host, self.cfg, self.L, self.nc = host, cfg, host.lib, host.ncl
+        self.ptr = self.L.nncp_model_new(C.byref(cfg))
+        self.dev = self.L.nncp_model_device(self.ptr)
+        self.cpu = self.L.nncp_model_cpu_device(self.ptr)
+        self.ctx = self.L.nncp_model_context(self.ptr)
+
+    def close(self):
+        if self.ptr:
+            self.L.nncp_model_free(self.ptr)
+            self.ptr = None
+
+    # -- tensors ---------------------------------------------------------
+    def _to_numpy(self, x):
+        d = (C.c_size_t * 8)()
+        n = self.nc.nc_tensor_get_dims(x, d)
+        dims = tuple(d[i] for i in range(n))
+        t = self.nc.nc_tensor_get_item_type(x)
+        h = self.nc.nc_tensor_to_cpu_device(self.nc.nc_dup_tensor(x))
+        cnt = int(np.prod(dims)) if dims else 1
+        ptr = self.nc.nc_tensor_get_ptr(h, None)
+        dt = np.dtype(B._NP[t])
+        buf = (C.c_char * (cnt * dt.itemsize)).from_address(ptr)
+        out = np.frombuffer(buf, dtype=dt).copy().reshape(tuple(reversed(dims)))
+        self.nc.nc_free_tensor(h)
+        return out
+
+    def _host_tensor(self, arr):
+        arr = np.ascontiguousarray(arr) if np.ndim(arr) else np.asarray(arr)
+        dims = (C.c_size_t * max(arr.ndim, 1))(*reversed(arr.shape))
+        x = self.nc.nc_new_tensor_nz(self.cpu, B._NC[arr.dtype], arr.ndim, dims)
+        C.memmove(self.nc.nc_tensor_get_ptr(x, None), arr.ctypes.data, arr.nbytes)
+        return x
+
+    def param_names(self):
+        n = self.L.nncp_model_param_count(self.ptr)
+        return [self.L.nncp_model_param_name(self.ptr, i).decode() for i in range(n)]
+
+    def get_param(self, name):
+        return self._to_numpy(self.L.nncp_model_param(self.ptr, name.encode())[0])
+
+    def set_param(self, name, arr):
+        slot = self.L.nncp_model_param(self.ptr, name.encode())
+        src = self.nc.nc_tensor_to_device(self._host_tensor(arr.astype(np.float32)), self.dev)
+        self.nc.nc_tensor_copy(slot[0], src)
+        self.nc.nc_free_tensor(src)
+
+    def params(self):
+        return {n: self.get_param(n) for n in self.param_names()}
+
+    # -- the model class ---------------------------------------------------
+    def eval(self, tokens, output_index=-1, keep=False):
+        """tokens: int array (T, B) [numpy order of the (B, T) input tensor].
+        Returns the probabilities as numpy (T|1, B, V)."""
+        inp = self._host_tensor(np.asarray(tokens, dtype=np.int32))
+        out = self.L.trf_eval(self.ptr, output_index, inp)
+        self.nc.nc_free_tensor(inp)
+        res = self._to_numpy(out)
+        self.nc.nc_free_tensor(out)
+        if not keep:
+            self.L.trf_eval_end(self.ptr)
+        return res
+
+    def logits(self):
+        return self._to_numpy(self.L.trf_last_logits(self.ptr))
+
+    def train_step(self, tokens, targets, lr):
+        """One full-segment evaluation + gradient + update; returns
+        (probabilities, loss in nats summed over the segment)."""
+        p = self.eval(tokens, -1, keep=True)
+        tgt = self._host_tensor(np.asarray(targets, dtype=np.int32))
+        self.L.trf_set_lr(self.ptr, lr)
+        loss = self.L.trf_eval_gradient(self.ptr, tgt)
+        self.nc.nc_free_tensor(tgt)
+        self.L.trf_update(self.ptr)
+        return p, -loss
+
+    def compress(self, syms, mode, lr=3e-4):
+        syms = np.ascontiguousarray(syms, dtype=np.uint16)
+        cap = syms.size * 4 + 1024
+        out = np.zeros(cap, dtype=np.uint8)
+        st = NNCPStats()
+        sched = constant_lr(lr) if not isinstance(lr, NNCPInterp) else lr
+        n = self.L.nncp_compress(self.ptr, syms.ctypes.data, syms.size, out.ctypes.data, cap, mode,
+                                 C.byref(sched), C.byref(st))
+        return out[:n].copy(), st
+
+    def decompress(self, data, n_syms, mode, lr=3e-4):
+        data = np.ascontiguousarray(data, dtype=np.uint8)
+        out = np.zeros(n_syms, dtype=np.uint16)
+        st = NNCPStats()
+        sched = constant_lr(lr) if not isinstance(lr, NNCPInterp) else lr
+        self.L.nncp_decompress(self.ptr, data.ctypes.data, data.size, out.ctypes.data, n_syms, mode,
+                               C.byref(sched), C.byref(st))
+        return out, st

@@ -1,0 +1,241 @@
+/*
+ * Block loop of the compressor / decompressor: process_block of the reference
+ * (nncp.c:2968-3147) restated over in-memory buffers.  A block of block_len
+ * symbols is cut into B contiguous sub-streams (the first block_len % B one
+ * symbol longer, nncp.c:2943-2965); each step codes one segment of T symbols
+ * of every stream from the model's probabilities, then trains on it; a tail
+ * shorter than T is coded without training.
+ *
+ * Modes (nncp_host.h): NNCP_MODE_SEQ_EVAL evaluates one timestep at a time on
+ * both sides, exactly as `nncp c` / `nncp d`.  NNCP_MODE_SEGMENT evaluates the
+ * whole segment at once when encoding (`nncp --encode_only`); the decoder then
+ * replays that same whole-segment evaluation once per timestep with the
+ * symbols known so far.  Column t of the evaluation depends only on inputs
+ * 0..t (causal mask; masked terms contribute exact zeros), so the replay
+ * reproduces the encoder's probabilities bit for bit.
+ */
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+#include "../../include/nncp_host.h"
+
+static double now_s(void)
+{
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return ts.tv_sec + 1e-9 * ts.tv_nsec;
+}
+
+typedef struct {
+    const uint16_t *rbuf;
+    uint16_t *wbuf;
+    int stride, rem;
+} BlockView;
+
+static int get_symb(const BlockView *v, int stream, int pos) /* nncp.c:2945-2954 */
+{
+    int e = stream < v->rem;
+    if (pos < 0 || pos >= v->stride + e)
+        return 0;
+    return v->rbuf[v->stride * stream + (v->rem < stream ? v->rem : stream) + pos];
+}
+
+static void put_symb(BlockView *v, int stream, int pos, int c) /* nncp.c:2956-2965 */
+{
+    int e = stream < v->rem;
+    if (pos < 0 || pos >= v->stride + e)
+        abort();
+    v->wbuf[v->stride * stream + (v->rem < stream ? v->rem : stream) + pos] = (uint16_t)c;
+}
+
+typedef struct {
+    NNCPModel *s;
+    NNCPPutBit *pb;
+    NNCPGetBit *gb;
+    BlockView view;
+    int is_decode, coder, n_symbols, B;
+    NNCPStats *st;
+} Coder;
+
+/* probabilities (or CDF rows) of one evaluation on the host: column index
+   col = t*B + stream for a segment evaluation, stream for a timestep */
+typedef struct {
+    NCTensor *host;
+    const float *prob;
+    const uint16_t *cdf;
+    size_t stride;
+} HostDist;
+
+static HostDist fetch_dist(Coder *c, NCTensor *output)
+{
+    HostDist d;
+    memset(&d, 0, sizeof(d));
+    if (c->coder == NNCP_CODER_CDF16) {
+        NCTensor *cdf = nc_soft_max_cdf16(nc_dup_tensor(trf_last_logits(c->s)));
+        nc_free_tensor(output);
+        d.host = nc_tensor_to_cpu_device(cdf);
+        d.cdf = nc_tensor_get_ptr(d.host, &d.stride);
+    } else {
+        d.host = nc_tensor_to_cpu_device(output);
+        d.prob = nc_tensor_get_ptr(d.host, &d.stride);
+    }
+    return d;
+}
+
+/* codes (or decodes) the symbol of `stream` at block position pos */
+static int code_symbol(Coder *c, const HostDist *d, size_t col, int stream, int pos)
+{
+    int sym;
+    if (!c->is_decode) {
+        sym = get_symb(&c->view, stream, pos);
+        if (d->cdf) nncp_write_sym_cdf(c->pb, d->cdf + col * d->stride, c->n_symbols, sym);
+        else nncp_write_sym(c->pb, d->prob + col * d->stride, c->n_symbols, sym);
+    } else {
+        if (d->cdf) sym = nncp_read_sym_cdf(c->gb, d->cdf + col * d->stride, c->n_symbols);
+        else sym = nncp_read_sym(c->gb, d->prob + col * d->stride, c->n_symbols);
+        put_symb(&c->view, stream, pos, sym);
+    }
+    return sym;
+}
+
+static int symbol_is_coded(int t, int stream, int len2, int rem, int full)
+{
+    return full || t < len2 || (t == len2 && stream < rem); /* nncp.c:3099-3100 */
+}
+
+/* One segment starting at block position idx: n_t timesteps are coded (T for a
+   full segment, fewer in the tail).  Fills `expected` when training follows. */
+static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int full,
+                         NCTensor *input, NCTensor *expected)
+{
+    NNCPModel *s = c->s;
+    int B = c->B;
+    double t0;
+    if (mode == NNCP_MODE_SEGMENT && !c->is_decode) {
+        /* nncp.c:3024-3046 */
+        for (int t = 0; t < n_t; t++)
+            for (int b = 0; b < B; b++)
+                nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
+        t0 = now_s();
+        NCTensor *out = trf_eval(s, -1, input);
+        HostDist d = fetch_dist(c, out);
+        c->st->t_eval += now_s() - t0;
+        t0 = now_s();
+        for (int t = 0; t < n_t; t++)
+            for (int b = 0; b < B; b++)
+                if (symbol_is_coded(t, b, len2, c->view.rem, full)) {
+                    int sym = code_symbol(c, &d, (size_t)t * B + b, b, idx + t);
+                    if (expected) nc_set1_i32_2d(expected, b, t, sym);
+                }
+        c->st->t_code += now_s() - t0;
+        nc_free_tensor(d.host);
+        return;
+    }
+    for (int t = 0; t < n_t; t++) {
+        /* nncp.c:2996-3022 (and 3087-3114 for the tail) */
+        for (int b = 0; b < B; b++)
+            nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
+        t0 = now_s();
+        NCTensor *out = trf_eval(s, mode == NNCP_MODE_SEGMENT ? -1 : t, input);
+        HostDist d = fetch_dist(c, out);
+        c->st->t_eval += now_s() - t0;
+        t0 = now_s();
+        for (int b = 0; b < B; b++)
+            if (symbol_is_coded(t, b, len2, c->view.rem, full)) {
+                size_t col = mode == NNCP_MODE_SEGMENT ? (size_t)t * B + b : (size_t)b;
+                int sym = code_symbol(c, &d, col, b, idx + t);
+                if (expected) nc_set1_i32_2d(expected, b, t, sym);
+            }
+        c->st->t_code += now_s() - t0;
+        nc_free_tensor(d.host);
+        /* replayed segment evaluations are discarded, except the last one of a
+           trained segment, whose graph the gradient needs */
+        if (mode == NNCP_MODE_SEGMENT && !(expected && t == n_t - 1))
+            trf_eval_end(s);
+    }
+    /* decoder in segment mode: the last replay was built once every input of
+       the segment was known (the last symbol is a target only), so its graph
+       is the one the encoder differentiated */
+}
+
+void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *block_buf,
+                        int block_len, int is_decode, int mode_flags, const NNCPInterp *lr,
+                        NNCPStats *st)
+{
+    NNCPStats local;
+    Coder c;
+    int mode = mode_flags & 1;
+    memset(&local, 0, sizeof(local));
+    memset(&c, 0, sizeof(c));
+    c.s = s; c.pb = pb; c.gb = gb; c.is_decode = is_decode;
+    c.coder = mode_flags & NNCP_CODER_CDF16;
+    c.st = st ? st : &local;
+
+    const NNCPConfig *cfg = nncp_model_config(s);
+    int B = cfg->batch_size, T = cfg->seg_len;
+    c.n_symbols = cfg->n_symbols;
+    c.B = B;
+    c.view.rbuf = block_buf; c.view.wbuf = block_buf;
+    c.view.stride = block_len / B;
+    c.view.rem = block_len % B;
+
+    NCDevice *cpu = nncp_model_cpu_device(s);
+    NCTensor *input = nc_new_tensor_2d(cpu, NC_TYPE_I32, B, T);
+    NCTensor *expected = nc_new_tensor_2d(cpu, NC_TYPE_I32, B, T);
+    trf_reset(s); /* nncp.c:2988 */
+
+    int idx = 0;
+    while (idx + T <= c.view.stride) { /* nncp.c:2993 */
+        code_segment(&c, mode, idx, T, T, 1, input, expected);
+        float rate = nncp_interp(lr, nncp_model_train_step(s)); /* nncp.c:3048-3050 */
+        trf_set_lr(s, rate);
+        double t0 = now_s();
+        float loss = trf_eval_gradient(s, expected);
+        c.st->t_grad += now_s() - t0;
+        t0 = now_s();
+        trf_update(s);
+        c.st->t_update += now_s() - t0;
+        c.st->loss_bits -= loss / log(2.0);
+        c.st->n_steps++;
+        c.st->n_symbols += (int64_t)T * B;
+        idx += T;
+    }
+    int len2 = c.view.stride - idx, len1 = len2 + (c.view.rem != 0); /* nncp.c:3076-3077 */
+    if (len1 > 0) {
+        for (int t = 0; t < T; t++)
+            for (int b = 0; b < B; b++)
+                nc_set1_i32_2d(input, b, t, 0);
+        code_segment(&c, mode, idx, len1, len2, 0, input, NULL);
+        trf_eval_end(s);
+        c.st->n_symbols += (int64_t)len2 * B + c.view.rem;
+    }
+    nc_free_tensor(expected);
+    nc_free_tensor(input);
+}
+
+size_t nncp_compress(NNCPModel *s, const uint16_t *syms, int n, uint8_t *out, size_t cap,
+                     int mode, const NNCPInterp *lr, NNCPStats *st)
+{
+    NNCPPutBit pb;
+    uint16_t *buf = nc_malloc(sizeof(uint16_t) * (n > 0 ? n : 1));
+    memcpy(buf, syms, sizeof(uint16_t) * n);
+    nncp_put_bit_init(&pb, out, cap);
+    nncp_process_block(s, &pb, NULL, buf, n, 0, mode, lr, st);
+    size_t len = nncp_put_bit_flush(&pb);
+    nc_free(buf);
+    if (pb.overflow) {
+        fprintf(stderr, "nncp_compress: output buffer too small (%zu needed)\n", len);
+        abort();
+    }
+    return len;
+}
+
+void nncp_decompress(NNCPModel *s, const uint8_t *in, size_t len, uint16_t *syms, int n,
+                     int mode, const NNCPInterp *lr, NNCPStats *st)
+{
+    NNCPGetBit gb;
+    nncp_get_bit_init(&gb, in, len);
+    nncp_process_block(s, NULL, &gb, syms, n, 1, mode, lr, st);
+}

@@ -1,0 +1,660 @@
+/*
+ * Transformer-XL model of NNCP on top of the libnc ABI: the `trf` model class
+ * (nncp.c:263-1562) restated as a library.  Two evaluation paths issue
+ * exactly the tensor ops the reference issues:
+ *   - reference path (cfg.fused = 0): the op-by-op sequence of trf_eval,
+ *     including the per-timestep (seq_eval) variant with its K/V caches and the
+ *     graph surgery of trf_eval_gradient;
+ *   - fused path (cfg.fused = 1): the same mathematics through nc_linear,
+ *     nc_relpos_attention and nc_fused_layer_norm (full-segment evaluation).
+ * Not supported (as in no BASELINE configuration): rotary position embedding,
+ * dropout / retrain, tied input-output embedding, sparse gradients.
+ */
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include "../../include/nncp_host.h"
+
+typedef struct {
+    NCTensor *w_q, *w_kv, *b_q, *w_o;
+    NCTensor *ff1, *ff2, *ff_bias1, *ff_bias2;
+    NCTensor *w_r, *b_r;
+    NCTensor *ln_g1, *ln_b1, *ln_g2, *ln_b2, *alpha;
+    /* per-timestep evaluation only */
+    NCTensor *mem_key, *mem_value, *tmp_w_r, *tmp_b_r, *attn_mask;
+    NCNode **key_nodes, **kq_nodes, **value_nodes, **va_nodes;
+} Layer;
+
+struct NNCPModel {
+    NNCPConfig cfg;
+    NCContext *ctx;
+    NCDevice *dev, *cpu;
+    NCRNDState *rnd;
+    NCParamList params;
+    Layer *layers;
+    NCTensor *ln_g, *ln_b, *embed, *embed_out, *out_bias;
+    NCTensor **mem_h, **train_h, **outputs;
+    NCTensor *logits;
+    NCSGDOptState *opt;
+    int seq_eval;
+    float embed_mult;
+    int64_t train_step;
+};
+
+static void die(const char *msg)
+{
+    fprintf(stderr, "nncp_host: %s\n", msg);
+    abort();
+}
+
+void nncp_config_default(NNCPConfig *c) /* the "default" profile, nncp.c:2471-2513 */
+{
+    memset(c, 0, sizeof(*c));
+    c->seed = 123;
+    c->batch_size = 16; c->seg_len = 32; c->n_symbols = 256;
+    c->n_layer = 4; c->d_model = 256; c->n_head = 8;
+    c->d_key = c->d_value = c->d_model / c->n_head;
+    c->d_inner = c->d_model * 2;
+    c->d_pos = 32; c->mem_len = 32;
+    for (int i = 0; i < c->n_layer; i++)
+        c->attn_len[i] = c->mem_len + c->seg_len;
+    c->init_range = 1.0f; c->embed_mult = 1.0f;
+    c->use_bias = 1; c->use_w_r = 1; c->tied_w_r = 1; c->tied_b_r = 1;
+    c->ln_flags = NNCP_LN_POST;
+    c->ff_act = NNCP_FF_GELU;
+    c->sgd_opt.algo = SGD_OPT_ADAM;
+    c->sgd_opt.u.adam.beta1 = 0.0f; c->sgd_opt.u.adam.beta2 = 0.9999f;
+    c->sgd_opt.u.adam.eps = 1e-8f; c->sgd_opt.u.adam.gradient_clip = 0.1f;
+    c->sgd_opt.lr = 3e-4f;
+    c->use_device = 1; c->fused = 0; c->nb_threads = 1;
+}
+
+static NCTensor *new_param(NNCPModel *s, NCTensor **slot, NCTensor *t, float init, const char *fmt, int idx)
+{
+    *slot = t;
+    nc_new_param(&s->params, slot, fmt, idx);
+    if (init > 0.0f)
+        nc_tensor_set_rnd_unif(t, 0, init, s->rnd);
+    return t;
+}
+
+static void new_layer_norm(NNCPModel *s, NCTensor **g, NCTensor **b, int idx) /* nncp.c:268-277 */
+{
+    new_param(s, g, nc_new_tensor_1d(s->dev, NC_TYPE_F32, s->cfg.d_model), 0, "ln_g_%d", idx);
+    nc_tensor_set_f32(*g, 1.0f);
+    new_param(s, b, nc_new_tensor_1d(s->dev, NC_TYPE_F32, s->cfg.d_model), 0, "ln_b_%d", idx);
+}
+
+NNCPModel *nncp_model_new(const NNCPConfig *cfg)
+{
+    NNCPModel *s = nc_mallocz(sizeof(*s));
+    const NNCPConfig *c;
+    s->cfg = *cfg;
+    c = &s->cfg;
+    if (c->n_layer < 1 || c->n_layer > NNCP_N_LAYER_MAX || c->d_model != c->d_key * c->n_head)
+        die("bad configuration (need d_model == d_key * n_head, 1 <= n_layer <= 32)");
+    int T = c->seg_len, M = c->mem_len, K = T + M, B = c->batch_size, H = c->n_head, D = c->d_model;
+    int gated = c->ff_act == NNCP_FF_GEGLU || c->ff_act == NNCP_FF_GATED_SILU;
+    /* nncp_init, nncp.c:2770-2779 */
+    s->ctx = nc_context_init(c->nb_threads);
+    s->cpu = nc_new_cpu_device(s->ctx);
+    s->dev = c->use_device ? nc_new_cuda_device(s->ctx, 0) : s->cpu;
+    s->rnd = nc_rnd_init(s->dev, c->seed);
+    /* trf_init, nncp.c:304-520 */
+    s->embed_mult = sqrtf((float)D) * c->embed_mult;
+    nc_param_list_init(s->ctx, &s->params);
+    float init = c->init_range / sqrtf((float)D);
+    s->layers = nc_mallocz(sizeof(Layer) * c->n_layer);
+    for (int l = 0; l < c->n_layer; l++) {
+        Layer *tl = &s->layers[l];
+        /* mask[j,i] = !(0 <= (i+M)-j < attn_len), nncp.c:352-365 */
+        NCTensor *mask = nc_new_tensor_2d(s->cpu, NC_TYPE_I8, K, T);
+        for (int i = 0; i < T; i++)
+            for (int j = 0; j < K; j++) {
+                int pos = i + M - j;
+                nc_set1_i32_2d(mask, j, i, !(pos >= 0 && pos < c->attn_len[l]));
+            }
+        tl->attn_mask = nc_tensor_to_device(mask, s->dev);
+        if (l == 0 || !c->tied_b_r)
+            new_param(s, &tl->b_r, nc_new_tensor_2d(s->dev, NC_TYPE_F32, K, H), 0, "b_r_%d", l);
+        if (c->use_w_r && (l == 0 || !c->tied_w_r))
+            new_param(s, &tl->w_r, nc_new_tensor_3d(s->dev, NC_TYPE_F32, c->d_key, c->d_pos, H), init, "w_r_%d", l);
+        new_param(s, &tl->w_q, nc_new_tensor_2d(s->dev, NC_TYPE_F32, H * c->d_key, D), init, "w_q_%d", l);
+        if (c->query_bias)
+            new_param(s, &tl->b_q, nc_new_tensor_1d(s->dev, NC_TYPE_F32, H * c->d_key), 0, "b_q_%d", l);
+        new_param(s, &tl->w_kv, nc_new_tensor_2d(s->dev, NC_TYPE_F32, H * c->d_key + H * c->d_value, D), init, "w_kv_%d", l);
+        if (c->d_value != D)
+            new_param(s, &tl->w_o, nc_new_tensor_2d(s->dev, NC_TYPE_F32, D, H * c->d_value), init, "w_o_%d", l);
+        int n1 = gated ? c->d_inner * 2 : c->d_inner;
+        new_param(s, &tl->ff1, nc_new_tensor_2d(s->dev, NC_TYPE_F32, n1, D), init, "ff1_%d", l);
+        if (c->use_bias)
+            new_param(s, &tl->ff_bias1, nc_new_tensor_1d(s->dev, NC_TYPE_F32, n1), 0, "ff_bias1_%d", l);
+        new_param(s, &tl->ff2, nc_new_tensor_2d(s->dev, NC_TYPE_F32, D, c->d_inner),
+                  init * sqrtf((float)D / (float)c->d_inner), "ff2_%d", l);
+        if (c->use_bias)
+            new_param(s, &tl->ff_bias2, nc_new_tensor_1d(s->dev, NC_TYPE_F32, D), 0, "ff_bias2_%d", l);
+        if (c->ln_flags & (NNCP_LN_POST | NNCP_LN_PRE)) {
+            new_layer_norm(s, &tl->ln_g1, &tl->ln_b1, l * 2);
+            new_layer_norm(s, &tl->ln_g2, &tl->ln_b2, l * 2 + 1);
+        }
+        if (c->ln_flags & NNCP_LN_COEF)
+            new_param(s, &tl->alpha, nc_new_scalar(s->dev, NC_TYPE_F32), 0, "alpha_%d", l);
+        /* caches and node tables of the per-timestep path, nncp.c:439-452 */
+        tl->mem_key = nc_new_tensor_4d(s->dev, NC_TYPE_F32, c->d_key, K, H, B);
+        tl->mem_value = nc_new_tensor_4d(s->dev, NC_TYPE_F32, c->d_value, K, H, B);
+        tl->key_nodes = nc_mallocz(sizeof(NCNode *) * (T + 1));
+        tl->kq_nodes = nc_mallocz(sizeof(NCNode *) * T);
+        tl->value_nodes = nc_mallocz(sizeof(NCNode *) * (T + 1));
+        tl->va_nodes = nc_mallocz(sizeof(NCNode *) * T);
+    }
+    if (c->ln_flags & NNCP_LN_FINAL)
+        new_layer_norm(s, &s->ln_g, &s->ln_b, c->n_layer * 2);
+    new_param(s, &s->embed, nc_new_tensor_2d(s->dev, NC_TYPE_F32, D, c->n_symbols), init, "embed", 0);
+    new_param(s, &s->embed_out, nc_new_tensor_2d(s->dev, NC_TYPE_F32, c->n_symbols, D), init, "embed_out", 0);
+    if (c->use_bias)
+        new_param(s, &s->out_bias, nc_new_tensor_1d(s->dev, NC_TYPE_F32, c->n_symbols), 0, "out_bias", 0);
+    s->mem_h = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
+    s->train_h = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
+    for (int l = 0; l < c->n_layer; l++) {
+        s->mem_h[l] = nc_new_tensor_3d(s->dev, NC_TYPE_F32, D, B, M);
+        s->train_h[l] = nc_new_tensor_3d(s->dev, NC_TYPE_F32, D, B, T);
+    }
+    s->outputs = nc_mallocz(sizeof(NCTensor *) * T);
+    s->opt = nc_sgd_opt_init(s->ctx, &c->sgd_opt);
+    nc_sgd_opt_set_all(&s->params, s->opt);
+    return s;
+}
+
+void nncp_model_free(NNCPModel *s) /* trf_end nncp.c:522-550, nncp_end nncp.c:2802-2809 */
+{
+    trf_eval_end(s);
+    for (int l = 0; l < s->cfg.n_layer; l++) {
+        Layer *tl = &s->layers[l];
+        nc_free_tensor(s->mem_h[l]); nc_free_tensor(s->train_h[l]);
+        nc_free_tensor(tl->mem_key); nc_free_tensor(tl->mem_value); nc_free_tensor(tl->attn_mask);
+        nc_free(tl->key_nodes); nc_free(tl->kq_nodes); nc_free(tl->value_nodes); nc_free(tl->va_nodes);
+    }
+    nc_free(s->mem_h); nc_free(s->train_h); nc_free(s->outputs);
+    nc_sgd_opt_set_all(&s->params, NULL);
+    nc_sgd_opt_end(s->opt);
+    nc_param_list_end(&s->params);
+    nc_free(s->layers);
+    nc_rnd_end(s->rnd);
+    nc_context_end(s->ctx);
+    nc_free(s);
+}
+
+const NNCPConfig *nncp_model_config(NNCPModel *s) { return &s->cfg; }
+NCContext *nncp_model_context(NNCPModel *s) { return s->ctx; }
+NCDevice *nncp_model_device(NNCPModel *s) { return s->dev; }
+NCDevice *nncp_model_cpu_device(NNCPModel *s) { return s->cpu; }
+int64_t nncp_model_train_step(NNCPModel *s) { return s->train_step; }
+
+NCTensor **nncp_model_param(NNCPModel *s, const char *name)
+{
+    for (struct list_head *el = s->params.param_list.next; el != &s->params.param_list; el = el->next) {
+        NCParam *p = (NCParam *)el;
+        if (!strcmp(p->name, name))
+            return p->pval;
+    }
+    return NULL;
+}
+
+int nncp_model_param_count(NNCPModel *s)
+{
+    int n = 0;
+    for (struct list_head *el = s->params.param_list.next; el != &s->params.param_list; el = el->next)
+        n++;
+    return n;
+}
+
+const char *nncp_model_param_name(NNCPModel *s, int index)
+{
+    int n = 0;
+    for (struct list_head *el = s->params.param_list.next; el != &s->params.param_list; el = el->next)
+        if (n++ == index)
+            return ((NCParam *)el)->name;
+    return NULL;
+}
+
+/* ---- pieces shared by the evaluation paths ----------------------------------- */
+
+static NCTensor *scalar(NNCPModel *s, float v) { return nc_new_f32(s->dev, v); }
+
+static NCTensor *layer_norm(NNCPModel *s, NCTensor *x, NCTensor *g, NCTensor *b) /* nncp.c:279-288 */
+{
+    int rms = s->cfg.ln_flags & NNCP_LN_RMSNORM;
+    if (s->cfg.fused)
+        return nc_fused_layer_norm(x, nc_dup_tensor(g), nc_dup_tensor(b), 1e-5f, !rms);
+    x = rms ? nc_rms_norm(x, 1e-5f) : nc_layer_norm(x, 1e-5f);
+    return nc_add(nc_mul(x, nc_dup_tensor(g)), nc_dup_tensor(b));
+}
+
+static NCTensor *split_head(NCTensor *x, int n_head) /* nncp.c:554-565 */
+{
+    size_t d[NC_N_DIMS_MAX];
+    nc_tensor_get_dims(x, d);
+    x = nc_reshape_4d(x, d[0] / n_head, n_head, d[1], d[2]);
+    return nc_permute_4d(x, 0, 3, 1, 2);
+}
+
+static NCTensor *concat_head(NCTensor *x) /* nncp.c:569-579 */
+{
+    size_t d[NC_N_DIMS_MAX];
+    x = nc_permute_4d(x, 0, 2, 3, 1);
+    nc_tensor_get_dims(x, d);
+    return nc_reshape_2d(x, d[0] * d[1], d[2] * d[3]);
+}
+
+/* store layer input into train_h (whole segment or one timestep), nncp.c:647-657 */
+static void save_layer_input(NNCPModel *s, int l, int output_index, NCTensor *x, int seg_len)
+{
+    NCTensor *dst = output_index < 0 ? nc_dup_tensor(s->train_h[l])
+                                     : nc_slice_alias(s->train_h[l], 2, output_index, output_index + 1);
+    NCTensor *src = nc_reshape_3d(nc_dup_tensor(x), s->cfg.d_model, s->cfg.batch_size, seg_len);
+    nc_tensor_copy(dst, src);
+    nc_free_tensor(src);
+    nc_free_tensor(dst);
+}
+
+/* position tensors of the reference path, built at the first timestep, nncp.c:728-761 */
+static void build_position_tensors(NNCPModel *s, int l)
+{
+    const NNCPConfig *c = &s->cfg;
+    Layer *tl = &s->layers[l];
+    if (c->use_w_r) {
+        if (l == 0 || !c->tied_w_r) {
+            NCTensor *w = nc_dup_tensor(tl->w_r);
+            w = c->batch_size > 1 ? nc_repeat_1d(w, c->batch_size)
+                                  : nc_reshape_4d(w, c->d_key, c->d_pos, c->n_head, 1);
+            tl->tmp_w_r = w;
+        } else {
+            tl->tmp_w_r = nc_dup_tensor(s->layers[0].tmp_w_r);
+        }
+    }
+    if (l == 0 || !c->tied_b_r) {
+        NCTensor *b = nc_mul(nc_dup_tensor(tl->b_r), scalar(s, sqrtf((float)(c->d_key * c->d_model))));
+        b = nc_repeat_2d(b, c->seg_len, c->batch_size);
+        tl->tmp_b_r = nc_permute_4d(b, 0, 2, 1, 3);
+    } else {
+        tl->tmp_b_r = nc_dup_tensor(s->layers[0].tmp_b_r);
+    }
+}
+
+/* reference attention, whole segment: nncp.c:763-800 */
+static NCTensor *attention_segment_ref(NNCPModel *s, int l, NCTensor *query, NCTensor *key, NCTensor *value)
+{
+    const NNCPConfig *c = &s->cfg;
+    Layer *tl = &s->layers[l];
+    NCTensor *t0 = nc_matmul_add(key, nc_dup_tensor(query), NULL, 1, 0, 1.0f), *rd;
+    if (c->use_w_r) {
+        rd = nc_matmul_add(nc_dup_tensor(tl->tmp_w_r), query, NULL, 1, 0, 1.0f);
+        rd = nc_pad(rd, c->mem_len + c->seg_len - c->d_pos, NC_PAD_DUP, 0, NC_PAD_ZERO);
+        rd = nc_add(rd, nc_dup_tensor(tl->tmp_b_r));
+    } else {
+        nc_free_tensor(query);
+        rd = nc_dup_tensor(tl->tmp_b_r);
+    }
+    rd = nc_rel_shift(rd, -(c->seg_len - 1), 1);
+    t0 = nc_add(rd, t0);
+    t0 = nc_mul(t0, scalar(s, 1.0f / sqrtf((float)c->d_key)));
+    t0 = nc_masked_fill(t0, nc_dup_tensor(tl->attn_mask), -INFINITY, 0);
+    t0 = nc_soft_max(t0);
+    return nc_matmul(value, t0);
+}
+
+/* reference attention, one timestep against the K/V caches: nncp.c:801-863 */
+static NCTensor *attention_timestep_ref(NNCPModel *s, int l, int t, NCTensor *query, NCTensor *key, NCTensor *value)
+{
+    const NNCPConfig *c = &s->cfg;
+    Layer *tl = &s->layers[l];
+    int row = c->mem_len + t;
+    NCTensor *slot, *t0, *t1, *rd;
+    NCNode *node;
+
+    tl->key_nodes[t + 1] = nc_dup_node(nc_get_node(key));
+    slot = nc_slice_alias(tl->mem_key, 1, row, row + 1);
+    nc_tensor_copy(slot, key);
+    nc_free_tensor(key); nc_free_tensor(slot);
+    key = nc_dup_tensor(tl->mem_key);
+
+    tl->value_nodes[t + 1] = nc_dup_node(nc_get_node(value));
+    slot = nc_slice_alias(tl->mem_value, 1, row, row + 1);
+    nc_tensor_copy(slot, value);
+    nc_free_tensor(value); nc_free_tensor(slot);
+    value = nc_dup_tensor(tl->mem_value);
+
+    t0 = nc_matmul_add(key, nc_dup_tensor(query), NULL, 1, 0, 1.0f);
+    node = nc_get_node(t0);
+    nc_node_set_arg(node, 1, query);
+    tl->kq_nodes[t] = node;
+    if (c->use_w_r) {
+        rd = nc_matmul_add(nc_dup_tensor(tl->tmp_w_r), query, NULL, 1, 0, 1.0f);
+        rd = nc_pad(rd, c->mem_len + c->seg_len - c->d_pos, NC_PAD_DUP, 0, NC_PAD_ZERO);
+        rd = nc_add(rd, nc_slice(nc_dup_tensor(tl->tmp_b_r), 1, t, t + 1));
+    } else {
+        nc_free_tensor(query);
+        rd = nc_slice(nc_dup_tensor(tl->tmp_b_r), 1, t, t + 1);
+    }
+    rd = nc_rel_shift(rd, -(c->seg_len - 1 - t), 1);
+    t0 = nc_add(rd, t0);
+    t0 = nc_mul(t0, scalar(s, 1.0f / sqrtf((float)c->d_key)));
+    t1 = nc_slice_alias(tl->attn_mask, 1, t, t + 1);
+    t0 = nc_masked_fill(t0, t1, -INFINITY, 0);
+    t1 = nc_soft_max(t0);
+    t0 = nc_matmul(value, nc_dup_tensor(t1));
+    node = nc_get_node(t0);
+    nc_node_set_arg(node, 1, t1);
+    nc_free_tensor(t1);
+    tl->va_nodes[t] = node;
+    return t0;
+}
+
+/* self-attention block of the reference path: nncp.c:659-890 */
+static NCTensor *attention_ref(NNCPModel *s, int l, int output_index, NCTensor *x, int seg_len)
+{
+    const NNCPConfig *c = &s->cfg;
+    Layer *tl = &s->layers[l];
+    int H = c->n_head, HDk = H * c->d_key, HDv = H * c->d_value, B = c->batch_size;
+    NCTensor *query, *key, *value, *t0;
+
+    query = nc_matmul(nc_dup_tensor(tl->w_q), nc_dup_tensor(x));
+    if (c->query_bias)
+        query = nc_add(query, nc_dup_tensor(tl->b_q));
+    t0 = nc_matmul(nc_dup_tensor(tl->w_kv), x);
+    key = nc_slice(nc_dup_tensor(t0), 0, 0, HDk);
+    value = nc_slice(t0, 0, HDk, HDk + HDv);
+    query = nc_reshape_3d(query, HDk, B, seg_len);
+    key = nc_reshape_3d(key, HDk, B, seg_len);
+    value = nc_reshape_3d(value, HDv, B, seg_len);
+
+    if (output_index <= 0) { /* keys / values of the memory, nncp.c:673-711 */
+        NCTensor *key0, *value0;
+        t0 = nc_reshape_2d(nc_dup_tensor(s->mem_h[l]), c->d_model, c->mem_len * B);
+        t0 = nc_matmul(nc_dup_tensor(tl->w_kv), t0);
+        key0 = nc_slice(nc_dup_tensor(t0), 0, 0, HDk);
+        value0 = nc_slice(t0, 0, HDk, HDk + HDv);
+        key0 = nc_reshape_3d(key0, HDk, B, c->mem_len);
+        value0 = nc_reshape_3d(value0, HDv, B, c->mem_len);
+        if (output_index < 0) {
+            NCTensor *tab[2];
+            tab[0] = key0; tab[1] = key;
+            key = nc_concat(tab, 2, 2);
+            tab[0] = value0; tab[1] = value;
+            value = nc_concat(tab, 2, 2);
+        } else {
+            NCTensor *slot = nc_slice_alias(tl->mem_key, 1, 0, c->mem_len);
+            key0 = split_head(key0, H);
+            tl->key_nodes[0] = nc_dup_node(nc_get_node(key0));
+            nc_tensor_copy(slot, key0);
+            nc_free_tensor(key0); nc_free_tensor(slot);
+            slot = nc_slice_alias(tl->mem_value, 1, 0, c->mem_len);
+            value0 = split_head(value0, H);
+            tl->value_nodes[0] = nc_dup_node(nc_get_node(value0));
+            nc_tensor_copy(slot, value0);
+            nc_free_tensor(value0); nc_free_tensor(slot);
+        }
+    }
+    key = split_head(key, H);
+    query = split_head(query, H);
+    value = split_head(value, H);
+    if (output_index <= 0)
+        build_position_tensors(s, l);
+    if (output_index < 0)
+        t0 = attention_segment_ref(s, l, query, key, value);
+    else
+        t0 = attention_timestep_ref(s, l, output_index, query, key, value);
+    if (tl->w_o) {
+        t0 = nc_matmul(nc_dup_tensor(tl->w_o), concat_head(t0));
+    } else { /* sum of the heads, nncp.c:875-890 */
+        int axis[4] = { 0, 3, 1, 2 };
+        t0 = nc_permute(t0, 4, axis);
+        t0 = nc_reduce_sum(NULL, t0, 3);
+        t0 = nc_mul(t0, scalar(s, 1.0f / sqrtf((float)H)));
+        t0 = nc_reshape_2d(t0, c->d_value, (size_t)seg_len * B);
+    }
+    return t0;
+}
+
+/* the same block through the fused entry points (full segment) */
+static NCTensor *attention_fused(NNCPModel *s, int l, NCTensor *x)
+{
+    const NNCPConfig *c = &s->cfg;
+    Layer *tl = &s->layers[l];
+    int H = c->n_head, HDk = H * c->d_key, HDv = H * c->d_value, B = c->batch_size, T = c->seg_len;
+    NCTensor *q, *kv, *kvm = NULL, *att;
+    Layer *pr = &s->layers[c->tied_w_r ? 0 : l], *pb = &s->layers[c->tied_b_r ? 0 : l];
+
+    q = nc_linear(nc_dup_tensor(tl->w_q), nc_dup_tensor(x), c->query_bias ? nc_dup_tensor(tl->b_q) : NULL, NC_ACT_NONE);
+    kv = nc_matmul(nc_dup_tensor(tl->w_kv), x);
+    if (c->mem_len > 0) {
+        kvm = nc_reshape_2d(nc_dup_tensor(s->mem_h[l]), c->d_model, (size_t)c->mem_len * B);
+        kvm = nc_matmul(nc_dup_tensor(tl->w_kv), kvm);
+        kvm = nc_reshape_3d(kvm, HDk + HDv, B, c->mem_len);
+    }
+    att = nc_relpos_attention(nc_reshape_3d(q, HDk, B, T), nc_reshape_3d(kv, HDk + HDv, B, T), kvm,
+                              c->use_w_r ? nc_dup_tensor(pr->w_r) : NULL, nc_dup_tensor(pb->b_r),
+                              H, c->d_key, c->attn_len[l], sqrtf((float)(c->d_key * c->d_model)));
+    att = nc_reshape_2d(att, HDv, (size_t)B * T);
+    if (!tl->w_o)
+        die("the fused path needs d_value != d_model (an output projection)");
+    return nc_matmul(nc_dup_tensor(tl->w_o), att);
+}
+
+/* feed-forward block: nncp.c:930-977 */
+static NCTensor *feed_forward(NNCPModel *s, int l, NCTensor *x)
+{
+    const NNCPConfig *c = &s->cfg;
+    Layer *tl = &s->layers[l];
+    NCTensor *t0, *tab[2];
+    int act = c->ff_act;
+    if (c->fused && (act == NNCP_FF_GELU || act == NNCP_FF_RELU)) {
+        t0 = nc_linear(nc_dup_tensor(tl->ff1), x, tl->ff_bias1 ? nc_dup_tensor(tl->ff_bias1) : NULL,
+                       act == NNCP_FF_GELU ? NC_ACT_GELU : NC_ACT_RELU);
+        return nc_linear(nc_dup_tensor(tl->ff2), t0, tl->ff_bias2 ? nc_dup_tensor(tl->ff_bias2) : NULL, NC_ACT_NONE);
+    }
+    t0 = nc_matmul(nc_dup_tensor(tl->ff1), x);
+    if (tl->ff_bias1)
+        t0 = nc_add(t0, nc_dup_tensor(tl->ff_bias1));
+    switch (act) {
+    case NNCP_FF_RELU: t0 = nc_relu(t0); break;
+    case NNCP_FF_GELU: t0 = nc_gelu(t0); break;
+    case NNCP_FF_GEGLU:
+        nc_split(tab, t0, 2, NULL, 0);
+        t0 = nc_mul(nc_gelu(tab[0]), tab[1]);
+        break;
+    case NNCP_FF_GATED_SILU:
+        nc_split(tab, t0, 2, NULL, 0);
+        t0 = nc_gated_swish(tab[1], tab[0], 1.0f);
+        break;
+    default: die("unknown ff_act");
+    }
+    t0 = nc_matmul(nc_dup_tensor(tl->ff2), t0);
+    if (tl->ff_bias2)
+        t0 = nc_add(t0, nc_dup_tensor(tl->ff_bias2));
+    return t0;
+}
+
+static void free_position_tensors(NNCPModel *s)
+{
+    for (int l = 0; l < s->cfg.n_layer; l++) {
+        nc_free_tensor(s->layers[l].tmp_w_r); s->layers[l].tmp_w_r = NULL;
+        nc_free_tensor(s->layers[l].tmp_b_r); s->layers[l].tmp_b_r = NULL;
+    }
+}
+
+NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
+{
+    const NNCPConfig *c = &s->cfg;
+    int seg_len, B = c->batch_size;
+    NCTensor *t0, *x, *output;
+
+    if (c->fused && output_index >= 0)
+        die("the fused path evaluates whole segments only (output_index < 0)");
+    if (output_index < 0) { /* nncp.c:612-623 */
+        t0 = nc_dup_tensor(input);
+        s->seq_eval = 0;
+        seg_len = c->seg_len;
+    } else {
+        t0 = nc_slice_alias(input, 1, output_index, output_index + 1);
+        s->seq_eval = 1;
+        seg_len = 1;
+    }
+    t0 = nc_tensor_to_device(t0, s->dev);
+    t0 = nc_reshape_1d(t0, (size_t)B * seg_len);
+    x = nc_get_col(nc_dup_tensor(s->embed), t0);
+    x = nc_mul(x, scalar(s, s->embed_mult));
+
+    for (int l = 0; l < c->n_layer; l++) {
+        Layer *tl = &s->layers[l];
+        NCTensor *x1 = nc_dup_tensor(x), *ff_in;
+        if (c->ln_flags & NNCP_LN_PRE)
+            x1 = layer_norm(s, x1, tl->ln_g1, tl->ln_b1);
+        save_layer_input(s, l, output_index, x1, seg_len);
+        t0 = c->fused ? attention_fused(s, l, x1) : attention_ref(s, l, output_index, x1, seg_len);
+        if (c->ln_flags & NNCP_LN_COEF)
+            t0 = nc_mul(t0, nc_dup_tensor(tl->alpha));
+        t0 = nc_add(t0, x); /* residual, nncp.c:896 */
+        if (c->ln_flags & NNCP_LN_POST)
+            t0 = layer_norm(s, t0, tl->ln_g1, tl->ln_b1);
+        ff_in = nc_dup_tensor(t0);
+        if (c->ln_flags & NNCP_LN_PRE)
+            t0 = layer_norm(s, t0, tl->ln_g2, tl->ln_b2);
+        t0 = feed_forward(s, l, t0);
+        if (c->ln_flags & NNCP_LN_COEF)
+            t0 = nc_mul(t0, nc_dup_tensor(tl->alpha));
+        t0 = nc_add(t0, ff_in); /* nncp.c:979 */
+        if (c->ln_flags & NNCP_LN_POST)
+            t0 = layer_norm(s, t0, tl->ln_g2, tl->ln_b2);
+        x = t0;
+    }
+    if (c->ln_flags & NNCP_LN_FINAL)
+        x = layer_norm(s, x, s->ln_g, s->ln_b);
+    /* logits and probabilities, nncp.c:1001-1009 */
+    if (c->fused) {
+        t0 = nc_linear(nc_dup_tensor(s->embed_out), x, s->out_bias ? nc_dup_tensor(s->out_bias) : NULL, NC_ACT_NONE);
+    } else {
+        t0 = nc_matmul(nc_dup_tensor(s->embed_out), x);
+        if (s->out_bias)
+            t0 = nc_add(t0, nc_dup_tensor(s->out_bias));
+    }
+    t0 = nc_reshape_3d(t0, c->n_symbols, B, seg_len);
+    nc_free_tensor(s->logits);
+    s->logits = nc_dup_tensor(t0);
+    output = nc_soft_max(t0);
+    if (s->outputs[output_index < 0 ? 0 : output_index])
+        die("trf_eval: previous evaluation not consumed (call trf_eval_gradient or trf_eval_end)");
+    s->outputs[output_index < 0 ? 0 : output_index] = nc_dup_tensor(output);
+    if (!c->fused && (output_index < 0 || output_index == c->seg_len - 1))
+        free_position_tensors(s);
+    return output;
+}
+
+NCTensor *trf_last_logits(NNCPModel *s) { return s->logits; }
+
+void trf_eval_end(NNCPModel *s) /* nncp.c:1032-1060 */
+{
+    free_position_tensors(s);
+    for (int l = 0; l < s->cfg.n_layer; l++) {
+        Layer *tl = &s->layers[l];
+        for (int i = 0; i <= s->cfg.seg_len; i++) {
+            nc_free_node(tl->key_nodes[i]); tl->key_nodes[i] = NULL;
+            nc_free_node(tl->value_nodes[i]); tl->value_nodes[i] = NULL;
+        }
+    }
+    for (int i = 0; i < s->cfg.seg_len; i++) {
+        nc_free_tensor(s->outputs[i]);
+        s->outputs[i] = NULL;
+    }
+    nc_free_tensor(s->logits);
+    s->logits = NULL;
+}
+
+static void backward_cb(void *opaque, NCTensor *yg, NCTensor *get_col_index) /* nncp.c:1078-1096 */
+{
+    sgd_opt_update_var(opaque, yg, get_col_index);
+}
+
+/* route the gradients of the T per-timestep products into one concatenated
+   key (value) tensor: nncp.c:1116-1158 */
+static NCNode *merge_timestep_nodes(NNCPModel *s, NCNode **src, NCNode **consumers)
+{
+    int T = s->cfg.seg_len;
+    size_t *ones = nc_malloc(sizeof(size_t) * T), two[2] = { (size_t)s->cfg.mem_len, (size_t)T };
+    NCNode *n, *n1, *pair[2];
+    for (int i = 0; i < T; i++)
+        ones[i] = 1;
+    n = nc_concat_node(s->ctx, src + 1, T, 1, ones);
+    pair[0] = src[0]; pair[1] = n;
+    n1 = nc_concat_node(s->ctx, pair, 2, 1, two);
+    for (int i = 0; i <= T; i++) {
+        nc_free_node(src[i]);
+        src[i] = NULL;
+    }
+    for (int i = 0; i < T; i++)
+        nc_node_set_parent(consumers[i], 0, n1);
+    nc_free_node(n);
+    nc_free_node(n1);
+    nc_free(ones);
+    return n;
+}
+
+float trf_eval_gradient(NNCPModel *s, const NCTensor *expected_output1) /* nncp.c:1099-1193 */
+{
+    const NNCPConfig *c = &s->cfg;
+    NCTensor *expected = nc_tensor_to_device(nc_dup_tensor(expected_output1), s->dev);
+    NCTensor *output, *loss;
+    float ret;
+    if (s->seq_eval) {
+        NCNode **tab = nc_malloc(sizeof(NCNode *) * (c->n_layer * 2 + 1));
+        int count = 0;
+        for (int l = 0; l < c->n_layer; l++) {
+            Layer *tl = &s->layers[l];
+            tab[count++] = merge_timestep_nodes(s, tl->key_nodes, tl->kq_nodes);
+            tab[count++] = merge_timestep_nodes(s, tl->value_nodes, tl->va_nodes);
+        }
+        output = nc_concat(s->outputs, c->seg_len, 2);
+        for (int i = 0; i < c->seg_len; i++)
+            s->outputs[i] = NULL;
+        tab[count++] = nc_get_node(output);
+        nc_concat_optimization(s->ctx, tab, count);
+        nc_free(tab);
+    } else {
+        output = s->outputs[0];
+        s->outputs[0] = NULL;
+    }
+    loss = nc_indexed_log(output, nc_dup_tensor(expected));
+    nc_free_tensor(expected);
+    loss = nc_sum(loss);
+    ret = nc_get_scalar_f32(loss);
+    loss = nc_mul(loss, nc_new_f32(nc_get_tensor_device(loss), -1.0f / (float)(c->seg_len * c->batch_size)));
+    nc_backward(loss, nc_new_f32(s->dev, 1.0f), backward_cb, 0);
+    nc_free_tensor(loss);
+    nc_free_tensor(s->logits);
+    s->logits = NULL;
+    return ret;
+}
+
+void trf_reset(NNCPModel *s) /* nncp.c:1195-1203 */
+{
+    for (int l = 0; l < s->cfg.n_layer; l++)
+        nc_tensor_set_zero(s->mem_h[l]);
+}
+
+void trf_update(NNCPModel *s) /* nncp.c:1224-1235 with mem_update nncp.c:1205-1221 */
+{
+    int M = s->cfg.mem_len, T = s->cfg.seg_len;
+    nc_sgd_opt_update(s->opt);
+    for (int l = 0; l < s->cfg.n_layer && M > 0; l++) {
+        if (M > T) {
+            nc_tensor_copy_slice(s->mem_h[l], s->mem_h[l], 2, 0, M - T, T);
+            nc_tensor_copy_slice(s->mem_h[l], s->train_h[l], 2, M - T, M, 0);
+        } else {
+            nc_tensor_copy_slice(s->mem_h[l], s->train_h[l], 2, 0, M, T - M);
+        }
+    }
+    s->train_step++;
+}
+
+void trf_set_lr(NNCPModel *s, float lr) { nc_sgd_opt_set_lr(s->opt, lr); }

@@ -1,0 +1,73 @@
+"""Helpers shared by the model-level tests: configurations, seeded data."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from conftest import ROOT, REF_LIB, load_pkg
+
+HOST_REF = os.path.join(ROOT, "oracle", "libnncp_host_ref.so")
+
+TINY = dict(n_layer=2, d_model=32, n_head=2, d_inner=64, d_pos=12, mem_len=8, seg_len=8,
+            batch_size=3, n_symbols=40, seed=7)
+# BASELINE config 1 (2 layers, d_model 128, 4 heads x 32, d_ff 512, T = M = 20, batch 4)
+C1 = dict(n_layer=2, d_model=128, n_head=4, d_inner=512, d_pos=40, mem_len=20, seg_len=20,
+          batch_size=4, n_symbols=256, seed=123)
+
+
+def ref_host():
+    pkg = load_pkg()
+    return pkg.host.Host(HOST_REF, REF_LIB)
+
+
+def hip_host():
+    pkg = load_pkg()
+    return pkg.host.Host()
+
+
+def rmsprop(lr=3e-4):
+    B = load_pkg().binding
+    return B.SGDOptParams(algo=B.SGD_OPT_RMSPROP, beta1=0.0, beta2=0.99, eps=1e-8, gradient_clip=0.0, lr=lr)
+
+
+def sgd(lr):
+    B = load_pkg().binding
+    return B.SGDOptParams(algo=B.SGD_OPT_BASIC, lr=lr)
+
+
+def markov1(n, n_symbols=256, seed=1234, s=1.1):
+    """Order-1 Markov source, each row Zipf(s) over a seeded permutation
+    (BASELINE config 1 data)."""
+    rng = np.random.default_rng(seed)
+    ranks = np.arange(1, n_symbols + 1, dtype=np.float64) ** -s
+    ranks /= ranks.sum()
+    cum = np.cumsum(ranks)
+    perms = np.stack([rng.permutation(n_symbols) for _ in range(n_symbols)])
+    u = rng.random(n)
+    out = np.zeros(n, dtype=np.uint16)
+    cur = 0
+    for i in range(n):
+        r = int(np.searchsorted(cum, u[i]))
+        cur = perms[cur, min(r, n_symbols - 1)]
+        out[i] = cur
+    return out
+
+
+def relerr(a, b):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return float(np.abs(a - b).max() / (np.abs(b).max() + 1e-30))
+
+
+def segment_batches(syms, B, T, n_steps):
+    """(tokens, targets) pairs laid out as process_block does for a block that
+    is an exact multiple of B*T: stream b owns syms[b*stride:(b+1)*stride]."""
+    stride = len(syms) // B
+    st = syms[:stride * B].reshape(B, stride).astype(np.int32)
+    out = []
+    for k in range(n_steps):
+        tgt = st[:, k * T:(k + 1) * T]                       # (B, T)
+        prev = np.concatenate([np.zeros((B, 1), np.int32) if k == 0 else st[:, k * T - 1:k * T],
+                               tgt[:, :-1]], axis=1)
+        out.append((prev.T.copy(), tgt.T.copy()))            # numpy (T, B)
+    return out
