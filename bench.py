@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path: NNCP's online train+code step on one MI355X.
+
+Workload (BASELINE.json configs[2]): Transformer-XL, 12 layers, d_model 512,
+8 heads x 64, d_ff 2048, seg_len 64, mem_len 64, batch 32 streams, 256 symbols,
+RMSProp (beta 0.99, eps 1e-8, lr 3e-4); data: a prefix of the seeded order-3
+Markov byte stream whose contexts draw next-byte distributions from
+Dirichlet(0.05); weights N(0, 0.02), seeded.
+
+One step = one batch of 32 x 64 = 2048 symbols through the whole path:
+whole-segment forward (fused HIP ops) -> logits -> 16-bit integer CDF on the
+GPU -> copy to pinned host memory -> host range coder (integer symbol coder)
+-> backward -> RMSProp update + memory shift.  The emitted stream is decodable
+(tests/test_gpu_model.py round-trips the same code path).
+
+Prints ONE JSON line (see the field list at the bottom).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+C3 = dict(n_layer=12, d_model=512, n_head=8, d_inner=2048, d_pos=128, mem_len=64, seg_len=64,
+          batch_size=32, n_symbols=256, seed=123)
+PEAK_TFLOPS = {"fp32": 157.3, "bf16": 2500.0}
+
+
+def markov3_dirichlet(n, seed=2024, alpha=0.05, n_symbols=256):
+    """Order-3 Markov source: every visited 3-symbol context draws its next-
+    symbol pmf from Dirichlet(alpha), lazily, seeded by (context, seed)."""
+    out = np.zeros(n, dtype=np.uint16)
+    cache = {}
+    rng = np.random.default_rng(seed)
+    u = rng.random(n)
+    ctx = (0, 0, 0)
+    for i in range(n):
+        cdf = cache.get(ctx)
+        if cdf is None:
+            h = (ctx[0] * 65536 + ctx[1] * 256 + ctx[2]) ^ (seed * 2654435761 & 0xffffffff)
+            p = np.random.default_rng(h).dirichlet(np.full(n_symbols, alpha))
+            cdf = np.cumsum(p)
+            cache[ctx] = cdf
+        s = min(int(np.searchsorted(cdf, u[i] * cdf[-1])), n_symbols - 1)
+        out[i] = s
+        ctx = (ctx[1], ctx[2], s)
+    return out
+
+
+def init_weights(model, seed=99, sigma=0.02):
+    """N(0, sigma) for every matrix, 1 for LayerNorm gains, 0 for biases."""
+    rng = np.random.default_rng(seed)
+    for name in model.param_names():
+        w = model.get_param(name)
+        if name.startswith("ln_g"):
+            new = np.ones_like(w)
+        elif w.ndim >= 2 and not name.startswith("b_r"):
+            new = rng.normal(0.0, sigma, size=w.shape).astype(np.float32)
+        else:
+            new = np.zeros_like(w)
+        model.set_param(name, new)
+
+
+def run_block(model, H, syms, mode):
+    """Codes syms (a multiple of B*T) as one block; returns (seconds, bytes, stats)."""
+    cap = syms.size * 4 + 4096
+    out = np.zeros(cap, dtype=np.uint8)
+    st = H.NNCPStats()
+    sched = H.constant_lr(3e-4)
+    model.nc.nc_synchronize(model.dev)
+    t0 = time.perf_counter()
+    n = model.L.nncp_compress(model.ptr, syms.ctypes.data, syms.size, out.ctypes.data, cap, mode,
+                              C.byref(sched), C.byref(st))
+    model.nc.nc_synchronize(model.dev)
+    return time.perf_counter() - t0, n, st
+
+
+def gemm_profile(model, H, syms, mode, hip_lib):
+    """Times every GEMM launch of a few extra steps with HIP events on the
+    launch stream; returns the per-instantiation rows."""
+    lib = C.CDLL(hip_lib)
+    lib.nchip_gemm_profile_enable(1)
+    run_block(model, H, syms, mode)
+    lib.nchip_gemm_profile_enable(0)
+    names = ((C.c_char * 48) * 16)()
+    launches = (C.c_int64 * 16)()
+    flops = (C.c_double * 16)()
+    secs = (C.c_double * 16)()
+    lib.nchip_gemm_profile_read.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    n = lib.nchip_gemm_profile_read(16, names, launches, flops, secs)
+    rows = []
+    for i in range(n):
+        rows.append(dict(kernel=names[i].value.decode(), launches=int(launches[i]),
+                         flops=float(flops[i]), seconds=float(secs[i])))
+    return rows
+
+
+def cpu_baseline(pkg, data, n_steps, threads):
+    """The CPU checker driving the reference op sequence (whole-segment
+    evaluation, float symbol coder: what `nncp --encode_only` does) on the
+    host cores, on the first n_steps batches of the same workload."""
+    H = pkg.host
+    host = H.Host(os.path.join(ROOT, "oracle", "libnncp_host_ref.so"),
+                  os.path.join(ROOT, "oracle", "libnc_ref.so"))
+    opt = pkg.binding.SGDOptParams(algo=pkg.binding.SGD_OPT_RMSPROP, beta2=0.99, eps=1e-8, lr=3e-4)
+    m = H.Model(host, H.make_config(**dict(C3, use_device=0, fused=0, nb_threads=threads, sgd_opt=opt)))
+    init_weights(m)
+    n = n_steps * C3["batch_size"] * C3["seg_len"]
+    sec, _, _ = run_block(m, H, data[:n], H.MODE_SEGMENT | H.CODER_FLOAT)
+    m.close()
+    return n / sec
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--variant", choices=["fp32", "bf16"], default="fp32")
+    ap.add_argument("--cpu-steps", type=int, default=2, help="0 skips the CPU baseline")
+    ap.add_argument("--profile-steps", type=int, default=2)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (one compression job per GPU, no "
+                 "collectives); run it with --gpus 1")
+
+    import __graft_entry__ as G
+    pkg = G._load_pkg()
+    H = pkg.host
+    if not os.path.exists(H.HOST_HIP_LIB) or not os.path.exists(pkg.binding.HIP_LIB):
+        G.build()
+    B, T = C3["batch_size"], C3["seg_len"]
+    per_step = B * T
+    total_steps = args.warmup + args.steps + args.profile_steps
+    data = markov3_dirichlet(max(total_steps, args.cpu_steps) * per_step)
+
+    opt = pkg.binding.SGDOptParams(algo=pkg.binding.SGD_OPT_RMSPROP, beta2=0.99, eps=1e-8, lr=3e-4)
+    model = H.Model(H.Host(), H.make_config(**dict(C3, use_device=1, fused=1, sgd_opt=opt)))
+    init_weights(model)
+    model.nc.nc_set_matmul_bf16(model.ctx, 1 if args.variant == "bf16" else 0)
+    mode = H.MODE_SEGMENT | H.CODER_CDF16
+
+    pos = 0
+    if args.warmup:
+        run_block(model, H, data[pos:pos + args.warmup * per_step], mode)
+        pos += args.warmup * per_step
+    l0 = model.nc.nc_get_launch_count(model.ctx)
+    sec, nbytes, st = run_block(model, H, data[pos:pos + args.steps * per_step], mode)
+    launches = model.nc.nc_get_launch_count(model.ctx) - l0
+    pos += args.steps * per_step
+    value = args.steps * per_step / sec
+
+    roof = None
+    if args.profile_steps:
+        rows = gemm_profile(model, H, data[pos:pos + args.profile_steps * per_step], mode,
+                            pkg.binding.HIP_LIB)
+        if rows:
+            dom = max(rows, key=lambda r: r["seconds"])
+            achieved = dom["flops"] / dom["seconds"] / 1e12
+            peak = PEAK_TFLOPS[args.variant]
+            tot_f = sum(r["flops"] for r in rows)
+            tot_s = sum(r["seconds"] for r in rows)
+            roof = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 3),
+                    "peak": peak, "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
+                    "traffic": None,
+                    "launches_per_step": dom["launches"] / args.profile_steps,
+                    "avg_launch_us": round(dom["seconds"] / dom["launches"] * 1e6, 2),
+                    "flops_per_launch": dom["flops"] / dom["launches"],
+                    "all_gemm_tflops": round(tot_f / tot_s / 1e12, 3),
+                    "all_gemm_ms_per_step": round(tot_s / args.profile_steps * 1e3, 3)}
+    model.close()
+
+    cpu = None
+    if args.cpu_steps:
+        threads = min(os.cpu_count() or 1, 16)
+        v = cpu_baseline(pkg, data, args.cpu_steps, threads)
+        cpu = {"value": round(v, 1), "unit": "symbols/s", "cores": threads, "kind": "port",
+               "sample": "first %d steps (%d symbols) of the same workload, CPU checker driving the "
+                         "reference op sequence, whole-segment evaluation, float symbol coder"
+                         % (args.cpu_steps, args.cpu_steps * per_step)}
+
+    print(json.dumps({
+        "metric": "symbols/sec compressed (train+code) 12L d512",
+        "value": round(value, 1), "unit": "symbols/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(sec / args.steps * 1e3, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if args.variant == "fp32" else "bf16-in/f32-acc", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[2]: 12L d512 8x64 ff2048 T64 M64 B32 V256, RMSProp, "
+                               "order-3 Markov Dirichlet(0.05) prefix, weights N(0,0.02)",
+                   "symbols_per_step": per_step, "coder": "gpu cdf16 + host range coder",
+                   "variant": args.variant},
+        "bits_per_symbol": round(nbytes * 8 / (args.steps * per_step), 4),
+        "kernel_launches_per_step": launches / args.steps,
+        "host_seconds": {"eval_and_copy": round(st.t_eval, 4), "code": round(st.t_code, 4),
+                         "grad": round(st.t_grad, 4), "update": round(st.t_update, 4)},
+        "roofline": roof, "cpu_baseline": cpu}))
+
+
+if __name__ == "__main__":
+    main()

@@ -53,6 +53,15 @@ int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, float alpha,
                 const float *bias, int act, float *pre, int precision,
                 int ksplit, float *workspace);
 
+/* Optional timing of every GEMM launch with HIP events recorded on the launch
+   stream.  After nchip_gemm_profile_enable(1), each nchip_gemm* call is
+   bracketed by an event pair; nchip_gemm_profile_read waits for them, sums
+   launches / flops (2*m*n*k*batch) / seconds per kernel instantiation, fills up
+   to max_variants rows and clears the records.  Returns the row count. */
+void nchip_gemm_profile_enable(int on);
+int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launches,
+                            double *flops, double *seconds);
+
 /* Chooses ksplit for nchip_gemm from the shape alone (never from data). */
 int nchip_gemm_pick_ksplit(int m, int n, int k, int batch);
 

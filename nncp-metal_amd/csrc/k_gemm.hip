@@ -18,6 +18,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <string.h>
+#include <vector>
 #include "../../include/nchip_kernels.h"
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -323,6 +325,15 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce(GemmArgs g)
     }
 }
 
+// ---- optional per-launch timing (HIP events on the launch stream) ----------
+struct ProfRec {
+    hipEvent_t start, stop;
+    int variant;
+    double flops;
+};
+bool g_prof_on = false;
+std::vector<ProfRec> g_prof;
+
 template <int BM, int BN, int BF16>
 void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g)
 {
@@ -387,12 +398,24 @@ extern "C" int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, fl
     // tile choice from the shape only: large tiles when they still fill the chip
     int64_t t128 = (int64_t)((m + 127) / 128) * ((n + 127) / 128) * batch * ksplit;
     bool big = (t128 >= 256) && m >= 128 && n >= 128;
+    ProfRec rec;
+    if (g_prof_on) {
+        (void)hipEventCreate(&rec.start);
+        (void)hipEventCreate(&rec.stop);
+        rec.variant = (big ? 8 : 0) | (ta ? 4 : 0) | (tb ? 2 : 0) | (precision == 1 ? 1 : 0);
+        rec.flops = 2.0 * m * n * (double)k * batch;
+        (void)hipEventRecord(rec.start, st);
+    }
     if (precision == 1) {
         if (big) launch_tile<128, 128, 1>(st, ta, tb, g);
         else launch_tile<64, 64, 1>(st, ta, tb, g);
     } else {
         if (big) launch_tile<128, 128, 0>(st, ta, tb, g);
         else launch_tile<64, 64, 0>(st, ta, tb, g);
+    }
+    if (g_prof_on) {
+        (void)hipEventRecord(rec.stop, st);
+        g_prof.push_back(rec);
     }
     if (ksplit > 1) {
         int64_t total = (int64_t)m * n;
@@ -418,4 +441,37 @@ extern "C" int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, flo
     return nchip_gemm2(stream, ta, tb, m, n, k, alpha, A, lda, stride_a, 0, B, ldb, stride_b, 0,
                        beta, C, ldc, stride_c, 0, batch, 1, bias, act, pre, precision, ksplit,
                        workspace);
+}
+
+// ---- profiling entry points ---------------------------------------------------
+extern "C" void nchip_gemm_profile_enable(int on)
+{
+    g_prof_on = on != 0;
+}
+
+extern "C" int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launches,
+                                       double *flops, double *seconds)
+{
+    double fl[16] = { 0 }, sec[16] = { 0 };
+    int64_t cnt[16] = { 0 };
+    for (ProfRec &r : g_prof) {
+        float ms = 0.0f;
+        (void)hipEventSynchronize(r.stop);
+        (void)hipEventElapsedTime(&ms, r.start, r.stop);
+        fl[r.variant] += r.flops;
+        sec[r.variant] += ms * 1e-3;
+        cnt[r.variant]++;
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+    }
+    g_prof.clear();
+    int n = 0;
+    for (int v = 0; v < 16 && n < max_variants; v++) {
+        if (!cnt[v]) continue;
+        int bt = (v & 8) ? 128 : 64;
+        snprintf(names[n], 48, "gemm_kernel<%d,%d,%d,%d,%d>", bt, bt, (v >> 2) & 1, (v >> 1) & 1, v & 1);
+        launches[n] = cnt[v]; flops[n] = fl[v]; seconds[n] = sec[v];
+        n++;
+    }
+    return n;
 }

@@ -71,3 +71,20 @@ def segment_batches(syms, B, T, n_steps):
                                tgt[:, :-1]], axis=1)
         out.append((prev.T.copy(), tgt.T.copy()))            # numpy (T, B)
     return out
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return float(np.linalg.norm(a - b) / (np.linalg.norm(b) + 1e-30))
+
+
+def tensors_close(a, b, tol=1e-5, max_factor=30):
+    """Agreement bar for gradient and weight tensors: relative L2 error <= tol.
+    The max-norm error is only bounded by max_factor*tol: single elements that
+    are sums of cancelling terms (tiny gradients), and weights moved by the
+    sign-like RMSProp update lr*g/(sqrt(v)+eps) of such elements, differ by
+    fp32 re-ordering noise that is large relative to the element but not to
+    the tensor (measured: gradients <= 5.4e-5, weights after 10 steps
+    <= 2.3e-4 max-norm, all <= 7.8e-6 in relative L2)."""
+    return rel_l2(a, b) <= tol and relerr(a, b) <= max_factor * tol
