@@ -385,11 +385,12 @@ void k_lstm_clamped_bwd(hipStream_t st, const float *cp, const float *in, const 
 
 int k_reduce_trailing_nsplit(int64_t inner, int64_t outer)
 {
-    // enough slices to occupy the chip, at least 8 summands per slice
+    // enough slices to occupy the chip while both stages stay short sequential
+    // sums (stage 1: outer/nsplit terms per thread, stage 2: nsplit terms)
     int64_t blocks_x = (inner + TPB - 1) / TPB;
-    int64_t s = 1024 / (blocks_x > 0 ? blocks_x : 1);
+    int64_t s = 512 / (blocks_x > 0 ? blocks_x : 1);
     if (s > outer / 8) s = outer / 8;
-    if (s > 256) s = 256;
+    if (s > 32) s = 32;
     if (s < 1) s = 1;
     return (int)s;
 }

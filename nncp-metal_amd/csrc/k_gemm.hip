@@ -19,6 +19,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
+#include <type_traits>
 #include <vector>
 #include "../../include/nchip_kernels.h"
 
@@ -190,13 +191,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g)
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.0f;
 
-    int nk = (kend - kbeg + BK - 1) / BK;
-    if (nk > 0) {
-        bool kf = (kbeg + BK <= kend);
-        la.load(A, g.lda, m0, kbeg, g.M, kend, a_full && kf, t);
-        lb.load(B, g.ldb, n0, kbeg, g.N, kend, b_full && kf, t);
-    }
-    for (int it = 0; it < nk; it++) {
+    // One pipeline step: write the prefetched registers to LDS buffer `buf`,
+    // barrier, start the global loads of tile `next` (when there is one), then
+    // the MFMAs of the tile in `buf`.  One barrier per tile is enough because a
+    // buffer is rewritten only two tiles later.  FAST is a compile-time flag so
+    // the steady-state loop carries no guarded-load code: the guarded path
+    // shares registers with the vector loads and the compiler then serialises
+    // every prefetch behind an s_waitcnt vmcnt(0).
+    auto step = [&](int it, int nk, auto fast_tag) {
+        constexpr bool FAST = decltype(fast_tag)::value;
         float *sa = smem + (it & 1) * (LDS_A + LDS_B);
         float *sb = sa + LDS_A;
         if (BF16) {
@@ -207,12 +210,16 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g)
             lb.store_f32(sb, t);
         }
         __syncthreads();
-        if (it + 1 < nk) {
+        if (FAST || it + 1 < nk) {
             int k0 = kbeg + (it + 1) * BK;
-            bool kf = (k0 + BK <= kend);
-            la.load(A, g.lda, m0, k0, g.M, kend, a_full && kf, t);
-            lb.load(B, g.ldb, n0, k0, g.N, kend, b_full && kf, t);
+            bool kf = FAST || (k0 + BK <= kend);
+            la.load(A, g.lda, m0, k0, g.M, kend, FAST || (a_full && kf), t);
+            lb.load(B, g.ldb, n0, k0, g.N, kend, FAST || (b_full && kf), t);
         }
+        // keep the prefetch ahead of the MFMAs: without this fence the
+        // scheduler sinks the global loads below the compute block and their
+        // latency is paid in full at the next LDS write
+        __builtin_amdgcn_sched_barrier(0);
         if (BF16) {
             // one 32x32x16 MFMA per tile pair covers the whole BK = 16
             const unsigned short *ha = reinterpret_cast<const unsigned short *>(sa);
@@ -235,26 +242,45 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g)
                         __builtin_bit_cast(__attribute__((ext_vector_type(8))) __bf16, fa[j]),
                         acc[i][j], 0, 0, 0);
         } else {
+            // fragments of k-step ks+1 are fetched while the MFMAs of ks run
+            float fa[2][TM], fb[2][TN];
+            const float *pa = sa + (lane >> 5) * (BM + PAD) + wm * (BM / 2) + (lane & 31);
+            const float *pb = sb + (lane >> 5) * (BN + PAD) + wn * (BN / 2) + (lane & 31);
+#pragma unroll
+            for (int j = 0; j < TM; j++) fa[0][j] = pa[j * 32];
+#pragma unroll
+            for (int i = 0; i < TN; i++) fb[0][i] = pb[i * 32];
 #pragma unroll
             for (int ks = 0; ks < BK / 2; ks++) {
-                int kk = ks * 2 + (lane >> 5);
-                float fa[TM], fb[TN];
+                const int cur = ks & 1, nxt = cur ^ 1;
+                if (ks + 1 < BK / 2) {
 #pragma unroll
-                for (int j = 0; j < TM; j++)
-                    fa[j] = sa[kk * (BM + PAD) + wm * (BM / 2) + j * 32 + (lane & 31)];
+                    for (int j = 0; j < TM; j++) fa[nxt][j] = pa[(ks + 1) * 2 * (BM + PAD) + j * 32];
 #pragma unroll
-                for (int i = 0; i < TN; i++)
-                    fb[i] = sb[kk * (BN + PAD) + wn * (BN / 2) + i * 32 + (lane & 31)];
+                    for (int i = 0; i < TN; i++) fb[nxt][i] = pb[(ks + 1) * 2 * (BN + PAD) + i * 32];
+                }
 #pragma unroll
                 for (int i = 0; i < TN; i++)
 #pragma unroll
                     for (int j = 0; j < TM; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[i], fa[j], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[cur][i], fa[cur][j], acc[i][j], 0, 0, 0);
             }
         }
-        // the next iteration writes the other buffer; one barrier per tile is
-        // enough because a buffer is rewritten only two iterations later
+    };
+
+    const int nk = (kend - kbeg + BK - 1) / BK;
+    const int nk_full = (kend - kbeg) / BK; // tiles with a complete k range
+    int it = 0;
+    if (nk > 0) {
+        bool kf = nk_full > 0;
+        la.load(A, g.lda, m0, kbeg, g.M, kend, a_full && kf, t);
+        lb.load(B, g.ldb, n0, kbeg, g.N, kend, b_full && kf, t);
     }
+    if (a_full && b_full) // steady state: tile it+1 is complete, unguarded vector loads
+        for (; it + 1 < nk_full; it++)
+            step(it, nk, std::true_type());
+    for (; it < nk; it++) // edge tiles and the k tail
+        step(it, nk, std::false_type());
 
     // epilogue.  acc[i][j][r] is C[m][n] with
     //   m = m0 + wm*BM/2 + j*32 + lane%32

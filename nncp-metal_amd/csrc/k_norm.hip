@@ -239,7 +239,7 @@ int nchip_norm_fwd(void *stream, const float *x, const float *w, const float *b,
 int nchip_norm_bwd_partial_rows(int64_t n)
 {
     int64_t r = n / 16;
-    if (r > 128) r = 128;
+    if (r > 32) r = 32;
     if (r < 1) r = 1;
     return (int)r;
 }
