@@ -88,12 +88,12 @@ def gemm_profile(model, H, syms, mode, hip_lib):
     lib.nchip_gemm_profile_enable(1)
     run_block(model, H, syms, mode)
     lib.nchip_gemm_profile_enable(0)
-    names = ((C.c_char * 48) * 16)()
-    launches = (C.c_int64 * 16)()
-    flops = (C.c_double * 16)()
-    secs = (C.c_double * 16)()
+    names = ((C.c_char * 48) * 24)()
+    launches = (C.c_int64 * 24)()
+    flops = (C.c_double * 24)()
+    secs = (C.c_double * 24)()
     lib.nchip_gemm_profile_read.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
-    n = lib.nchip_gemm_profile_read(16, names, launches, flops, secs)
+    n = lib.nchip_gemm_profile_read(24, names, launches, flops, secs)
     rows = []
     for i in range(n):
         rows.append(dict(kernel=names[i].value.decode(), launches=int(launches[i]),

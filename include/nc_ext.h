@@ -69,6 +69,15 @@ float nc_exp_det(float x);
    Returns the previous setting.  libnc_ref.so emulates the same rounding. */
 int nc_set_matmul_bf16(NCContext *m, int enable);
 
+/* When non-zero, nc_backward() postpones the weight-gradient GEMMs
+   dW = dY X^T of plain linear layers (weight used once in the graph) and runs
+   them all in one grouped launch just before it returns.  The gradient
+   tensors passed to the NCParamUpdateFunc for those parameters then hold valid
+   data only after nc_backward() has returned - fine for callbacks that just
+   forward to sgd_opt_update_var (nncp.c:1078-1096).  Returns the previous
+   setting.  No effect in libnc_ref.so. */
+int nc_set_deferred_weight_grad(NCContext *m, int enable);
+
 /* Number of kernel launches issued so far (0 in libnc_ref.so). */
 int64_t nc_get_launch_count(NCContext *m);
 

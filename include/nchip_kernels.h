@@ -53,6 +53,24 @@ int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, float alpha,
                 const float *bias, int act, float *pre, int precision,
                 int ksplit, float *workspace);
 
+/* Many independent GEMMs C_p = alpha_p * op(A_p) * op(B_p) in ONE launch (same
+   transposition flags, 128x128 tiles, no bias/activation, beta = 0).  The
+   weight-gradient GEMMs dW = dY X^T of a whole backward pass are issued this
+   way: each is too small to fill 256 CUs on its own.  dev_table lives in
+   device memory; tile_start is the running sum of
+   nchip_gemm_grouped_tiles(m, n) over the preceding problems. */
+typedef struct {
+    const float *A, *B;
+    float *C;
+    int m, n, k;
+    int lda, ldb, ldc;
+    int tile_start;
+    float alpha;
+} NchipGemmProblem;
+int nchip_gemm_grouped_tiles(int m, int n);
+int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmProblem *dev_table,
+                       int n_problems, int total_tiles, int precision);
+
 /* Optional timing of every GEMM launch with HIP events recorded on the launch
    stream.  After nchip_gemm_profile_enable(1), each nchip_gemm* call is
    bracketed by an event pair; nchip_gemm_profile_read waits for them, sums
@@ -128,6 +146,22 @@ int nchip_add_col(void *stream, const float *g, const int32_t *idx, float *dw, i
 int nchip_opt_update(void *stream, int algo, float *w, float *m, float *v, const float *g,
                      int64_t n, float lr, float beta1, float beta2, float eps, float clip,
                      float c1, float c2);
+
+/* The same update for many parameter tensors in ONE launch (the optimiser is
+   pure bandwidth: 16 B per parameter for RMSProp).  dev_table[n_tensors] and
+   dev_chunk_prefix[n_tensors + 1] live in device memory; tensor i owns the
+   workgroups chunk_prefix[i] .. chunk_prefix[i+1]-1, each covering `chunk`
+   consecutive elements.  m may be NULL (beta1 == 0), v may be NULL (SGD). */
+typedef struct {
+    float *w, *m, *v;
+    const float *g;
+    int64_t n;
+    float lr;
+    int pad_;
+} NchipOptTensor;
+int nchip_opt_update_multi(void *stream, int algo, const NchipOptTensor *dev_table,
+                           const int *dev_chunk_prefix, int n_tensors, int total_chunks, int chunk,
+                           float beta1, float beta2, float eps, float clip, float c1, float c2);
 
 /* logits (v, n) f32 -> cdf (v, n) u16 as specified in nc_ext.h
    (nc_soft_max_cdf16); bit-identical to the CPU checker. */

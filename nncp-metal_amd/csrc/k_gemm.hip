@@ -18,6 +18,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 #include <type_traits>
 #include <vector>
@@ -29,7 +30,7 @@ typedef short shortx8 __attribute__((ext_vector_type(8)));
 
 namespace {
 
-constexpr int BK = 16;
+constexpr int KALIGN = 16; // split-K chunk granularity
 constexpr int PAD = 4;   // keeps 16-byte alignment of LDS rows, staggers banks
 constexpr int NXCD = 8;
 
@@ -46,6 +47,8 @@ struct GemmArgs {
     float alpha, beta;
     int act;
     int tiles_m, tiles_n;
+    const NchipGemmProblem *grp; // grouped launch: one problem per table row
+    int n_grp;
 };
 
 __device__ __forceinline__ float gelu_tanh(float x)
@@ -72,9 +75,10 @@ __device__ __forceinline__ unsigned short f32_to_bf16(float f)
 // MAJOR = 1: the tile's long axis (m or n) is contiguous in memory
 //            (A with ta = 0, B with tb = 1);  element (i, k) at p[i + k*ld].
 // MAJOR = 0: k is contiguous (A with ta = 1, B with tb = 0); (i, k) at p[k + i*ld].
-template <int BT, int MAJOR>
+template <int BT, int BK, int MAJOR, int NT>
 struct TileLoader {
-    static constexpr int NV = BT * BK / 4 / 256; // float4 per thread
+    static constexpr int NV = BT * BK / 4 / NT; // float4 per thread
+    static_assert(NV >= 1 && NV * NT * 4 == BT * BK, "tile must divide evenly over the threads");
     floatx4 r[NV];
 
     __device__ __forceinline__ void load(const float *p, int64_t ld, int i0, int k0,
@@ -82,7 +86,7 @@ struct TileLoader {
     {
 #pragma unroll
         for (int v = 0; v < NV; v++) {
-            int idx = t + v * 256;
+            int idx = t + v * NT;
             int i, k;
             if (MAJOR) { i = (idx % (BT / 4)) * 4; k = idx / (BT / 4); }
             else       { i = idx % BT;             k = (idx / BT) * 4; }
@@ -111,7 +115,7 @@ struct TileLoader {
     {
 #pragma unroll
         for (int v = 0; v < NV; v++) {
-            int idx = t + v * 256;
+            int idx = t + v * NT;
             if (MAJOR) {
                 int i = (idx % (BT / 4)) * 4, k = idx / (BT / 4);
                 *reinterpret_cast<floatx4 *>(lds + k * (BT + PAD) + i) = r[v];
@@ -130,7 +134,7 @@ struct TileLoader {
     {
 #pragma unroll
         for (int v = 0; v < NV; v++) {
-            int idx = t + v * 256;
+            int idx = t + v * NT;
             if (MAJOR) {
                 int i = (idx % (BT / 4)) * 4, k = idx / (BT / 4);
 #pragma unroll
@@ -146,23 +150,43 @@ struct TileLoader {
     }
 };
 
-template <int BM, int BN, int TA, int TB, int BF16>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g)
+template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs g0)
 {
-    constexpr int TM = BM / 64, TN = BN / 64; // 32x32 MFMA tiles per wavefront
+    GemmArgs g = g0;
+    constexpr int NT = 64 * WM * WN;                      // threads: WM x WN wavefronts
+    constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN); // 32x32 MFMA tiles per wavefront
+    constexpr int WTM = BM / WM, WTN = BN / WN;           // wavefront tile
     constexpr int LDS_A = BF16 ? BM * (BK + 8) / 2 : BK * (BM + PAD); // in floats
     constexpr int LDS_B = BF16 ? BN * (BK + 8) / 2 : BK * (BN + PAD);
     __shared__ __attribute__((aligned(16))) float smem[2 * (LDS_A + LDS_B)];
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave % WM, wn = wave / WM;
 
     // XCD-aware tile order: the hardware deals consecutive workgroup ids round
     // robin over the 8 XCDs; give each XCD a contiguous run of tiles so tiles
     // that share an A/B panel also share an L2.
-    int ntiles = g.tiles_m * g.tiles_n;
     int bid = blockIdx.x;
-    if (ntiles % NXCD == 0)
+    if (g.grp) {
+        // grouped launch: find the problem that owns this workgroup
+        int lo = 0, hi = g.n_grp; // grp[lo].tile_start <= bid < grp[hi].tile_start
+        while (hi - lo > 1) {
+            int mid = (lo + hi) >> 1;
+            if (g.grp[mid].tile_start <= bid) lo = mid; else hi = mid;
+        }
+        const NchipGemmProblem pr = g.grp[lo];
+        bid -= pr.tile_start;
+        g.A = pr.A; g.B = pr.B; g.C = pr.C;
+        g.M = pr.m; g.N = pr.n; g.K = pr.k;
+        g.lda = pr.lda; g.ldb = pr.ldb; g.ldc = pr.ldc;
+        g.alpha = pr.alpha;
+        g.kchunk = pr.k;
+        g.tiles_m = (pr.m + BM - 1) / BM;
+        g.tiles_n = (pr.n + BN - 1) / BN;
+    }
+    int ntiles = g.tiles_m * g.tiles_n;
+    if (!g.grp && ntiles % NXCD == 0)
         bid = (bid % NXCD) * (ntiles / NXCD) + bid / NXCD;
     const int tile_m = bid % g.tiles_m, tile_n = bid / g.tiles_m;
     const int bz = blockIdx.y;
@@ -179,8 +203,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g)
     const bool a_full = (m0 + BM <= g.M) && (g.lda % 4 == 0) && (((uintptr_t)A & 15) == 0);
     const bool b_full = (n0 + BN <= g.N) && (g.ldb % 4 == 0) && (((uintptr_t)B & 15) == 0);
 
-    TileLoader<BM, TA ? 0 : 1> la;
-    TileLoader<BN, TB ? 1 : 0> lb;
+    TileLoader<BM, BK, TA ? 0 : 1, NT> la;
+    TileLoader<BN, BK, TB ? 1 : 0, NT> lb;
 
     floatx16 acc[TN][TM];
 #pragma unroll
@@ -221,31 +245,34 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g)
         // latency is paid in full at the next LDS write
         __builtin_amdgcn_sched_barrier(0);
         if (BF16) {
-            // one 32x32x16 MFMA per tile pair covers the whole BK = 16
+            // one 32x32x16 MFMA per tile pair per 16 k
             const unsigned short *ha = reinterpret_cast<const unsigned short *>(sa);
             const unsigned short *hb = reinterpret_cast<const unsigned short *>(sb);
-            shortx8 fa[TM], fb[TN];
 #pragma unroll
-            for (int j = 0; j < TM; j++)
-                fa[j] = *reinterpret_cast<const shortx8 *>(
-                    ha + (wm * (BM / 2) + j * 32 + (lane & 31)) * (BK + 8) + (lane >> 5) * 8);
-#pragma unroll
-            for (int i = 0; i < TN; i++)
-                fb[i] = *reinterpret_cast<const shortx8 *>(
-                    hb + (wn * (BN / 2) + i * 32 + (lane & 31)) * (BK + 8) + (lane >> 5) * 8);
-#pragma unroll
-            for (int i = 0; i < TN; i++)
+            for (int kb = 0; kb < BK / 16; kb++) {
+                shortx8 fa[TM], fb[TN];
 #pragma unroll
                 for (int j = 0; j < TM; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(__attribute__((ext_vector_type(8))) __bf16, fb[i]),
-                        __builtin_bit_cast(__attribute__((ext_vector_type(8))) __bf16, fa[j]),
-                        acc[i][j], 0, 0, 0);
+                    fa[j] = *reinterpret_cast<const shortx8 *>(
+                        ha + (wm * WTM + j * 32 + (lane & 31)) * (BK + 8) + kb * 16 + (lane >> 5) * 8);
+#pragma unroll
+                for (int i = 0; i < TN; i++)
+                    fb[i] = *reinterpret_cast<const shortx8 *>(
+                        hb + (wn * WTN + i * 32 + (lane & 31)) * (BK + 8) + kb * 16 + (lane >> 5) * 8);
+#pragma unroll
+                for (int i = 0; i < TN; i++)
+#pragma unroll
+                    for (int j = 0; j < TM; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(__attribute__((ext_vector_type(8))) __bf16, fb[i]),
+                            __builtin_bit_cast(__attribute__((ext_vector_type(8))) __bf16, fa[j]),
+                            acc[i][j], 0, 0, 0);
+            }
         } else {
             // fragments of k-step ks+1 are fetched while the MFMAs of ks run
             float fa[2][TM], fb[2][TN];
-            const float *pa = sa + (lane >> 5) * (BM + PAD) + wm * (BM / 2) + (lane & 31);
-            const float *pb = sb + (lane >> 5) * (BN + PAD) + wn * (BN / 2) + (lane & 31);
+            const float *pa = sa + (lane >> 5) * (BM + PAD) + wm * WTM + (lane & 31);
+            const float *pb = sb + (lane >> 5) * (BN + PAD) + wn * WTN + (lane & 31);
 #pragma unroll
             for (int j = 0; j < TM; j++) fa[0][j] = pa[j * 32];
 #pragma unroll
@@ -285,8 +312,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs g)
     // epilogue.  acc[i][j][r] is C[m][n] with
     //   m = m0 + wm*BM/2 + j*32 + lane%32
     //   n = n0 + wn*BN/2 + i*32 + (r/4)*8 + (lane/32)*4 + r%4
-    const int mm_base = m0 + wm * (BM / 2) + (lane & 31);
-    const int nn_base = n0 + wn * (BN / 2) + (lane >> 5) * 4;
+    const int mm_base = m0 + wm * WTM + (lane & 31);
+    const int nn_base = n0 + wn * WTN + (lane >> 5) * 4;
     if (g.ksplit > 1) {
         float *ws = g.ws + ((int64_t)(kz * g.batch + b)) * g.M * g.N;
 #pragma unroll
@@ -360,16 +387,16 @@ struct ProfRec {
 bool g_prof_on = false;
 std::vector<ProfRec> g_prof;
 
-template <int BM, int BN, int BF16>
+template <int BM, int BN, int BK, int WM, int WN, int BF16>
 void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
-    dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(256);
-    if (!ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, 0, 0, BF16>), grid, block, 0, st, g);
-    else if (ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, 1, 0, BF16>), grid, block, 0, st, g);
-    else if (!ta && tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, 0, 1, BF16>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((gemm_kernel<BM, BN, 1, 1, BF16>), grid, block, 0, st, g);
+    dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(64 * WM * WN);
+    if (!ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 0, 0, BF16>), grid, block, 0, st, g);
+    else if (ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 1, 0, BF16>), grid, block, 0, st, g);
+    else if (!ta && tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 0, 1, BF16>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 1, 1, BF16>), grid, block, 0, st, g);
 }
 
 } // namespace
@@ -417,29 +444,56 @@ extern "C" int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, fl
     g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.sa = sa_out; g.sb = sb_out; g.sc = sc_out;
     g.sa_in = sa_in; g.sb_in = sb_in; g.sc_in = sc_in; g.batch_in = batch_in;
     g.M = m; g.N = n; g.K = k; g.batch = batch; g.ksplit = ksplit;
-    g.kchunk = ((k + ksplit - 1) / ksplit + BK - 1) / BK * BK;
-    if (g.kchunk < BK) g.kchunk = BK;
+    g.kchunk = ((k + ksplit - 1) / ksplit + KALIGN - 1) / KALIGN * KALIGN;
+    if (g.kchunk < KALIGN) g.kchunk = KALIGN;
     g.alpha = alpha; g.beta = beta; g.act = act;
+    g.grp = nullptr; g.n_grp = 0;
     hipStream_t st = (hipStream_t)stream;
     // tile choice from the shape only: large tiles when they still fill the chip
     int64_t t128 = (int64_t)((m + 127) / 128) * ((n + 127) / 128) * batch * ksplit;
-    bool big = (t128 >= 256) && m >= 128 && n >= 128;
     ProfRec rec;
     if (g_prof_on) {
         (void)hipEventCreate(&rec.start);
         (void)hipEventCreate(&rec.stop);
-        rec.variant = (big ? 8 : 0) | (ta ? 4 : 0) | (tb ? 2 : 0) | (precision == 1 ? 1 : 0);
+        rec.variant = -1;
         rec.flops = 2.0 * m * n * (double)k * batch;
         (void)hipEventRecord(rec.start, st);
     }
+    // Tile configuration from the shape alone.  Measured on MI355X (fp32):
+    // small outputs want the most workgroups (64x64, 4 wavefronts); once
+    // 128x64 tiles still give >= 256 workgroups, 8 wavefronts of 32x32 on a
+    // 128x64x32 tile win; very large problems use 128x128x32 with 8 wavefronts.
+    static const char *ecfg = getenv("NCHIP_GEMM_CFG"); // tuning aid: forces a configuration
+    int cfg = ecfg ? atoi(ecfg) : 0;
+    int64_t nb = (int64_t)batch * ksplit;
+    int64_t t128x64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64) * nb;
+    if (!cfg) {
+        if (t128 >= 512 && m >= 128 && n >= 128) cfg = 7;
+        else if (t128x64 >= 256 && m >= 128 && n >= 64) cfg = 4;
+        else cfg = 5;
+    }
     if (precision == 1) {
-        if (big) launch_tile<128, 128, 1>(st, ta, tb, g);
-        else launch_tile<64, 64, 1>(st, ta, tb, g);
+        if (cfg == 7) launch_tile<128, 128, 32, 4, 2, 1>(st, ta, tb, g);
+        else if (cfg == 4) launch_tile<128, 64, 32, 4, 2, 1>(st, ta, tb, g);
+        else launch_tile<64, 64, 32, 2, 2, 1>(st, ta, tb, g);
+    } else if (cfg == 1) {
+        launch_tile<128, 128, 16, 2, 2, 0>(st, ta, tb, g);
+    } else if (cfg == 2) {
+        launch_tile<128, 128, 16, 4, 2, 0>(st, ta, tb, g);
+    } else if (cfg == 3) {
+        launch_tile<128, 64, 16, 2, 2, 0>(st, ta, tb, g);
+    } else if (cfg == 4) {
+        launch_tile<128, 64, 32, 4, 2, 0>(st, ta, tb, g);
+    } else if (cfg == 6) {
+        launch_tile<64, 128, 16, 2, 2, 0>(st, ta, tb, g);
+    } else if (cfg == 7) {
+        launch_tile<128, 128, 32, 4, 2, 0>(st, ta, tb, g);
     } else {
-        if (big) launch_tile<128, 128, 0>(st, ta, tb, g);
-        else launch_tile<64, 64, 0>(st, ta, tb, g);
+        launch_tile<64, 64, 16, 2, 2, 0>(st, ta, tb, g);
     }
     if (g_prof_on) {
+        int tile = cfg == 7 ? 2 : (cfg == 4 ? 1 : 0);
+        rec.variant = tile * 8 + (ta ? 4 : 0) + (tb ? 2 : 0) + (precision == 1 ? 1 : 0);
         (void)hipEventRecord(rec.stop, st);
         g_prof.push_back(rec);
     }
@@ -478,26 +532,60 @@ extern "C" void nchip_gemm_profile_enable(int on)
 extern "C" int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launches,
                                        double *flops, double *seconds)
 {
-    double fl[16] = { 0 }, sec[16] = { 0 };
-    int64_t cnt[16] = { 0 };
+    double fl[24] = { 0 }, sec[24] = { 0 };
+    int64_t cnt[24] = { 0 };
     for (ProfRec &r : g_prof) {
         float ms = 0.0f;
         (void)hipEventSynchronize(r.stop);
         (void)hipEventElapsedTime(&ms, r.start, r.stop);
-        fl[r.variant] += r.flops;
-        sec[r.variant] += ms * 1e-3;
-        cnt[r.variant]++;
+        if (r.variant >= 0 && r.variant < 24) {
+            fl[r.variant] += r.flops;
+            sec[r.variant] += ms * 1e-3;
+            cnt[r.variant]++;
+        }
         (void)hipEventDestroy(r.start);
         (void)hipEventDestroy(r.stop);
     }
     g_prof.clear();
+    static const char *tiles[3] = { "64,64,16,2,2", "128,64,32,4,2", "128,128,32,4,2" };
     int n = 0;
-    for (int v = 0; v < 16 && n < max_variants; v++) {
+    for (int v = 0; v < 24 && n < max_variants; v++) {
         if (!cnt[v]) continue;
-        int bt = (v & 8) ? 128 : 64;
-        snprintf(names[n], 48, "gemm_kernel<%d,%d,%d,%d,%d>", bt, bt, (v >> 2) & 1, (v >> 1) & 1, v & 1);
+        snprintf(names[n], 48, "gemm_kernel<%s,%d,%d,%d>", tiles[v / 8], (v >> 2) & 1, (v >> 1) & 1, v & 1);
         launches[n] = cnt[v]; flops[n] = fl[v]; seconds[n] = sec[v];
         n++;
     }
     return n;
+}
+
+// ---- grouped launch ---------------------------------------------------------------
+extern "C" int nchip_gemm_grouped_tiles(int m, int n)
+{
+    return ((m + 127) / 128) * ((n + 127) / 128);
+}
+
+extern "C" int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmProblem *dev_table,
+                                  int n_problems, int total_tiles, int precision)
+{
+    if (n_problems <= 0 || total_tiles <= 0) return 0;
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.grp = dev_table; g.n_grp = n_problems;
+    g.batch = 1; g.batch_in = 1; g.ksplit = 1;
+    g.beta = 0.0f; g.act = 0;
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid(total_tiles, 1), block(512);
+#define GRP(TA, TB, BF) hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, 0, st, g)
+    if (precision == 1) {
+        if (!ta && !tb) GRP(0, 0, 1); else if (ta && !tb) GRP(1, 0, 1); else if (!ta && tb) GRP(0, 1, 1); else GRP(1, 1, 1);
+    } else {
+        if (!ta && !tb) GRP(0, 0, 0); else if (ta && !tb) GRP(1, 0, 0); else if (!ta && tb) GRP(0, 1, 0); else GRP(1, 1, 0);
+    }
+#undef GRP
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        fprintf(stderr, "nchip_gemm_grouped: launch failed: %s\n", hipGetErrorString(e));
+        return -2;
+    }
+    return 0;
 }

@@ -206,6 +206,48 @@ __global__ void opt_update_kernel(int algo, float *w, float *m, float *v, const 
     }
 }
 
+__device__ __forceinline__ void opt_step(int algo, float &w, float *m, float &v, float gi, float lr,
+                                         float b1, float b2, float eps, float clip, float c1, float c2)
+{
+    if (algo == 0) {
+        w -= lr * gi;
+    } else if (algo == 1) {
+        if (clip != 0.0f) gi = fminf(fmaxf(gi, -clip), clip);
+        float mi = gi;
+        if (m) { mi = b1 * *m + (1.0f - b1) * gi; *m = mi; }
+        float vi = b2 * v + (1.0f - b2) * gi * gi;
+        v = vi;
+        w -= lr * (mi * c1) / (sqrtf(vi * c2) + eps);
+    } else {
+        float vi = b2 * v + (1.0f - b2) * gi * gi;
+        v = vi;
+        w -= lr * gi / (sqrtf(vi) + eps);
+    }
+}
+
+// One launch for every parameter: block -> (tensor, chunk) through a prefix
+// table of chunk counts; element-wise, so the result equals the per-tensor kernel.
+__global__ __launch_bounds__(TPB) void opt_update_multi_kernel(const NchipOptTensor *tab,
+                                                               const int *chunk_prefix, int n_tensors,
+                                                               int chunk, int algo, float b1, float b2,
+                                                               float eps, float clip, float c1, float c2)
+{
+    int bid = blockIdx.x, lo = 0, hi = n_tensors; // chunk_prefix[lo] <= bid < chunk_prefix[hi]
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (chunk_prefix[mid] <= bid) lo = mid; else hi = mid;
+    }
+    NchipOptTensor t = tab[lo];
+    int64_t e0 = (int64_t)(bid - chunk_prefix[lo]) * chunk;
+    int64_t e1 = e0 + chunk < t.n ? e0 + chunk : t.n;
+    for (int64_t i = e0 + threadIdx.x; i < e1; i += TPB) {
+        float w = t.w[i], v = t.v ? t.v[i] : 0.0f;
+        opt_step(algo, w, t.m ? t.m + i : nullptr, v, t.g[i], t.lr, b1, b2, eps, clip, c1, c2);
+        t.w[i] = w;
+        if (t.v) t.v[i] = v;
+    }
+}
+
 inline int grid_for(int64_t n, int cap = 8192)
 {
     int64_t b = (n + TPB - 1) / TPB;
@@ -305,6 +347,17 @@ int nchip_add_col(void *stream, const float *g, const int32_t *idx, float *dw, i
     if (v <= 0 || d <= 0) return 0;
     hipLaunchKernelGGL(add_col_kernel, dim3(v), dim3(TPB), 0, (hipStream_t)stream, g, idx, dw, d, n);
     return check("nchip_add_col");
+}
+
+int nchip_opt_update_multi(void *stream, int algo, const NchipOptTensor *dev_table,
+                            const int *dev_chunk_prefix, int n_tensors, int total_chunks, int chunk,
+                            float beta1, float beta2, float eps, float clip, float c1, float c2)
+{
+    if (n_tensors <= 0 || total_chunks <= 0) return 0;
+    if (algo != 0 && algo != 1 && algo != 16) { fprintf(stderr, "nchip_opt_update_multi: unknown algo %d\n", algo); return -1; }
+    hipLaunchKernelGGL(opt_update_multi_kernel, dim3(total_chunks), dim3(TPB), 0, (hipStream_t)stream,
+                       dev_table, dev_chunk_prefix, n_tensors, chunk, algo, beta1, beta2, eps, clip, c1, c2);
+    return check("nchip_opt_update_multi");
 }
 
 int nchip_opt_update(void *stream, int algo, float *w, float *m, float *v, const float *g, int64_t n,

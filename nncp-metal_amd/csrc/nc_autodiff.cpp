@@ -119,6 +119,7 @@ static void count_edges(NCNode *root, int epoch)
                 stack.push_back(p);
             }
             p->pending++;
+            p->consumers = p->pending;
         }
     }
 }
@@ -179,4 +180,5 @@ extern "C" void nc_backward(const NCTensor *x, NCTensor *grad, NCParamUpdateFunc
         nc_free_tensor(g);
         nc_free_node(nd);
     }
+    nc_flush_deferred(m);
 }

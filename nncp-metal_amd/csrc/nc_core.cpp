@@ -105,6 +105,9 @@ extern "C" NCContext *nc_context_init(int nb_threads)
     m->launches = 0;
     m->node_seq = 0;
     m->epoch = 0;
+    m->defer_wgrad = false;
+    m->grp_staging = nullptr;
+    m->grp_staging_cap = 0;
     const char *e = getenv("NCHIP_MATMUL_BF16");
     if (e && atoi(e) != 0)
         m->matmul_bf16 = 1;
@@ -168,6 +171,13 @@ extern "C" int nc_set_matmul_bf16(NCContext *m, int enable)
 }
 
 extern "C" int64_t nc_get_launch_count(NCContext *m) { return m->launches; }
+
+extern "C" int nc_set_deferred_weight_grad(NCContext *m, int enable)
+{
+    int old = m->defer_wgrad;
+    m->defer_wgrad = enable != 0;
+    return old;
+}
 
 // ---- tensors ----------------------------------------------------------------
 size_t nc_type_size(NCTypeEnum t)
@@ -640,6 +650,8 @@ struct NCSGDOptState {
     SGDOptParams p;
     int64_t step;
     std::vector<SGDOptVarState *> vars;
+    void *staging = nullptr; // pinned table of the previous update, recycled one update later
+    size_t staging_cap = 0;
 };
 
 extern "C" NCSGDOptState *nc_sgd_opt_init(NCContext *m, const SGDOptParams *p)
@@ -649,7 +661,11 @@ extern "C" NCSGDOptState *nc_sgd_opt_init(NCContext *m, const SGDOptParams *p)
     return s;
 }
 
-extern "C" void nc_sgd_opt_end(NCSGDOptState *s) { delete s; }
+extern "C" void nc_sgd_opt_end(NCSGDOptState *s)
+{
+    if (s->staging) s->ctx->host_pool.put(s->staging, s->staging_cap);
+    delete s;
+}
 
 extern "C" void nc_sgd_opt_set_all(NCParamList *pl, NCSGDOptState *s)
 {
@@ -714,17 +730,48 @@ extern "C" void nc_sgd_opt_update(NCSGDOptState *s)
     s->step++;
     float c1 = 1.0f / (1.0f - powf(b1, (float)s->step));
     float c2 = 1.0f / (1.0f - powf(b2, (float)s->step));
+    // one launch over every parameter that received a gradient
+    const int chunk = 8192;
+    std::vector<NchipOptTensor> tab;
+    std::vector<int> prefix(1, 0);
     for (SGDOptVarState *vs : s->vars) {
         if (!vs->has_grad) continue;
         NCTensor *w = *vs->param->pval;
         need_dev(w, "nc_sgd_opt_update");
-        // with beta1 == 0 the first moment equals the gradient; m is not stored
-        float *mp = vs->m ? nc_f32(vs->m) : (vs->v ? nc_f32(vs->v) : nullptr);
-        if (nchip_opt_update(s->ctx->stream, (int)p->algo, nc_f32(w), mp, vs->v ? nc_f32(vs->v) : nullptr,
-                             nc_f32(vs->g), (int64_t)vs->n, p->lr * vs->param->lr_mult,
-                             vs->m ? b1 : 0.0f, b2, p->u.adam.eps, p->u.adam.gradient_clip, c1, c2))
-            nc_fatal("optimiser update failed");
-        s->ctx->launches++;
+        NchipOptTensor t;
+        t.w = nc_f32(w);
+        t.m = vs->m ? nc_f32(vs->m) : nullptr; // with beta1 == 0 the first moment is the gradient
+        t.v = vs->v ? nc_f32(vs->v) : nullptr;
+        t.g = nc_f32(vs->g);
+        t.n = (int64_t)vs->n;
+        t.lr = p->lr * vs->param->lr_mult;
+        t.pad_ = 0;
+        tab.push_back(t);
+        prefix.push_back(prefix.back() + (int)((vs->n + chunk - 1) / chunk));
+    }
+    if (tab.empty()) return;
+    NCContext *m = s->ctx;
+    size_t tb = tab.size() * sizeof(NchipOptTensor), pb = prefix.size() * sizeof(int);
+    size_t hcap, dcap;
+    // pinned staging and device table; both go back to the pools only after
+    // the stream has consumed them (the synchronize below is cheap here: the
+    // host has nothing else to enqueue before the next step's token upload)
+    uint8_t *host = (uint8_t *)m->host_pool.get(tb + pb, &hcap);
+    uint8_t *dev = (uint8_t *)m->dev_pool.get(tb + pb, &dcap);
+    memcpy(host, tab.data(), tb);
+    memcpy(host + tb, prefix.data(), pb);
+    hip_check(hipMemcpyAsync(dev, host, tb + pb, hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync opt table");
+    if (nchip_opt_update_multi(m->stream, (int)p->algo, (const NchipOptTensor *)dev, (const int *)(dev + tb),
+                               (int)tab.size(), prefix.back(), chunk, b1, b2, p->u.adam.eps,
+                               p->u.adam.gradient_clip, c1, c2))
+        nc_fatal("optimiser update failed");
+    m->launches++;
+    // the copy must have read the staging buffer before it is recycled
+    if (s->staging) m->host_pool.put(s->staging, s->staging_cap);
+    s->staging = host; s->staging_cap = hcap;
+    m->dev_pool.put(dev, dcap); // stream ordered: next user is enqueued after the kernel
+    for (SGDOptVarState *vs : s->vars) {
+        if (!vs->has_grad) continue;
         nc_free_tensor(vs->g);
         vs->g = nullptr;
         vs->has_grad = false;

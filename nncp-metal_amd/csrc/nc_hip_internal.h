@@ -42,6 +42,13 @@ struct NCDevice {
     bool is_hip;
 };
 
+// weight-gradient GEMM postponed to one grouped launch at the end of nc_backward
+struct DeferredGemm {
+    NCTensor *a, *b, *c; // c (m x n) = alpha * a (m x k) * b^T (b is n x k)
+    int m, n, k;
+    float alpha;
+};
+
 struct NCContext {
     int nb_threads;
     NCDevice cpu, hip;
@@ -52,6 +59,10 @@ struct NCContext {
     int64_t launches;
     int64_t node_seq;
     int epoch;
+    bool defer_wgrad;
+    std::vector<DeferredGemm> deferred;
+    void *grp_staging;
+    size_t grp_staging_cap;
 };
 
 struct NCTensorBuffer {
@@ -95,6 +106,7 @@ struct NCNode {
     // backward-walk state
     NCTensor *grad = nullptr;
     int pending = 0;
+    int consumers = 0; // edges into this node in the current backward walk
     int mark = 0;
 };
 
@@ -122,5 +134,6 @@ NCTensor *nc_reshape_view(NCTensor *x, int nd, const size_t *dims); // consumes,
 NCNode *nc_new_node(NCContext *m, int op, int n_args, NCTensor **args);
 NCTensor *nc_finish(NCTensor *y, NCNode *n, NCTensor **args, int n_args);
 void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga); // nc_ops.cpp
+void nc_flush_deferred(NCContext *m);                          // nc_ops.cpp
 
 #endif

@@ -582,6 +582,15 @@ static void matmul_bw(NCNode *nd, NCTensor *g, NCTensor **ga, int ia, int ib)
     MMShape s = mm_shape(a, b, ta, tb);
     if (nd->parents[ia]) {
         NCTensor *da = nc_alloc_like(a);
+        NCNode *pa = nd->parents[ia];
+        if (m->defer_wgrad && !ta && !tb && s.batch == 1 && pa->op == OP_PARAM && pa->consumers == 1) {
+            // dW = alpha * dY * X^T of a plain linear layer whose weight is used
+            // once: postponed to the grouped launch at the end of nc_backward
+            DeferredGemm d;
+            d.a = nc_contig(nc_dup_tensor(g)); d.b = nc_dup_tensor(b); d.c = nc_dup_tensor(da);
+            d.m = (int)s.m; d.n = (int)s.k; d.k = (int)s.n; d.alpha = alpha;
+            m->deferred.push_back(d);
+        } else
         if (!ta) dev_gemm(m, false, !tb, s.m, s.k, s.n, alpha, g, b, 0.0f, da, s.batch, nullptr, 0, nullptr);
         else     dev_gemm(m, tb, true, s.k, s.m, s.n, alpha, b, g, 0.0f, da, s.batch, nullptr, 0, nullptr);
         ga[ia] = da;
@@ -892,6 +901,42 @@ extern "C" float nc_exp_det(float x)
     union { float f; uint32_t u; } v = { p };
     v.u += (uint32_t)((int32_t)n * (1 << 23));
     return v.f;
+}
+
+// Runs every postponed weight-gradient GEMM in one grouped launch.  The
+// gradient tensors were handed to the parameter callback earlier, so with
+// nc_set_deferred_weight_grad() enabled they hold valid data only once
+// nc_backward() has returned.
+void nc_flush_deferred(NCContext *m)
+{
+    if (m->deferred.empty()) return;
+    std::vector<NchipGemmProblem> tab;
+    int tiles = 0;
+    for (DeferredGemm &d : m->deferred) {
+        NchipGemmProblem p;
+        p.A = nc_f32(d.a); p.B = nc_f32(d.b); p.C = nc_f32(d.c);
+        p.m = d.m; p.n = d.n; p.k = d.k;
+        p.lda = d.m; p.ldb = d.n; p.ldc = d.m;
+        p.tile_start = tiles; p.alpha = d.alpha;
+        tiles += nchip_gemm_grouped_tiles(d.m, d.n);
+        tab.push_back(p);
+    }
+    size_t bytes = tab.size() * sizeof(NchipGemmProblem), hcap, dcap;
+    void *host = m->host_pool.get(bytes, &hcap);
+    void *dev = m->dev_pool.get(bytes, &dcap);
+    memcpy(host, tab.data(), bytes);
+    hip_check(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync gemm table");
+    if (nchip_gemm_grouped(m->stream, 0, 1, (const NchipGemmProblem *)dev, (int)tab.size(), tiles, m->matmul_bf16))
+        nc_fatal("grouped weight-gradient GEMM failed");
+    m->launches++;
+    // pinned staging is recycled one flush later (the copy has long run by then)
+    if (m->grp_staging) m->host_pool.put(m->grp_staging, m->grp_staging_cap);
+    m->grp_staging = host; m->grp_staging_cap = hcap;
+    m->dev_pool.put(dev, dcap);
+    for (DeferredGemm &d : m->deferred) {
+        nc_free_tensor(d.a); nc_free_tensor(d.b); nc_free_tensor(d.c);
+    }
+    m->deferred.clear();
 }
 
 // ---- backward dispatch --------------------------------------------------------

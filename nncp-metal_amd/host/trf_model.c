@@ -101,6 +101,8 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
     s->cpu = nc_new_cpu_device(s->ctx);
     s->dev = c->use_device ? nc_new_cuda_device(s->ctx, 0) : s->cpu;
     s->rnd = nc_rnd_init(s->dev, c->seed);
+    if (c->fused)
+        nc_set_deferred_weight_grad(s->ctx, 1); /* backward_cb only forwards to sgd_opt_update_var */
     /* trf_init, nncp.c:304-520 */
     s->embed_mult = sqrtf((float)D) * c->embed_mult;
     nc_param_list_init(s->ctx, &s->params);
