@@ -97,6 +97,10 @@ int nchip_relpos_attn_fwd(void *stream, const float *q, int64_t ldq,
                           int H, int dk, int dv, int B, int T, int M, int d_pos,
                           int attn_len, float b_r_scale, int precision);
 
+/* Kernel launches issued by the calling thread's last successful
+   nchip_relpos_attn_fwd (1 when the head fits the single-kernel path). */
+int nchip_relpos_attn_last_launches(void);
+
 /* Backward of the above from the saved probs.  dq, dkv, dkvm are fully
    overwritten; dw_r (dk, d_pos, H) and db_r (K, H) are overwritten with the
    sums over streams, reduced in a fixed order (no atomics).  scratch needs

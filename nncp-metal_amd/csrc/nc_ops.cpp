@@ -801,7 +801,7 @@ extern "C" NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv
                                    m->matmul_bf16);
     if (rel) nc_tmp_free(m, rel, cap);
     if (rc) nc_fatal("nc_relpos_attention: kernel rejected the shapes");
-    m->launches += 6;
+    m->launches += nchip_relpos_attn_last_launches();
     NCNode *n = nc_new_node(m, OP_ATTN, 5, all);
     bool graph = false;
     for (int i = 0; i < 5; i++)
@@ -844,7 +844,7 @@ static void attn_bw(NCNode *nd, NCTensor *g, NCTensor **ga)
                                    nd->ia[2], nd->fa[0], m->matmul_bf16, scratch);
     nc_tmp_free(m, scratch, cap);
     if (rc) nc_fatal("nc_relpos_attention backward failed");
-    m->launches += 14;
+    m->launches += nchip_relpos_attn_last_launches();
     nc_free_tensor(gc);
     NCTensor *out[5] = { dq, dkv, dkvm, dwr, dbr };
     for (int i = 0; i < 5; i++) {
