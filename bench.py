@@ -101,6 +101,84 @@ def gemm_profile(model, H, syms, mode, hip_lib):
     return rows
 
 
+def attention_c2(pkg, iters=50):
+    """Isolated rel-pos attention forward+backward at BASELINE configs[1]
+    (B 32, H 8, d_head 64, 64 queries x 128 keys, sinusoidal position table,
+    learned bias), through the raw kernel entry points on the null stream,
+    timed with a HIP event pair around `iters` forward+backward pairs.
+    Algorithmic bytes: fwd Q + K + V + P_table + O, bwd Q,K,V,O,dO in and
+    dQ,dK,dV out = 72 MiB; dense flops 11 GEMM-likes x 268 M = 2.95 G."""
+    nc = pkg.binding.NC(pkg.binding.HIP_LIB)
+    lib = C.CDLL(pkg.binding.HIP_LIB)
+    hip = C.CDLL("libamdhip64.so")
+    B, Hh, dk, T, M = 32, 8, 64, 64, 64
+    K, d_pos = M + T, M + T
+    rng = np.random.default_rng(0)
+    q = rng.normal(0, 0.125, (T, B, Hh * dk)).astype(np.float32)
+    kv = rng.normal(0, 0.125, (T, B, 2 * Hh * dk)).astype(np.float32)
+    kvm = rng.normal(0, 0.125, (M, B, 2 * Hh * dk)).astype(np.float32)
+    delta = (d_pos - 1 - np.arange(d_pos))[:, None]
+    inv = 1.0 / 10000 ** (np.arange(0, dk, 2) / dk)
+    tab = np.zeros((d_pos, dk), np.float32)
+    tab[:, 0::2] = np.sin(delta * inv)
+    tab[:, 1::2] = np.cos(delta * inv)
+    w_r = np.broadcast_to(tab, (Hh, d_pos, dk)).copy()
+    b_r = rng.normal(0, 0.02, (Hh, K)).astype(np.float32)
+    dout = rng.normal(0, 1, (T, B, Hh * dk)).astype(np.float32)
+    host = dict(q=q, kv=kv, kvm=kvm, w_r=w_r, b_r=b_r, dout=dout)
+    dev = {k: nc.tensor(v) for k, v in host.items()}
+    lib.nchip_relpos_attn_bwd_scratch.restype = C.c_size_t
+    nscr = lib.nchip_relpos_attn_bwd_scratch(Hh, dk, B, T, M, d_pos)
+    outs = dict(out=q.shape, probs=(B, Hh, T, K), rel=(B, Hh, T, d_pos), dq=q.shape, dkv=kv.shape,
+                dkvm=kvm.shape, dw_r=w_r.shape, db_r=b_r.shape, scratch=(nscr,))
+    for k, shp in outs.items():
+        dev[k] = nc.tensor(np.zeros(shp, np.float32))
+    P = {k: C.c_void_p(nc.lib.nc_tensor_get_ptr(v, None)) for k, v in dev.items()}
+    i64, f32, i32 = C.c_int64, C.c_float, C.c_int
+    ld, ldkv = i64(Hh * dk), i64(2 * Hh * dk)
+
+    def fwd():
+        return lib.nchip_relpos_attn_fwd(None, P["q"], ld, P["kv"], P["kvm"], ldkv, P["w_r"], P["b_r"],
+                                         P["out"], ld, P["probs"], P["rel"], i32(Hh), i32(dk), i32(dk),
+                                         i32(B), i32(T), i32(M), i32(d_pos), i32(K), f32(1.0), i32(0))
+
+    def bwd():
+        return lib.nchip_relpos_attn_bwd(None, P["q"], ld, P["kv"], P["kvm"], ldkv, P["w_r"], P["probs"],
+                                         P["dout"], ld, P["dq"], P["dkv"], P["dkvm"], P["dw_r"], P["db_r"],
+                                         i32(Hh), i32(dk), i32(dk), i32(B), i32(T), i32(M), i32(d_pos),
+                                         i32(K), f32(1.0), i32(0), P["scratch"])
+
+    def timed(fns):
+        e0, e1 = C.c_void_p(), C.c_void_p()
+        hip.hipEventCreate(C.byref(e0))
+        hip.hipEventCreate(C.byref(e1))
+        for f in fns:
+            assert f() == 0
+        hip.hipDeviceSynchronize()
+        hip.hipEventRecord(e0, None)
+        for _ in range(iters):
+            for f in fns:
+                f()
+        hip.hipEventRecord(e1, None)
+        hip.hipEventSynchronize(e1)
+        ms = C.c_float()
+        hip.hipEventElapsedTime(C.byref(ms), e0, e1)
+        hip.hipEventDestroy(e0)
+        hip.hipEventDestroy(e1)
+        return ms.value * 1e3 / iters
+
+    us_f, us_b, us = timed([fwd]), timed([bwd]), timed([fwd, bwd])
+    for v in dev.values():
+        nc.free(v)
+    nc.close()
+    nbytes, flops = 72 * 2 ** 20, 2.95e9
+    return {"workload": "BASELINE configs[1]: B32 H8 d64 T64 K128 fwd+bwd fp32",
+            "us_fwd": round(us_f, 2), "us_bwd": round(us_b, 2), "us_fwd_bwd": round(us, 2),
+            "algorithmic_GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / 8000, 4),
+            "dense_TFLOPs": round(flops / us / 1e6, 2), "mfma_fp32_frac": round(flops / us / 1e6 / 157.3, 4),
+            "binding_bound": "mfma (39 flop/B > fp32 ridge 20)"}
+
+
 def cpu_baseline(pkg, data, n_steps, threads):
     """The CPU checker driving the reference op sequence (whole-segment
     evaluation, float symbol coder: what `nncp --encode_only` does) on the
@@ -125,6 +203,7 @@ def main():
     ap.add_argument("--variant", choices=["fp32", "bf16"], default="fp32")
     ap.add_argument("--cpu-steps", type=int, default=2, help="0 skips the CPU baseline")
     ap.add_argument("--profile-steps", type=int, default=2)
+    ap.add_argument("--attention-iters", type=int, default=50, help="0 skips the isolated attention timing")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (one compression job per GPU, no "
@@ -175,6 +254,7 @@ def main():
                     "all_gemm_tflops": round(tot_f / tot_s / 1e12, 3),
                     "all_gemm_ms_per_step": round(tot_s / args.profile_steps * 1e3, 3)}
     model.close()
+    attn = attention_c2(pkg, args.attention_iters) if args.attention_iters else None
 
     cpu = None
     if args.cpu_steps:
@@ -199,7 +279,7 @@ def main():
         "kernel_launches_per_step": launches / args.steps,
         "host_seconds": {"eval_and_copy": round(st.t_eval, 4), "code": round(st.t_code, 4),
                          "grad": round(st.t_grad, 4), "update": round(st.t_update, 4)},
-        "roofline": roof, "cpu_baseline": cpu}))
+        "roofline": roof, "attention": attn, "cpu_baseline": cpu}))
 
 
 if __name__ == "__main__":

@@ -1,0 +1,670 @@
+// Relative-position causal attention (nncp.c:722-800 and its gradient) as ONE
+// kernel per direction for heads that fit in LDS: d_head 32 or 64, up to 64
+// queries and 128 keys / relative positions.
+//
+// A workgroup (4 wavefronts) owns one (stream, head).  Q, the position vectors
+// w_r[:, :, h], K and V of that head are staged once in LDS as [token][feature]
+// rows of DK + 4 floats: with that stride both fragment shapes of
+// v_mfma_f32_16x16x4_f32 read LDS at the 2-lanes-per-bank minimum
+// ("row = token, k = feature": bank 4*il + g; "row = feature, k = token
+// 4g + r": bank 16g + il).  Every tile is zero-filled to its full static size,
+// so the compute phases are straight-line code without bounds branches: rows
+// and columns outside the problem contribute exact zeros or are masked by
+// selects, and only the global stores are guarded.  (Branches around MFMA
+// groups make the compiler shuttle accumulators between AGPRs and VGPRs, which
+// drains the matrix pipeline; skipping the causally dead key tiles would not
+// shorten the workgroup, whose last wavefront sees every key.)
+//
+// Forward, wavefront w = query columns 16w..16w+15:
+//   rel = w_r^T q -> per-wavefront LDS strip;  S = K^T q + shifted rel + bias
+//   (1/sqrt(dk) folded into q), causal/window mask, all in registers;  softmax
+//   over the keys with two xor-shuffles (a column lives in lanes l, l^16, l^32,
+//   l^48);  O = V P with P fed to the MFMA straight from the score registers.
+// Backward: dA = V^T dO and dS in registers, dq = K dS + w_r dRel (dRel = the
+// rel-shift adjoint of dS, scattered into an LDS strip that replaces V); then
+// P^T and dS^T are parked in LDS over K / w_r and the wavefronts switch to
+// owning key tiles (dK = Q dS^T, dV = dO P^T) and position tiles
+// (dw_r[b,h] = Q dRel^T).  Per-(stream, head) dw_r / db_r partials go to scratch
+// and a second kernel sums them over streams in stream order.  No atomics.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include "k_internal.h"
+
+namespace {
+
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+constexpr int FA_TMAX = 64;     // queries per head
+constexpr int FA_RSTRIDE = 131; // rel strip row: shifted reads and tile writes both <= 4 lanes per bank
+constexpr int FA_PSTRIDE = 65;  // transposed P / dS tiles of the backward
+constexpr int FA_NB = 256;      // bias row: K entries, zero up to the largest index a masked key can form
+
+__device__ __forceinline__ floatx4_t mfma16(float a, float b, floatx4_t c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ void wave_lds_sync()
+{
+    // same-wavefront LDS exchange: earlier writes of any lane before later reads
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Staging of a [ROWS][DK + 4] LDS tile from global rows of DK floats, split in
+// two so that the loads of every tile are in flight before the first LDS store
+// waits on one: fetch_rows issues the float4 loads (rows >= rows_valid read as
+// zero), put_rows stores the whole tile.  src(row) is the row address; src(0)
+// must be readable even when rows_valid is 0.
+template <int DK, int ROWS, typename F>
+__device__ __forceinline__ void fetch_rows(floatx4_t (&v)[ROWS * (DK / 4) / 256], int rows_valid, F src)
+{
+    constexpr int C4 = DK / 4;
+#pragma unroll
+    for (int it = 0; it < ROWS * C4 / 256; it++) {
+        int idx = threadIdx.x + it * 256;
+        int row = idx / C4, c = (idx % C4) * 4;
+        // always load (from a clamped, valid row) and select afterwards: a load
+        // under a divergent branch would be waited for before the next is issued
+        int rc = row < rows_valid ? row : rows_valid - 1;
+        floatx4_t x = *reinterpret_cast<const floatx4_t *>(src(rc < 0 ? 0 : rc) + c);
+        v[it] = row < rows_valid ? x : floatx4_t{ 0, 0, 0, 0 };
+    }
+}
+
+template <int DK, int ROWS>
+__device__ __forceinline__ void put_rows(float *dst, const floatx4_t (&v)[ROWS * (DK / 4) / 256])
+{
+    constexpr int RS = DK + 4, C4 = DK / 4;
+#pragma unroll
+    for (int it = 0; it < ROWS * C4 / 256; it++) {
+        int idx = threadIdx.x + it * 256;
+        int row = idx / C4, c = (idx % C4) * 4;
+        *reinterpret_cast<floatx4_t *>(dst + row * RS + c) = v[it];
+    }
+}
+
+// Optional per-phase shader-clock stamps of one workgroup (debug builds only).
+#ifdef NCHIP_ATTN_PHASE_CLOCKS
+__device__ long long *g_phase_clk = nullptr;
+#define PHASE_MARK(k)                                                                          \
+    do {                                                                                       \
+        if (g_phase_clk && blockIdx.x == 0 && (threadIdx.x & 63) == 0)                         \
+            g_phase_clk[(threadIdx.x >> 6) * 16 + (k)] = clock64();                            \
+    } while (0)
+#else
+#define PHASE_MARK(k) do { } while (0)
+#endif
+
+// Keeps the LDS reads of the next tile ahead of the MFMAs of the current one:
+// without the fence the scheduler sinks each read next to its use and every
+// MFMA pair then waits a full LDS round trip.
+#define PIPELINE_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// A operands of one 16-row tile for a DK-deep contraction (row = il, k-slot g)
+template <int NS>
+__device__ __forceinline__ void load_afrag(float (&f)[NS], const float *row_g)
+{
+#pragma unroll
+    for (int s = 0; s < NS; s++) f[s] = row_g[4 * s];
+}
+
+// A operands of 4 k-steps (tokens tile*16 + 4g + r) x ND feature tiles
+template <int ND, int RS>
+__device__ __forceinline__ void load_tokfrag(float (&f)[ND][4], const float *base, int tile, int g, int il)
+{
+#pragma unroll
+    for (int dt = 0; dt < ND; dt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) f[dt][r] = base[(tile * 16 + 4 * g + r) * RS + dt * 16 + il];
+}
+
+// NT = key / position tiles of 16 (4: up to 64 keys, 8: up to 128)
+template <int DK, int NT>
+struct FwdLayout {
+    static constexpr int RS = DK + 4, KR = NT * 16;
+    static constexpr int q = 0, w = q + FA_TMAX * RS, k = w + KR * RS, v = k + KR * RS,
+                         r = v + KR * RS, b = r + 4 * 16 * FA_RSTRIDE, floats = b + FA_NB;
+};
+
+template <int DK, int NT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    using L = FwdLayout<DK, NT>;
+    constexpr int RS = DK + 4, NS = DK / 4, ND = DK / 16, KR = NT * 16;
+    float *Qs = lds + L::q, *Ws = lds + L::w, *Ks = lds + L::k, *Vs = lds + L::v;
+    float *Rs = lds + L::r; // [4][16][FA_RSTRIDE]
+    float *Bs = lds + L::b; // bias * b_r_scale / sqrt(dk), zero past K
+
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    // consecutive workgroups (one per XCD in turn) take consecutive streams, so
+    // an XCD fetches whole token columns (every head of its streams)
+    const int b = blockIdx.x % a.B, h = blockIdx.x / a.B;
+    const int il = lane & 15, g = lane >> 4;
+    const int i = 16 * w + il;
+    const bool has_w = a.w_r != nullptr;
+    PHASE_MARK(0);
+
+    // All global loads are issued up front; each tile is parked in LDS just
+    // before the phase that needs it, so K and V arrive under the rel phase.
+    floatx4_t vq[FA_TMAX * (DK / 4) / 256], vw[KR * (DK / 4) / 256], vk[KR * (DK / 4) / 256],
+        vv[KR * (DK / 4) / 256];
+    {
+        auto kvrow = [&](int r) {
+            return (r < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * r)
+                            : a.kv + a.ldkv * (b + (int64_t)a.B * (r - a.M))) + (int64_t)h * DK;
+        };
+        fetch_rows<DK, FA_TMAX>(vq, a.T, [&](int r) { return a.q + (int64_t)h * DK + a.ldq * (b + (int64_t)a.B * r); });
+        fetch_rows<DK, KR>(vw, has_w ? a.d_pos : 0, [&](int r) { return has_w ? a.w_r + ((int64_t)h * a.d_pos + r) * DK : a.q; });
+        fetch_rows<DK, KR>(vk, a.K, kvrow);
+        fetch_rows<DK, KR>(vv, a.K, [&](int r) { return kvrow(r) + (int64_t)a.H * DK; });
+    }
+    if (t < FA_NB) Bs[t] = (a.b_r && t < a.K) ? a.b_r[(int64_t)h * a.K + t] * (a.b_r_scale * a.scale) : 0.0f;
+    put_rows<DK, FA_TMAX>(Qs, vq);
+    put_rows<DK, KR>(Ws, vw);
+    __syncthreads();
+    PHASE_MARK(1);
+
+    // query fragments: B operand (k-slot g, column il) of every 4-wide k-step
+    float qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) qf[s] = Qs[i * RS + 4 * s + g] * a.scale; // 1/sqrt(dk) folded in
+
+    float *Rw = Rs + (w * 16 + il) * FA_RSTRIDE; // this lane's column of rel
+    {
+        float af[2][NS];
+        load_afrag<NS>(af[0], Ws + il * RS + g);
+#pragma unroll
+        for (int pt = 0; pt < NT; pt++) {
+            if (pt + 1 < NT) load_afrag<NS>(af[(pt + 1) & 1], Ws + ((pt + 1) * 16 + il) * RS + g);
+            PIPELINE_FENCE();
+            floatx4_t acc = { 0, 0, 0, 0 };
+#pragma unroll
+            for (int s = 0; s < NS; s++) acc = mfma16(af[pt & 1][s], qf[s], acc);
+#pragma unroll
+            for (int r = 0; r < 4; r++) Rw[pt * 16 + 4 * g + r] = acc[r];
+        }
+        wave_lds_sync();
+    }
+    put_rows<DK, KR>(Ks, vk);
+    __syncthreads();
+    PHASE_MARK(2);
+
+    float sc[NT][4];
+    float mx = -INFINITY;
+    {
+        const int dbase = i + a.M - 4 * g;      // delta of key 4g of tile 0
+        const int pbase = a.d_pos - 1 - dbase;  // its rel row before clamping
+        const int pmax = a.d_pos - 1;
+        const unsigned dlim = i < a.T ? (unsigned)a.attn_len : 0u;
+        float af[2][NS];
+        load_afrag<NS>(af[0], Ks + il * RS + g);
+#pragma unroll
+        for (int jt = 0; jt < NT; jt++) {
+            if (jt + 1 < NT) load_afrag<NS>(af[(jt + 1) & 1], Ks + ((jt + 1) * 16 + il) * RS + g);
+            PIPELINE_FENCE();
+            // shifted rel and bias of the 4 keys of this lane: loaded unconditionally
+            // (clamped / padded, always inside the arrays) and selected afterwards
+            float relv[4], bv[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                int delta = dbase - (jt * 16 + r);
+                int pi = pbase + (jt * 16 + r); // d_pos-1-delta
+                pi = pi < 0 ? 0 : (pi > pmax ? pmax : pi);
+                relv[r] = Rw[pi];
+                bv[r] = Bs[(a.K - 1 - delta) & (FA_NB - 1)];
+            }
+            floatx4_t acc = { 0, 0, 0, 0 };
+#pragma unroll
+            for (int s = 0; s < NS; s++) acc = mfma16(af[jt & 1][s], qf[s], acc);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                // key j < K is implied: delta >= 0 > i - T for a real column
+                unsigned delta = (unsigned)(dbase - (jt * 16 + r));
+                float v = delta < dlim ? acc[r] + relv[r] + bv[r] : -INFINITY;
+                sc[jt][r] = v;
+                mx = fmaxf(mx, v);
+            }
+        }
+    }
+    PHASE_MARK(3);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    if (mx == -INFINITY) mx = 0.0f; // padding column
+    float sum = 0.0f;
+#pragma unroll
+    for (int jt = 0; jt < NT; jt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float e = __expf(sc[jt][r] - mx); // exp(-inf) = 0 for masked keys
+            sc[jt][r] = e;
+            sum += e;
+        }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+#pragma unroll
+    for (int jt = 0; jt < NT; jt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) sc[jt][r] *= inv;
+
+    if (a.probs && i < a.T) {
+        float *pc = a.probs + (((int64_t)b * a.H + h) * a.T + i) * a.K;
+        const bool vec = (a.K & 3) == 0;
+#pragma unroll
+        for (int jt = 0; jt < NT; jt++) {
+            int j0 = jt * 16 + 4 * g;
+            if (vec && j0 < a.K) {
+                floatx4_t v = { sc[jt][0], sc[jt][1], sc[jt][2], sc[jt][3] };
+                *reinterpret_cast<floatx4_t *>(pc + j0) = v;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (j0 + r < a.K) pc[j0 + r] = sc[jt][r];
+            }
+        }
+    }
+    put_rows<DK, KR>(Vs, vv);
+    __syncthreads();
+    PHASE_MARK(4);
+
+    // O = V P: the ND feature tiles are independent accumulation chains
+    {
+        floatx4_t acc[ND];
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++) acc[dt] = floatx4_t{ 0, 0, 0, 0 };
+        float vf[2][ND][4];
+        load_tokfrag<ND, RS>(vf[0], Vs, 0, g, il);
+#pragma unroll
+        for (int jt = 0; jt < NT; jt++) {
+            if (jt + 1 < NT) load_tokfrag<ND, RS>(vf[(jt + 1) & 1], Vs, jt + 1, g, il);
+            PIPELINE_FENCE();
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++) acc[dt] = mfma16(vf[jt & 1][dt][r], sc[jt][r], acc[dt]);
+        }
+        if (i < a.T) {
+#pragma unroll
+            for (int dt = 0; dt < ND; dt++) {
+                float *o = a.out + (int64_t)h * DK + dt * 16 + 4 * g + a.ldo * (b + (int64_t)a.B * i);
+                *reinterpret_cast<floatx4_t *>(o) = acc[dt];
+            }
+        }
+    }
+    PHASE_MARK(5);
+}
+
+template <int DK, int NT>
+struct BwdLayout {
+    static constexpr int RS = DK + 4, KR = NT * 16;
+    static constexpr int kw_a = 2 * KR * RS, kw_b = 2 * KR * FA_PSTRIDE, kw = kw_a > kw_b ? kw_a : kw_b;
+    static constexpr int v_a = KR * RS, v_b = FA_TMAX * FA_RSTRIDE, vsz = v_a > v_b ? v_a : v_b;
+    static constexpr int q = 0, o = q + FA_TMAX * RS, k = o + FA_TMAX * RS, w = k + KR * RS,
+                         v = k + kw, floats = v + vsz;
+    static constexpr int pt = k, st = k + KR * FA_PSTRIDE; // over K / w_r once they are dead
+    static constexpr int red = o;                          // db_r halves, over dO once it is dead
+};
+
+template <int DK, int NT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void relpos_attn_bwd_fused(FusedAttnBwdArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    using L = BwdLayout<DK, NT>;
+    constexpr int RS = DK + 4, NS = DK / 4, ND = DK / 16, KR = NT * 16, PS = FA_PSTRIDE;
+    constexpr int NSQ = FA_TMAX / 4;
+    float *Qs = lds + L::q, *Os = lds + L::o, *Ks = lds + L::k, *Ws = lds + L::w, *Vs = lds + L::v;
+    float *Rs = Vs;           // [64][FA_RSTRIDE] dRel, once V is dead
+    float *Pt = lds + L::pt;  // [KR][PS] P^T
+    float *St = lds + L::st;  // [KR][PS] dS^T
+
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int b = blockIdx.x % a.B, h = blockIdx.x / a.B; // as in the forward
+    const bool has_w = a.w_r != nullptr;
+    const int il = lane & 15, g = lane >> 4;
+    const int i = 16 * w + il;
+    PHASE_MARK(0);
+
+    // every global load is issued up front, in the order the phases need the
+    // tiles; each tile is parked in LDS just before its first use
+    floatx4_t vq[FA_TMAX * (DK / 4) / 256], vo[FA_TMAX * (DK / 4) / 256], vw[KR * (DK / 4) / 256],
+        vk[KR * (DK / 4) / 256], vv[KR * (DK / 4) / 256];
+    float p[NT][4], ds[NT][4];
+    {
+        auto kvrow = [&](int r) {
+            return (r < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * r)
+                            : a.kv + a.ldkv * (b + (int64_t)a.B * (r - a.M))) + (int64_t)h * DK;
+        };
+        fetch_rows<DK, FA_TMAX>(vo, a.T, [&](int r) { return a.dout + (int64_t)h * DK + a.ldo * (b + (int64_t)a.B * r); });
+        fetch_rows<DK, KR>(vv, a.K, [&](int r) { return kvrow(r) + (int64_t)a.H * DK; });
+        const float *pc = a.probs + (((int64_t)b * a.H + h) * a.T + (i < a.T ? i : 0)) * a.K;
+        const bool vec = (a.K & 3) == 0;
+#pragma unroll
+        for (int jt = 0; jt < NT; jt++) {
+            floatx4_t pv = { 0, 0, 0, 0 };
+            int j0 = jt * 16 + 4 * g;
+            if (vec) { // unconditional load from a clamped address, then select
+                floatx4_t x = *reinterpret_cast<const floatx4_t *>(pc + (j0 < a.K ? j0 : 0));
+                if (i < a.T && j0 < a.K) pv = x;
+            } else if (i < a.T) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (j0 + r < a.K) pv[r] = pc[j0 + r];
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) p[jt][r] = pv[r];
+        }
+        fetch_rows<DK, KR>(vk, a.K, kvrow);
+        fetch_rows<DK, KR>(vw, has_w ? a.d_pos : 0, [&](int r) { return has_w ? a.w_r + ((int64_t)h * a.d_pos + r) * DK : a.q; });
+        fetch_rows<DK, FA_TMAX>(vq, a.T, [&](int r) { return a.q + (int64_t)h * DK + a.ldq * (b + (int64_t)a.B * r); });
+    }
+    put_rows<DK, FA_TMAX>(Os, vo);
+    put_rows<DK, KR>(Vs, vv);
+    __syncthreads();
+    PHASE_MARK(1);
+
+    // dA = V^T dO, then dS = P (dA - colsum(P dA)) / sqrt(dk)
+    {
+        float dof[NS];
+#pragma unroll
+        for (int s = 0; s < NS; s++) dof[s] = Os[i * RS + 4 * s + g];
+        float af[2][NS];
+        load_afrag<NS>(af[0], Vs + il * RS + g);
+        float dot = 0.0f;
+#pragma unroll
+        for (int jt = 0; jt < NT; jt++) {
+            if (jt + 1 < NT) load_afrag<NS>(af[(jt + 1) & 1], Vs + ((jt + 1) * 16 + il) * RS + g);
+            PIPELINE_FENCE();
+            floatx4_t acc = { 0, 0, 0, 0 };
+#pragma unroll
+            for (int s = 0; s < NS; s++) acc = mfma16(af[jt & 1][s], dof[s], acc);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                ds[jt][r] = acc[r];
+                dot += p[jt][r] * acc[r];
+            }
+        }
+        dot += __shfl_xor(dot, 16, 64);
+        dot += __shfl_xor(dot, 32, 64);
+#pragma unroll
+        for (int jt = 0; jt < NT; jt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) ds[jt][r] = p[jt][r] * (ds[jt][r] - dot) * a.scale; // masked: p = 0
+    }
+    PHASE_MARK(2);
+    put_rows<DK, KR>(Ks, vk);
+    put_rows<DK, KR>(Ws, vw);
+    put_rows<DK, FA_TMAX>(Qs, vq);
+    __syncthreads(); // K, w_r, Q visible; every wavefront is done with V: its space becomes the dRel strip
+    PHASE_MARK(3);
+
+    float *Rw = Rs + i * FA_RSTRIDE;
+    {
+        // dRel[pi(delta), i] = sum of dS over the keys that read that row
+        for (int pp = g; pp < KR; pp += 4) Rw[pp] = 0.0f;
+        wave_lds_sync();
+        const int dbase = i + a.M - 4 * g, pbase = a.d_pos - 1 - dbase;
+        const unsigned dlim = (i < a.T && has_w) ? (unsigned)a.attn_len : 0u;
+        float acc0 = 0.0f;
+#pragma unroll
+        for (int jt = 0; jt < NT; jt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                unsigned delta = (unsigned)(dbase - (jt * 16 + r));
+                int pi = pbase + (jt * 16 + r);
+                // rows >= 1 receive exactly one key; row 0 collects the far keys;
+                // masked keys go to a dump slot past the strip (never read)
+                const bool on = delta < dlim;
+                Rw[(on && pi >= 1) ? pi : FA_RSTRIDE - 1] = ds[jt][r];
+                acc0 += (on && pi < 1) ? ds[jt][r] : 0.0f;
+            }
+        acc0 += __shfl_xor(acc0, 16, 64);
+        acc0 += __shfl_xor(acc0, 32, 64);
+        if (g == 0) Rw[0] = acc0;
+        wave_lds_sync();
+    }
+    // dq = K dS + w_r dRel: ND independent accumulation chains
+    {
+        floatx4_t dqa[ND];
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++) dqa[dt] = floatx4_t{ 0, 0, 0, 0 };
+        float kf[2][ND][4], rf[2][4];
+        load_tokfrag<ND, RS>(kf[0], Ks, 0, g, il);
+#pragma unroll
+        for (int jt = 0; jt < NT; jt++) {
+            if (jt + 1 < NT) load_tokfrag<ND, RS>(kf[(jt + 1) & 1], Ks, jt + 1, g, il);
+            else {
+                load_tokfrag<ND, RS>(kf[(jt + 1) & 1], Ws, 0, g, il);
+#pragma unroll
+                for (int r = 0; r < 4; r++) rf[(jt + 1) & 1][r] = Rw[4 * g + r];
+            }
+            PIPELINE_FENCE();
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++) dqa[dt] = mfma16(kf[jt & 1][dt][r], ds[jt][r], dqa[dt]);
+        }
+#pragma unroll
+        for (int pt = 0; pt < NT; pt++) {
+            constexpr int o = NT & 1; // buffer parity continues from the key loop
+            if (pt + 1 < NT) {
+                load_tokfrag<ND, RS>(kf[(pt + 1 + o) & 1], Ws, pt + 1, g, il);
+#pragma unroll
+                for (int r = 0; r < 4; r++) rf[(pt + 1 + o) & 1][r] = Rw[(pt + 1) * 16 + 4 * g + r];
+            }
+            PIPELINE_FENCE();
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++)
+                    dqa[dt] = mfma16(kf[(pt + o) & 1][dt][r], rf[(pt + o) & 1][r], dqa[dt]);
+        }
+        if (i < a.T) {
+#pragma unroll
+            for (int dt = 0; dt < ND; dt++) {
+                float *o = a.dq + (int64_t)h * DK + dt * 16 + 4 * g + a.ldq * (b + (int64_t)a.B * i);
+                *reinterpret_cast<floatx4_t *>(o) = dqa[dt];
+            }
+        }
+    }
+    PHASE_MARK(4);
+    __syncthreads(); // K and w_r are dead: park P^T and dS^T over them
+#pragma unroll
+    for (int jt = 0; jt < NT; jt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            int j = jt * 16 + 4 * g + r;
+            Pt[j * PS + i] = p[jt][r];
+            St[j * PS + i] = ds[jt][r];
+        }
+    __syncthreads();
+    PHASE_MARK(5);
+
+    // the contraction now runs over the query index; k-slot g of step s is
+    // query 16*(s/4) + 4g + s%4, which keeps the Q / dO reads conflict-free
+    auto load_qd = [&](float (&f)[ND], const float *base, int s) {
+        int iq = 16 * (s >> 2) + 4 * g + (s & 3);
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++) f[dt] = base[iq * RS + dt * 16 + il];
+    };
+    // dK = Q dS^T, dV = dO P^T: wavefront w owns key tiles w, w+4, ...
+#pragma unroll
+    for (int u = 0; u < NT / 4; u++) {
+        const int jt = w + 4 * u;
+        float sb[NSQ], pb[NSQ];
+#pragma unroll
+        for (int s = 0; s < NSQ; s++) {
+            int iq = 16 * (s >> 2) + 4 * g + (s & 3);
+            sb[s] = St[(jt * 16 + il) * PS + iq];
+            pb[s] = Pt[(jt * 16 + il) * PS + iq];
+        }
+        floatx4_t ak[ND], av[ND];
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++) { ak[dt] = floatx4_t{ 0, 0, 0, 0 }; av[dt] = floatx4_t{ 0, 0, 0, 0 }; }
+        float qa[2][ND], oa[2][ND];
+        load_qd(qa[0], Qs, 0);
+        load_qd(oa[0], Os, 0);
+#pragma unroll
+        for (int s = 0; s < NSQ; s++) {
+            if (s + 1 < NSQ) { load_qd(qa[(s + 1) & 1], Qs, s + 1); load_qd(oa[(s + 1) & 1], Os, s + 1); }
+            PIPELINE_FENCE();
+#pragma unroll
+            for (int dt = 0; dt < ND; dt++) {
+                ak[dt] = mfma16(qa[s & 1][dt], sb[s], ak[dt]);
+                av[dt] = mfma16(oa[s & 1][dt], pb[s], av[dt]);
+            }
+        }
+        const int j = jt * 16 + il;
+        if (j < a.K) {
+            float *dst = (j < a.M ? a.dkvm + a.ldkv * (b + (int64_t)a.B * j)
+                                  : a.dkv + a.ldkv * (b + (int64_t)a.B * (j - a.M))) + (int64_t)h * DK;
+#pragma unroll
+            for (int dt = 0; dt < ND; dt++) {
+                *reinterpret_cast<floatx4_t *>(dst + dt * 16 + 4 * g) = ak[dt];
+                *reinterpret_cast<floatx4_t *>(dst + (int64_t)a.H * DK + dt * 16 + 4 * g) = av[dt];
+            }
+        }
+    }
+    PHASE_MARK(6);
+    // dw_r partial of this (stream, head): Q dRel^T, wavefront w owns position tiles w, w+4, ...
+    if (has_w) {
+        float *dwz = a.dwp + ((int64_t)b * a.H + h) * a.d_pos * DK;
+#pragma unroll
+        for (int u = 0; u < NT / 4; u++) {
+            const int pt = w + 4 * u;
+            float rb[NSQ];
+#pragma unroll
+            for (int s = 0; s < NSQ; s++) {
+                int iq = 16 * (s >> 2) + 4 * g + (s & 3);
+                rb[s] = Rs[iq * FA_RSTRIDE + pt * 16 + il];
+            }
+            floatx4_t acc[ND];
+#pragma unroll
+            for (int dt = 0; dt < ND; dt++) acc[dt] = floatx4_t{ 0, 0, 0, 0 };
+            float qa[2][ND];
+            load_qd(qa[0], Qs, 0);
+#pragma unroll
+            for (int s = 0; s < NSQ; s++) {
+                if (s + 1 < NSQ) load_qd(qa[(s + 1) & 1], Qs, s + 1);
+                PIPELINE_FENCE();
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++) acc[dt] = mfma16(qa[s & 1][dt], rb[s], acc[dt]);
+            }
+            const int pp = pt * 16 + il;
+            if (pp < a.d_pos) {
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++)
+                    *reinterpret_cast<floatx4_t *>(dwz + (int64_t)pp * DK + dt * 16 + 4 * g) = acc[dt];
+            }
+        }
+    }
+    PHASE_MARK(7);
+    // db_r partial: row K-1-delta collects the diagonal delta of dS.  Threads
+    // t and t+128 sum the two halves of the query range; the halves meet in LDS
+    // (over dO, dead once every wavefront has left the dK/dV phase).
+    if (a.dbp) {
+        __syncthreads();
+        float *red = lds + L::red;
+        const int delta = t & 127, half = t >> 7;
+        float acc = 0.0f;
+        if (delta < a.K) {
+#pragma unroll 8
+            for (int q8 = 0; q8 < FA_TMAX / 2; q8++) {
+                int iq = half * (FA_TMAX / 2) + q8;
+                int j = iq + a.M - delta;
+                bool on = iq < a.T && j >= 0 && j < a.K;
+                float v = St[(on ? j : 0) * PS + iq];
+                acc += on ? v : 0.0f;
+            }
+        }
+        if (half) red[delta] = acc;
+        __syncthreads();
+        if (!half && delta < a.K)
+            a.dbp[((int64_t)b * a.H + h) * a.K + (a.K - 1 - delta)] = a.b_r_scale * (acc + red[delta]);
+    }
+    PHASE_MARK(8);
+}
+
+// dw_r (n_w) and db_r (n_b) = sums over the B per-stream partials, in stream order
+__global__ __launch_bounds__(256) void attn_param_grad_reduce(const float *dwp, float *dw, int64_t n_w,
+                                                              const float *dbp, float *db, int64_t n_b, int B)
+{
+    int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const float *src;
+    float *dst;
+    int64_t n;
+    if (e < n_w) { src = dwp + e; dst = dw + e; n = n_w; }
+    else if (e < n_w + n_b) { src = dbp + (e - n_w); dst = db + (e - n_w); n = n_b; }
+    else return;
+    float acc = 0.0f;
+    for (int b = 0; b < B; b++) acc += src[(int64_t)b * n];
+    *dst = acc;
+}
+
+template <typename KernelT>
+bool allow_lds(KernelT kern, size_t bytes)
+{
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return true;
+}
+
+template <int DK, int NT>
+int launch_fwd(hipStream_t st, const FusedAttnFwdArgs &a)
+{
+    constexpr size_t bytes = sizeof(float) * FwdLayout<DK, NT>::floats;
+    static_assert(bytes <= 160 * 1024, "forward tiles exceed LDS");
+    static const bool ok = allow_lds(relpos_attn_fwd_fused<DK, NT>, bytes);
+    if (!ok) return -1;
+    hipLaunchKernelGGL((relpos_attn_fwd_fused<DK, NT>), dim3(a.B * a.H), dim3(256), bytes, st, a);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <int DK, int NT>
+int launch_bwd(hipStream_t st, const FusedAttnBwdArgs &a)
+{
+    constexpr size_t bytes = sizeof(float) * BwdLayout<DK, NT>::floats;
+    static_assert(bytes <= 160 * 1024, "backward tiles exceed LDS");
+    static const bool ok = allow_lds(relpos_attn_bwd_fused<DK, NT>, bytes);
+    if (!ok) return -1;
+    hipLaunchKernelGGL((relpos_attn_bwd_fused<DK, NT>), dim3(a.B * a.H), dim3(256), bytes, st, a);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+} // namespace
+
+bool k_attn_fused_shape_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr)
+{
+    return dk == dv && (dk == 64 || dk == 32) && T <= FA_TMAX && K <= 128 && (!has_wr || d_pos <= 128);
+}
+
+int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk)
+{
+    const bool small = a.K <= 64 && a.d_pos <= 64;
+    if (dk == 64) return small ? launch_fwd<64, 4>(st, a) : launch_fwd<64, 8>(st, a);
+    return small ? launch_fwd<32, 4>(st, a) : launch_fwd<32, 8>(st, a);
+}
+
+int k_attn_fused_bwd(hipStream_t st, const FusedAttnBwdArgs &a, int dk, float *dw_r, float *db_r,
+                     int64_t n_w, int64_t n_b, int *launches)
+{
+    const bool small = a.K <= 64 && a.d_pos <= 64;
+    int rc = dk == 64 ? (small ? launch_bwd<64, 4>(st, a) : launch_bwd<64, 8>(st, a))
+                      : (small ? launch_bwd<32, 4>(st, a) : launch_bwd<32, 8>(st, a));
+    if (rc) return rc;
+    *launches = 1;
+    if (n_w + n_b > 0) {
+        hipLaunchKernelGGL(attn_param_grad_reduce, dim3((unsigned)((n_w + n_b + 255) / 256)), dim3(256), 0, st,
+                           (const float *)a.dwp, dw_r, n_w, (const float *)a.dbp, db_r, n_b, a.B);
+        *launches = 2;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}

@@ -72,4 +72,25 @@ void k_pad_bwd(hipStream_t st, const float *gy, float *gx, int64_t n_in, int64_t
                int64_t left, int lop, int64_t right, int rop);
 }
 
+// single-kernel rel-pos attention for heads that fit in LDS (k_attn_fused.hip)
+struct FusedAttnFwdArgs {
+    const float *q, *kv, *kvm, *w_r, *b_r;
+    float *out, *probs;
+    int64_t ldq, ldkv, ldo;
+    int H, B, T, M, K, d_pos, attn_len;
+    float b_r_scale, scale;
+};
+struct FusedAttnBwdArgs {
+    const float *q, *kv, *kvm, *w_r, *probs, *dout;
+    float *dq, *dkv, *dkvm, *dwp, *dbp; // dwp / dbp: per-stream partials in scratch
+    int64_t ldq, ldkv, ldo;
+    int H, B, T, M, K, d_pos, attn_len;
+    float b_r_scale, scale;
+};
+bool k_attn_fused_shape_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr);
+int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk);
+// returns 0, -1 (path unavailable, nothing launched) or -2 (launch failed)
+int k_attn_fused_bwd(hipStream_t st, const FusedAttnBwdArgs &a, int dk, float *dw_r, float *db_r,
+                     int64_t n_w, int64_t n_b, int *launches);
+
 #endif
