@@ -80,6 +80,11 @@ void nchip_gemm_profile_enable(int on);
 int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launches,
                             double *flops, double *seconds);
 
+/* Tuning aid: forces tile configuration `cfg` (an index into the table in
+   k_gemm.hip) for every later nchip_gemm* call; 0 restores the automatic
+   choice.  The environment variable NCHIP_GEMM_CFG sets the initial value. */
+void nchip_gemm_force_config(int cfg);
+
 /* Chooses ksplit for nchip_gemm from the shape alone (never from data). */
 int nchip_gemm_pick_ksplit(int m, int n, int k, int batch);
 

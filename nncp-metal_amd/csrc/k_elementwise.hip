@@ -179,7 +179,9 @@ __global__ void lstm_clamped_bwd_kernel(const float *cp, const float *in, const 
     }
 }
 
-// stage 1: tmp[s][i] = sum over the s-th slice of the outer axis (sequential)
+// stage 1: tmp[s][i] = sum over the s-th slice of the outer axis.  Four
+// interleaved chains (rows o0+u, o0+u+4, ...) keep four loads in flight; they
+// are combined in chain order.
 __global__ void reduce_trailing_stage1(const float *x, float *tmp, int64_t inner, int64_t outer,
                                        int nsplit)
 {
@@ -188,20 +190,36 @@ __global__ void reduce_trailing_stage1(const float *x, float *tmp, int64_t inner
     if (i >= inner) return;
     int64_t per = (outer + nsplit - 1) / nsplit;
     int64_t o0 = s * per, o1 = o0 + per < outer ? o0 + per : outer;
-    float acc = 0.0f;
-    for (int64_t o = o0; o < o1; o++)
-        acc += x[i + o * inner];
-    tmp[(int64_t)s * inner + i] = acc;
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+    int64_t o = o0;
+    for (; o + 3 < o1; o += 4) {
+        a0 += x[i + o * inner];
+        a1 += x[i + (o + 1) * inner];
+        a2 += x[i + (o + 2) * inner];
+        a3 += x[i + (o + 3) * inner];
+    }
+    for (; o < o1; o++) a0 += x[i + o * inner];
+    tmp[(int64_t)s * inner + i] = (a0 + a1) + (a2 + a3);
 }
 
-__global__ void reduce_trailing_stage2(const float *tmp, const float *y0, float *out,
-                                       int64_t inner, int nsplit)
+// stage 2: out[i] = y0[i] + sum_s tmp[s][i]; 4 interleaved slice groups per
+// element (sequential inside a group), combined in group order
+__global__ __launch_bounds__(256) void reduce_trailing_stage2(const float *tmp, const float *y0, float *out,
+                                                              int64_t inner, int nsplit)
 {
-    GRID_STRIDE(i, inner) {
-        float acc = y0 ? y0[i] : 0.0f;
-        for (int s = 0; s < nsplit; s++)
-            acc += tmp[(int64_t)s * inner + i];
-        out[i] = acc;
+    __shared__ float sh[3][64];
+    const int ig = threadIdx.x & 63, rg = threadIdx.x >> 6;
+    const int64_t i = (int64_t)blockIdx.x * 64 + ig;
+    float acc = 0.0f;
+    if (i < inner) {
+#pragma unroll 4
+        for (int s = rg; s < nsplit; s += 4) acc += tmp[(int64_t)s * inner + i];
+    }
+    if (rg > 0) sh[rg - 1][ig] = acc;
+    __syncthreads();
+    if (rg == 0 && i < inner) {
+        acc = (acc + sh[0][ig]) + (sh[1][ig] + sh[2][ig]);
+        out[i] = y0 ? y0[i] + acc : acc;
     }
 }
 
@@ -390,7 +408,7 @@ int k_reduce_trailing_nsplit(int64_t inner, int64_t outer)
     int64_t blocks_x = (inner + TPB - 1) / TPB;
     int64_t s = 512 / (blocks_x > 0 ? blocks_x : 1);
     if (s > outer / 8) s = outer / 8;
-    if (s > 32) s = 32;
+    if (s > 64) s = 64;
     if (s < 1) s = 1;
     return (int)s;
 }
@@ -401,7 +419,7 @@ void k_reduce_trailing(hipStream_t st, const float *x, const float *y0, float *o
     int ns = k_reduce_trailing_nsplit(inner, outer);
     dim3 grid((unsigned)((inner + TPB - 1) / TPB), ns);
     hipLaunchKernelGGL(reduce_trailing_stage1, grid, dim3(TPB), 0, st, x, tmp, inner, outer, ns);
-    hipLaunchKernelGGL(reduce_trailing_stage2, dim3(nblocks(inner)), dim3(TPB), 0, st, (const float *)tmp, y0, out, inner, ns);
+    hipLaunchKernelGGL(reduce_trailing_stage2, dim3((unsigned)((inner + 63) / 64)), dim3(256), 0, st, (const float *)tmp, y0, out, inner, ns);
 }
 
 void k_reduce_all(hipStream_t st, const float *x, float *out, float *tmp, int64_t n)

@@ -150,18 +150,25 @@ struct TileLoader {
     }
 };
 
-template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16>
-__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs g0)
+// KW = 2 doubles the wavefronts of a workgroup without shrinking its tile: the
+// two groups of WM x WN wavefronts share the LDS tiles and split every 32-deep
+// k slab, group 0 taking k%32 < 16 and group 1 the rest; group 1 hands its
+// accumulators over through LDS at the end (C = chain0 + chain1, fixed order).
+template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16, int KW = 1>
+__global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 {
     GemmArgs g = g0;
-    constexpr int NT = 64 * WM * WN;                      // threads: WM x WN wavefronts
+    static_assert(KW == 1 || (KW == 2 && BK % 32 == 0), "k groups split 32-deep slabs");
+    constexpr int NT = 64 * WM * WN * KW;                 // threads: KW groups of WM x WN wavefronts
     constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN); // 32x32 MFMA tiles per wavefront
     constexpr int WTM = BM / WM, WTN = BN / WN;           // wavefront tile
     constexpr int LDS_A = BF16 ? BM * (BK + 8) / 2 : BK * (BM + PAD); // in floats
     constexpr int LDS_B = BF16 ? BN * (BK + 8) / 2 : BK * (BN + PAD);
+    static_assert(KW == 1 || BM * BN <= 2 * (LDS_A + LDS_B), "accumulator hand-over must fit in the tile buffers");
     __shared__ __attribute__((aligned(16))) float smem[2 * (LDS_A + LDS_B)];
 
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int t = threadIdx.x, lane = t & 63;
+    const int kg = (t >> 6) / (WM * WN), wave = (t >> 6) % (WM * WN);
     const int wm = wave % WM, wn = wave / WM;
 
     // XCD-aware tile order: the hardware deals consecutive workgroup ids round
@@ -245,20 +252,21 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs g0)
         // latency is paid in full at the next LDS write
         __builtin_amdgcn_sched_barrier(0);
         if (BF16) {
-            // one 32x32x16 MFMA per tile pair per 16 k
+            // one 32x32x16 MFMA per tile pair per 16 k; group kg takes every KW-th
             const unsigned short *ha = reinterpret_cast<const unsigned short *>(sa);
             const unsigned short *hb = reinterpret_cast<const unsigned short *>(sb);
 #pragma unroll
-            for (int kb = 0; kb < BK / 16; kb++) {
+            for (int u = 0; u < BK / 16 / KW; u++) {
+                const int kofs = (u * KW + kg) * 16;
                 shortx8 fa[TM], fb[TN];
 #pragma unroll
                 for (int j = 0; j < TM; j++)
                     fa[j] = *reinterpret_cast<const shortx8 *>(
-                        ha + (wm * WTM + j * 32 + (lane & 31)) * (BK + 8) + kb * 16 + (lane >> 5) * 8);
+                        ha + (wm * WTM + j * 32 + (lane & 31)) * (BK + 8) + kofs + (lane >> 5) * 8);
 #pragma unroll
                 for (int i = 0; i < TN; i++)
                     fb[i] = *reinterpret_cast<const shortx8 *>(
-                        hb + (wn * WTN + i * 32 + (lane & 31)) * (BK + 8) + kb * 16 + (lane >> 5) * 8);
+                        hb + (wn * WTN + i * 32 + (lane & 31)) * (BK + 8) + kofs + (lane >> 5) * 8);
 #pragma unroll
                 for (int i = 0; i < TN; i++)
 #pragma unroll
@@ -269,22 +277,26 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs g0)
                             acc[i][j], 0, 0, 0);
             }
         } else {
-            // fragments of k-step ks+1 are fetched while the MFMAs of ks run
+            // fragments of k-step u+1 are fetched while the MFMAs of u run.
+            // LDS row of step u: 2u (KW = 1), or the u-th pair of this group's
+            // half of each 32-deep slab (KW = 2)
+            constexpr int NSTEP = BK / 2 / KW;
+            auto krow = [](int u) { return KW == 1 ? 2 * u : (u >> 3) * 32 + 2 * (u & 7); };
             float fa[2][TM], fb[2][TN];
-            const float *pa = sa + (lane >> 5) * (BM + PAD) + wm * WTM + (lane & 31);
-            const float *pb = sb + (lane >> 5) * (BN + PAD) + wn * WTN + (lane & 31);
+            const float *pa = sa + ((lane >> 5) + kg * 16) * (BM + PAD) + wm * WTM + (lane & 31);
+            const float *pb = sb + ((lane >> 5) + kg * 16) * (BN + PAD) + wn * WTN + (lane & 31);
 #pragma unroll
             for (int j = 0; j < TM; j++) fa[0][j] = pa[j * 32];
 #pragma unroll
             for (int i = 0; i < TN; i++) fb[0][i] = pb[i * 32];
 #pragma unroll
-            for (int ks = 0; ks < BK / 2; ks++) {
-                const int cur = ks & 1, nxt = cur ^ 1;
-                if (ks + 1 < BK / 2) {
+            for (int u = 0; u < NSTEP; u++) {
+                const int cur = u & 1, nxt = cur ^ 1;
+                if (u + 1 < NSTEP) {
 #pragma unroll
-                    for (int j = 0; j < TM; j++) fa[nxt][j] = pa[(ks + 1) * 2 * (BM + PAD) + j * 32];
+                    for (int j = 0; j < TM; j++) fa[nxt][j] = pa[krow(u + 1) * (BM + PAD) + j * 32];
 #pragma unroll
-                    for (int i = 0; i < TN; i++) fb[nxt][i] = pb[(ks + 1) * 2 * (BN + PAD) + i * 32];
+                    for (int i = 0; i < TN; i++) fb[nxt][i] = pb[krow(u + 1) * (BN + PAD) + i * 32];
                 }
 #pragma unroll
                 for (int i = 0; i < TN; i++)
@@ -308,6 +320,28 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs g0)
             step(it, nk, std::true_type());
     for (; it < nk; it++) // edge tiles and the k tail
         step(it, nk, std::false_type());
+
+    if (KW == 2) {
+        // group 1 parks its accumulators in LDS (the tiles are dead), group 0 adds them
+        __syncthreads();
+        float *red = smem + (size_t)wave * (TN * TM * 16 * 64) + lane;
+        if (kg == 1) {
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+#pragma unroll
+                for (int j = 0; j < TM; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) red[((i * TM + j) * 16 + r) * 64] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (kg == 1) return;
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int j = 0; j < TM; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] += red[((i * TM + j) * 16 + r) * 64];
+    }
 
     // epilogue.  acc[i][j][r] is C[m][n] with
     //   m = m0 + wm*BM/2 + j*32 + lane%32
@@ -385,18 +419,19 @@ struct ProfRec {
     double flops;
 };
 bool g_prof_on = false;
+int g_force_cfg = getenv("NCHIP_GEMM_CFG") ? atoi(getenv("NCHIP_GEMM_CFG")) : 0;
 std::vector<ProfRec> g_prof;
 
-template <int BM, int BN, int BK, int WM, int WN, int BF16>
+template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1>
 void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
-    dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(64 * WM * WN);
-    if (!ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 0, 0, BF16>), grid, block, 0, st, g);
-    else if (ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 1, 0, BF16>), grid, block, 0, st, g);
-    else if (!ta && tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 0, 1, BF16>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 1, 1, BF16>), grid, block, 0, st, g);
+    dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(64 * WM * WN * KW);
+    if (!ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 0, 0, BF16, KW>), grid, block, 0, st, g);
+    else if (ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 1, 0, BF16, KW>), grid, block, 0, st, g);
+    else if (!ta && tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 0, 1, BF16, KW>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 1, 1, BF16, KW>), grid, block, 0, st, g);
 }
 
 } // namespace
@@ -460,17 +495,17 @@ extern "C" int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, fl
         (void)hipEventRecord(rec.start, st);
     }
     // Tile configuration from the shape alone.  Measured on MI355X (fp32):
-    // small outputs want the most workgroups (64x64, 4 wavefronts); once
+    // small outputs want the most workgroups and the most wavefronts per
+    // workgroup (64x64x32, two k groups of 4 wavefronts); once
     // 128x64 tiles still give >= 256 workgroups, 8 wavefronts of 32x32 on a
     // 128x64x32 tile win; very large problems use 128x128x32 with 8 wavefronts.
-    static const char *ecfg = getenv("NCHIP_GEMM_CFG"); // tuning aid: forces a configuration
-    int cfg = ecfg ? atoi(ecfg) : 0;
+    int cfg = g_force_cfg; // tuning aid: 0 = choose from the shape
     int64_t nb = (int64_t)batch * ksplit;
     int64_t t128x64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64) * nb;
     if (!cfg) {
         if (t128 >= 512 && m >= 128 && n >= 128) cfg = 7;
         else if (t128x64 >= 256 && m >= 128 && n >= 64) cfg = 4;
-        else cfg = 5;
+        else cfg = 8;
     }
     if (precision == 1) {
         if (cfg == 7) launch_tile<128, 128, 32, 4, 2, 1>(st, ta, tb, g);
@@ -488,11 +523,15 @@ extern "C" int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, fl
         launch_tile<64, 128, 16, 2, 2, 0>(st, ta, tb, g);
     } else if (cfg == 7) {
         launch_tile<128, 128, 32, 4, 2, 0>(st, ta, tb, g);
+    } else if (cfg == 8) {
+        launch_tile<64, 64, 32, 2, 2, 0, 2>(st, ta, tb, g);
+    } else if (cfg == 9) {
+        launch_tile<64, 64, 64, 2, 2, 0, 2>(st, ta, tb, g);
     } else {
         launch_tile<64, 64, 16, 2, 2, 0>(st, ta, tb, g);
     }
     if (g_prof_on) {
-        int tile = cfg == 7 ? 2 : (cfg == 4 ? 1 : 0);
+        int tile = cfg == 7 ? 2 : (cfg == 4 ? 1 : (cfg == 8 ? 3 : 0));
         rec.variant = tile * 8 + (ta ? 4 : 0) + (tb ? 2 : 0) + (precision == 1 ? 1 : 0);
         (void)hipEventRecord(rec.stop, st);
         g_prof.push_back(rec);
@@ -523,6 +562,12 @@ extern "C" int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, flo
                        workspace);
 }
 
+// tuning aid: forces tile configuration `cfg` for every later call (0 = automatic)
+extern "C" void nchip_gemm_force_config(int cfg)
+{
+    g_force_cfg = cfg;
+}
+
 // ---- profiling entry points ---------------------------------------------------
 extern "C" void nchip_gemm_profile_enable(int on)
 {
@@ -532,13 +577,13 @@ extern "C" void nchip_gemm_profile_enable(int on)
 extern "C" int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launches,
                                        double *flops, double *seconds)
 {
-    double fl[24] = { 0 }, sec[24] = { 0 };
-    int64_t cnt[24] = { 0 };
+    double fl[32] = { 0 }, sec[32] = { 0 };
+    int64_t cnt[32] = { 0 };
     for (ProfRec &r : g_prof) {
         float ms = 0.0f;
         (void)hipEventSynchronize(r.stop);
         (void)hipEventElapsedTime(&ms, r.start, r.stop);
-        if (r.variant >= 0 && r.variant < 24) {
+        if (r.variant >= 0 && r.variant < 32) {
             fl[r.variant] += r.flops;
             sec[r.variant] += ms * 1e-3;
             cnt[r.variant]++;
@@ -547,11 +592,12 @@ extern "C" int nchip_gemm_profile_read(int max_variants, char (*names)[48], int6
         (void)hipEventDestroy(r.stop);
     }
     g_prof.clear();
-    static const char *tiles[3] = { "64,64,16,2,2", "128,64,32,4,2", "128,128,32,4,2" };
+    static const char *tiles[4] = { "64,64,16,2,2", "128,64,32,4,2", "128,128,32,4,2", "64,64,32,2,2" };
     int n = 0;
-    for (int v = 0; v < 24 && n < max_variants; v++) {
+    for (int v = 0; v < 32 && n < max_variants; v++) {
         if (!cnt[v]) continue;
-        snprintf(names[n], 48, "gemm_kernel<%s,%d,%d,%d>", tiles[v / 8], (v >> 2) & 1, (v >> 1) & 1, v & 1);
+        snprintf(names[n], 48, "gemm_kernel<%s,%d,%d,%d%s>", tiles[v / 8], (v >> 2) & 1, (v >> 1) & 1, v & 1,
+                 v / 8 == 3 ? ",2" : "");
         launches[n] = cnt[v]; flops[n] = fl[v]; seconds[n] = sec[v];
         n++;
     }

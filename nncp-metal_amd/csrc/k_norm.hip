@@ -93,17 +93,87 @@ __global__ __launch_bounds__(TPB) void norm_bwd_wb_stage1(const float *g, const 
     partial[((int64_t)s * 2 + 1) * d + i] = ab;
 }
 
-__global__ void norm_bwd_wb_stage2(const float *partial, float *dw, float *db, int d, int rows)
+// d = 64*NV: dx and the per-block dw / db partials in ONE pass over g and xhat.
+// A wavefront walks cw consecutive columns keeping them in registers; its
+// per-lane dw / db sums are combined over the 4 wavefronts in wavefront order
+// and written as partial row blockIdx.x.
+template <int NV>
+__global__ __launch_bounds__(TPB) void norm_bwd_fused(const float *g, const float *xhat, const float *rstd,
+                                                      const float *w, float *dx, float *partial,
+                                                      int64_t n, int avg, int cw)
 {
-    int i = blockIdx.x * TPB + threadIdx.x;
-    if (i >= d) return;
-    float aw = 0.0f, ab = 0.0f;
-    for (int s = 0; s < rows; s++) {
-        aw += partial[((int64_t)s * 2) * d + i];
-        ab += partial[((int64_t)s * 2 + 1) * d + i];
+    constexpr int D = NV * 64;
+    __shared__ float sh[WPB - 1][2][D];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    float wr[NV], aw[NV], ab[NV];
+#pragma unroll
+    for (int v = 0; v < NV; v++) { wr[v] = w ? w[lane + 64 * v] : 1.0f; aw[v] = 0.0f; ab[v] = 0.0f; }
+    const int64_t c0 = ((int64_t)blockIdx.x * WPB + wv) * cw;
+    for (int k = 0; k < cw; k++) {
+        const int64_t c = c0 + k;
+        if (c >= n) break;
+        float gv[NV], hv[NV];
+#pragma unroll
+        for (int v = 0; v < NV; v++) { gv[v] = g[c * D + lane + 64 * v]; hv[v] = xhat[c * D + lane + 64 * v]; }
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            float gh = gv[v] * wr[v];
+            s1 += gh;
+            s2 += gh * hv[v];
+            aw[v] += gv[v] * hv[v];
+            ab[v] += gv[v];
+        }
+        if (dx) {
+            s1 = avg ? wave_sum(s1) / (float)D : 0.0f;
+            s2 = wave_sum(s2) / (float)D;
+            const float r = rstd[c];
+#pragma unroll
+            for (int v = 0; v < NV; v++) dx[c * D + lane + 64 * v] = r * (gv[v] * wr[v] - s1 - hv[v] * s2);
+        }
     }
-    if (dw) dw[i] = aw;
-    if (db) db[i] = ab;
+    if (!partial) return;
+    if (wv > 0) {
+#pragma unroll
+        for (int v = 0; v < NV; v++) { sh[wv - 1][0][lane + 64 * v] = aw[v]; sh[wv - 1][1][lane + 64 * v] = ab[v]; }
+    }
+    __syncthreads();
+    if (wv == 0) {
+        float *pw = partial + (int64_t)blockIdx.x * 2 * D, *pb = pw + D;
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            float a = aw[v], b = ab[v];
+#pragma unroll
+            for (int u = 0; u < WPB - 1; u++) { a += sh[u][0][lane + 64 * v]; b += sh[u][1][lane + 64 * v]; }
+            pw[lane + 64 * v] = a;
+            pb[lane + 64 * v] = b;
+        }
+    }
+}
+
+// dw[i], db[i] = sum of the partial rows: 4 interleaved row groups per element
+// (sequential inside a group), combined in group order
+__global__ __launch_bounds__(TPB) void norm_bwd_wb_stage2(const float *partial, float *dw, float *db, int d, int rows)
+{
+    __shared__ float sh[WPB - 1][2][64];
+    const int ig = threadIdx.x & 63, rg = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + ig;
+    float aw = 0.0f, ab = 0.0f;
+    if (i < d) {
+#pragma unroll 4
+        for (int s = rg; s < rows; s += WPB) {
+            aw += partial[((int64_t)s * 2) * d + i];
+            ab += partial[((int64_t)s * 2 + 1) * d + i];
+        }
+    }
+    if (rg > 0) { sh[rg - 1][0][ig] = aw; sh[rg - 1][1][ig] = ab; }
+    __syncthreads();
+    if (rg == 0 && i < d) {
+#pragma unroll
+        for (int u = 0; u < WPB - 1; u++) { aw += sh[u][0][ig]; ab += sh[u][1][ig]; }
+        if (dw) dw[i] = aw;
+        if (db) db[i] = ab;
+    }
 }
 
 __global__ __launch_bounds__(TPB) void softmax_fwd_kernel(const float *x, float *y, int v, int64_t n)
@@ -168,10 +238,45 @@ __global__ void get_col_kernel(const float *w, const int32_t *idx, float *y, int
     }
 }
 
-// one block per vocabulary entry; the token loop is sequential so that columns
-// sharing a symbol are added in increasing token order
+// Embedding gradient dw[:, sym] = sum of the columns whose token is sym, added
+// in increasing token order.  One block per vocabulary entry: the block first
+// lists its columns in order (each thread scans a contiguous slice of the
+// tokens, an exclusive prefix over the threads places its hits), then every
+// thread sums its feature rows down the list, so each column of g is read once.
+constexpr int ADD_COL_MAX_N = 8192; // tokens whose indices fit the LDS list
+
 __global__ __launch_bounds__(TPB) void add_col_kernel(const float *g, const int32_t *idx, float *dw,
                                                       int d, int64_t n)
+{
+    __shared__ int list[ADD_COL_MAX_N];
+    __shared__ int cnt[TPB + 1];
+    const int sym = blockIdx.x, t = threadIdx.x;
+    const int per = (int)((n + TPB - 1) / TPB);
+    const int c0 = t * per, c1 = (int)(c0 + per < n ? c0 + per : n);
+    int mine = 0;
+    for (int c = c0; c < c1; c++) mine += idx[c] == sym;
+    cnt[t + 1] = mine;
+    if (t == 0) cnt[0] = 0;
+    __syncthreads();
+    if (t == 0)
+        for (int k = 1; k <= TPB; k++) cnt[k] += cnt[k - 1];
+    __syncthreads();
+    int pos = cnt[t];
+    for (int c = c0; c < c1; c++)
+        if (idx[c] == sym) list[pos++] = c;
+    __syncthreads();
+    const int total = cnt[TPB];
+    for (int i = t; i < d; i += TPB) {
+        float acc = 0.0f;
+#pragma unroll 4
+        for (int k = 0; k < total; k++) acc += g[(int64_t)list[k] * d + i];
+        dw[(int64_t)sym * d + i] = acc;
+    }
+}
+
+// any n: every block scans all tokens for every feature slice
+__global__ __launch_bounds__(TPB) void add_col_scan_kernel(const float *g, const int32_t *idx, float *dw,
+                                                           int d, int64_t n)
 {
     int sym = blockIdx.x;
     for (int i0 = 0; i0 < d; i0 += TPB) {
@@ -278,12 +383,19 @@ int nchip_norm_fwd(void *stream, const float *x, const float *w, const float *b,
     return check("nchip_norm_fwd");
 }
 
+// columns per wavefront of the fused backward: 2, more when that would give
+// more than 1024 partial rows
+static int norm_bwd_cw(int64_t n)
+{
+    int64_t cw = (n + (int64_t)WPB * 1024 - 1) / ((int64_t)WPB * 1024);
+    return (int)(cw < 2 ? 2 : cw);
+}
+
 int nchip_norm_bwd_partial_rows(int64_t n)
 {
-    int64_t r = n / 16;
-    if (r > 32) r = 32;
-    if (r < 1) r = 1;
-    return (int)r;
+    int cw = norm_bwd_cw(n);
+    int64_t r = (n + (int64_t)WPB * cw - 1) / ((int64_t)WPB * cw);
+    return (int)(r < 32 ? 32 : r); // the generic path uses up to 32 slices
 }
 
 int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float *rstd, const float *w,
@@ -291,15 +403,28 @@ int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float 
 {
     if (n <= 0 || d <= 0) return 0;
     hipStream_t st = (hipStream_t)stream;
+    const bool wb = dw || db;
+    if (wb && !partial) { fprintf(stderr, "nchip_norm_bwd: partial buffer missing\n"); return -1; }
+    if (d == 128 || d == 256 || d == 512 || d == 1024) {
+        const int cw = norm_bwd_cw(n);
+        const int rows = (int)((n + (int64_t)WPB * cw - 1) / ((int64_t)WPB * cw));
+        float *pp = wb ? partial : nullptr;
+#define NORM_BWD(NV) hipLaunchKernelGGL(norm_bwd_fused<NV>, dim3(rows), dim3(TPB), 0, st, g, xhat, rstd, w, dx, pp, n, avg, cw)
+        if (d == 128) NORM_BWD(2); else if (d == 256) NORM_BWD(4); else if (d == 512) NORM_BWD(8); else NORM_BWD(16);
+#undef NORM_BWD
+        if (wb)
+            hipLaunchKernelGGL(norm_bwd_wb_stage2, dim3((d + 63) / 64), dim3(TPB), 0, st,
+                               (const float *)partial, dw, db, d, rows);
+        return check("nchip_norm_bwd");
+    }
     if (dx)
         hipLaunchKernelGGL(norm_bwd_dx_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, st,
                            g, xhat, rstd, w, dx, d, n, avg);
-    if (dw || db) {
-        if (!partial) { fprintf(stderr, "nchip_norm_bwd: partial buffer missing\n"); return -1; }
-        int rows = nchip_norm_bwd_partial_rows(n);
+    if (wb) {
+        int rows = (int)(n / 16 > 32 ? 32 : (n / 16 < 1 ? 1 : n / 16));
         hipLaunchKernelGGL(norm_bwd_wb_stage1, dim3((d + TPB - 1) / TPB, rows), dim3(TPB), 0, st,
                            g, xhat, partial, d, n, rows);
-        hipLaunchKernelGGL(norm_bwd_wb_stage2, dim3((d + TPB - 1) / TPB), dim3(TPB), 0, st,
+        hipLaunchKernelGGL(norm_bwd_wb_stage2, dim3((d + 63) / 64), dim3(TPB), 0, st,
                            (const float *)partial, dw, db, d, rows);
     }
     return check("nchip_norm_bwd");
@@ -345,7 +470,10 @@ int nchip_get_col(void *stream, const float *w, const int32_t *idx, float *y, in
 int nchip_add_col(void *stream, const float *g, const int32_t *idx, float *dw, int d, int v, int64_t n)
 {
     if (v <= 0 || d <= 0) return 0;
-    hipLaunchKernelGGL(add_col_kernel, dim3(v), dim3(TPB), 0, (hipStream_t)stream, g, idx, dw, d, n);
+    if (n <= ADD_COL_MAX_N)
+        hipLaunchKernelGGL(add_col_kernel, dim3(v), dim3(TPB), 0, (hipStream_t)stream, g, idx, dw, d, n);
+    else
+        hipLaunchKernelGGL(add_col_scan_kernel, dim3(v), dim3(TPB), 0, (hipStream_t)stream, g, idx, dw, d, n);
     return check("nchip_add_col");
 }
 

@@ -193,3 +193,62 @@ def test_host_tensor_compute_is_refused(pkg):
             "nc.nc_add(a, nc.dup(a))") % (__file__.rsplit("/", 1)[0],)
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
     assert r.returncode != 0 and "GPU only" in r.stderr
+
+
+def _run_graph(nc, arrays, build, weight):
+    hs = [nc.param(a, "p%d" % i) for i, a in enumerate(arrays)]
+    y = build(nc, *[nc.dup(h.value) for h, _ in hs])
+    out = nc.numpy(y)
+    loss = nc.nc_sum(nc.nc_mul(y, nc.tensor(weight)))
+    g = nc.backward(loss)
+    nc.free(loss)
+    return out, [g[p] for _, p in hs]
+
+
+@pytest.mark.parametrize("d,n", [(128, 80), (256, 37), (512, 2048), (512, 100), (1024, 64), (96, 50)])
+@pytest.mark.parametrize("avg", [0, 1])
+def test_norm_model_shapes(hip, ref, rng, d, n, avg):
+    """LayerNorm / RMSNorm with affine at the widths the single-pass backward
+    is specialised for (and one it is not), ragged column counts included."""
+    arrays = [rng.standard_normal((n, d)).astype(np.float32),
+              (1 + 0.1 * rng.standard_normal(d)).astype(np.float32),
+              (0.1 * rng.standard_normal(d)).astype(np.float32)]
+    weight = rng.standard_normal((n, d)).astype(np.float32)
+    build = lambda nc, x, w, b: nc.nc_fused_layer_norm(x, w, b, 1e-5, avg)
+    (oh, gh), (orf, gr) = (_run_graph(nc, arrays, build, weight) for nc in (hip, ref))
+    assert relerr(oh, orf) <= TOL
+    for a, b in zip(gh, gr):
+        assert relerr(a, b) <= 5 * TOL
+
+
+@pytest.mark.parametrize("v,d,n", [(256, 512, 2048), (50, 128, 333), (16, 40, 9000)])
+def test_embedding_gradient_model_shapes(hip, ref, rng, v, d, n):
+    """get_col backward (deterministic scatter-add), including a token count
+    beyond the in-LDS index list."""
+    w = rng.standard_normal((v, d)).astype(np.float32)
+    idx = rng.integers(0, v, size=n).astype(np.int32)
+    idx[: min(n, 7)] = 3  # repeated symbol
+    weight = rng.standard_normal((n, d)).astype(np.float32)
+    res = []
+    for nc in (hip, ref):
+        build = lambda nc, w_: nc.nc_get_col(w_, nc.tensor(idx))
+        res.append(_run_graph(nc, [w], build, weight))
+    assert np.array_equal(res[0][0], res[1][0])
+    assert relerr(res[0][1][0], res[1][1][0]) <= 5 * TOL
+    # same inputs, same bits
+    again = _run_graph(hip, [w], lambda nc, w_: nc.nc_get_col(w_, nc.tensor(idx)), weight)
+    assert np.array_equal(again[1][0], res[0][1][0])
+
+
+@pytest.mark.parametrize("f,n", [(2048, 2048), (512, 2048), (256, 77), (1000, 513)])
+def test_bias_gradient_model_shapes(hip, ref, rng, f, n):
+    """Column-sum reductions behind the bias gradients (two-stage, fixed order)."""
+    x = rng.standard_normal((n, f)).astype(np.float32)
+    b = rng.standard_normal(f).astype(np.float32)
+    weight = rng.standard_normal((n, f)).astype(np.float32)
+    build = lambda nc, x_, b_: nc.nc_add(x_, b_)
+    (oh, gh), (orf, gr) = (_run_graph(nc, [x, b], build, weight) for nc in (hip, ref))
+    assert relerr(oh, orf) <= TOL
+    exact = weight.astype(np.float64).sum(axis=0)
+    assert relerr(gh[1], exact) <= TOL
+    assert relerr(gh[1], gr[1]) <= 5 * TOL
