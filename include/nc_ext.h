@@ -26,6 +26,11 @@ extern "C" {
    the matmul + bias pairs at nncp.c:659-661, 970-972, 1002-1004. */
 NCTensor *nc_linear(NCTensor *w, NCTensor *x, NCTensor *bias, int act);
 
+/* y = act(w * x + bias) + res, res shaped like the result: the linear layer
+   together with the residual connection that follows it (nncp.c:896, 979).
+   Gradients flow to w, x, bias and res. */
+NCTensor *nc_linear_add(NCTensor *w, NCTensor *x, NCTensor *bias, int act, NCTensor *res);
+
 /* Relative-position causal attention over memory + current segment, all
    heads and streams in one call.  Replaces nncp.c:722-800 and the
    split_head/concat_head copies (nncp.c:554-579).

@@ -41,6 +41,17 @@ int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, float alpha,
                const float *bias, int act, float *pre, int precision,
                int ksplit, float *workspace);
 
+/* C = act(alpha * op(A) * op(B) + bias) + addend, with addend laid out like C
+   (ldc, stride_c; may alias nothing written by the call).  Used for residual
+   connections (nncp.c:803, 975) and to add an incoming gradient in the same
+   pass instead of a separate element-wise sum. */
+int nchip_gemm_add(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                   const float *A, int64_t lda, int64_t stride_a,
+                   const float *B, int64_t ldb, int64_t stride_b,
+                   float *C, int64_t ldc, int64_t stride_c, int batch,
+                   const float *bias, int act, float *pre, const float *addend,
+                   int precision, int ksplit, float *workspace);
+
 /* Same with two-level batching: batch index z addresses
    A + (z / batch_in)*sa_out + (z % batch_in)*sa_in (likewise B and C).  Lets
    per-(stream, head) products read the (features, streams, time) activations
@@ -125,12 +136,13 @@ int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
 int nchip_norm_fwd(void *stream, const float *x, const float *w, const float *b,
                    float *y, float *xhat, float *rstd, int d, int64_t n,
                    float eps, int avg);
-/* dx (d,n); dw, db (d) overwritten (may be NULL when w is NULL).  partial
-   needs nchip_norm_bwd_partial_rows(n) * 2 * d floats. */
+/* dx (d,n) = gradient of the input, plus dx_add (d,n) when that is not NULL;
+   dw, db (d) overwritten (may be NULL when w is NULL).  partial needs
+   nchip_norm_bwd_partial_rows(n) * 2 * d floats. */
 int nchip_norm_bwd_partial_rows(int64_t n);
 int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float *rstd,
-                   const float *w, float *dx, float *dw, float *db, float *partial,
-                   int d, int64_t n, int avg);
+                   const float *w, float *dx, const float *dx_add, float *dw, float *db,
+                   float *partial, int d, int64_t n, int avg);
 
 /* softmax over axis 0 of (v, n) and its backward dx = y*(g - sum(g*y))
    (libnc.h:382; nncp.c:796, 1008). */

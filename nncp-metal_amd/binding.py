@@ -113,6 +113,7 @@ _PROTOS = {
     "vec_sum_f32": (_F, [C.POINTER(_F), _SZ]),
     # nc_ext.h
     "nc_linear": (_P, [_P, _P, _P, _I]),
+    "nc_linear_add": (_P, [_P, _P, _P, _I, _P]),
     "nc_relpos_attention": (_P, [_P, _P, _P, _P, _P, _I, _I, _I, _F]),
     "nc_soft_max_cdf16": (_P, [_P]), "nc_cdf_lookup": (_P, [_P, _P]),
     "nc_exp_det": (_F, [_F]),

@@ -38,6 +38,7 @@ struct GemmArgs {
     const float *A, *B;
     float *C;
     const float *bias;
+    const float *add; // same layout as C, added after the activation (may be NULL)
     float *pre;
     float *ws;
     int64_t lda, ldb, ldc, sa, sb, sc;   // outer batch strides
@@ -210,8 +211,10 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     const bool a_full = (m0 + BM <= g.M) && (g.lda % 4 == 0) && (((uintptr_t)A & 15) == 0);
     const bool b_full = (n0 + BN <= g.N) && (g.ldb % 4 == 0) && (((uintptr_t)B & 15) == 0);
 
-    TileLoader<BM, BK, TA ? 0 : 1, NT> la;
-    TileLoader<BN, BK, TB ? 1 : 0, NT> lb;
+    // two register sets: while tile it is computed, tile it+1 has arrived (or is
+    // about to) and tile it+2 is in flight, so a load has two compute phases to land
+    TileLoader<BM, BK, TA ? 0 : 1, NT> la0, la1;
+    TileLoader<BN, BK, TB ? 1 : 0, NT> lb0, lb1;
 
     floatx16 acc[TN][TM];
 #pragma unroll
@@ -222,14 +225,14 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.0f;
 
-    // One pipeline step: write the prefetched registers to LDS buffer `buf`,
-    // barrier, start the global loads of tile `next` (when there is one), then
-    // the MFMAs of the tile in `buf`.  One barrier per tile is enough because a
-    // buffer is rewritten only two tiles later.  FAST is a compile-time flag so
-    // the steady-state loop carries no guarded-load code: the guarded path
-    // shares registers with the vector loads and the compiler then serialises
-    // every prefetch behind an s_waitcnt vmcnt(0).
-    auto step = [&](int it, int nk, auto fast_tag) {
+    // One pipeline step: write the register set holding tile `it` to LDS buffer
+    // it&1, barrier, refill that set with tile it+2 (when there is one), then
+    // the MFMAs of tile `it`.  One barrier per tile is enough because a buffer
+    // is rewritten only two tiles later.  FAST is a compile-time flag so the
+    // steady-state loop carries no guarded-load code: the guarded path shares
+    // registers with the vector loads and the compiler then serialises every
+    // prefetch behind an s_waitcnt vmcnt(0).
+    auto step = [&](int it, int nk, auto fast_tag, auto &la, auto &lb) {
         constexpr bool FAST = decltype(fast_tag)::value;
         float *sa = smem + (it & 1) * (LDS_A + LDS_B);
         float *sb = sa + LDS_A;
@@ -241,8 +244,8 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
             lb.store_f32(sb, t);
         }
         __syncthreads();
-        if (FAST || it + 1 < nk) {
-            int k0 = kbeg + (it + 1) * BK;
+        if (FAST || it + 2 < nk) {
+            int k0 = kbeg + (it + 2) * BK;
             bool kf = FAST || (k0 + BK <= kend);
             la.load(A, g.lda, m0, k0, g.M, kend, FAST || (a_full && kf), t);
             lb.load(B, g.ldb, n0, k0, g.N, kend, FAST || (b_full && kf), t);
@@ -282,21 +285,28 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
             // half of each 32-deep slab (KW = 2)
             constexpr int NSTEP = BK / 2 / KW;
             auto krow = [](int u) { return KW == 1 ? 2 * u : (u >> 3) * 32 + 2 * (u & 7); };
-            float fa[2][TM], fb[2][TN];
+            // FD-1 k-steps of fragments are in flight ahead of the MFMAs: with one
+            // 32x32 tile per wavefront a k-step is a single 64-cycle MFMA, shorter
+            // than an LDS round trip
+            constexpr int FD = NSTEP < 4 ? NSTEP : 4;
+            float fa[FD][TM], fb[FD][TN];
             const float *pa = sa + ((lane >> 5) + kg * 16) * (BM + PAD) + wm * WTM + (lane & 31);
             const float *pb = sb + ((lane >> 5) + kg * 16) * (BN + PAD) + wn * WTN + (lane & 31);
 #pragma unroll
-            for (int j = 0; j < TM; j++) fa[0][j] = pa[j * 32];
+            for (int u = 0; u < FD - 1; u++) {
 #pragma unroll
-            for (int i = 0; i < TN; i++) fb[0][i] = pb[i * 32];
+                for (int j = 0; j < TM; j++) fa[u][j] = pa[krow(u) * (BM + PAD) + j * 32];
+#pragma unroll
+                for (int i = 0; i < TN; i++) fb[u][i] = pb[krow(u) * (BN + PAD) + i * 32];
+            }
 #pragma unroll
             for (int u = 0; u < NSTEP; u++) {
-                const int cur = u & 1, nxt = cur ^ 1;
-                if (u + 1 < NSTEP) {
+                const int cur = u % FD, nxt = (u + FD - 1) % FD;
+                if (u + FD - 1 < NSTEP) {
 #pragma unroll
-                    for (int j = 0; j < TM; j++) fa[nxt][j] = pa[krow(u + 1) * (BM + PAD) + j * 32];
+                    for (int j = 0; j < TM; j++) fa[nxt][j] = pa[krow(u + FD - 1) * (BM + PAD) + j * 32];
 #pragma unroll
-                    for (int i = 0; i < TN; i++) fb[nxt][i] = pb[krow(u + 1) * (BN + PAD) + i * 32];
+                    for (int i = 0; i < TN; i++) fb[nxt][i] = pb[krow(u + FD - 1) * (BN + PAD) + i * 32];
                 }
 #pragma unroll
                 for (int i = 0; i < TN; i++)
@@ -312,14 +322,23 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     int it = 0;
     if (nk > 0) {
         bool kf = nk_full > 0;
-        la.load(A, g.lda, m0, kbeg, g.M, kend, a_full && kf, t);
-        lb.load(B, g.ldb, n0, kbeg, g.N, kend, b_full && kf, t);
+        la0.load(A, g.lda, m0, kbeg, g.M, kend, a_full && kf, t);
+        lb0.load(B, g.ldb, n0, kbeg, g.N, kend, b_full && kf, t);
     }
-    if (a_full && b_full) // steady state: tile it+1 is complete, unguarded vector loads
-        for (; it + 1 < nk_full; it++)
-            step(it, nk, std::true_type());
-    for (; it < nk; it++) // edge tiles and the k tail
-        step(it, nk, std::false_type());
+    if (nk > 1) {
+        bool kf = nk_full > 1;
+        la1.load(A, g.lda, m0, kbeg + BK, g.M, kend, a_full && kf, t);
+        lb1.load(B, g.ldb, n0, kbeg + BK, g.N, kend, b_full && kf, t);
+    }
+    if (a_full && b_full) // steady state: tiles it+2, it+3 are complete, unguarded vector loads
+        for (; it + 3 < nk_full; it += 2) {
+            step(it, nk, std::true_type(), la0, lb0);
+            step(it + 1, nk, std::true_type(), la1, lb1);
+        }
+    for (; it < nk; it++) { // edge tiles and the k tail (it is even when the loop starts)
+        if (it & 1) step(it, nk, std::false_type(), la1, lb1);
+        else step(it, nk, std::false_type(), la0, lb0);
+    }
 
     if (KW == 2) {
         // group 1 parks its accumulators in LDS (the tiles are dead), group 0 adds them
@@ -368,6 +387,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     const int64_t coff = (int64_t)b_out * g.sc + (int64_t)b_in * g.sc_in;
     float *C = g.C + coff;
     float *P = g.pre ? g.pre + coff : nullptr;
+    const float *Radd = g.add ? g.add + coff : nullptr;
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
@@ -384,7 +404,9 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
                 if (g.beta != 0.0f) v += g.beta * C[off];
                 v += bv;
                 if (P) P[off] = v;
-                C[off] = apply_act(v, g.act);
+                v = apply_act(v, g.act);
+                if (Radd) v += Radd[off];
+                C[off] = v;
             }
         }
 }
@@ -397,6 +419,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce(GemmArgs g)
     const int64_t coff = (int64_t)(b / g.batch_in) * g.sc + (int64_t)(b % g.batch_in) * g.sc_in;
     float *C = g.C + coff;
     float *P = g.pre ? g.pre + coff : nullptr;
+    const float *Radd = g.add ? g.add + coff : nullptr;
     for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
         int m = (int)(e % g.M);
         int64_t n = e / g.M;
@@ -408,7 +431,9 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce(GemmArgs g)
         if (g.beta != 0.0f) v += g.beta * C[off];
         if (g.bias) v += g.bias[m];
         if (P) P[off] = v;
-        C[off] = apply_act(v, g.act);
+        v = apply_act(v, g.act);
+        if (Radd) v += Radd[off];
+        C[off] = v;
     }
 }
 
@@ -450,13 +475,13 @@ extern "C" int nchip_gemm_pick_ksplit(int m, int n, int k, int batch)
     return s < 1 ? 1 : s;
 }
 
-extern "C" int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, float alpha,
-                           const float *A, int64_t lda, int64_t sa_out, int64_t sa_in,
-                           const float *B, int64_t ldb, int64_t sb_out, int64_t sb_in,
-                           float beta, float *C, int64_t ldc, int64_t sc_out, int64_t sc_in,
-                           int batch, int batch_in,
-                           const float *bias, int act, float *pre, int precision,
-                           int ksplit, float *workspace)
+static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                      const float *A, int64_t lda, int64_t sa_out, int64_t sa_in,
+                      const float *B, int64_t ldb, int64_t sb_out, int64_t sb_in,
+                      float beta, float *C, int64_t ldc, int64_t sc_out, int64_t sc_in,
+                      int batch, int batch_in,
+                      const float *bias, int act, float *pre, const float *addend, int precision,
+                      int ksplit, float *workspace)
 {
     if (m <= 0 || n <= 0 || batch <= 0)
         return 0;
@@ -475,7 +500,7 @@ extern "C" int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, fl
         return -1;
     }
     GemmArgs g;
-    g.A = A; g.B = B; g.C = C; g.bias = bias; g.pre = pre; g.ws = workspace;
+    g.A = A; g.B = B; g.C = C; g.bias = bias; g.add = addend; g.pre = pre; g.ws = workspace;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.sa = sa_out; g.sb = sb_out; g.sc = sc_out;
     g.sa_in = sa_in; g.sb_in = sb_in; g.sc_in = sc_in; g.batch_in = batch_in;
     g.M = m; g.N = n; g.K = k; g.batch = batch; g.ksplit = ksplit;
@@ -548,6 +573,31 @@ extern "C" int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, fl
         return -2;
     }
     return 0;
+}
+
+extern "C" int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                           const float *A, int64_t lda, int64_t sa_out, int64_t sa_in,
+                           const float *B, int64_t ldb, int64_t sb_out, int64_t sb_in,
+                           float beta, float *C, int64_t ldc, int64_t sc_out, int64_t sc_in,
+                           int batch, int batch_in,
+                           const float *bias, int act, float *pre, int precision,
+                           int ksplit, float *workspace)
+{
+    return gemm2_impl(stream, ta, tb, m, n, k, alpha, A, lda, sa_out, sa_in, B, ldb, sb_out, sb_in,
+                      beta, C, ldc, sc_out, sc_in, batch, batch_in, bias, act, pre, nullptr, precision,
+                      ksplit, workspace);
+}
+
+extern "C" int nchip_gemm_add(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                              const float *A, int64_t lda, int64_t stride_a,
+                              const float *B, int64_t ldb, int64_t stride_b,
+                              float *C, int64_t ldc, int64_t stride_c, int batch,
+                              const float *bias, int act, float *pre, const float *addend,
+                              int precision, int ksplit, float *workspace)
+{
+    return gemm2_impl(stream, ta, tb, m, n, k, alpha, A, lda, stride_a, 0, B, ldb, stride_b, 0,
+                      0.0f, C, ldc, stride_c, 0, batch, 1, bias, act, pre, addend, precision, ksplit,
+                      workspace);
 }
 
 extern "C" int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, float alpha,

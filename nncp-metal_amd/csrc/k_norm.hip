@@ -54,7 +54,7 @@ __global__ __launch_bounds__(TPB) void norm_fwd_kernel(const float *x, const flo
 // dx = rstd * (gh - mean(gh) - xhat * mean(gh * xhat)),  gh = g * w
 __global__ __launch_bounds__(TPB) void norm_bwd_dx_kernel(const float *g, const float *xhat,
                                                           const float *rstd, const float *w,
-                                                          float *dx, int d, int64_t n, int avg)
+                                                          float *dx, const float *dx_add, int d, int64_t n, int avg)
 {
     int lane = threadIdx.x & 63;
     int64_t c = (int64_t)blockIdx.x * WPB + (threadIdx.x >> 6);
@@ -71,7 +71,8 @@ __global__ __launch_bounds__(TPB) void norm_bwd_dx_kernel(const float *g, const 
     float r = rstd[c];
     for (int i = lane; i < d; i += 64) {
         float gh = w ? gc[i] * w[i] : gc[i];
-        dx[c * d + i] = r * (gh - s1 - hc[i] * s2);
+        float v = r * (gh - s1 - hc[i] * s2);
+        dx[c * d + i] = dx_add ? dx_add[c * d + i] + v : v;
     }
 }
 
@@ -99,8 +100,8 @@ __global__ __launch_bounds__(TPB) void norm_bwd_wb_stage1(const float *g, const 
 // and written as partial row blockIdx.x.
 template <int NV>
 __global__ __launch_bounds__(TPB) void norm_bwd_fused(const float *g, const float *xhat, const float *rstd,
-                                                      const float *w, float *dx, float *partial,
-                                                      int64_t n, int avg, int cw)
+                                                      const float *w, float *dx, const float *dx_add,
+                                                      float *partial, int64_t n, int avg, int cw)
 {
     constexpr int D = NV * 64;
     __shared__ float sh[WPB - 1][2][D];
@@ -129,7 +130,10 @@ __global__ __launch_bounds__(TPB) void norm_bwd_fused(const float *g, const floa
             s2 = wave_sum(s2) / (float)D;
             const float r = rstd[c];
 #pragma unroll
-            for (int v = 0; v < NV; v++) dx[c * D + lane + 64 * v] = r * (gv[v] * wr[v] - s1 - hv[v] * s2);
+            for (int v = 0; v < NV; v++) {
+                float val = r * (gv[v] * wr[v] - s1 - hv[v] * s2);
+                dx[c * D + lane + 64 * v] = dx_add ? dx_add[c * D + lane + 64 * v] + val : val;
+            }
         }
     }
     if (!partial) return;
@@ -399,7 +403,8 @@ int nchip_norm_bwd_partial_rows(int64_t n)
 }
 
 int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float *rstd, const float *w,
-                   float *dx, float *dw, float *db, float *partial, int d, int64_t n, int avg)
+                   float *dx, const float *dx_add, float *dw, float *db, float *partial, int d, int64_t n,
+                   int avg)
 {
     if (n <= 0 || d <= 0) return 0;
     hipStream_t st = (hipStream_t)stream;
@@ -409,7 +414,7 @@ int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float 
         const int cw = norm_bwd_cw(n);
         const int rows = (int)((n + (int64_t)WPB * cw - 1) / ((int64_t)WPB * cw));
         float *pp = wb ? partial : nullptr;
-#define NORM_BWD(NV) hipLaunchKernelGGL(norm_bwd_fused<NV>, dim3(rows), dim3(TPB), 0, st, g, xhat, rstd, w, dx, pp, n, avg, cw)
+#define NORM_BWD(NV) hipLaunchKernelGGL(norm_bwd_fused<NV>, dim3(rows), dim3(TPB), 0, st, g, xhat, rstd, w, dx, dx_add, pp, n, avg, cw)
         if (d == 128) NORM_BWD(2); else if (d == 256) NORM_BWD(4); else if (d == 512) NORM_BWD(8); else NORM_BWD(16);
 #undef NORM_BWD
         if (wb)
@@ -419,7 +424,7 @@ int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float 
     }
     if (dx)
         hipLaunchKernelGGL(norm_bwd_dx_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, st,
-                           g, xhat, rstd, w, dx, d, n, avg);
+                           g, xhat, rstd, w, dx, dx_add, d, n, avg);
     if (wb) {
         int rows = (int)(n / 16 > 32 ? 32 : (n / 16 < 1 ? 1 : n / 16));
         hipLaunchKernelGGL(norm_bwd_wb_stage1, dim3((d + TPB - 1) / TPB, rows), dim3(TPB), 0, st,

@@ -170,13 +170,31 @@ extern "C" void nc_backward(const NCTensor *x, NCTensor *grad, NCParamUpdateFunc
             continue;
         }
         std::vector<NCTensor *> ga(nd->n_args > 0 ? nd->n_args : 1, nullptr);
+        // offer the gradients the parents already hold: a backward kernel that
+        // can add one in its epilogue returns the finished sum (existing + new,
+        // the same two terms accumulate() would add)
+        for (int i = 0; i < NC_BW_ARGS; i++) {
+            NCNode *p = i < nd->n_args ? nd->parents[i] : nullptr;
+            bool again = false; // the same parent twice: only the first slot may take it
+            for (int j = 0; j < i && p; j++) again |= nd->parents[j] == p;
+            m->bw_prev[i] = (p && !again) ? p->grad : nullptr;
+            m->bw_used[i] = false;
+        }
         if (g) nc_node_backward(nd, g, ga.data());
         for (int i = 0; i < nd->n_args; i++) {
             NCNode *p = nd->parents[i];
             if (!p) { nc_free_tensor(ga[i]); continue; }
-            if (ga[i]) accumulate(p, ga[i]);
+            if (ga[i]) {
+                if (i < NC_BW_ARGS && m->bw_used[i]) {
+                    nc_free_tensor(p->grad);
+                    p->grad = ga[i];
+                } else {
+                    accumulate(p, ga[i]);
+                }
+            }
             if (--p->pending == 0) ready.push_back(p);
         }
+        for (int i = 0; i < NC_BW_ARGS; i++) { m->bw_prev[i] = nullptr; m->bw_used[i] = false; }
         nc_free_tensor(g);
         nc_free_node(nd);
     }

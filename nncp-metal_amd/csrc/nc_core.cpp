@@ -106,6 +106,7 @@ extern "C" NCContext *nc_context_init(int nb_threads)
     m->node_seq = 0;
     m->epoch = 0;
     m->defer_wgrad = false;
+    for (int i = 0; i < NC_BW_ARGS; i++) { m->bw_prev[i] = nullptr; m->bw_used[i] = false; }
     m->grp_staging = nullptr;
     m->grp_staging_cap = 0;
     const char *e = getenv("NCHIP_MATMUL_BF16");

@@ -49,6 +49,8 @@ struct DeferredGemm {
     float alpha;
 };
 
+#define NC_BW_ARGS 8 // node arguments for which nc_backward offers the existing gradient
+
 struct NCContext {
     int nb_threads;
     NCDevice cpu, hip;
@@ -60,6 +62,10 @@ struct NCContext {
     int64_t node_seq;
     int epoch;
     bool defer_wgrad;
+    // set by nc_backward around each node: gradients its parents already hold
+    // (bw_prev) and whether the node's backward folded them in (bw_used)
+    NCTensor *bw_prev[NC_BW_ARGS];
+    bool bw_used[NC_BW_ARGS];
     std::vector<DeferredGemm> deferred;
     void *grp_staging;
     size_t grp_staging_cap;

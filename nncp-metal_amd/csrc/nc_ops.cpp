@@ -518,15 +518,24 @@ static MMShape mm_shape(const NCTensor *a, const NCTensor *b, bool ta, bool tb)
 }
 
 // C (contiguous m x n per batch) = alpha op(A) op(B) + beta C [+ bias, act]
+// `addend` (laid out like C, or NULL) is added after the activation; beta must be 0 with it
 static void dev_gemm(NCContext *m, bool ta, bool tb, size_t M, size_t N, size_t K, float alpha,
                      const NCTensor *a, const NCTensor *b, float beta, NCTensor *c, size_t batch,
-                     const float *bias, int act, float *pre)
+                     const float *bias, int act, float *pre, const float *addend = nullptr)
 {
     int ks = nchip_gemm_pick_ksplit((int)M, (int)N, (int)K, (int)batch);
     size_t cap = 0;
     float *ws = nullptr;
     if (ks > 1) ws = nc_tmp_f32(m, batch * ks * M * N, &cap);
-    int rc = nchip_gemm(m->stream, ta, tb, (int)M, (int)N, (int)K, alpha,
+    int rc;
+    if (addend)
+        rc = nchip_gemm_add(m->stream, ta, tb, (int)M, (int)N, (int)K, alpha,
+                            nc_f32(a), (int64_t)(ta ? K : M), (int64_t)(M * K),
+                            nc_f32(b), (int64_t)(tb ? N : K), (int64_t)(K * N),
+                            nc_f32(c), (int64_t)M, (int64_t)(M * N), (int)batch,
+                            bias, act, pre, addend, m->matmul_bf16, ks, ws);
+    else
+        rc = nchip_gemm(m->stream, ta, tb, (int)M, (int)N, (int)K, alpha,
                         nc_f32(a), (int64_t)(ta ? K : M), (int64_t)(M * K),
                         nc_f32(b), (int64_t)(tb ? N : K), (int64_t)(K * N),
                         beta, nc_f32(c), (int64_t)M, (int64_t)(M * N), (int)batch,
@@ -552,10 +561,10 @@ extern "C" NCTensor *nc_matmul_add(NCTensor *a, NCTensor *b, NCTensor *c, BOOL t
         c = nc_contig(c);
         need_f32(c, "nc_matmul_add");
         if (nc_numel(c) != nc_numel(y)) nc_fatal("nc_matmul_add: addend shape mismatch");
-        hip_check(hipMemcpyAsync(nc_data(y), nc_data(c), nc_numel(y) * sizeof(float),
-                                 hipMemcpyDeviceToDevice, m->stream), "hipMemcpyAsync");
     }
-    dev_gemm(m, ta != 0, tb != 0, s.m, s.n, s.k, alpha, a, b, c ? 1.0f : 0.0f, y, s.batch, nullptr, 0, nullptr);
+    // the addend is read in the GEMM epilogue: no copy, no second pass
+    dev_gemm(m, ta != 0, tb != 0, s.m, s.n, s.k, alpha, a, b, 0.0f, y, s.batch, nullptr, 0, nullptr,
+             c ? nc_f32(c) : nullptr);
     NCTensor *args[3] = { a, b, c };
     NCNode *n = nc_new_node(m, OP_MATMUL, 3, args);
     if (a->node || b->node || (c && c->node)) {
@@ -570,6 +579,18 @@ extern "C" NCTensor *nc_matmul_add(NCTensor *a, NCTensor *b, NCTensor *c, BOOL t
 }
 
 extern "C" NCTensor *nc_matmul(NCTensor *w, NCTensor *x) { return nc_matmul_add(w, x, nullptr, 0, 0, 1.0f); }
+
+// During nc_backward: the gradient already delivered to parent `arg` of the
+// node being processed, when a kernel can add it in its own epilogue instead of
+// a separate element-wise sum.  Taking it marks it as consumed.
+static const float *nc_bw_addend(NCContext *m, int arg, size_t numel)
+{
+    if (arg >= NC_BW_ARGS || !m->bw_prev[arg]) return nullptr;
+    NCTensor *p = m->bw_prev[arg];
+    if (p->type != NC_TYPE_F32 || !nc_is_contig(p) || nc_numel(p) != numel) return nullptr;
+    m->bw_used[arg] = true;
+    return nc_f32(p);
+}
 
 // gradients of alpha op(A) op(B): the four transposition cases
 static void matmul_bw(NCNode *nd, NCTensor *g, NCTensor **ga, int ia, int ib)
@@ -597,14 +618,16 @@ static void matmul_bw(NCNode *nd, NCTensor *g, NCTensor **ga, int ia, int ib)
     }
     if (nd->parents[ib]) {
         NCTensor *db = nc_alloc_like(b);
-        if (!tb) dev_gemm(m, !ta, false, s.k, s.n, s.m, alpha, a, g, 0.0f, db, s.batch, nullptr, 0, nullptr);
-        else     dev_gemm(m, true, ta, s.n, s.k, s.m, alpha, g, a, 0.0f, db, s.batch, nullptr, 0, nullptr);
+        // a gradient already delivered to this parent is added in the epilogue
+        const float *prev = nc_bw_addend(m, ib, nc_numel(db));
+        if (!tb) dev_gemm(m, !ta, false, s.k, s.n, s.m, alpha, a, g, 0.0f, db, s.batch, nullptr, 0, nullptr, prev);
+        else     dev_gemm(m, true, ta, s.n, s.k, s.m, alpha, g, a, 0.0f, db, s.batch, nullptr, 0, nullptr, prev);
         ga[ib] = db;
     }
 }
 
-// y = act(w x + bias) in one GEMM with a fused epilogue (nc_ext.h)
-extern "C" NCTensor *nc_linear(NCTensor *w, NCTensor *x, NCTensor *bias, int act)
+// y = act(w x + bias) [+ res] in one GEMM with a fused epilogue (nc_ext.h)
+static NCTensor *linear_impl(NCTensor *w, NCTensor *x, NCTensor *bias, int act, NCTensor *res)
 {
     w = nc_contig(w); x = nc_contig(x);
     need_f32(w, "nc_linear"); need_f32(x, "nc_linear");
@@ -620,12 +643,17 @@ extern "C" NCTensor *nc_linear(NCTensor *w, NCTensor *x, NCTensor *bias, int act
     memcpy(dims, x->dims, sizeof(size_t) * x->n_dims);
     dims[0] = s.m;
     NCTensor *y = new_f32(w, x->n_dims, dims);
-    bool graph = w->node || x->node || (bias && bias->node);
+    if (res) {
+        res = nc_contig(res);
+        need_f32(res, "nc_linear_add");
+        if (nc_numel(res) != nc_numel(y)) nc_fatal("nc_linear_add: res must have the shape of the result");
+    }
+    bool graph = w->node || x->node || (bias && bias->node) || (res && res->node);
     NCTensor *pre = (act != NC_ACT_NONE && graph) ? nc_alloc_like(y) : nullptr;
     dev_gemm(m, false, false, s.m, s.n, s.k, 1.0f, w, x, 0.0f, y, 1, bias ? nc_f32(bias) : nullptr, act,
-             pre ? nc_f32(pre) : nullptr);
-    NCTensor *args[3] = { w, x, bias };
-    NCNode *n = nc_new_node(m, OP_LINEAR, 3, args);
+             pre ? nc_f32(pre) : nullptr, res ? nc_f32(res) : nullptr);
+    NCTensor *args[4] = { w, x, bias, res };
+    NCNode *n = nc_new_node(m, OP_LINEAR, 4, args);
     if (graph) {
         n->saved[0] = nc_view(w);
         n->saved[1] = nc_view(x);
@@ -634,10 +662,20 @@ extern "C" NCTensor *nc_linear(NCTensor *w, NCTensor *x, NCTensor *bias, int act
     }
     n->ia[0] = 0; n->ia[1] = 0; n->ia[2] = 1; n->ia[3] = act;
     n->fa[0] = 1.0f;
-    y = nc_finish(y, n, args, 3);
+    y = nc_finish(y, n, args, 4);
     nc_free_tensor(pre);
-    nc_free_tensor(w); nc_free_tensor(x); nc_free_tensor(bias);
+    nc_free_tensor(w); nc_free_tensor(x); nc_free_tensor(bias); nc_free_tensor(res);
     return y;
+}
+
+extern "C" NCTensor *nc_linear(NCTensor *w, NCTensor *x, NCTensor *bias, int act)
+{
+    return linear_impl(w, x, bias, act, nullptr);
+}
+
+extern "C" NCTensor *nc_linear_add(NCTensor *w, NCTensor *x, NCTensor *bias, int act, NCTensor *res)
+{
+    return linear_impl(w, x, bias, act, res);
 }
 
 // ---- embedding, softmax, loss, norms ----------------------------------------
@@ -1068,6 +1106,7 @@ void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
         if (nd->parents[2]) ga[2] = nc_dup_tensor(g);
         break;
     case OP_LINEAR: {
+        if (nd->n_args > 3 && nd->parents[3]) ga[3] = nc_dup_tensor(g); // residual input
         NCTensor *gz = nc_dup_tensor(g);
         if (nd->ia[3] != NC_ACT_NONE) {
             NCTensor *t = nc_alloc_like(g);
@@ -1123,8 +1162,9 @@ void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
         NCTensor *dw = (w && nd->parents[1]) ? nc_alloc(g->dev, NC_TYPE_F32, 1, &dd, false) : nullptr;
         NCTensor *db = (w && nd->parents[2]) ? nc_alloc(g->dev, NC_TYPE_F32, 1, &dd, false) : nullptr;
         float *partial = (dw || db) ? nc_tmp_f32(m, (size_t)nchip_norm_bwd_partial_rows(cols) * 2 * d, &cap) : nullptr;
+        const float *prev = dx ? nc_bw_addend(m, 0, nc_numel(dx)) : nullptr;
         if (nchip_norm_bwd(st, nc_f32(g), nc_f32(xhat), nc_f32(rstd), w ? nc_f32(w) : nullptr,
-                           dx ? nc_f32(dx) : nullptr, dw ? nc_f32(dw) : nullptr, db ? nc_f32(db) : nullptr,
+                           dx ? nc_f32(dx) : nullptr, prev, dw ? nc_f32(dw) : nullptr, db ? nc_f32(db) : nullptr,
                            partial, d, cols, nd->ia[0]))
             nc_fatal("layer norm backward failed");
         if (partial) nc_tmp_free(m, partial, cap);

@@ -420,7 +420,8 @@ static NCTensor *attention_ref(NNCPModel *s, int l, int output_index, NCTensor *
 }
 
 /* the same block through the fused entry points (full segment) */
-static NCTensor *attention_fused(NNCPModel *s, int l, NCTensor *x)
+/* res (or NULL) is the residual input, added by the output projection itself */
+static NCTensor *attention_fused(NNCPModel *s, int l, NCTensor *x, NCTensor *res)
 {
     const NNCPConfig *c = &s->cfg;
     Layer *tl = &s->layers[l];
@@ -441,11 +442,12 @@ static NCTensor *attention_fused(NNCPModel *s, int l, NCTensor *x)
     att = nc_reshape_2d(att, HDv, (size_t)B * T);
     if (!tl->w_o)
         die("the fused path needs d_value != d_model (an output projection)");
-    return nc_matmul(nc_dup_tensor(tl->w_o), att);
+    return nc_matmul_add(nc_dup_tensor(tl->w_o), att, res, 0, 0, 1.0f);
 }
 
-/* feed-forward block: nncp.c:930-977 */
-static NCTensor *feed_forward(NNCPModel *s, int l, NCTensor *x)
+/* feed-forward block: nncp.c:930-977; res (fused path only, or NULL) is the
+   residual input, added by the second linear layer itself */
+static NCTensor *feed_forward(NNCPModel *s, int l, NCTensor *x, NCTensor *res)
 {
     const NNCPConfig *c = &s->cfg;
     Layer *tl = &s->layers[l];
@@ -454,8 +456,13 @@ static NCTensor *feed_forward(NNCPModel *s, int l, NCTensor *x)
     if (c->fused && (act == NNCP_FF_GELU || act == NNCP_FF_RELU)) {
         t0 = nc_linear(nc_dup_tensor(tl->ff1), x, tl->ff_bias1 ? nc_dup_tensor(tl->ff_bias1) : NULL,
                        act == NNCP_FF_GELU ? NC_ACT_GELU : NC_ACT_RELU);
+        if (res)
+            return nc_linear_add(nc_dup_tensor(tl->ff2), t0, tl->ff_bias2 ? nc_dup_tensor(tl->ff_bias2) : NULL,
+                                 NC_ACT_NONE, res);
         return nc_linear(nc_dup_tensor(tl->ff2), t0, tl->ff_bias2 ? nc_dup_tensor(tl->ff_bias2) : NULL, NC_ACT_NONE);
     }
+    if (res)
+        die("feed_forward: the residual is fused only on the fused GELU/ReLU path");
     t0 = nc_matmul(nc_dup_tensor(tl->ff1), x);
     if (tl->ff_bias1)
         t0 = nc_add(t0, nc_dup_tensor(tl->ff_bias1));
@@ -514,19 +521,31 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
         if (c->ln_flags & NNCP_LN_PRE)
             x1 = layer_norm(s, x1, tl->ln_g1, tl->ln_b1);
         save_layer_input(s, l, output_index, x1, seg_len);
-        t0 = c->fused ? attention_fused(s, l, x1) : attention_ref(s, l, output_index, x1, seg_len);
-        if (c->ln_flags & NNCP_LN_COEF)
-            t0 = nc_mul(t0, nc_dup_tensor(tl->alpha));
-        t0 = nc_add(t0, x); /* residual, nncp.c:896 */
+        /* the fused path folds the residual sums (nncp.c:896, 979) into the
+           GEMMs that produce their other operand */
+        int fold = c->fused && !(c->ln_flags & NNCP_LN_COEF);
+        int fold_ff = fold && (c->ff_act == NNCP_FF_GELU || c->ff_act == NNCP_FF_RELU);
+        if (fold) {
+            t0 = attention_fused(s, l, x1, x);
+        } else {
+            t0 = c->fused ? attention_fused(s, l, x1, NULL) : attention_ref(s, l, output_index, x1, seg_len);
+            if (c->ln_flags & NNCP_LN_COEF)
+                t0 = nc_mul(t0, nc_dup_tensor(tl->alpha));
+            t0 = nc_add(t0, x); /* residual, nncp.c:896 */
+        }
         if (c->ln_flags & NNCP_LN_POST)
             t0 = layer_norm(s, t0, tl->ln_g1, tl->ln_b1);
         ff_in = nc_dup_tensor(t0);
         if (c->ln_flags & NNCP_LN_PRE)
             t0 = layer_norm(s, t0, tl->ln_g2, tl->ln_b2);
-        t0 = feed_forward(s, l, t0);
-        if (c->ln_flags & NNCP_LN_COEF)
-            t0 = nc_mul(t0, nc_dup_tensor(tl->alpha));
-        t0 = nc_add(t0, ff_in); /* nncp.c:979 */
+        if (fold_ff) {
+            t0 = feed_forward(s, l, t0, ff_in);
+        } else {
+            t0 = feed_forward(s, l, t0, NULL);
+            if (c->ln_flags & NNCP_LN_COEF)
+                t0 = nc_mul(t0, nc_dup_tensor(tl->alpha));
+            t0 = nc_add(t0, ff_in); /* nncp.c:979 */
+        }
         if (c->ln_flags & NNCP_LN_POST)
             t0 = layer_norm(s, t0, tl->ln_g2, tl->ln_b2);
         x = t0;

@@ -919,6 +919,13 @@ NCTensor *nc_linear(NCTensor *w, NCTensor *x, NCTensor *bias, int act)
     return y;
 }
 
+/* y = act(w x + bias) + res: a linear layer with its residual connection
+   (nncp.c:896, 979; see nc_ext.h) */
+NCTensor *nc_linear_add(NCTensor *w, NCTensor *x, NCTensor *bias, int act, NCTensor *res)
+{
+    return nc_add(nc_linear(w, x, bias, act), res);
+}
+
 /* ------------------------------------------------------------------------ */
 /* embedding, softmax, loss, norms                                          */
 

@@ -324,6 +324,12 @@ _add("linear_gelu", [(5, 7), (3, 5), (7,)],
      lambda nc, w, x, b: nc.nc_linear(w, x, b, 1), lambda w, x, b: U.gelu(x @ w + b))
 _add("linear_nobias", [(5, 7), (3, 5)],
      lambda nc, w, x: nc.nc_linear(w, x, None, 0), lambda w, x: x @ w)
+_add("linear_add_gelu", [(5, 7), (3, 5), (7,), (3, 7)],
+     lambda nc, w, x, b, r: nc.nc_linear_add(w, x, b, 1, r), lambda w, x, b, r: U.gelu(x @ w + b) + r)
+_add("linear_add_nobias", [(5, 7), (3, 5), (3, 7)],
+     lambda nc, w, x, r: nc.nc_linear_add(w, x, None, 0, r), lambda w, x, r: x @ w + r)
+_add("matmul_add_residual", [(5, 7), (3, 5), (3, 7)],
+     lambda nc, w, x, r: nc.nc_matmul_add(w, x, r, 0, 0, 0.5), lambda w, x, r: 0.5 * (x @ w) + r)
 _add("linear_relu", [(5, 7), (3, 5), (7,)],
      lambda nc, w, x, b: nc.nc_linear(w, x, b, 2), lambda w, x, b: np.maximum(x @ w + b, 0))
 
