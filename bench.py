@@ -204,6 +204,9 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=2, help="0 skips the CPU baseline")
     ap.add_argument("--profile-steps", type=int, default=2)
     ap.add_argument("--attention-iters", type=int, default=50, help="0 skips the isolated attention timing")
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="first issue one device-to-device copy of this many MiB (a kernel of known "
+                         "traffic, to scale FETCH_SIZE / WRITE_SIZE readings of a counter run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (one compression job per GPU, no "
@@ -224,6 +227,19 @@ def main():
     init_weights(model)
     model.nc.nc_set_matmul_bf16(model.ctx, 1 if args.variant == "bf16" else 0)
     mode = H.MODE_SEGMENT | H.CODER_CDF16
+
+    if args.calibrate_copy_mib:
+        hip = C.CDLL("libamdhip64.so")
+        nbytes_cal = args.calibrate_copy_mib << 20
+        src, dst = C.c_void_p(), C.c_void_p()
+        assert hip.hipMalloc(C.byref(src), C.c_size_t(nbytes_cal)) == 0
+        assert hip.hipMalloc(C.byref(dst), C.c_size_t(nbytes_cal)) == 0
+        hip.hipMemset(src, 1, C.c_size_t(nbytes_cal))
+        hip.hipDeviceSynchronize()
+        assert hip.hipMemcpy(dst, src, C.c_size_t(nbytes_cal), 3) == 0  # hipMemcpyDeviceToDevice
+        hip.hipDeviceSynchronize()
+        hip.hipFree(src)
+        hip.hipFree(dst)
 
     pos = 0
     if args.warmup:

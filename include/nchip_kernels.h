@@ -69,22 +69,25 @@ int nchip_gemm2(void *stream, int ta, int tb, int m, int n, int k, float alpha,
    weight-gradient GEMMs dW = dY X^T of a whole backward pass are issued this
    way: each is too small to fill 256 CUs on its own.  dev_table lives in
    device memory; tile_start is the running sum of
-   nchip_gemm_grouped_tiles(m, n) over the preceding problems. */
+   nchip_gemm_grouped_tiles(m, n) over the preceding problems.  total_flops
+   (sum of 2*m*n*k) is only recorded by the optional launch timing. */
 typedef struct {
     const float *A, *B;
     float *C;
-    int m, n, k;
-    int lda, ldb, ldc;
+    const float *A2, *B2; /* optional second k range: C = alpha*(op(A)op(B) + op(A2)op(B2)) */
+    int m, n, k, k2;      /* k2 = 0 without A2/B2; with them k must be a multiple of 64 */
+    int lda, ldb, ldc;    /* A2 / B2 use lda / ldb too */
     int tile_start;
     float alpha;
 } NchipGemmProblem;
 int nchip_gemm_grouped_tiles(int m, int n);
 int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmProblem *dev_table,
-                       int n_problems, int total_tiles, int precision);
+                       int n_problems, int total_tiles, int precision, double total_flops);
 
-/* Optional timing of every GEMM launch with HIP events recorded on the launch
-   stream.  After nchip_gemm_profile_enable(1), each nchip_gemm* call is
-   bracketed by an event pair; nchip_gemm_profile_read waits for them, sums
+/* Optional timing of every GEMM launch with HIP events on the launch stream.
+   After nchip_gemm_profile_enable(1), each nchip_gemm* dispatch carries an
+   event pair bound to its own start / stop timestamps (hipExtLaunchKernelGGL;
+   a split-K reduction pass is not included); nchip_gemm_profile_read waits for them, sums
    launches / flops (2*m*n*k*batch) / seconds per kernel instantiation, fills up
    to max_variants rows and clears the records.  Returns the row count. */
 void nchip_gemm_profile_enable(int on);

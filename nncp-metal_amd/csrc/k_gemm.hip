@@ -16,6 +16,7 @@
 // precision 1 rounds both operands to bf16 (nearest-even) while they are
 // written to LDS and feeds v_mfma_f32_32x32x16_bf16 (fp32 accumulate).
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -176,6 +177,9 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     // robin over the 8 XCDs; give each XCD a contiguous run of tiles so tiles
     // that share an A/B panel also share an L2.
     int bid = blockIdx.x;
+    // second k range of a grouped problem: k tiles from k1 on read A2 / B2
+    const float *A2 = nullptr, *B2 = nullptr;
+    int k1 = 0x7fffffff;
     if (g.grp) {
         // grouped launch: find the problem that owns this workgroup
         int lo = 0, hi = g.n_grp; // grp[lo].tile_start <= bid < grp[hi].tile_start
@@ -186,10 +190,11 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
         const NchipGemmProblem pr = g.grp[lo];
         bid -= pr.tile_start;
         g.A = pr.A; g.B = pr.B; g.C = pr.C;
-        g.M = pr.m; g.N = pr.n; g.K = pr.k;
+        g.M = pr.m; g.N = pr.n; g.K = pr.k + pr.k2;
+        if (pr.k2 > 0) { A2 = pr.A2; B2 = pr.B2; k1 = pr.k; }
         g.lda = pr.lda; g.ldb = pr.ldb; g.ldc = pr.ldc;
         g.alpha = pr.alpha;
-        g.kchunk = pr.k;
+        g.kchunk = pr.k + pr.k2;
         g.tiles_m = (pr.m + BM - 1) / BM;
         g.tiles_n = (pr.n + BN - 1) / BN;
     }
@@ -247,8 +252,11 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
         if (FAST || it + 2 < nk) {
             int k0 = kbeg + (it + 2) * BK;
             bool kf = FAST || (k0 + BK <= kend);
-            la.load(A, g.lda, m0, k0, g.M, kend, FAST || (a_full && kf), t);
-            lb.load(B, g.ldb, n0, k0, g.N, kend, FAST || (b_full && kf), t);
+            const bool second = k0 >= k1; // uniform
+            const float *Ak = second ? A2 : A, *Bk = second ? B2 : B;
+            const int kr = second ? k0 - k1 : k0, ke = second ? kend - k1 : (kend < k1 ? kend : k1);
+            la.load(Ak, g.lda, m0, kr, g.M, ke, FAST || (a_full && kf), t);
+            lb.load(Bk, g.ldb, n0, kr, g.N, ke, FAST || (b_full && kf), t);
         }
         // keep the prefetch ahead of the MFMAs: without this fence the
         // scheduler sinks the global loads below the compute block and their
@@ -447,16 +455,26 @@ bool g_prof_on = false;
 int g_force_cfg = getenv("NCHIP_GEMM_CFG") ? atoi(getenv("NCHIP_GEMM_CFG")) : 0;
 std::vector<ProfRec> g_prof;
 
+// With `rec` the kernel's own start / stop timestamps are bound to the record's
+// events (hipExtLaunchKernelGGL), so the measured time is the dispatch alone,
+// as a kernel trace reports it, without the marker packets of hipEventRecord.
 template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1>
-void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g)
+void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(64 * WM * WN * KW);
-    if (!ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 0, 0, BF16, KW>), grid, block, 0, st, g);
-    else if (ta && !tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 1, 0, BF16, KW>), grid, block, 0, st, g);
-    else if (!ta && tb) hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 0, 1, BF16, KW>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, 1, 1, BF16, KW>), grid, block, 0, st, g);
+#define LAUNCH(TA, TB)                                                                                     \
+    do {                                                                                                   \
+        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW>), grid, block, 0, \
+                                       st, rec->start, rec->stop, 0, g);                                   \
+        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW>), grid, block, 0, st, g); \
+    } while (0)
+    if (!ta && !tb) LAUNCH(0, 0);
+    else if (ta && !tb) LAUNCH(1, 0);
+    else if (!ta && tb) LAUNCH(0, 1);
+    else LAUNCH(1, 1);
+#undef LAUNCH
 }
 
 } // namespace
@@ -517,8 +535,8 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
         (void)hipEventCreate(&rec.stop);
         rec.variant = -1;
         rec.flops = 2.0 * m * n * (double)k * batch;
-        (void)hipEventRecord(rec.start, st);
     }
+    ProfRec *pr = g_prof_on ? &rec : nullptr;
     // Tile configuration from the shape alone.  Measured on MI355X (fp32):
     // small outputs want the most workgroups and the most wavefronts per
     // workgroup (64x64x32, two k groups of 4 wavefronts); once
@@ -533,32 +551,31 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
         else cfg = 8;
     }
     if (precision == 1) {
-        if (cfg == 7) launch_tile<128, 128, 32, 4, 2, 1>(st, ta, tb, g);
-        else if (cfg == 4) launch_tile<128, 64, 32, 4, 2, 1>(st, ta, tb, g);
-        else launch_tile<64, 64, 32, 2, 2, 1>(st, ta, tb, g);
+        if (cfg == 7) launch_tile<128, 128, 32, 4, 2, 1>(st, ta, tb, g, pr);
+        else if (cfg == 4) launch_tile<128, 64, 32, 4, 2, 1>(st, ta, tb, g, pr);
+        else launch_tile<64, 64, 32, 2, 2, 1>(st, ta, tb, g, pr);
     } else if (cfg == 1) {
-        launch_tile<128, 128, 16, 2, 2, 0>(st, ta, tb, g);
+        launch_tile<128, 128, 16, 2, 2, 0>(st, ta, tb, g, pr);
     } else if (cfg == 2) {
-        launch_tile<128, 128, 16, 4, 2, 0>(st, ta, tb, g);
+        launch_tile<128, 128, 16, 4, 2, 0>(st, ta, tb, g, pr);
     } else if (cfg == 3) {
-        launch_tile<128, 64, 16, 2, 2, 0>(st, ta, tb, g);
+        launch_tile<128, 64, 16, 2, 2, 0>(st, ta, tb, g, pr);
     } else if (cfg == 4) {
-        launch_tile<128, 64, 32, 4, 2, 0>(st, ta, tb, g);
+        launch_tile<128, 64, 32, 4, 2, 0>(st, ta, tb, g, pr);
     } else if (cfg == 6) {
-        launch_tile<64, 128, 16, 2, 2, 0>(st, ta, tb, g);
+        launch_tile<64, 128, 16, 2, 2, 0>(st, ta, tb, g, pr);
     } else if (cfg == 7) {
-        launch_tile<128, 128, 32, 4, 2, 0>(st, ta, tb, g);
+        launch_tile<128, 128, 32, 4, 2, 0>(st, ta, tb, g, pr);
     } else if (cfg == 8) {
-        launch_tile<64, 64, 32, 2, 2, 0, 2>(st, ta, tb, g);
+        launch_tile<64, 64, 32, 2, 2, 0, 2>(st, ta, tb, g, pr);
     } else if (cfg == 9) {
-        launch_tile<64, 64, 64, 2, 2, 0, 2>(st, ta, tb, g);
+        launch_tile<64, 64, 64, 2, 2, 0, 2>(st, ta, tb, g, pr);
     } else {
-        launch_tile<64, 64, 16, 2, 2, 0>(st, ta, tb, g);
+        launch_tile<64, 64, 16, 2, 2, 0>(st, ta, tb, g, pr);
     }
     if (g_prof_on) {
         int tile = cfg == 7 ? 2 : (cfg == 4 ? 1 : (cfg == 8 ? 3 : 0));
         rec.variant = tile * 8 + (ta ? 4 : 0) + (tb ? 2 : 0) + (precision == 1 ? 1 : 0);
-        (void)hipEventRecord(rec.stop, st);
         g_prof.push_back(rec);
     }
     if (ksplit > 1) {
@@ -661,7 +678,7 @@ extern "C" int nchip_gemm_grouped_tiles(int m, int n)
 }
 
 extern "C" int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmProblem *dev_table,
-                                  int n_problems, int total_tiles, int precision)
+                                  int n_problems, int total_tiles, int precision, double total_flops)
 {
     if (n_problems <= 0 || total_tiles <= 0) return 0;
     GemmArgs g;
@@ -671,13 +688,26 @@ extern "C" int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmP
     g.beta = 0.0f; g.act = 0;
     hipStream_t st = (hipStream_t)stream;
     dim3 grid(total_tiles, 1), block(512);
-#define GRP(TA, TB, BF) hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, 0, st, g)
+    ProfRec rec;
+    if (g_prof_on) {
+        (void)hipEventCreate(&rec.start);
+        (void)hipEventCreate(&rec.stop);
+        rec.variant = 2 * 8 + (ta ? 4 : 0) + (tb ? 2 : 0) + (precision == 1 ? 1 : 0);
+        rec.flops = total_flops;
+    }
+#define GRP(TA, TB, BF)                                                                                    \
+    do {                                                                                                   \
+        if (g_prof_on) hipExtLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, 0, st, \
+                                             rec.start, rec.stop, 0, g);                                   \
+        else hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, 0, st, g);      \
+    } while (0)
     if (precision == 1) {
         if (!ta && !tb) GRP(0, 0, 1); else if (ta && !tb) GRP(1, 0, 1); else if (!ta && tb) GRP(0, 1, 1); else GRP(1, 1, 1);
     } else {
         if (!ta && !tb) GRP(0, 0, 0); else if (ta && !tb) GRP(1, 0, 0); else if (!ta && tb) GRP(0, 1, 0); else GRP(1, 1, 0);
     }
 #undef GRP
+    if (g_prof_on) g_prof.push_back(rec);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         fprintf(stderr, "nchip_gemm_grouped: launch failed: %s\n", hipGetErrorString(e));

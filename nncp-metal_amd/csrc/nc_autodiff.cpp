@@ -128,6 +128,8 @@ static void accumulate(NCNode *p, NCTensor *g)
 {
     g = nc_contig(g);
     if (!p->grad) { p->grad = g; return; }
+    // a postponed weight gradient holds no data yet: run it before summing
+    if (p->op == OP_PARAM && nc_has_deferred(p->ctx, p)) nc_flush_deferred(p->ctx);
     size_t n = nc_numel(g);
     if (n != nc_numel(p->grad))
         nc_fatal("backward: gradient size mismatch at op %d (%zu vs %zu)", p->op, n, nc_numel(p->grad));
@@ -177,7 +179,7 @@ extern "C" void nc_backward(const NCTensor *x, NCTensor *grad, NCParamUpdateFunc
             NCNode *p = i < nd->n_args ? nd->parents[i] : nullptr;
             bool again = false; // the same parent twice: only the first slot may take it
             for (int j = 0; j < i && p; j++) again |= nd->parents[j] == p;
-            m->bw_prev[i] = (p && !again) ? p->grad : nullptr;
+            m->bw_prev[i] = (p && !again && p->op != OP_PARAM) ? p->grad : nullptr;
             m->bw_used[i] = false;
         }
         if (g) nc_node_backward(nd, g, ga.data());

@@ -43,10 +43,13 @@ struct NCDevice {
 };
 
 // weight-gradient GEMM postponed to one grouped launch at the end of nc_backward
+struct NCNode;
 struct DeferredGemm {
-    NCTensor *a, *b, *c; // c (m x n) = alpha * a (m x k) * b^T (b is n x k)
-    int m, n, k;
+    NCTensor *a, *b, *c;   // c (m x n) = alpha * (a (m x k) * b^T + a2 (m x k2) * b2^T), b is n x k
+    NCTensor *a2, *b2;     // second use of the same weight (or NULL)
+    int m, n, k, k2;
     float alpha;
+    const NCNode *param;   // the parameter this gradient belongs to
 };
 
 #define NC_BW_ARGS 8 // node arguments for which nc_backward offers the existing gradient
@@ -141,5 +144,6 @@ NCNode *nc_new_node(NCContext *m, int op, int n_args, NCTensor **args);
 NCTensor *nc_finish(NCTensor *y, NCNode *n, NCTensor **args, int n_args);
 void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga); // nc_ops.cpp
 void nc_flush_deferred(NCContext *m);                          // nc_ops.cpp
+bool nc_has_deferred(const NCContext *m, const NCNode *param);  // nc_ops.cpp
 
 #endif

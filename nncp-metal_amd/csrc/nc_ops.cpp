@@ -5,6 +5,7 @@
 // aborts (see need_dev).
 #include <math.h>
 #include "nc_hip_internal.h"
+#include <algorithm>
 
 #define LAUNCHED(x) (nc_ctx(x)->launches++)
 
@@ -604,17 +605,33 @@ static void matmul_bw(NCNode *nd, NCTensor *g, NCTensor **ga, int ia, int ib)
     if (nd->parents[ia]) {
         NCTensor *da = nc_alloc_like(a);
         NCNode *pa = nd->parents[ia];
-        if (m->defer_wgrad && !ta && !tb && s.batch == 1 && pa->op == OP_PARAM && pa->consumers == 1) {
-            // dW = alpha * dY * X^T of a plain linear layer whose weight is used
-            // once: postponed to the grouped launch at the end of nc_backward
+        // dW = alpha * dY * X^T of a plain linear layer whose weight is used once
+        // or twice (K/V of the segment and of the memory): postponed to the
+        // grouped launch at the end of nc_backward; the second use joins the
+        // first as a second k range of the same problem
+        DeferredGemm *open_entry = nullptr;
+        for (DeferredGemm &e : m->deferred)
+            if (e.param == pa) open_entry = &e;
+        const bool plain = m->defer_wgrad && !ta && !tb && s.batch == 1 && pa->op == OP_PARAM;
+        if (plain && !open_entry && pa->consumers <= 2) {
             DeferredGemm d;
             d.a = nc_contig(nc_dup_tensor(g)); d.b = nc_dup_tensor(b); d.c = nc_dup_tensor(da);
+            d.a2 = d.b2 = nullptr; d.k2 = 0;
             d.m = (int)s.m; d.n = (int)s.k; d.k = (int)s.n; d.alpha = alpha;
+            d.param = pa;
             m->deferred.push_back(d);
-        } else
-        if (!ta) dev_gemm(m, false, !tb, s.m, s.k, s.n, alpha, g, b, 0.0f, da, s.batch, nullptr, 0, nullptr);
-        else     dev_gemm(m, tb, true, s.k, s.m, s.n, alpha, b, g, 0.0f, da, s.batch, nullptr, 0, nullptr);
-        ga[ia] = da;
+            ga[ia] = da;
+        } else if (plain && open_entry && !open_entry->a2 && open_entry->m == (int)s.m &&
+                   open_entry->n == (int)s.k && open_entry->k % 64 == 0 && open_entry->alpha == alpha) {
+            open_entry->a2 = nc_contig(nc_dup_tensor(g));
+            open_entry->b2 = nc_dup_tensor(b);
+            open_entry->k2 = (int)s.n;
+            nc_free_tensor(da); // the first use's tensor receives the whole gradient
+        } else {
+            if (!ta) dev_gemm(m, false, !tb, s.m, s.k, s.n, alpha, g, b, 0.0f, da, s.batch, nullptr, 0, nullptr);
+            else     dev_gemm(m, tb, true, s.k, s.m, s.n, alpha, b, g, 0.0f, da, s.batch, nullptr, 0, nullptr);
+            ga[ia] = da;
+        }
     }
     if (nd->parents[ib]) {
         NCTensor *db = nc_alloc_like(b);
@@ -950,10 +967,18 @@ void nc_flush_deferred(NCContext *m)
     if (m->deferred.empty()) return;
     std::vector<NchipGemmProblem> tab;
     int tiles = 0;
+    double flops = 0.0;
+    // longest reductions first: their tiles run longest and would otherwise
+    // form the tail of the launch
+    std::stable_sort(m->deferred.begin(), m->deferred.end(), [](const DeferredGemm &x, const DeferredGemm &y) {
+        return x.k + (x.a2 ? x.k2 : 0) > y.k + (y.a2 ? y.k2 : 0);
+    });
     for (DeferredGemm &d : m->deferred) {
         NchipGemmProblem p;
         p.A = nc_f32(d.a); p.B = nc_f32(d.b); p.C = nc_f32(d.c);
-        p.m = d.m; p.n = d.n; p.k = d.k;
+        p.A2 = d.a2 ? nc_f32(d.a2) : nullptr; p.B2 = d.b2 ? nc_f32(d.b2) : nullptr;
+        p.m = d.m; p.n = d.n; p.k = d.k; p.k2 = d.a2 ? d.k2 : 0;
+        flops += 2.0 * d.m * d.n * (double)(d.k + p.k2);
         p.lda = d.m; p.ldb = d.n; p.ldc = d.m;
         p.tile_start = tiles; p.alpha = d.alpha;
         tiles += nchip_gemm_grouped_tiles(d.m, d.n);
@@ -964,7 +989,7 @@ void nc_flush_deferred(NCContext *m)
     void *dev = m->dev_pool.get(bytes, &dcap);
     memcpy(host, tab.data(), bytes);
     hip_check(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync gemm table");
-    if (nchip_gemm_grouped(m->stream, 0, 1, (const NchipGemmProblem *)dev, (int)tab.size(), tiles, m->matmul_bf16))
+    if (nchip_gemm_grouped(m->stream, 0, 1, (const NchipGemmProblem *)dev, (int)tab.size(), tiles, m->matmul_bf16, flops))
         nc_fatal("grouped weight-gradient GEMM failed");
     m->launches++;
     // pinned staging is recycled one flush later (the copy has long run by then)
@@ -973,8 +998,16 @@ void nc_flush_deferred(NCContext *m)
     m->dev_pool.put(dev, dcap);
     for (DeferredGemm &d : m->deferred) {
         nc_free_tensor(d.a); nc_free_tensor(d.b); nc_free_tensor(d.c);
+        nc_free_tensor(d.a2); nc_free_tensor(d.b2);
     }
     m->deferred.clear();
+}
+
+bool nc_has_deferred(const NCContext *m, const NCNode *param)
+{
+    for (const DeferredGemm &e : m->deferred)
+        if (e.param == param) return true;
+    return false;
 }
 
 // ---- backward dispatch --------------------------------------------------------
