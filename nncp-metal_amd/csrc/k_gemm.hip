@@ -35,6 +35,11 @@ constexpr int KALIGN = 16; // split-K chunk granularity
 constexpr int PAD = 4;   // keeps 16-byte alignment of LDS rows, staggers banks
 constexpr int NXCD = 8;
 
+#ifdef NCHIP_GEMM_CLOCKS
+// debug builds: shader-clock and wall-clock span of the k loop of workgroup 0
+__device__ long long *g_gemm_clk = nullptr;
+#endif
+
 struct GemmArgs {
     const float *A, *B;
     float *C;
@@ -129,24 +134,92 @@ struct TileLoader {
             }
         }
     }
+};
 
-    // bf16 LDS tile: rows are i (m or n), BK + 8 halves each, k contiguous so a
-    // lane can fetch its 8 consecutive k for v_mfma_f32_32x32x16_bf16 in one read
-    __device__ __forceinline__ void store_bf16(unsigned short *lds, int t) const
+// bf16 variant of the loader.  LDS holds 32-bit words of two bf16 values that
+// are consecutive in k: word (kp, i) = (x[i][2kp], x[i][2kp+1]), rows kp of
+// BT + PAD words.  A lane of v_mfma_f32_32x32x16_bf16 (row i, k group kg) reads
+// the 4 words kp = kb*8 + kg*4 .. +3 of column i: 8 consecutive k, lanes on
+// consecutive banks.  Operands whose long axis is contiguous in memory are
+// fetched as two float4 from rows k, k+1 and stored as one 16-byte LDS write;
+// k-contiguous operands give two words per float4.  Rounding is to nearest
+// even (v_cvt_pk_bf16_f32).
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
+{
+    floatx2_t f = { lo, hi };
+    bf16x2_t h = __builtin_convertvector(f, bf16x2_t);
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+template <int BT, int BK, int MAJOR, int NT>
+struct TileLoaderBf16 {
+    static constexpr int NV = BT * BK / 4 / NT; // float4 per thread
+    static_assert(NV >= 1 && NV * NT * 4 == BT * BK, "tile must divide evenly over the threads");
+    static_assert(!MAJOR || NV % 2 == 0, "row pairs need an even number of float4 per thread");
+    floatx4 r[NV];
+
+    __device__ __forceinline__ static void coords(int v, int t, int &i, int &k)
+    {
+        if (MAJOR) { // entries 2p, 2p+1 are rows k, k+1 of the same 4 columns
+            int idx = t + (v >> 1) * NT;
+            i = (idx % (BT / 4)) * 4;
+            k = (idx / (BT / 4)) * 2 + (v & 1);
+        } else {
+            int idx = t + v * NT;
+            i = idx % BT;
+            k = (idx / BT) * 4;
+        }
+    }
+
+    __device__ __forceinline__ void load(const float *p, int64_t ld, int i0, int k0,
+                                         int imax, int kmax, bool fast, int t)
     {
 #pragma unroll
         for (int v = 0; v < NV; v++) {
-            int idx = t + v * NT;
-            if (MAJOR) {
-                int i = (idx % (BT / 4)) * 4, k = idx / (BT / 4);
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    lds[(i + e) * (BK + 8) + k] = f32_to_bf16(r[v][e]);
+            int i, k;
+            coords(v, t, i, k);
+            if (fast) {
+                const float *src = MAJOR ? p + (int64_t)(k0 + k) * ld + (i0 + i)
+                                         : p + (int64_t)(i0 + i) * ld + (k0 + k);
+                r[v] = *reinterpret_cast<const floatx4 *>(src);
             } else {
-                int i = idx % BT, k = (idx / BT) * 4;
+                floatx4 tmp;
 #pragma unroll
-                for (int e = 0; e < 4; e++)
-                    lds[i * (BK + 8) + k + e] = f32_to_bf16(r[v][e]);
+                for (int e = 0; e < 4; e++) {
+                    int ii = MAJOR ? i + e : i, kk = MAJOR ? k : k + e;
+                    float val = 0.0f;
+                    if (i0 + ii < imax && k0 + kk < kmax)
+                        val = MAJOR ? p[(int64_t)(k0 + kk) * ld + (i0 + ii)]
+                                    : p[(int64_t)(i0 + ii) * ld + (k0 + kk)];
+                    tmp[e] = val;
+                }
+                r[v] = tmp;
+            }
+        }
+    }
+
+    __device__ __forceinline__ void store(uint32_t *lds, int t) const
+    {
+        if (MAJOR) {
+#pragma unroll
+            for (int v = 0; v < NV; v += 2) {
+                int i, k;
+                coords(v, t, i, k);
+                uint32_t w[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[e] = pack_bf16(r[v][e], r[v + 1][e]);
+                *reinterpret_cast<uint4 *>(lds + (k >> 1) * (BT + PAD) + i) = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < NV; v++) {
+                int i, k;
+                coords(v, t, i, k);
+                lds[(k >> 1) * (BT + PAD) + i] = pack_bf16(r[v][0], r[v][1]);
+                lds[((k >> 1) + 1) * (BT + PAD) + i] = pack_bf16(r[v][2], r[v][3]);
             }
         }
     }
@@ -156,7 +229,7 @@ struct TileLoader {
 // two groups of WM x WN wavefronts share the LDS tiles and split every 32-deep
 // k slab, group 0 taking k%32 < 16 and group 1 the rest; group 1 hands its
 // accumulators over through LDS at the end (C = chain0 + chain1, fixed order).
-template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16, int KW = 1>
+template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16, int KW = 1, int PF = 2>
 __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 {
     GemmArgs g = g0;
@@ -164,8 +237,8 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     constexpr int NT = 64 * WM * WN * KW;                 // threads: KW groups of WM x WN wavefronts
     constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN); // 32x32 MFMA tiles per wavefront
     constexpr int WTM = BM / WM, WTN = BN / WN;           // wavefront tile
-    constexpr int LDS_A = BF16 ? BM * (BK + 8) / 2 : BK * (BM + PAD); // in floats
-    constexpr int LDS_B = BF16 ? BN * (BK + 8) / 2 : BK * (BN + PAD);
+    constexpr int LDS_A = BF16 ? (BK / 2) * (BM + PAD) : BK * (BM + PAD); // in 32-bit words
+    constexpr int LDS_B = BF16 ? (BK / 2) * (BN + PAD) : BK * (BN + PAD);
     static_assert(KW == 1 || BM * BN <= 2 * (LDS_A + LDS_B), "accumulator hand-over must fit in the tile buffers");
     __shared__ __attribute__((aligned(16))) float smem[2 * (LDS_A + LDS_B)];
 
@@ -216,10 +289,13 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     const bool a_full = (m0 + BM <= g.M) && (g.lda % 4 == 0) && (((uintptr_t)A & 15) == 0);
     const bool b_full = (n0 + BN <= g.N) && (g.ldb % 4 == 0) && (((uintptr_t)B & 15) == 0);
 
-    // two register sets: while tile it is computed, tile it+1 has arrived (or is
-    // about to) and tile it+2 is in flight, so a load has two compute phases to land
-    TileLoader<BM, BK, TA ? 0 : 1, NT> la0, la1;
-    TileLoader<BN, BK, TB ? 1 : 0, NT> lb0, lb1;
+    // PF register sets: while tile it is computed, tiles it+1 .. it+PF are landing
+    // or in flight, so a load has PF compute phases to arrive.  Two sets are
+    // enough on MI355X: four or six measured no faster on any model shape.
+    using LoaderA = std::conditional_t<BF16 != 0, TileLoaderBf16<BM, BK, TA ? 0 : 1, NT>, TileLoader<BM, BK, TA ? 0 : 1, NT>>;
+    using LoaderB = std::conditional_t<BF16 != 0, TileLoaderBf16<BN, BK, TB ? 1 : 0, NT>, TileLoader<BN, BK, TB ? 1 : 0, NT>>;
+    LoaderA la[PF];
+    LoaderB lb[PF];
 
     floatx16 acc[TN][TM];
 #pragma unroll
@@ -231,7 +307,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
                 acc[i][j][r] = 0.0f;
 
     // One pipeline step: write the register set holding tile `it` to LDS buffer
-    // it&1, barrier, refill that set with tile it+2 (when there is one), then
+    // it&1, barrier, refill that set with tile it+PF (when there is one), then
     // the MFMAs of tile `it`.  One barrier per tile is enough because a buffer
     // is rewritten only two tiles later.  FAST is a compile-time flag so the
     // steady-state loop carries no guarded-load code: the guarded path shares
@@ -241,16 +317,16 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
         constexpr bool FAST = decltype(fast_tag)::value;
         float *sa = smem + (it & 1) * (LDS_A + LDS_B);
         float *sb = sa + LDS_A;
-        if (BF16) {
-            la.store_bf16(reinterpret_cast<unsigned short *>(sa), t);
-            lb.store_bf16(reinterpret_cast<unsigned short *>(sb), t);
+        if constexpr (BF16 != 0) {
+            la.store(reinterpret_cast<uint32_t *>(sa), t);
+            lb.store(reinterpret_cast<uint32_t *>(sb), t);
         } else {
             la.store_f32(sa, t);
             lb.store_f32(sb, t);
         }
         __syncthreads();
-        if (FAST || it + 2 < nk) {
-            int k0 = kbeg + (it + 2) * BK;
+        if (FAST || it + PF < nk) {
+            int k0 = kbeg + (it + PF) * BK;
             bool kf = FAST || (k0 + BK <= kend);
             const bool second = k0 >= k1; // uniform
             const float *Ak = second ? A2 : A, *Bk = second ? B2 : B;
@@ -262,22 +338,24 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
         // scheduler sinks the global loads below the compute block and their
         // latency is paid in full at the next LDS write
         __builtin_amdgcn_sched_barrier(0);
-        if (BF16) {
-            // one 32x32x16 MFMA per tile pair per 16 k; group kg takes every KW-th
-            const unsigned short *ha = reinterpret_cast<const unsigned short *>(sa);
-            const unsigned short *hb = reinterpret_cast<const unsigned short *>(sb);
+        if constexpr (BF16 != 0) {
+            // one 32x32x16 MFMA per tile pair per 16 k; group kg takes every KW-th block
+            const uint32_t *wa = reinterpret_cast<const uint32_t *>(sa) + (lane >> 5) * 4 * (BM + PAD) + wm * WTM + (lane & 31);
+            const uint32_t *wb = reinterpret_cast<const uint32_t *>(sb) + (lane >> 5) * 4 * (BN + PAD) + wn * WTN + (lane & 31);
 #pragma unroll
             for (int u = 0; u < BK / 16 / KW; u++) {
-                const int kofs = (u * KW + kg) * 16;
-                shortx8 fa[TM], fb[TN];
+                const int row0 = (u * KW + kg) * 8; // word row of this 16-k block
+                uint4 fa[TM], fb[TN];
 #pragma unroll
-                for (int j = 0; j < TM; j++)
-                    fa[j] = *reinterpret_cast<const shortx8 *>(
-                        ha + (wm * WTM + j * 32 + (lane & 31)) * (BK + 8) + kofs + (lane >> 5) * 8);
+                for (int j = 0; j < TM; j++) {
+                    const uint32_t *q = wa + row0 * (BM + PAD) + j * 32;
+                    fa[j] = make_uint4(q[0], q[BM + PAD], q[2 * (BM + PAD)], q[3 * (BM + PAD)]);
+                }
 #pragma unroll
-                for (int i = 0; i < TN; i++)
-                    fb[i] = *reinterpret_cast<const shortx8 *>(
-                        hb + (wn * WTN + i * 32 + (lane & 31)) * (BK + 8) + kofs + (lane >> 5) * 8);
+                for (int i = 0; i < TN; i++) {
+                    const uint32_t *q = wb + row0 * (BN + PAD) + i * 32;
+                    fb[i] = make_uint4(q[0], q[BN + PAD], q[2 * (BN + PAD)], q[3 * (BN + PAD)]);
+                }
 #pragma unroll
                 for (int i = 0; i < TN; i++)
 #pragma unroll
@@ -325,29 +403,36 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
         }
     };
 
+#ifdef NCHIP_GEMM_CLOCKS
+    long long dbg_c0 = clock64(), dbg_w0 = wall_clock64();
+#endif
     const int nk = (kend - kbeg + BK - 1) / BK;
     const int nk_full = (kend - kbeg) / BK; // tiles with a complete k range
     int it = 0;
-    if (nk > 0) {
-        bool kf = nk_full > 0;
-        la0.load(A, g.lda, m0, kbeg, g.M, kend, a_full && kf, t);
-        lb0.load(B, g.ldb, n0, kbeg, g.N, kend, b_full && kf, t);
-    }
-    if (nk > 1) {
-        bool kf = nk_full > 1;
-        la1.load(A, g.lda, m0, kbeg + BK, g.M, kend, a_full && kf, t);
-        lb1.load(B, g.ldb, n0, kbeg + BK, g.N, kend, b_full && kf, t);
-    }
-    if (a_full && b_full) // steady state: tiles it+2, it+3 are complete, unguarded vector loads
-        for (; it + 3 < nk_full; it += 2) {
-            step(it, nk, std::true_type(), la0, lb0);
-            step(it + 1, nk, std::true_type(), la1, lb1);
+#pragma unroll
+    for (int j = 0; j < PF; j++)
+        if (j < nk) {
+            bool kf = nk_full > j;
+            la[j].load(A, g.lda, m0, kbeg + j * BK, g.M, kend, a_full && kf, t);
+            lb[j].load(B, g.ldb, n0, kbeg + j * BK, g.N, kend, b_full && kf, t);
         }
-    for (; it < nk; it++) { // edge tiles and the k tail (it is even when the loop starts)
-        if (it & 1) step(it, nk, std::false_type(), la1, lb1);
-        else step(it, nk, std::false_type(), la0, lb0);
+    if (a_full && b_full) // steady state: tiles it+PF .. it+2PF-1 are complete, unguarded vector loads
+        for (; it + 2 * PF - 1 < nk_full; it += PF) {
+#pragma unroll
+            for (int j = 0; j < PF; j++) step(it + j, nk, std::true_type(), la[j], lb[j]);
+        }
+    for (; it < nk; it++) { // edge tiles and the k tail (it is a multiple of PF when the loop starts)
+#pragma unroll
+        for (int j = 0; j < PF; j++)
+            if (it % PF == j) step(it, nk, std::false_type(), la[j], lb[j]);
     }
 
+#ifdef NCHIP_GEMM_CLOCKS
+    if (g_gemm_clk && blockIdx.x == 0 && blockIdx.y == 0 && t == 0) {
+        g_gemm_clk[0] = clock64() - dbg_c0;       // shader cycles of the k loop
+        g_gemm_clk[1] = wall_clock64() - dbg_w0;  // 100 MHz ticks of the same span
+    }
+#endif
     if (KW == 2) {
         // group 1 parks its accumulators in LDS (the tiles are dead), group 0 adds them
         __syncthreads();
@@ -458,7 +543,7 @@ std::vector<ProfRec> g_prof;
 // With `rec` the kernel's own start / stop timestamps are bound to the record's
 // events (hipExtLaunchKernelGGL), so the measured time is the dispatch alone,
 // as a kernel trace reports it, without the marker packets of hipEventRecord.
-template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1>
+template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1, int PF = 2>
 void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
@@ -466,9 +551,9 @@ void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
     dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(64 * WM * WN * KW);
 #define LAUNCH(TA, TB)                                                                                     \
     do {                                                                                                   \
-        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW>), grid, block, 0, \
+        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>), grid, block, 0, \
                                        st, rec->start, rec->stop, 0, g);                                   \
-        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW>), grid, block, 0, st, g); \
+        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>), grid, block, 0, st, g); \
     } while (0)
     if (!ta && !tb) LAUNCH(0, 0);
     else if (ta && !tb) LAUNCH(1, 0);
@@ -552,8 +637,8 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     }
     if (precision == 1) {
         if (cfg == 7) launch_tile<128, 128, 32, 4, 2, 1>(st, ta, tb, g, pr);
-        else if (cfg == 4) launch_tile<128, 64, 32, 4, 2, 1>(st, ta, tb, g, pr);
-        else launch_tile<64, 64, 32, 2, 2, 1>(st, ta, tb, g, pr);
+        else if (cfg == 4) launch_tile<128, 64, 64, 4, 2, 1>(st, ta, tb, g, pr);
+        else launch_tile<64, 64, 64, 2, 2, 1, 2>(st, ta, tb, g, pr);
     } else if (cfg == 1) {
         launch_tile<128, 128, 16, 2, 2, 0>(st, ta, tb, g, pr);
     } else if (cfg == 2) {
@@ -570,6 +655,9 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
         launch_tile<64, 64, 32, 2, 2, 0, 2>(st, ta, tb, g, pr);
     } else if (cfg == 9) {
         launch_tile<64, 64, 64, 2, 2, 0, 2>(st, ta, tb, g, pr);
+    } else if (cfg == 10) {
+        launch_tile<64, 64, 32, 2, 2, 0, 2, 4>(st, ta, tb, g, pr);
+
     } else {
         launch_tile<64, 64, 16, 2, 2, 0>(st, ta, tb, g, pr);
     }
@@ -659,12 +747,14 @@ extern "C" int nchip_gemm_profile_read(int max_variants, char (*names)[48], int6
         (void)hipEventDestroy(r.stop);
     }
     g_prof.clear();
-    static const char *tiles[4] = { "64,64,16,2,2", "128,64,32,4,2", "128,128,32,4,2", "64,64,32,2,2" };
+    static const char *tiles_f32[4] = { "64,64,16,2,2", "128,64,32,4,2", "128,128,32,4,2", "64,64,32,2,2" };
+    static const char *tiles_bf16[4] = { "64,64,64,2,2", "128,64,64,4,2", "128,128,32,4,2", "64,64,64,2,2" };
     int n = 0;
     for (int v = 0; v < 32 && n < max_variants; v++) {
         if (!cnt[v]) continue;
-        snprintf(names[n], 48, "gemm_kernel<%s,%d,%d,%d%s>", tiles[v / 8], (v >> 2) & 1, (v >> 1) & 1, v & 1,
-                 v / 8 == 3 ? ",2" : "");
+        const bool two_groups = v / 8 == 3 || ((v & 1) && v / 8 == 0);
+        snprintf(names[n], 48, "gemm_kernel<%s,%d,%d,%d%s>", (v & 1) ? tiles_bf16[v / 8] : tiles_f32[v / 8],
+                 (v >> 2) & 1, (v >> 1) & 1, v & 1, two_groups ? ",2" : "");
         launches[n] = cnt[v]; flops[n] = fl[v]; seconds[n] = sec[v];
         n++;
     }

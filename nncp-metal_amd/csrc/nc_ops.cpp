@@ -853,7 +853,7 @@ extern "C" NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv
                                    all[3] ? nc_f32(all[3]) : nullptr, all[4] ? nc_f32(all[4]) : nullptr,
                                    nc_f32(y), (int64_t)od[0], nc_f32(probs), rel,
                                    a.H, a.dk, a.dv, a.B, a.T, a.M, a.d_pos, attn_len, b_r_scale,
-                                   m->matmul_bf16);
+                                   0 /* attention stays fp32 in the bf16 variant */);
     if (rel) nc_tmp_free(m, rel, cap);
     if (rc) nc_fatal("nc_relpos_attention: kernel rejected the shapes");
     m->launches += nchip_relpos_attn_last_launches();
@@ -896,7 +896,7 @@ static void attn_bw(NCNode *nd, NCTensor *g, NCTensor **ga)
                                    (int64_t)gc->dims[0], nc_f32(dq), nc_f32(dkv),
                                    dkvm ? nc_f32(dkvm) : nullptr, dwr ? nc_f32(dwr) : nullptr,
                                    dbr ? nc_f32(dbr) : nullptr, a.H, a.dk, a.dv, a.B, a.T, a.M, a.d_pos,
-                                   nd->ia[2], nd->fa[0], m->matmul_bf16, scratch);
+                                   nd->ia[2], nd->fa[0], 0, scratch);
     nc_tmp_free(m, scratch, cap);
     if (rc) nc_fatal("nc_relpos_attention backward failed");
     m->launches += nchip_relpos_attn_last_launches();
