@@ -141,7 +141,7 @@ struct TileLoader {
 // BT + PAD words.  A lane of v_mfma_f32_32x32x16_bf16 (row i, k group kg) reads
 // the 4 words kp = kb*8 + kg*4 .. +3 of column i: 8 consecutive k, lanes on
 // consecutive banks.  Operands whose long axis is contiguous in memory are
-// fetched as two float4 from rows k, k+1 and stored as one 16-byte LDS write;
+// fetched as 2 columns x 2 rows (k, k+1) and stored as one 8-byte LDS write;
 // k-contiguous operands give two words per float4.  Rounding is to nearest
 // even (v_cvt_pk_bf16_f32).
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -156,22 +156,17 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
 
 template <int BT, int BK, int MAJOR, int NT>
 struct TileLoaderBf16 {
-    static constexpr int NV = BT * BK / 4 / NT; // float4 per thread
+    static constexpr int NV = BT * BK / 4 / NT; // 4-float units per thread
     static_assert(NV >= 1 && NV * NT * 4 == BT * BK, "tile must divide evenly over the threads");
-    static_assert(!MAJOR || NV % 2 == 0, "row pairs need an even number of float4 per thread");
     floatx4 r[NV];
 
+    // MAJOR = 1: a unit is 2 columns x 2 consecutive k rows, r = (x[i][k], x[i+1][k], x[i][k+1], x[i+1][k+1]);
+    // MAJOR = 0: a unit is 4 consecutive k of one column
     __device__ __forceinline__ static void coords(int v, int t, int &i, int &k)
     {
-        if (MAJOR) { // entries 2p, 2p+1 are rows k, k+1 of the same 4 columns
-            int idx = t + (v >> 1) * NT;
-            i = (idx % (BT / 4)) * 4;
-            k = (idx / (BT / 4)) * 2 + (v & 1);
-        } else {
-            int idx = t + v * NT;
-            i = idx % BT;
-            k = (idx / BT) * 4;
-        }
+        int idx = t + v * NT;
+        if (MAJOR) { i = (idx % (BT / 2)) * 2; k = (idx / (BT / 2)) * 2; }
+        else       { i = idx % BT;             k = (idx / BT) * 4; }
     }
 
     __device__ __forceinline__ void load(const float *p, int64_t ld, int i0, int k0,
@@ -182,14 +177,19 @@ struct TileLoaderBf16 {
             int i, k;
             coords(v, t, i, k);
             if (fast) {
-                const float *src = MAJOR ? p + (int64_t)(k0 + k) * ld + (i0 + i)
-                                         : p + (int64_t)(i0 + i) * ld + (k0 + k);
-                r[v] = *reinterpret_cast<const floatx4 *>(src);
+                if (MAJOR) {
+                    const float *src = p + (int64_t)(k0 + k) * ld + (i0 + i);
+                    floatx2_t a = *reinterpret_cast<const floatx2_t *>(src);
+                    floatx2_t b = *reinterpret_cast<const floatx2_t *>(src + ld);
+                    r[v] = floatx4{ a[0], a[1], b[0], b[1] };
+                } else {
+                    r[v] = *reinterpret_cast<const floatx4 *>(p + (int64_t)(i0 + i) * ld + (k0 + k));
+                }
             } else {
                 floatx4 tmp;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    int ii = MAJOR ? i + e : i, kk = MAJOR ? k : k + e;
+                    int ii = MAJOR ? i + (e & 1) : i, kk = MAJOR ? k + (e >> 1) : k + e;
                     float val = 0.0f;
                     if (i0 + ii < imax && k0 + kk < kmax)
                         val = MAJOR ? p[(int64_t)(k0 + kk) * ld + (i0 + ii)]
@@ -203,21 +203,14 @@ struct TileLoaderBf16 {
 
     __device__ __forceinline__ void store(uint32_t *lds, int t) const
     {
-        if (MAJOR) {
 #pragma unroll
-            for (int v = 0; v < NV; v += 2) {
-                int i, k;
-                coords(v, t, i, k);
-                uint32_t w[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) w[e] = pack_bf16(r[v][e], r[v + 1][e]);
-                *reinterpret_cast<uint4 *>(lds + (k >> 1) * (BT + PAD) + i) = make_uint4(w[0], w[1], w[2], w[3]);
-            }
-        } else {
-#pragma unroll
-            for (int v = 0; v < NV; v++) {
-                int i, k;
-                coords(v, t, i, k);
+        for (int v = 0; v < NV; v++) {
+            int i, k;
+            coords(v, t, i, k);
+            if (MAJOR) {
+                uint2 w = make_uint2(pack_bf16(r[v][0], r[v][2]), pack_bf16(r[v][1], r[v][3]));
+                *reinterpret_cast<uint2 *>(lds + (k >> 1) * (BT + PAD) + i) = w;
+            } else {
                 lds[(k >> 1) * (BT + PAD) + i] = pack_bf16(r[v][0], r[v][1]);
                 lds[((k >> 1) + 1) * (BT + PAD) + i] = pack_bf16(r[v][2], r[v][3]);
             }
@@ -428,9 +421,13 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     }
 
 #ifdef NCHIP_GEMM_CLOCKS
-    if (g_gemm_clk && blockIdx.x == 0 && blockIdx.y == 0 && t == 0) {
-        g_gemm_clk[0] = clock64() - dbg_c0;       // shader cycles of the k loop
-        g_gemm_clk[1] = wall_clock64() - dbg_w0;  // 100 MHz ticks of the same span
+    if (g_gemm_clk && blockIdx.y == 0 && t == 0) {
+        if (blockIdx.x == 0) {
+            g_gemm_clk[0] = clock64() - dbg_c0;       // shader cycles of the k loop
+            g_gemm_clk[1] = wall_clock64() - dbg_w0;  // 100 MHz ticks of the same span
+        }
+        g_gemm_clk[4 + 3 * blockIdx.x] = dbg_w0;          // per workgroup: start,
+        g_gemm_clk[5 + 3 * blockIdx.x] = wall_clock64();  // end of the k loop
     }
 #endif
     if (KW == 2) {
@@ -481,27 +478,72 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     float *C = g.C + coff;
     float *P = g.pre ? g.pre + coff : nullptr;
     const float *Radd = g.add ? g.add + coff : nullptr;
+    // The 16 values of a 32x32 accumulator tile go to 16 columns of C.  Everything
+    // read here (addend, beta*C) is fetched for all 16 first, so the loads are in
+    // flight together, and the uniform option tests are hoisted out of the
+    // element loop: a branch per element with a load behind it costs one memory
+    // round trip each.
+    const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N); // uniform
+    const bool plain = !g.bias && !P && !Radd && g.beta == 0.0f && g.act == NCHIP_ACT_NONE;
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
         for (int j = 0; j < TM; j++) {
-            int m = mm_base + j * 32;
-            if (m >= g.M) continue;
-            float bv = g.bias ? g.bias[m] : 0.0f;
+            const int m = mm_base + j * 32;
+            const int nb = nn_base + i * 32;
+            if (!full && m >= g.M) continue;
+            float *Cp = C + (int64_t)nb * g.ldc + m; // element r lives at Cp + nofs(r)*ldc
+            auto nofs = [](int r) { return (r >> 2) * 8 + (r & 3); };
+            if (plain && full) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) Cp[(int64_t)nofs(r) * g.ldc] = g.alpha * acc[i][j][r];
+                continue;
+            }
+            bool ok[16];
+#pragma unroll
+            for (int r = 0; r < 16; r++) ok[r] = full || nb + nofs(r) < g.N;
+            float extra[16]; // beta*C + addend
+#pragma unroll
+            for (int r = 0; r < 16; r++) extra[r] = 0.0f;
+            if (Radd) {
+                const float *Ap = Radd + (int64_t)nb * g.ldc + m;
+#pragma unroll
+                for (int r = 0; r < 16; r++) extra[r] = ok[r] ? Ap[(int64_t)nofs(r) * g.ldc] : 0.0f;
+            }
+            float prev[16];
+            const bool has_beta = g.beta != 0.0f;
+            if (has_beta) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) prev[r] = ok[r] ? Cp[(int64_t)nofs(r) * g.ldc] : 0.0f;
+            }
+            const float bv = g.bias ? g.bias[m] : 0.0f;
+            float v[16];
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                int n = nn_base + i * 32 + (r >> 2) * 8 + (r & 3);
-                if (n >= g.N) continue;
-                int64_t off = (int64_t)n * g.ldc + m;
-                float v = g.alpha * acc[i][j][r];
-                if (g.beta != 0.0f) v += g.beta * C[off];
-                v += bv;
-                if (P) P[off] = v;
-                v = apply_act(v, g.act);
-                if (Radd) v += Radd[off];
-                C[off] = v;
+                v[r] = g.alpha * acc[i][j][r];
+                if (has_beta) v[r] += g.beta * prev[r];
+                v[r] += bv;
             }
+            if (P) {
+                float *Pp = P + (int64_t)nb * g.ldc + m;
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (ok[r]) Pp[(int64_t)nofs(r) * g.ldc] = v[r];
+            }
+            if (g.act == NCHIP_ACT_GELU) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) v[r] = gelu_tanh(v[r]);
+            } else if (g.act == NCHIP_ACT_RELU) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) v[r] = v[r] > 0.0f ? v[r] : 0.0f;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r] + extra[r];
         }
+#ifdef NCHIP_GEMM_CLOCKS
+    if (g_gemm_clk && blockIdx.y == 0 && t == 0) g_gemm_clk[6 + 3 * blockIdx.x] = wall_clock64(); // stores issued
+#endif
 }
 
 // sums the ksplit partial tiles in increasing k order, then the same epilogue
@@ -637,8 +679,9 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     }
     if (precision == 1) {
         if (cfg == 7) launch_tile<128, 128, 32, 4, 2, 1>(st, ta, tb, g, pr);
-        else if (cfg == 4) launch_tile<128, 64, 64, 4, 2, 1>(st, ta, tb, g, pr);
-        else launch_tile<64, 64, 64, 2, 2, 1, 2>(st, ta, tb, g, pr);
+        else if (cfg == 4) launch_tile<128, 64, 32, 4, 2, 1>(st, ta, tb, g, pr);
+        else if (cfg == 9) launch_tile<64, 64, 64, 2, 2, 1, 2>(st, ta, tb, g, pr);
+        else launch_tile<64, 64, 32, 2, 2, 1, 2>(st, ta, tb, g, pr);
     } else if (cfg == 1) {
         launch_tile<128, 128, 16, 2, 2, 0>(st, ta, tb, g, pr);
     } else if (cfg == 2) {
@@ -748,7 +791,7 @@ extern "C" int nchip_gemm_profile_read(int max_variants, char (*names)[48], int6
     }
     g_prof.clear();
     static const char *tiles_f32[4] = { "64,64,16,2,2", "128,64,32,4,2", "128,128,32,4,2", "64,64,32,2,2" };
-    static const char *tiles_bf16[4] = { "64,64,64,2,2", "128,64,64,4,2", "128,128,32,4,2", "64,64,64,2,2" };
+    static const char *tiles_bf16[4] = { "64,64,32,2,2", "128,64,32,4,2", "128,128,32,4,2", "64,64,32,2,2" };
     int n = 0;
     for (int v = 0; v < 32 && n < max_variants; v++) {
         if (!cnt[v]) continue;
