@@ -52,6 +52,16 @@ int nchip_gemm_add(void *stream, int ta, int tb, int m, int n, int k, float alph
                    const float *bias, int act, float *pre, const float *addend,
                    int precision, int ksplit, float *workspace);
 
+/* C = (alpha * op(A) * op(B)) .* act'(pre_act): the input gradient of a linear
+   layer whose input came out of an activation (pre_act = the values before
+   that activation, laid out like C).  One GEMM instead of a GEMM and an
+   element-wise pass; the product is rounded to fp32 before the multiplication,
+   as the two-pass form does. */
+int nchip_gemm_dact(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                    const float *A, int64_t lda, const float *B, int64_t ldb,
+                    float *C, int64_t ldc, const float *pre_act, int act,
+                    int precision, int ksplit, float *workspace);
+
 /* Same with two-level batching: batch index z addresses
    A + (z / batch_in)*sa_out + (z % batch_in)*sa_in (likewise B and C).  Lets
    per-(stream, head) products read the (features, streams, time) activations

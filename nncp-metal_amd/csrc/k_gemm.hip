@@ -45,6 +45,8 @@ struct GemmArgs {
     float *C;
     const float *bias;
     const float *add; // same layout as C, added after the activation (may be NULL)
+    const float *dpre; // same layout as C: the result is multiplied by act'(dpre) (may be NULL)
+    int dact;
     float *pre;
     float *ws;
     int64_t lda, ldb, ldc, sa, sb, sc;   // outer batch strides
@@ -62,6 +64,17 @@ __device__ __forceinline__ float gelu_tanh(float x)
 {
     const float c0 = 0.7978845608f, c1 = 0.044715f;
     return 0.5f * x * (1.0f + tanhf(c0 * (x + c1 * x * x * x)));
+}
+
+__device__ __forceinline__ float act_grad(float x, int act)
+{
+    if (act == NCHIP_ACT_GELU) {
+        const float c0 = 0.7978845608f, c1 = 0.044715f;
+        float t = tanhf(c0 * (x + c1 * x * x * x));
+        return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * c0 * (1.0f + 3.0f * c1 * x * x);
+    }
+    if (act == NCHIP_ACT_RELU) return x > 0.0f ? 1.0f : 0.0f;
+    return 1.0f;
 }
 
 __device__ __forceinline__ float apply_act(float v, int act)
@@ -484,7 +497,8 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     // element loop: a branch per element with a load behind it costs one memory
     // round trip each.
     const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N); // uniform
-    const bool plain = !g.bias && !P && !Radd && g.beta == 0.0f && g.act == NCHIP_ACT_NONE;
+    const float *Dp = g.dpre ? g.dpre + coff : nullptr;
+    const bool plain = !g.bias && !P && !Radd && !Dp && g.beta == 0.0f && g.act == NCHIP_ACT_NONE;
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
@@ -537,6 +551,18 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 #pragma unroll
                 for (int r = 0; r < 16; r++) v[r] = v[r] > 0.0f ? v[r] : 0.0f;
             }
+            if (Dp) { // gradient through an activation: times act'(pre-activation)
+                const float *Dq = Dp + (int64_t)nb * g.ldc + m;
+                float pz[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) pz[r] = ok[r] ? Dq[(int64_t)nofs(r) * g.ldc] : 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; r++) v[r] = (v[r] + extra[r]) * act_grad(pz[r], g.dact);
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r];
+                continue;
+            }
 #pragma unroll
             for (int r = 0; r < 16; r++)
                 if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r] + extra[r];
@@ -568,6 +594,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce(GemmArgs g)
         if (P) P[off] = v;
         v = apply_act(v, g.act);
         if (Radd) v += Radd[off];
+        if (g.dpre) v *= act_grad(g.dpre[coff + off], g.dact);
         C[off] = v;
     }
 }
@@ -626,7 +653,7 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
                       float beta, float *C, int64_t ldc, int64_t sc_out, int64_t sc_in,
                       int batch, int batch_in,
                       const float *bias, int act, float *pre, const float *addend, int precision,
-                      int ksplit, float *workspace)
+                      int ksplit, float *workspace, const float *dpre = nullptr, int dact = 0)
 {
     if (m <= 0 || n <= 0 || batch <= 0)
         return 0;
@@ -646,6 +673,7 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     }
     GemmArgs g;
     g.A = A; g.B = B; g.C = C; g.bias = bias; g.add = addend; g.pre = pre; g.ws = workspace;
+    g.dpre = dpre; g.dact = dact;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.sa = sa_out; g.sb = sb_out; g.sc = sc_out;
     g.sa_in = sa_in; g.sb_in = sb_in; g.sc_in = sc_in; g.batch_in = batch_in;
     g.M = m; g.N = n; g.K = k; g.batch = batch; g.ksplit = ksplit;
@@ -746,6 +774,15 @@ extern "C" int nchip_gemm_add(void *stream, int ta, int tb, int m, int n, int k,
     return gemm2_impl(stream, ta, tb, m, n, k, alpha, A, lda, stride_a, 0, B, ldb, stride_b, 0,
                       0.0f, C, ldc, stride_c, 0, batch, 1, bias, act, pre, addend, precision, ksplit,
                       workspace);
+}
+
+extern "C" int nchip_gemm_dact(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                               const float *A, int64_t lda, const float *B, int64_t ldb,
+                               float *C, int64_t ldc, const float *pre_act, int act,
+                               int precision, int ksplit, float *workspace)
+{
+    return gemm2_impl(stream, ta, tb, m, n, k, alpha, A, lda, 0, 0, B, ldb, 0, 0, 0.0f, C, ldc, 0, 0, 1, 1,
+                      nullptr, 0, nullptr, nullptr, precision, ksplit, workspace, pre_act, act);
 }
 
 extern "C" int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, float alpha,

@@ -637,6 +637,23 @@ static void matmul_bw(NCNode *nd, NCTensor *g, NCTensor **ga, int ia, int ib)
         NCTensor *db = nc_alloc_like(b);
         // a gradient already delivered to this parent is added in the epilogue
         const float *prev = nc_bw_addend(m, ib, nc_numel(db));
+        // x came out of nc_linear's activation and feeds nothing else: its
+        // backward step (times act'(pre)) rides in this GEMM's epilogue
+        NCNode *px = nd->parents[ib];
+        if (!prev && !tb && s.batch == 1 && px->op == OP_LINEAR && px->ia[3] != NC_ACT_NONE && px->consumers == 1 &&
+            px->saved[2] && nc_numel(px->saved[2]) == nc_numel(db) && nc_is_contig(px->saved[2])) {
+            int ks = nchip_gemm_pick_ksplit((int)s.k, (int)s.n, (int)s.m, 1);
+            size_t cap = 0;
+            float *ws = ks > 1 ? nc_tmp_f32(m, (size_t)ks * s.k * s.n, &cap) : nullptr;
+            if (nchip_gemm_dact(m->stream, !ta, 0, (int)s.k, (int)s.n, (int)s.m, alpha,
+                                nc_f32(a), (int64_t)(!ta ? s.m : s.k), nc_f32(g), (int64_t)s.m,
+                                nc_f32(db), (int64_t)s.k, nc_f32(px->saved[2]), px->ia[3],
+                                m->matmul_bf16, ks, ws))
+                nc_fatal("gemm failed (activation-gradient epilogue)");
+            if (ws) nc_tmp_free(m, ws, cap);
+            m->launches += ks > 1 ? 2 : 1;
+            px->ia[5] = 1; // the gradient delivered to px is already d(pre-activation)
+        } else
         if (!tb) dev_gemm(m, !ta, false, s.k, s.n, s.m, alpha, a, g, 0.0f, db, s.batch, nullptr, 0, nullptr, prev);
         else     dev_gemm(m, true, ta, s.n, s.k, s.m, alpha, g, a, 0.0f, db, s.batch, nullptr, 0, nullptr, prev);
         ga[ib] = db;
@@ -1141,7 +1158,9 @@ void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
     case OP_LINEAR: {
         if (nd->n_args > 3 && nd->parents[3]) ga[3] = nc_dup_tensor(g); // residual input
         NCTensor *gz = nc_dup_tensor(g);
-        if (nd->ia[3] != NC_ACT_NONE) {
+        const bool already = nd->ia[5] != 0; // the producer of g applied act'(pre) in its epilogue
+        nd->ia[5] = 0;
+        if (nd->ia[3] != NC_ACT_NONE && !already) {
             NCTensor *t = nc_alloc_like(g);
             k_unary_bwd(st, nd->ia[3] == NC_ACT_GELU ? KU_GELU : KU_RELU, nc_f32(nd->saved[2]), nc_f32(g), nc_f32(t), cnt);
             m->launches++;

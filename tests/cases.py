@@ -330,6 +330,12 @@ _add("linear_add_nobias", [(5, 7), (3, 5), (3, 7)],
      lambda nc, w, x, r: nc.nc_linear_add(w, x, None, 0, r), lambda w, x, r: x @ w + r)
 _add("matmul_add_residual", [(5, 7), (3, 5), (3, 7)],
      lambda nc, w, x, r: nc.nc_matmul_add(w, x, r, 0, 0, 0.5), lambda w, x, r: 0.5 * (x @ w) + r)
+_add("mlp_gelu_linear", [(5, 7), (3, 5), (7,), (7, 4), (4,)],
+     lambda nc, w1, x, b1, w2, b2: nc.nc_linear(w2, nc.nc_linear(w1, x, b1, 1), b2, 0),
+     lambda w1, x, b1, w2, b2: U.gelu(x @ w1 + b1) @ w2 + b2)
+_add("mlp_relu_linear_add", [(5, 7), (3, 5), (7, 4), (3, 4)],
+     lambda nc, w1, x, w2, r: nc.nc_linear_add(w2, nc.nc_linear(w1, x, None, 2), None, 0, r),
+     lambda w1, x, w2, r: np.maximum(x @ w1, 0) @ w2 + r)
 _add("linear_relu", [(5, 7), (3, 5), (7,)],
      lambda nc, w, x, b: nc.nc_linear(w, x, b, 2), lambda w, x, b: np.maximum(x @ w + b, 0))
 
