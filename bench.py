@@ -160,7 +160,7 @@ def attention_c2(pkg, iters=50):
         return lib.nchip_relpos_attn_bwd(None, P["q"], ld, P["kv"], P["kvm"], ldkv, P["w_r"], P["probs"],
                                          P["dout"], ld, P["dq"], P["dkv"], P["dkvm"], P["dw_r"], P["db_r"],
                                          i32(Hh), i32(dk), i32(dk), i32(B), i32(T), i32(M), i32(d_pos),
-                                         i32(K), f32(1.0), i32(0), P["scratch"])
+                                         i32(K), f32(1.0), i32(0), P["scratch"], i32(0))
 
     def timed(fns):
         e0, e1 = C.c_void_p(), C.c_void_p()

@@ -133,7 +133,12 @@ int nchip_relpos_attn_last_launches(void);
 /* Backward of the above from the saved probs.  dq, dkv, dkvm are fully
    overwritten; dw_r (dk, d_pos, H) and db_r (K, H) are overwritten with the
    sums over streams, reduced in a fixed order (no atomics).  scratch needs
-   nchip_relpos_attn_bwd_scratch() floats. */
+   nchip_relpos_attn_bwd_scratch() floats.  Returns 0, a negative error, or 1
+   when keep_partials was set and the single-kernel path ran: then dw_r / db_r
+   are NOT written and the per-stream partials stay in scratch for the caller
+   to sum over the B rows: the dw_r partial of stream b at scratch[b*n_w + i]
+   (n_w = dk*d_pos*H), the db_r partial at scratch[B*n_w + b*n_b + i]
+   (n_b = K*H). */
 size_t nchip_relpos_attn_bwd_scratch(int H, int dk, int B, int T, int M, int d_pos);
 int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
                           const float *kv, const float *kvm, int64_t ldkv,
@@ -141,7 +146,8 @@ int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
                           const float *dout, int64_t ldo,
                           float *dq, float *dkv, float *dkvm, float *dw_r, float *db_r,
                           int H, int dk, int dv, int B, int T, int M, int d_pos,
-                          int attn_len, float b_r_scale, int precision, float *scratch);
+                          int attn_len, float b_r_scale, int precision, float *scratch,
+                          int keep_partials);
 
 /* LayerNorm / RMSNorm over axis 0 of (d, n) with optional affine
    (nncp.c:279-288; libnc.h:389-395).  xhat (d, n) and rstd (n) are saved for
@@ -153,6 +159,11 @@ int nchip_norm_fwd(void *stream, const float *x, const float *w, const float *b,
    dw, db (d) overwritten (may be NULL when w is NULL).  partial needs
    nchip_norm_bwd_partial_rows(n) * 2 * d floats. */
 int nchip_norm_bwd_partial_rows(int64_t n);
+/* Rows of `partial` actually written for (d, n): row r holds the dw partial at
+   partial[(2r)*d + i] and the db partial at partial[(2r+1)*d + i].  With
+   partial given and dw == db == NULL the sums over the rows are left to the
+   caller (they can be batched over many calls). */
+int nchip_norm_bwd_rows(int d, int64_t n);
 int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float *rstd,
                    const float *w, float *dx, const float *dx_add, float *dw, float *db,
                    float *partial, int d, int64_t n, int avg);

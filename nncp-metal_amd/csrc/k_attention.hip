@@ -265,7 +265,8 @@ extern "C" int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
                                      const float *dout, int64_t ldo,
                                      float *dq, float *dkv, float *dkvm, float *dw_r, float *db_r,
                                      int H, int dk, int dv, int B, int T, int M, int d_pos,
-                                     int attn_len, float b_r_scale, int precision, float *scratch)
+                                     int attn_len, float b_r_scale, int precision, float *scratch,
+                                     int keep_partials)
 {
     if (check_shapes(H, dk, dv, B, T, M, d_pos, attn_len, w_r != nullptr)) return -1;
     if (!q || !kv || !probs || !dout || !dq || !dkv || !scratch || (M > 0 && (!kvm || !dkvm)) ||
@@ -291,9 +292,9 @@ extern "C" int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
         a.H = H; a.B = B; a.T = T; a.M = M; a.K = K; a.d_pos = w_r ? d_pos : 1; a.attn_len = attn_len;
         a.b_r_scale = b_r_scale; a.scale = 1.0f / sqrtf((float)dk);
         int nl = 0;
-        int frc = k_attn_fused_bwd(st, a, dk, dw_r, db_r, n_w, n_b, &nl);
+        int frc = k_attn_fused_bwd(st, a, dk, dw_r, db_r, n_w, n_b, &nl, keep_partials != 0);
         if (frc == -2) return bad("kernel launch failed");
-        if (frc == 0) { g_last_launches = nl; return 0; }
+        if (frc == 0) { g_last_launches = nl; return (keep_partials && n_w + n_b > 0) ? 1 : 0; }
     }
     const float *vm = kvm ? kvm + (int64_t)H * dk : nullptr, *vc = kv + (int64_t)H * dk;
     // dA = V^T dO

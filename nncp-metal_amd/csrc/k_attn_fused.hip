@@ -654,14 +654,14 @@ int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk)
 }
 
 int k_attn_fused_bwd(hipStream_t st, const FusedAttnBwdArgs &a, int dk, float *dw_r, float *db_r,
-                     int64_t n_w, int64_t n_b, int *launches)
+                     int64_t n_w, int64_t n_b, int *launches, bool keep_partials)
 {
     const bool small = a.K <= 64 && a.d_pos <= 64;
     int rc = dk == 64 ? (small ? launch_bwd<64, 4>(st, a) : launch_bwd<64, 8>(st, a))
                       : (small ? launch_bwd<32, 4>(st, a) : launch_bwd<32, 8>(st, a));
     if (rc) return rc;
     *launches = 1;
-    if (n_w + n_b > 0) {
+    if (n_w + n_b > 0 && !keep_partials) {
         hipLaunchKernelGGL(attn_param_grad_reduce, dim3((unsigned)((n_w + n_b + 255) / 256)), dim3(256), 0, st,
                            (const float *)a.dwp, dw_r, n_w, (const float *)a.dbp, db_r, n_b, a.B);
         *launches = 2;

@@ -223,6 +223,23 @@ __global__ __launch_bounds__(256) void reduce_trailing_stage2(const float *tmp, 
     }
 }
 
+__global__ __launch_bounds__(256) void reduce_rows_multi_kernel(const KReduceRowsEntry *table)
+{
+    __shared__ float sh[3][64];
+    const KReduceRowsEntry e = table[blockIdx.y];
+    const int ig = threadIdx.x & 63, rg = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + ig;
+    if (blockIdx.x * 64 >= e.n) return; // uniform per block
+    float acc = 0.0f;
+    if (i < e.n) {
+#pragma unroll 4
+        for (int r = rg; r < e.rows; r += 4) acc += e.src[(int64_t)r * e.stride + i];
+    }
+    if (rg > 0) sh[rg - 1][ig] = acc;
+    __syncthreads();
+    if (rg == 0 && i < e.n) e.dst[i] = (acc + sh[0][ig]) + (sh[1][ig] + sh[2][ig]);
+}
+
 // block-level fixed tree sum of 256 partials
 __device__ __forceinline__ float block_tree_sum(float v, float *sh)
 {
@@ -420,6 +437,21 @@ void k_reduce_trailing(hipStream_t st, const float *x, const float *y0, float *o
     dim3 grid((unsigned)((inner + TPB - 1) / TPB), ns);
     hipLaunchKernelGGL(reduce_trailing_stage1, grid, dim3(TPB), 0, st, x, tmp, inner, outer, ns);
     hipLaunchKernelGGL(reduce_trailing_stage2, dim3((unsigned)((inner + 63) / 64)), dim3(256), 0, st, (const float *)tmp, y0, out, inner, ns);
+}
+
+int k_reduce_trailing_partials(hipStream_t st, const float *x, float *tmp, int64_t inner, int64_t outer)
+{
+    if (inner <= 0) return 0;
+    int ns = k_reduce_trailing_nsplit(inner, outer);
+    dim3 grid((unsigned)((inner + TPB - 1) / TPB), ns);
+    hipLaunchKernelGGL(reduce_trailing_stage1, grid, dim3(TPB), 0, st, x, tmp, inner, outer, ns);
+    return ns;
+}
+
+void k_reduce_rows_multi(hipStream_t st, const KReduceRowsEntry *dev_table, int n_entries, int max_n)
+{
+    if (n_entries <= 0 || max_n <= 0) return;
+    hipLaunchKernelGGL(reduce_rows_multi_kernel, dim3((unsigned)((max_n + 63) / 64), n_entries), dim3(256), 0, st, dev_table);
 }
 
 void k_reduce_all(hipStream_t st, const float *x, float *out, float *tmp, int64_t n)

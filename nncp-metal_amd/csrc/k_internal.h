@@ -56,6 +56,18 @@ void k_lstm_clamped_bwd(hipStream_t st, const float *cp, const float *in, const 
 int k_reduce_trailing_nsplit(int64_t inner, int64_t outer);
 void k_reduce_trailing(hipStream_t st, const float *x, const float *y0, float *out, float *tmp,
                        int64_t inner, int64_t outer);
+// stage 1 only: tmp[s][i] for s < k_reduce_trailing_nsplit(inner, outer); returns that count
+int k_reduce_trailing_partials(hipStream_t st, const float *x, float *tmp, int64_t inner, int64_t outer);
+// many row sums in one launch: dst[i] = sum_{r < rows} src[r*stride + i], i < n,
+// per table entry (table in device memory); 4 interleaved row groups per
+// element, sequential inside a group, combined in group order
+struct KReduceRowsEntry {
+    const float *src;
+    float *dst;
+    int64_t stride;
+    int rows, n;
+};
+void k_reduce_rows_multi(hipStream_t st, const KReduceRowsEntry *dev_table, int n_entries, int max_n);
 // out[0] = sum of all n elements (fixed tree); tmp: 1024 floats
 void k_reduce_all(hipStream_t st, const float *x, float *out, float *tmp, int64_t n);
 // general un-broadcast: out (numel nout, dims d.dims with strides d.sb over the
@@ -91,6 +103,6 @@ bool k_attn_fused_shape_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr)
 int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk);
 // returns 0, -1 (path unavailable, nothing launched) or -2 (launch failed)
 int k_attn_fused_bwd(hipStream_t st, const FusedAttnBwdArgs &a, int dk, float *dw_r, float *db_r,
-                     int64_t n_w, int64_t n_b, int *launches);
+                     int64_t n_w, int64_t n_b, int *launches, bool keep_partials);
 
 #endif

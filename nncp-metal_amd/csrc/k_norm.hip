@@ -402,6 +402,16 @@ int nchip_norm_bwd_partial_rows(int64_t n)
     return (int)(r < 32 ? 32 : r); // the generic path uses up to 32 slices
 }
 
+// exact number of partial rows nchip_norm_bwd writes for (d, n)
+int nchip_norm_bwd_rows(int d, int64_t n)
+{
+    if (d == 128 || d == 256 || d == 512 || d == 1024) {
+        const int cw = norm_bwd_cw(n);
+        return (int)((n + (int64_t)WPB * cw - 1) / ((int64_t)WPB * cw));
+    }
+    return (int)(n / 16 > 32 ? 32 : (n / 16 < 1 ? 1 : n / 16));
+}
+
 int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float *rstd, const float *w,
                    float *dx, const float *dx_add, float *dw, float *db, float *partial, int d, int64_t n,
                    int avg)
@@ -410,10 +420,11 @@ int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float 
     hipStream_t st = (hipStream_t)stream;
     const bool wb = dw || db;
     if (wb && !partial) { fprintf(stderr, "nchip_norm_bwd: partial buffer missing\n"); return -1; }
+    // partial given without dw / db: the partial rows are left for the caller to sum
     if (d == 128 || d == 256 || d == 512 || d == 1024) {
         const int cw = norm_bwd_cw(n);
-        const int rows = (int)((n + (int64_t)WPB * cw - 1) / ((int64_t)WPB * cw));
-        float *pp = wb ? partial : nullptr;
+        const int rows = nchip_norm_bwd_rows(d, n);
+        float *pp = partial;
 #define NORM_BWD(NV) hipLaunchKernelGGL(norm_bwd_fused<NV>, dim3(rows), dim3(TPB), 0, st, g, xhat, rstd, w, dx, dx_add, pp, n, avg, cw)
         if (d == 128) NORM_BWD(2); else if (d == 256) NORM_BWD(4); else if (d == 512) NORM_BWD(8); else NORM_BWD(16);
 #undef NORM_BWD
@@ -425,12 +436,13 @@ int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float 
     if (dx)
         hipLaunchKernelGGL(norm_bwd_dx_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, st,
                            g, xhat, rstd, w, dx, dx_add, d, n, avg);
-    if (wb) {
-        int rows = (int)(n / 16 > 32 ? 32 : (n / 16 < 1 ? 1 : n / 16));
+    if (partial) {
+        int rows = nchip_norm_bwd_rows(d, n);
         hipLaunchKernelGGL(norm_bwd_wb_stage1, dim3((d + TPB - 1) / TPB, rows), dim3(TPB), 0, st,
                            g, xhat, partial, d, n, rows);
-        hipLaunchKernelGGL(norm_bwd_wb_stage2, dim3((d + 63) / 64), dim3(TPB), 0, st,
-                           (const float *)partial, dw, db, d, rows);
+        if (wb)
+            hipLaunchKernelGGL(norm_bwd_wb_stage2, dim3((d + 63) / 64), dim3(TPB), 0, st,
+                               (const float *)partial, dw, db, d, rows);
     }
     return check("nchip_norm_bwd");
 }

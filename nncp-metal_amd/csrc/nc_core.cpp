@@ -109,6 +109,8 @@ extern "C" NCContext *nc_context_init(int nb_threads)
     for (int i = 0; i < NC_BW_ARGS; i++) { m->bw_prev[i] = nullptr; m->bw_used[i] = false; }
     m->grp_staging = nullptr;
     m->grp_staging_cap = 0;
+    m->red_staging = nullptr;
+    m->red_staging_cap = 0;
     const char *e = getenv("NCHIP_MATMUL_BF16");
     if (e && atoi(e) != 0)
         m->matmul_bf16 = 1;

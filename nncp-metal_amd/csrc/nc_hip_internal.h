@@ -52,6 +52,17 @@ struct DeferredGemm {
     const NCNode *param;   // the parameter this gradient belongs to
 };
 
+// a gradient that is a sum of partial rows, summed with all others of its kind
+// in one launch at the end of nc_backward
+struct DeferredReduce {
+    const float *src;
+    float *dst;
+    int64_t stride;
+    int rows, n;
+    const NCNode *param;
+};
+struct DeferredTmp { float *ptr; size_t cap; };
+
 #define NC_BW_ARGS 8 // node arguments for which nc_backward offers the existing gradient
 
 struct NCContext {
@@ -70,8 +81,13 @@ struct NCContext {
     NCTensor *bw_prev[NC_BW_ARGS];
     bool bw_used[NC_BW_ARGS];
     std::vector<DeferredGemm> deferred;
+    std::vector<DeferredReduce> deferred_red;
+    std::vector<DeferredTmp> deferred_tmp;    // scratch the partial rows live in
+    std::vector<NCTensor *> deferred_keep;    // destination tensors
     void *grp_staging;
     size_t grp_staging_cap;
+    void *red_staging;
+    size_t red_staging_cap;
 };
 
 struct NCTensorBuffer {
@@ -145,5 +161,6 @@ NCTensor *nc_finish(NCTensor *y, NCNode *n, NCTensor **args, int n_args);
 void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga); // nc_ops.cpp
 void nc_flush_deferred(NCContext *m);                          // nc_ops.cpp
 bool nc_has_deferred(const NCContext *m, const NCNode *param);  // nc_ops.cpp
+bool nc_can_defer_sum(const NCContext *m, const NCNode *parent); // nc_ops.cpp
 
 #endif

@@ -82,7 +82,12 @@ static NCTensor *dev_binary(int op, const NCTensor *a, const NCTensor *b)
 }
 
 // sums g (consumed) down to `target` (each target dim equals g's or is 1/missing)
-static NCTensor *dev_unbroadcast(NCTensor *g, const Shape &target)
+static void defer_sum(NCContext *m, const float *src, NCTensor *dst, int rows, int64_t stride, int n,
+                      const NCNode *param);
+
+// defer_param: the parameter node the result is the gradient of, when its
+// final sum over partial rows may wait for the end of nc_backward
+static NCTensor *dev_unbroadcast(NCTensor *g, const Shape &target, const NCNode *defer_param = nullptr)
 {
     size_t nt = 1;
     for (int i = 0; i < target.nd; i++) nt *= target.d[i];
@@ -106,8 +111,16 @@ static NCTensor *dev_unbroadcast(NCTensor *g, const Shape &target)
     } else if (prefix) {
         int64_t inner = (int64_t)nt, outer = (int64_t)(nc_numel(g) / nt);
         float *tmp = nc_tmp_f32(m, (size_t)k_reduce_trailing_nsplit(inner, outer) * inner, &cap);
-        k_reduce_trailing(m->stream, nc_f32(g), nullptr, nc_f32(y), tmp, inner, outer);
-        nc_tmp_free(m, tmp, cap);
+        if (defer_param && nc_can_defer_sum(m, defer_param) && inner < (1 << 30)) {
+            int ns = k_reduce_trailing_partials(m->stream, nc_f32(g), tmp, inner, outer);
+            defer_sum(m, tmp, y, ns, inner, (int)inner, defer_param);
+            DeferredTmp dt = { tmp, cap };
+            m->deferred_tmp.push_back(dt);
+        } else {
+            k_reduce_trailing(m->stream, nc_f32(g), nullptr, nc_f32(y), tmp, inner, outer);
+            nc_tmp_free(m, tmp, cap);
+            m->launches++; // second stage
+        }
     } else {
         // general case: one thread per kept element loops over the reduced axes
         NdDesc keep, red;
@@ -907,15 +920,26 @@ static void attn_bw(NCNode *nd, NCTensor *g, NCTensor **ga)
     NCTensor *dbr = nd->ia[4] ? new_f32(q, 2, bd) : nullptr;
     size_t cap;
     float *scratch = nc_tmp_f32(m, nchip_relpos_attn_bwd_scratch(a.H, a.dk, a.B, a.T, a.M, a.d_pos), &cap);
+    const int keep = (dwr || dbr) && (!dwr || nc_can_defer_sum(m, nd->parents[3])) &&
+                     (!dbr || nc_can_defer_sum(m, nd->parents[4]));
     int rc = nchip_relpos_attn_bwd(m->stream, nc_f32(q), (int64_t)q->dims[0], nc_f32(kv),
                                    kvm ? nc_f32(kvm) : nullptr, (int64_t)kv->dims[0],
                                    w_r ? nc_f32(w_r) : nullptr, nc_f32(probs), nc_f32(gc),
                                    (int64_t)gc->dims[0], nc_f32(dq), nc_f32(dkv),
                                    dkvm ? nc_f32(dkvm) : nullptr, dwr ? nc_f32(dwr) : nullptr,
                                    dbr ? nc_f32(dbr) : nullptr, a.H, a.dk, a.dv, a.B, a.T, a.M, a.d_pos,
-                                   nd->ia[2], nd->fa[0], 0, scratch);
-    nc_tmp_free(m, scratch, cap);
-    if (rc) nc_fatal("nc_relpos_attention backward failed");
+                                   nd->ia[2], nd->fa[0], 0, scratch, keep);
+    if (rc < 0) nc_fatal("nc_relpos_attention backward failed");
+    if (rc == 1) {
+        // per-stream dw_r / db_r partials stay in scratch until the batched sum
+        const int64_t n_w = dwr ? (int64_t)nc_numel(dwr) : 0, n_b = dbr ? (int64_t)nc_numel(dbr) : 0;
+        if (dwr) defer_sum(m, scratch, dwr, a.B, n_w, (int)n_w, nd->parents[3]);
+        if (dbr) defer_sum(m, scratch + n_w * a.B, dbr, a.B, n_b, (int)n_b, nd->parents[4]);
+        DeferredTmp dt = { scratch, cap };
+        m->deferred_tmp.push_back(dt);
+    } else {
+        nc_tmp_free(m, scratch, cap);
+    }
     m->launches += nchip_relpos_attn_last_launches();
     nc_free_tensor(gc);
     NCTensor *out[5] = { dq, dkv, dkvm, dwr, dbr };
@@ -975,11 +999,7 @@ extern "C" float nc_exp_det(float x)
     return v.f;
 }
 
-// Runs every postponed weight-gradient GEMM in one grouped launch.  The
-// gradient tensors were handed to the parameter callback earlier, so with
-// nc_set_deferred_weight_grad() enabled they hold valid data only once
-// nc_backward() has returned.
-void nc_flush_deferred(NCContext *m)
+static void flush_deferred_gemms(NCContext *m)
 {
     if (m->deferred.empty()) return;
     std::vector<NchipGemmProblem> tab;
@@ -1020,11 +1040,64 @@ void nc_flush_deferred(NCContext *m)
     m->deferred.clear();
 }
 
+static void flush_deferred_sums(NCContext *m)
+{
+    if (m->deferred_red.empty()) return;
+    std::vector<KReduceRowsEntry> tab;
+    int max_n = 0;
+    for (DeferredReduce &d : m->deferred_red) {
+        KReduceRowsEntry e;
+        e.src = d.src; e.dst = d.dst; e.stride = d.stride; e.rows = d.rows; e.n = d.n;
+        if (d.n > max_n) max_n = d.n;
+        tab.push_back(e);
+    }
+    size_t bytes = tab.size() * sizeof(KReduceRowsEntry), hcap, dcap;
+    void *host = m->host_pool.get(bytes, &hcap);
+    void *dev = m->dev_pool.get(bytes, &dcap);
+    memcpy(host, tab.data(), bytes);
+    hip_check(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync sum table");
+    k_reduce_rows_multi(m->stream, (const KReduceRowsEntry *)dev, (int)tab.size(), max_n);
+    m->launches++;
+    if (m->red_staging) m->host_pool.put(m->red_staging, m->red_staging_cap);
+    m->red_staging = host; m->red_staging_cap = hcap;
+    m->dev_pool.put(dev, dcap);
+    for (DeferredTmp &t : m->deferred_tmp) nc_tmp_free(m, t.ptr, t.cap);
+    for (NCTensor *t : m->deferred_keep) nc_free_tensor(t);
+    m->deferred_red.clear(); m->deferred_tmp.clear(); m->deferred_keep.clear();
+}
+
+// Runs every postponed weight-gradient GEMM in one grouped launch and every
+// postponed sum of partial rows in another.  The gradient tensors were handed
+// to the parameter callback earlier, so with nc_set_deferred_weight_grad()
+// enabled they hold valid data only once nc_backward() has returned.
+void nc_flush_deferred(NCContext *m)
+{
+    flush_deferred_gemms(m);
+    flush_deferred_sums(m);
+}
+
 bool nc_has_deferred(const NCContext *m, const NCNode *param)
 {
     for (const DeferredGemm &e : m->deferred)
         if (e.param == param) return true;
+    for (const DeferredReduce &e : m->deferred_red)
+        if (e.param == param) return true;
     return false;
+}
+
+// a gradient that goes straight to a parameter used once may be finished late
+bool nc_can_defer_sum(const NCContext *m, const NCNode *parent)
+{
+    return m->defer_wgrad && parent && parent->op == OP_PARAM && parent->consumers == 1;
+}
+
+static void defer_sum(NCContext *m, const float *src, NCTensor *dst, int rows, int64_t stride, int n,
+                      const NCNode *param)
+{
+    DeferredReduce d;
+    d.src = src; d.dst = nc_f32(dst); d.rows = rows; d.stride = stride; d.n = n; d.param = param;
+    m->deferred_red.push_back(d);
+    m->deferred_keep.push_back(nc_dup_tensor(dst));
 }
 
 // ---- backward dispatch --------------------------------------------------------
@@ -1171,7 +1244,7 @@ void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
         if (nd->parents[2]) {
             Shape bs;
             bs.nd = 1; bs.d[0] = nd->saved[0]->dims[0];
-            ga[2] = dev_unbroadcast(nc_dup_tensor(gz), bs);
+            ga[2] = dev_unbroadcast(nc_dup_tensor(gz), bs, nd->parents[2]);
         }
         nc_free_tensor(gz);
         break;
@@ -1215,12 +1288,24 @@ void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
         NCTensor *db = (w && nd->parents[2]) ? nc_alloc(g->dev, NC_TYPE_F32, 1, &dd, false) : nullptr;
         float *partial = (dw || db) ? nc_tmp_f32(m, (size_t)nchip_norm_bwd_partial_rows(cols) * 2 * d, &cap) : nullptr;
         const float *prev = dx ? nc_bw_addend(m, 0, nc_numel(dx)) : nullptr;
+        // dw / db that go straight to once-used parameters: their sums over the
+        // partial rows join the batched sum at the end of nc_backward
+        const bool late = dw && db && nc_can_defer_sum(m, nd->parents[1]) && nc_can_defer_sum(m, nd->parents[2]);
         if (nchip_norm_bwd(st, nc_f32(g), nc_f32(xhat), nc_f32(rstd), w ? nc_f32(w) : nullptr,
-                           dx ? nc_f32(dx) : nullptr, prev, dw ? nc_f32(dw) : nullptr, db ? nc_f32(db) : nullptr,
-                           partial, d, cols, nd->ia[0]))
+                           dx ? nc_f32(dx) : nullptr, prev, (dw && !late) ? nc_f32(dw) : nullptr,
+                           (db && !late) ? nc_f32(db) : nullptr, partial, d, cols, nd->ia[0]))
             nc_fatal("layer norm backward failed");
-        if (partial) nc_tmp_free(m, partial, cap);
-        m->launches += 3;
+        if (late) {
+            const int rows = nchip_norm_bwd_rows(d, cols);
+            defer_sum(m, partial, dw, rows, 2 * (int64_t)d, d, nd->parents[1]);
+            defer_sum(m, partial + d, db, rows, 2 * (int64_t)d, d, nd->parents[2]);
+            DeferredTmp dt = { partial, cap };
+            m->deferred_tmp.push_back(dt);
+            m->launches += 1;
+        } else {
+            if (partial) nc_tmp_free(m, partial, cap);
+            m->launches += (dw || db) ? 2 : 1;
+        }
         ga[0] = dx; ga[1] = dw; ga[2] = db;
         break;
     }
