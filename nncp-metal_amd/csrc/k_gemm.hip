@@ -729,6 +729,7 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     } else if (cfg == 10) {
         launch_tile<64, 64, 32, 2, 2, 0, 2, 4>(st, ta, tb, g, pr);
 
+
     } else {
         launch_tile<64, 64, 16, 2, 2, 0>(st, ta, tb, g, pr);
     }

@@ -137,3 +137,44 @@ def test_fused_segment_stream_round_trip_and_size_c1(hosts):
     ref.close()
     assert abs(len(data) - len(data_ref)) <= 0.005 * len(data_ref), (len(data), len(data_ref))
     assert abs(st.loss_bits - st_ref.loss_bits) <= 1e-4 * st_ref.loss_bits
+
+
+PROFILE_VARIANTS = {
+    # nncp's enwik profile features (nncp.c:2515-2572) at a small size: pre + final
+    # RMSNorm, GEGLU, untied position parameters, d_pos = K
+    "enwik_like": dict(n_layer=2, d_model=128, n_head=4, d_inner=256, d_pos=48, mem_len=24, seg_len=24,
+                       batch_size=3, n_symbols=64, ln_flags=2 | 4 | 16, ff_act=2, tied_w_r=0, tied_b_r=0),
+    # more keys than the single-kernel attention holds in LDS (K = 144): batched-GEMM attention
+    "long_memory": dict(n_layer=2, d_model=128, n_head=4, d_inner=256, d_pos=144, mem_len=112, seg_len=32,
+                        batch_size=2, n_symbols=64),
+    # head size outside {32, 64}, gated SiLU, query bias, per-layer attention windows, no w_r
+    "odd_heads": dict(n_layer=2, d_model=96, n_head=4, d_inner=192, d_pos=20, mem_len=12, seg_len=16,
+                      batch_size=3, n_symbols=50, ff_act=3, query_bias=1, use_w_r=0, attn_len=[9, 28]),
+    # ReLU with LN_COEF scaling (residual folding is off on that path)
+    "relu_coef": dict(n_layer=2, d_model=64, n_head=2, d_inner=128, d_pos=16, mem_len=16, seg_len=16,
+                      batch_size=4, n_symbols=32, ff_act=0, ln_flags=1 | 8),
+}
+
+
+@pytest.mark.parametrize("name", sorted(PROFILE_VARIANTS))
+@pytest.mark.parametrize("fused", [0, 1])
+def test_profile_variants_match_checker(hosts, name, fused):
+    """The model-class options beyond the default profile, product vs checker
+    after 1 and 4 training steps.  With fused = 1 the attention is always the
+    fused op; gated feed-forward forms keep the reference op sequence."""
+    cfg = dict(PROFILE_VARIANTS[name])
+    cfg.setdefault("seed", 321)
+    hip, ref = _pair(hosts, cfg, fused=fused, sgd_opt=M.rmsprop(3e-4))
+    B, T, V = cfg["batch_size"], cfg["seg_len"], cfg["n_symbols"]
+    syms = M.markov1(B * T * 4, V, seed=77)
+    for step, (tok, tgt) in enumerate(M.segment_batches(syms, B, T, 4), 1):
+        ph, lh = hip.train_step(tok, tgt, 3e-4)
+        pr, lr_ = ref.train_step(tok, tgt, 3e-4)
+        if step in (1, 4):
+            assert M.relerr(ph, pr) <= 1e-5, (name, step)
+            assert abs(lh - lr_) <= 1e-5 * abs(lr_), (name, step)
+    w_h, w_r = hip.params(), ref.params()
+    for k in w_r:
+        assert M.tensors_close(w_h[k], w_r[k], 1e-5), (name, k, M.rel_l2(w_h[k], w_r[k]))
+    hip.close()
+    ref.close()
