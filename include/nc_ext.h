@@ -49,6 +49,24 @@ NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv_mem,
                               NCTensor *w_r, NCTensor *b_r, int n_head,
                               int d_key, int attn_len, float b_r_scale);
 
+/* One query position of nc_relpos_attention: q (H*dk, B) is the query of
+   position t, kv_cache (H*dk+H*dv, B, T) holds the keys / values of positions
+   0..t of the current segment (later columns finite, e.g. zero), kv_mem, w_r,
+   b_r as above.  Result (H*dv, B), bit-identical to column t of the
+   whole-segment call once the segment is complete (the decoder's view of
+   nncp.c:801-863).  No gradient. */
+NCTensor *nc_relpos_attention_step(NCTensor *q, NCTensor *kv_cache, NCTensor *kv_mem,
+                                   NCTensor *w_r, NCTensor *b_r, int n_head, int d_key,
+                                   int attn_len, float b_r_scale, int t);
+
+/* When non-zero, the forward products of nc_matmul / nc_matmul_add / nc_linear
+   use one tile class and one reduction order whatever the number of columns,
+   so evaluating a single token column reproduces, bit for bit, that column of a
+   whole-segment evaluation (what a per-timestep decoder needs against a
+   whole-segment encoder).  Returns the previous setting.  No effect in
+   libnc_ref.so, whose products are column-independent by construction. */
+int nc_set_matmul_width_invariant(NCContext *m, int enable);
+
 /* Integer CDF for the arithmetic coder (anchor: nc_soft_max_int libnc.h:384).
    logits (V, n) f32 -> (V, n) NC_TYPE_U16 with, per column,
      cdf[0] = 0, cdf[i+1] - cdf[i] >= 1, implicit cdf[V] = 65536.

@@ -22,6 +22,11 @@ extern "C" {
 #define NCHIP_ACT_GELU 1
 #define NCHIP_ACT_RELU 2
 
+/* or-ed into `precision`: use the tile class and reduction order that do not
+   depend on m or n (64x64 tiles, two interleaved k chains, no split-K), so a
+   column computed alone is bit-identical to the same column of a wide product */
+#define NCHIP_GEMM_WIDTH_INVARIANT 0x100
+
 /* C = act(alpha * op(A) * op(B) + beta * C + bias), batched.
    Replaces nc_matmul / nc_matmul_add (libnc.h:365-373, call sites
    nncp.c:659-1004).  op(A) is m x k: A is (m,k) when ta == 0, (k,m) when
@@ -125,6 +130,19 @@ int nchip_relpos_attn_fwd(void *stream, const float *q, int64_t ldq,
                           float *out, int64_t ldo, float *probs, float *rel,
                           int H, int dk, int dv, int B, int T, int M, int d_pos,
                           int attn_len, float b_r_scale, int precision);
+
+/* The same for ONE query position t of the segment (the per-timestep step of a
+   decoder, nncp.c:801-863): q and out are single token columns (H*dk, B) and
+   (H*dv, B); kv is the segment's K/V cache (H*dk+H*dv, B, T) whose columns
+   0..t are filled (later columns must hold finite values; they are masked).
+   The result is bit-identical to column t of nchip_relpos_attn_fwd on the
+   completed segment.  Only shapes of the single-kernel path (d_head 32 or 64,
+   T <= 64, K <= 128, d_pos <= 128). */
+int nchip_relpos_attn_fwd_step(void *stream, const float *q, int64_t ldq,
+                               const float *kv, const float *kvm, int64_t ldkv,
+                               const float *w_r, const float *b_r, float *out, int64_t ldo,
+                               int H, int dk, int dv, int B, int T, int M, int d_pos,
+                               int attn_len, float b_r_scale, int t);
 
 /* Kernel launches issued by the calling thread's last successful
    nchip_relpos_attn_fwd (1 when the head fits the single-kernel path). */

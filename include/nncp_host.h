@@ -114,11 +114,27 @@ void trf_update(NNCPModel *s);                                             /* nn
 void trf_set_lr(NNCPModel *s, float lr);                                   /* nncp.c:1243 */
 /* logits of the last trf_eval (V, B, T|1), borrowed; used by the CDF path */
 NCTensor *trf_last_logits(NNCPModel *s);
+/* Per-timestep evaluation with K/V caches through the fused entry points (the
+   decoder's view of a segment, nncp.c:801-863; cfg.fused = 1 and the shapes of
+   the single-kernel attention).  trf_step_begin once per segment, then
+   trf_eval_step(t, input) for t = 0, 1, ...: evaluates the one token column t of
+   input (B, T) against the memory and the columns evaluated so far and returns
+   the owned probabilities (V, B, 1); no graph is kept.  With
+   nc_set_matmul_width_invariant() on for both sides, its logits equal column t
+   of the whole-segment trf_eval bit for bit. */
+void trf_step_begin(NNCPModel *s);
+NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input);
+void trf_step_end(NNCPModel *s);
 
 /* ---- block loop (process_block, nncp.c:2968-3147) ------------------------------ */
 #define NNCP_MODE_SEQ_EVAL 0   /* one trf_eval per timestep: decodable, as nncp c/d */
 #define NNCP_MODE_SEGMENT 1    /* one trf_eval per segment (nncp --encode_only); the
                                   decoder replays the same segment evaluation T times */
+#define NNCP_MODE_STEP_DECODE 4 /* with NNCP_MODE_SEGMENT: the decoder evaluates one token
+                                  column per timestep against K/V caches (trf_eval_step)
+                                  instead of replaying the segment; both sides then run
+                                  their forward products width-invariant, so the flag is
+                                  part of the stream's format */
 #define NNCP_CODER_FLOAT 0     /* write_sym on float probabilities */
 #define NNCP_CODER_CDF16 2     /* nc_soft_max_cdf16 + integer symbol coder */
 

@@ -216,6 +216,7 @@ extern "C" int nchip_relpos_attn_fwd(void *stream, const float *q, int64_t ldq,
         a.ldq = ldq; a.ldkv = ldkv; a.ldo = ldo;
         a.H = H; a.B = B; a.T = T; a.M = M; a.K = K; a.d_pos = w_r ? d_pos : 1; a.attn_len = attn_len;
         a.b_r_scale = b_r_scale; a.scale = 1.0f / sqrtf((float)dk);
+        a.q_only = -1;
         if (k_attn_fused_fwd((hipStream_t)stream, a, dk) == 0) { g_last_launches = 1; return 0; }
     }
     if (w_r) // rel = w_r[h]^T q
@@ -250,6 +251,30 @@ extern "C" int nchip_relpos_attn_fwd(void *stream, const float *q, int64_t ldq,
 }
 
 extern "C" int nchip_relpos_attn_last_launches(void) { return g_last_launches; }
+
+extern "C" int nchip_relpos_attn_fwd_step(void *stream, const float *q, int64_t ldq,
+                                          const float *kv, const float *kvm, int64_t ldkv,
+                                          const float *w_r, const float *b_r, float *out, int64_t ldo,
+                                          int H, int dk, int dv, int B, int T, int M, int d_pos,
+                                          int attn_len, float b_r_scale, int t)
+{
+    if (check_shapes(H, dk, dv, B, T, M, d_pos, attn_len, w_r != nullptr)) return -1;
+    if (!q || !kv || !out || (M > 0 && !kvm)) return bad("null pointer");
+    if (t < 0 || t >= T) return bad("query position outside the segment");
+    const int K = M + T;
+    if (!k_attn_fused_shape_ok(dk, dv, T, K, d_pos, w_r != nullptr) || ldq % 4 || ldkv % 4 || ldo % 4 ||
+        !al16(q) || !al16(kv) || (kvm && !al16(kvm)) || (w_r && !al16(w_r)) || !al16(out))
+        return bad("single-query attention needs the single-kernel shapes (d_head 32/64, T <= 64, K <= 128)");
+    FusedAttnFwdArgs a;
+    a.q = q; a.kv = kv; a.kvm = kvm; a.w_r = w_r; a.b_r = b_r; a.out = out; a.probs = nullptr;
+    a.ldq = ldq; a.ldkv = ldkv; a.ldo = ldo;
+    a.H = H; a.B = B; a.T = T; a.M = M; a.K = K; a.d_pos = w_r ? d_pos : 1; a.attn_len = attn_len;
+    a.b_r_scale = b_r_scale; a.scale = 1.0f / sqrtf((float)dk);
+    a.q_only = t;
+    if (k_attn_fused_fwd((hipStream_t)stream, a, dk)) return bad("kernel launch failed");
+    g_last_launches = 1;
+    return 0;
+}
 
 extern "C" size_t nchip_relpos_attn_bwd_scratch(int H, int dk, int B, int T, int M, int d_pos)
 {

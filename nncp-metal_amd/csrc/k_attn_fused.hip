@@ -158,7 +158,11 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
             return (r < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * r)
                             : a.kv + a.ldkv * (b + (int64_t)a.B * (r - a.M))) + (int64_t)h * DK;
         };
-        fetch_rows<DK, FA_TMAX>(vq, a.T, [&](int r) { return a.q + (int64_t)h * DK + a.ldq * (b + (int64_t)a.B * r); });
+        // single-query mode: every row of the Q tile is the one query; its column
+        // q_only goes through exactly the arithmetic of a whole-segment call
+        fetch_rows<DK, FA_TMAX>(vq, a.T, [&](int r) {
+            return a.q + (int64_t)h * DK + a.ldq * (b + (a.q_only >= 0 ? 0 : (int64_t)a.B * r));
+        });
         fetch_rows<DK, KR>(vw, has_w ? a.d_pos : 0, [&](int r) { return has_w ? a.w_r + ((int64_t)h * a.d_pos + r) * DK : a.q; });
         fetch_rows<DK, KR>(vk, a.K, kvrow);
         fetch_rows<DK, KR>(vv, a.K, [&](int r) { return kvrow(r) + (int64_t)a.H * DK; });
@@ -288,10 +292,11 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
 #pragma unroll
                 for (int dt = 0; dt < ND; dt++) acc[dt] = mfma16(vf[jt & 1][dt][r], sc[jt][r], acc[dt]);
         }
-        if (i < a.T) {
+        if (a.q_only >= 0 ? i == a.q_only : i < a.T) {
 #pragma unroll
             for (int dt = 0; dt < ND; dt++) {
-                float *o = a.out + (int64_t)h * DK + dt * 16 + 4 * g + a.ldo * (b + (int64_t)a.B * i);
+                float *o = a.out + (int64_t)h * DK + dt * 16 + 4 * g +
+                           a.ldo * (b + (a.q_only >= 0 ? 0 : (int64_t)a.B * i));
                 *reinterpret_cast<floatx4_t *>(o) = acc[dt];
             }
         }

@@ -662,7 +662,9 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
                 m, n, k, (long)lda, (long)ldb, (long)ldc);
         return -1;
     }
-    if (ksplit < 1) ksplit = 1;
+    const bool invariant = (precision & NCHIP_GEMM_WIDTH_INVARIANT) != 0;
+    precision &= 0xff;
+    if (ksplit < 1 || invariant) ksplit = 1;
     if (ksplit > 1 && !workspace) {
         fprintf(stderr, "nchip_gemm: ksplit=%d needs a workspace\n", ksplit);
         return -1;
@@ -697,7 +699,7 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     // workgroup (64x64x32, two k groups of 4 wavefronts); once
     // 128x64 tiles still give >= 256 workgroups, 8 wavefronts of 32x32 on a
     // 128x64x32 tile win; very large problems use 128x128x32 with 8 wavefronts.
-    int cfg = g_force_cfg; // tuning aid: 0 = choose from the shape
+    int cfg = invariant ? 8 : g_force_cfg; // tuning aid: 0 = choose from the shape
     int64_t nb = (int64_t)batch * ksplit;
     int64_t t128x64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64) * nb;
     if (!cfg) {

@@ -91,6 +91,7 @@ struct FusedAttnFwdArgs {
     int64_t ldq, ldkv, ldo;
     int H, B, T, M, K, d_pos, attn_len;
     float b_r_scale, scale;
+    int q_only; // >= 0: q and out are single (features, B) columns holding query position q_only
 };
 struct FusedAttnBwdArgs {
     const float *q, *kv, *kvm, *w_r, *probs, *dout;

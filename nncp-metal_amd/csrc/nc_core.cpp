@@ -102,6 +102,7 @@ extern "C" NCContext *nc_context_init(int nb_threads)
     m->dev_pool.device = true;
     m->host_pool.device = false;
     m->matmul_bf16 = 0;
+    m->matmul_invariant = 0;
     m->launches = 0;
     m->node_seq = 0;
     m->epoch = 0;
@@ -165,6 +166,13 @@ extern "C" void nc_synchronize(NCDevice *d)
 }
 
 extern "C" void nc_prof_dump(void) {}
+
+extern "C" int nc_set_matmul_width_invariant(NCContext *m, int enable) // nc_ext.h
+{
+    int old = m->matmul_invariant;
+    m->matmul_invariant = enable != 0;
+    return old;
+}
 
 extern "C" int nc_set_matmul_bf16(NCContext *m, int enable)
 {

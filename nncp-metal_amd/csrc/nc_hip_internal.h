@@ -72,6 +72,7 @@ struct NCContext {
     hipStream_t stream;
     Pool dev_pool, host_pool;
     int matmul_bf16;
+    int matmul_invariant; // forward products use the width-invariant GEMM class
     int64_t launches;
     int64_t node_seq;
     int epoch;

@@ -533,11 +533,15 @@ static MMShape mm_shape(const NCTensor *a, const NCTensor *b, bool ta, bool tb)
 
 // C (contiguous m x n per batch) = alpha op(A) op(B) + beta C [+ bias, act]
 // `addend` (laid out like C, or NULL) is added after the activation; beta must be 0 with it
+// forward: a product of the forward pass (honours nc_set_matmul_width_invariant)
 static void dev_gemm(NCContext *m, bool ta, bool tb, size_t M, size_t N, size_t K, float alpha,
                      const NCTensor *a, const NCTensor *b, float beta, NCTensor *c, size_t batch,
-                     const float *bias, int act, float *pre, const float *addend = nullptr)
+                     const float *bias, int act, float *pre, const float *addend = nullptr,
+                     bool forward = false)
 {
-    int ks = nchip_gemm_pick_ksplit((int)M, (int)N, (int)K, (int)batch);
+    const bool invariant = forward && m->matmul_invariant;
+    const int prec = m->matmul_bf16 | (invariant ? NCHIP_GEMM_WIDTH_INVARIANT : 0);
+    int ks = invariant ? 1 : nchip_gemm_pick_ksplit((int)M, (int)N, (int)K, (int)batch);
     size_t cap = 0;
     float *ws = nullptr;
     if (ks > 1) ws = nc_tmp_f32(m, batch * ks * M * N, &cap);
@@ -547,13 +551,13 @@ static void dev_gemm(NCContext *m, bool ta, bool tb, size_t M, size_t N, size_t 
                             nc_f32(a), (int64_t)(ta ? K : M), (int64_t)(M * K),
                             nc_f32(b), (int64_t)(tb ? N : K), (int64_t)(K * N),
                             nc_f32(c), (int64_t)M, (int64_t)(M * N), (int)batch,
-                            bias, act, pre, addend, m->matmul_bf16, ks, ws);
+                            bias, act, pre, addend, prec, ks, ws);
     else
         rc = nchip_gemm(m->stream, ta, tb, (int)M, (int)N, (int)K, alpha,
                         nc_f32(a), (int64_t)(ta ? K : M), (int64_t)(M * K),
                         nc_f32(b), (int64_t)(tb ? N : K), (int64_t)(K * N),
                         beta, nc_f32(c), (int64_t)M, (int64_t)(M * N), (int)batch,
-                        bias, act, pre, m->matmul_bf16, ks, ws);
+                        bias, act, pre, prec, ks, ws);
     if (ws) nc_tmp_free(m, ws, cap);
     if (rc) nc_fatal("gemm failed (m=%zu n=%zu k=%zu)", M, N, K);
     m->launches += ks > 1 ? 2 : 1;
@@ -578,7 +582,7 @@ extern "C" NCTensor *nc_matmul_add(NCTensor *a, NCTensor *b, NCTensor *c, BOOL t
     }
     // the addend is read in the GEMM epilogue: no copy, no second pass
     dev_gemm(m, ta != 0, tb != 0, s.m, s.n, s.k, alpha, a, b, 0.0f, y, s.batch, nullptr, 0, nullptr,
-             c ? nc_f32(c) : nullptr);
+             c ? nc_f32(c) : nullptr, true);
     NCTensor *args[3] = { a, b, c };
     NCNode *n = nc_new_node(m, OP_MATMUL, 3, args);
     if (a->node || b->node || (c && c->node)) {
@@ -698,7 +702,7 @@ static NCTensor *linear_impl(NCTensor *w, NCTensor *x, NCTensor *bias, int act, 
     bool graph = w->node || x->node || (bias && bias->node) || (res && res->node);
     NCTensor *pre = (act != NC_ACT_NONE && graph) ? nc_alloc_like(y) : nullptr;
     dev_gemm(m, false, false, s.m, s.n, s.k, 1.0f, w, x, 0.0f, y, 1, bias ? nc_f32(bias) : nullptr, act,
-             pre ? nc_f32(pre) : nullptr, res ? nc_f32(res) : nullptr);
+             pre ? nc_f32(pre) : nullptr, res ? nc_f32(res) : nullptr, true);
     NCTensor *args[4] = { w, x, bias, res };
     NCNode *n = nc_new_node(m, OP_LINEAR, 4, args);
     if (graph) {
@@ -902,6 +906,37 @@ extern "C" NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv
     n->fa[0] = b_r_scale;
     y = nc_finish(y, n, all, 5);
     nc_free_tensor(probs);
+    for (int i = 0; i < 5; i++) nc_free_tensor(all[i]);
+    return y;
+}
+
+// nc_ext.h: one query position against the segment's K/V cache; no graph
+extern "C" NCTensor *nc_relpos_attention_step(NCTensor *q, NCTensor *kv_cache, NCTensor *kv_mem,
+                                              NCTensor *w_r, NCTensor *b_r, int n_head, int d_key,
+                                              int attn_len, float b_r_scale, int t)
+{
+    NCTensor *all[5] = { q, kv_cache, kv_mem, w_r, b_r };
+    for (int i = 0; i < 5; i++)
+        if (all[i]) { all[i] = nc_contig(all[i]); need_f32(all[i], "nc_relpos_attention_step"); }
+    NCContext *m = nc_ctx(all[0]);
+    if (all[0]->n_dims != 2 || all[1]->n_dims != 3 || all[0]->dims[1] != all[1]->dims[1])
+        nc_fatal("nc_relpos_attention_step: q (H*dk, B) and kv_cache (H*dk+H*dv, B, T) expected");
+    const size_t B = all[1]->dims[1], T = all[1]->dims[2];
+    // the shape checks of the whole-segment op, on a view of q as one of T positions
+    size_t qd[3] = { all[0]->dims[0], B, T };
+    NCTensor qshape = *all[0];
+    qshape.n_dims = 3;
+    memcpy(qshape.dims, qd, sizeof(qd));
+    AttnDims a = attn_dims(&qshape, all[1], all[2], all[3], all[4], n_head, d_key);
+    size_t od[2] = { (size_t)a.H * a.dv, B };
+    NCTensor *y = new_f32(all[0], 2, od);
+    int rc = nchip_relpos_attn_fwd_step(m->stream, nc_f32(all[0]), (int64_t)all[0]->dims[0],
+                                        nc_f32(all[1]), all[2] ? nc_f32(all[2]) : nullptr, (int64_t)all[1]->dims[0],
+                                        all[3] ? nc_f32(all[3]) : nullptr, all[4] ? nc_f32(all[4]) : nullptr,
+                                        nc_f32(y), (int64_t)od[0], a.H, a.dk, a.dv, a.B, a.T, a.M, a.d_pos,
+                                        attn_len, b_r_scale, t);
+    if (rc) nc_fatal("nc_relpos_attention_step: kernel rejected the shapes");
+    m->launches++;
     for (int i = 0; i < 5; i++) nc_free_tensor(all[i]);
     return y;
 }

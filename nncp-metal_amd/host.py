@@ -11,7 +11,7 @@ from . import binding as B
 HERE = os.path.dirname(os.path.abspath(__file__))
 HOST_HIP_LIB = os.path.join(HERE, "host", "libnncp_host_hip.so")
 
-MODE_SEQ_EVAL, MODE_SEGMENT = 0, 1
+MODE_SEQ_EVAL, MODE_SEGMENT, MODE_STEP_DECODE = 0, 1, 4
 CODER_FLOAT, CODER_CDF16 = 0, 2
 LN_POST, LN_PRE, LN_FINAL, LN_COEF, LN_RMSNORM = 1, 2, 4, 8, 16
 FF_RELU, FF_GELU, FF_GEGLU, FF_GATED_SILU = 0, 1, 2, 3
@@ -115,6 +115,10 @@ class Host:
         L.trf_set_lr.argtypes = [_P, C.c_float]
         L.trf_last_logits.restype = _P
         L.trf_last_logits.argtypes = [_P]
+        L.trf_step_begin.argtypes = [_P]
+        L.trf_step_end.argtypes = [_P]
+        L.trf_eval_step.restype = _P
+        L.trf_eval_step.argtypes = [_P, C.c_int, _P]
         L.nncp_compress.restype = C.c_size_t
         L.nncp_compress.argtypes = [_P, _P, C.c_int, _P, C.c_size_t, C.c_int,
                                     C.POINTER(NNCPInterp), C.POINTER(NNCPStats)]
@@ -207,6 +211,23 @@ class Model:
 
     def logits(self):
         return self._to_numpy(self.L.trf_last_logits(self.ptr))
+
+    def eval_steps(self, tokens):
+        """Per-timestep cached evaluation of a whole segment (trf_step_begin +
+        trf_eval_step for every position).  Returns (probabilities (T, B, V),
+        logits (T, B, V)) assembled from the single-column results."""
+        tokens = np.asarray(tokens, dtype=np.int32)
+        inp = self._host_tensor(tokens)
+        self.L.trf_step_begin(self.ptr)
+        probs, logits = [], []
+        for t in range(tokens.shape[0]):
+            out = self.L.trf_eval_step(self.ptr, t, inp)
+            probs.append(self._to_numpy(out)[0])
+            logits.append(self.logits()[0])
+            self.nc.nc_free_tensor(out)
+        self.L.trf_step_end(self.ptr)
+        self.nc.nc_free_tensor(inp)
+        return np.stack(probs), np.stack(logits)
 
     def train_step(self, tokens, targets, lr):
         """One full-segment evaluation + gradient + update; returns

@@ -21,6 +21,12 @@
 #include <time.h>
 #include "../../include/nncp_host.h"
 
+static void die_stream(const char *msg)
+{
+    fprintf(stderr, "nncp_host: %s\n", msg);
+    abort();
+}
+
 static double now_s(void)
 {
     struct timespec ts;
@@ -55,7 +61,7 @@ typedef struct {
     NNCPPutBit *pb;
     NNCPGetBit *gb;
     BlockView view;
-    int is_decode, coder, n_symbols, B;
+    int is_decode, coder, n_symbols, B, step_decode;
     NNCPStats *st;
 } Coder;
 
@@ -133,6 +139,33 @@ static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int ful
         nc_free_tensor(d.host);
         return;
     }
+    if (mode == NNCP_MODE_SEGMENT && c->step_decode) {
+        /* decoder, one token column per timestep against the K/V caches */
+        trf_step_begin(s);
+        for (int t = 0; t < n_t; t++) {
+            for (int b = 0; b < B; b++)
+                nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
+            t0 = now_s();
+            NCTensor *out = trf_eval_step(s, t, input);
+            HostDist d = fetch_dist(c, out);
+            c->st->t_eval += now_s() - t0;
+            t0 = now_s();
+            for (int b = 0; b < B; b++)
+                if (symbol_is_coded(t, b, len2, c->view.rem, full)) {
+                    int sym = code_symbol(c, &d, (size_t)b, b, idx + t);
+                    if (expected) nc_set1_i32_2d(expected, b, t, sym);
+                }
+            c->st->t_code += now_s() - t0;
+            nc_free_tensor(d.host);
+        }
+        trf_step_end(s);
+        if (expected) { /* the graph the encoder differentiated: one whole-segment evaluation */
+            t0 = now_s();
+            nc_free_tensor(trf_eval(s, -1, input));
+            c->st->t_eval += now_s() - t0;
+        }
+        return;
+    }
     for (int t = 0; t < n_t; t++) {
         /* nncp.c:2996-3022 (and 3087-3114 for the tail) */
         for (int b = 0; b < B; b++)
@@ -171,6 +204,13 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
     memset(&c, 0, sizeof(c));
     c.s = s; c.pb = pb; c.gb = gb; c.is_decode = is_decode;
     c.coder = mode_flags & NNCP_CODER_CDF16;
+    if (mode_flags & NNCP_MODE_STEP_DECODE) {
+        if (mode != NNCP_MODE_SEGMENT)
+            die_stream("NNCP_MODE_STEP_DECODE goes with NNCP_MODE_SEGMENT");
+        /* both sides: products whose columns do not depend on how many are computed together */
+        nc_set_matmul_width_invariant(nncp_model_context(s), 1);
+        c.step_decode = is_decode;
+    }
     c.st = st ? st : &local;
 
     const NNCPConfig *cfg = nncp_model_config(s);

@@ -35,6 +35,7 @@ struct NNCPModel {
     Layer *layers;
     NCTensor *ln_g, *ln_b, *embed, *embed_out, *out_bias;
     NCTensor **mem_h, **train_h, **outputs;
+    NCTensor **step_kv, **step_kvm; /* per-timestep decoding: K/V of the segment so far, K/V of the memory */
     NCTensor *logits;
     NCSGDOptState *opt;
     int seq_eval;
@@ -177,6 +178,8 @@ void nncp_model_free(NNCPModel *s) /* trf_end nncp.c:522-550, nncp_end nncp.c:28
         nc_free_tensor(tl->mem_key); nc_free_tensor(tl->mem_value); nc_free_tensor(tl->attn_mask);
         nc_free(tl->key_nodes); nc_free(tl->kq_nodes); nc_free(tl->value_nodes); nc_free(tl->va_nodes);
     }
+    trf_step_end(s);
+    nc_free(s->step_kv); nc_free(s->step_kvm);
     nc_free(s->mem_h); nc_free(s->train_h); nc_free(s->outputs);
     nc_sgd_opt_set_all(&s->params, NULL);
     nc_sgd_opt_end(s->opt);
@@ -573,6 +576,108 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
 }
 
 NCTensor *trf_last_logits(NNCPModel *s) { return s->logits; }
+
+/* ---- per-timestep evaluation with K/V caches (the decoder's view, nncp.c:801-863,
+   through the fused entry points) ------------------------------------------------
+   trf_step_begin once per segment, then trf_eval_step(t) for t = 0, 1, ...: each
+   call evaluates ONE token column (the symbols of position t-1 of every stream)
+   against the memory and the columns seen so far.  With
+   nc_set_matmul_width_invariant() on in both the encoder and the decoder its
+   logits are bit-identical to column t of the whole-segment trf_eval. */
+void trf_step_end(NNCPModel *s)
+{
+    if (!s->step_kv) return;
+    for (int l = 0; l < s->cfg.n_layer; l++) {
+        nc_free_tensor(s->step_kv[l]); s->step_kv[l] = NULL;
+        nc_free_tensor(s->step_kvm[l]); s->step_kvm[l] = NULL;
+    }
+}
+
+void trf_step_begin(NNCPModel *s)
+{
+    const NNCPConfig *c = &s->cfg;
+    if (!c->fused)
+        die("per-timestep cached evaluation needs the fused path (cfg.fused = 1)");
+    if (!s->step_kv) {
+        s->step_kv = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
+        s->step_kvm = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
+    }
+    trf_step_end(s);
+    for (int l = 0; l < c->n_layer; l++) /* zero: columns not yet reached are masked but must be finite */
+        s->step_kv[l] = nc_new_tensor_3d(s->dev, NC_TYPE_F32, (size_t)c->n_head * (c->d_key + c->d_value),
+                                         c->batch_size, c->seg_len);
+}
+
+NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
+{
+    const NNCPConfig *c = &s->cfg;
+    int B = c->batch_size, H = c->n_head, HDk = H * c->d_key, HDv = H * c->d_value;
+    NCTensor *t0, *x;
+    if (!s->step_kv || !s->step_kv[0])
+        die("trf_eval_step: call trf_step_begin first");
+    if (t < 0 || t >= c->seg_len)
+        die("trf_eval_step: position outside the segment");
+    t0 = nc_slice_alias(input, 1, t, t + 1);
+    t0 = nc_tensor_to_device(t0, s->dev);
+    t0 = nc_reshape_1d(t0, (size_t)B);
+    x = nc_get_col(nc_dup_tensor(s->embed), t0);
+    x = nc_mul(x, scalar(s, s->embed_mult));
+    for (int l = 0; l < c->n_layer; l++) {
+        Layer *tl = &s->layers[l];
+        Layer *pr = &s->layers[c->tied_w_r ? 0 : l], *pb = &s->layers[c->tied_b_r ? 0 : l];
+        NCTensor *x1 = nc_dup_tensor(x), *ff_in, *q, *kv, *att;
+        if (c->ln_flags & NNCP_LN_PRE)
+            x1 = layer_norm(s, x1, tl->ln_g1, tl->ln_b1);
+        if (t == 0 && c->mem_len > 0) { /* K/V of the memory: once per segment */
+            NCTensor *m2 = nc_reshape_2d(nc_dup_tensor(s->mem_h[l]), c->d_model, (size_t)c->mem_len * B);
+            m2 = nc_matmul(nc_dup_tensor(tl->w_kv), m2);
+            s->step_kvm[l] = nc_reshape_3d(m2, HDk + HDv, B, c->mem_len);
+        }
+        q = nc_linear(nc_dup_tensor(tl->w_q), nc_dup_tensor(x1), c->query_bias ? nc_dup_tensor(tl->b_q) : NULL, NC_ACT_NONE);
+        kv = nc_matmul(nc_dup_tensor(tl->w_kv), x1);
+        kv = nc_reshape_3d(kv, HDk + HDv, B, 1);
+        nc_tensor_copy_slice(s->step_kv[l], kv, 2, t, t + 1, 0);
+        nc_free_tensor(kv);
+        att = nc_relpos_attention_step(q, nc_dup_tensor(s->step_kv[l]),
+                                       c->mem_len > 0 ? nc_dup_tensor(s->step_kvm[l]) : NULL,
+                                       c->use_w_r ? nc_dup_tensor(pr->w_r) : NULL, nc_dup_tensor(pb->b_r),
+                                       H, c->d_key, c->attn_len[l], sqrtf((float)(c->d_key * c->d_model)), t);
+        if (!tl->w_o)
+            die("the fused path needs d_value != d_model (an output projection)");
+        int fold = !(c->ln_flags & NNCP_LN_COEF);
+        int fold_ff = fold && (c->ff_act == NNCP_FF_GELU || c->ff_act == NNCP_FF_RELU);
+        if (fold) {
+            t0 = nc_matmul_add(nc_dup_tensor(tl->w_o), att, x, 0, 0, 1.0f);
+        } else {
+            t0 = nc_matmul_add(nc_dup_tensor(tl->w_o), att, NULL, 0, 0, 1.0f);
+            t0 = nc_mul(t0, nc_dup_tensor(tl->alpha));
+            t0 = nc_add(t0, x);
+        }
+        if (c->ln_flags & NNCP_LN_POST)
+            t0 = layer_norm(s, t0, tl->ln_g1, tl->ln_b1);
+        ff_in = nc_dup_tensor(t0);
+        if (c->ln_flags & NNCP_LN_PRE)
+            t0 = layer_norm(s, t0, tl->ln_g2, tl->ln_b2);
+        if (fold_ff) {
+            t0 = feed_forward(s, l, t0, ff_in);
+        } else {
+            t0 = feed_forward(s, l, t0, NULL);
+            if (c->ln_flags & NNCP_LN_COEF)
+                t0 = nc_mul(t0, nc_dup_tensor(tl->alpha));
+            t0 = nc_add(t0, ff_in);
+        }
+        if (c->ln_flags & NNCP_LN_POST)
+            t0 = layer_norm(s, t0, tl->ln_g2, tl->ln_b2);
+        x = t0;
+    }
+    if (c->ln_flags & NNCP_LN_FINAL)
+        x = layer_norm(s, x, s->ln_g, s->ln_b);
+    t0 = nc_linear(nc_dup_tensor(s->embed_out), x, s->out_bias ? nc_dup_tensor(s->out_bias) : NULL, NC_ACT_NONE);
+    t0 = nc_reshape_3d(t0, c->n_symbols, B, 1);
+    nc_free_tensor(s->logits);
+    s->logits = nc_dup_tensor(t0);
+    return nc_soft_max(t0);
+}
 
 void trf_eval_end(NNCPModel *s) /* nncp.c:1032-1060 */
 {

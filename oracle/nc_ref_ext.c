@@ -150,6 +150,30 @@ NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv_mem,
     return y;
 }
 
+/* one query position: the whole-segment routine on a query tensor that holds
+   the query in column t, then that column of the result (see nc_ext.h) */
+NCTensor *nc_relpos_attention_step(NCTensor *q, NCTensor *kv_cache, NCTensor *kv_mem,
+                                   NCTensor *w_r, NCTensor *b_r, int n_head, int d_key,
+                                   int attn_len, float b_r_scale, int t)
+{
+    size_t dims[3], B, T;
+    NCTensor *qf, *y;
+    q = nc_contig(q);
+    if (q->n_dims != 2 || kv_cache->n_dims != 3)
+        nc_fatal("relpos_attention_step: q (H*dk, B) and kv_cache (.., B, T) expected");
+    B = kv_cache->dims[1]; T = kv_cache->dims[2];
+    if (q->dims[1] != B || t < 0 || (size_t)t >= T)
+        nc_fatal("relpos_attention_step: stream count or position out of range");
+    dims[0] = q->dims[0]; dims[1] = B; dims[2] = T;
+    qf = nc_alloc(q->dev, NC_TYPE_F32, 3, dims, 1);
+    memcpy(nc_f32(qf) + (size_t)t * dims[0] * B, nc_f32(q), sizeof(float) * dims[0] * B);
+    nc_free_tensor(q);
+    y = nc_relpos_attention(qf, kv_cache, kv_mem, w_r, b_r, n_head, d_key, attn_len, b_r_scale);
+    y = nc_contig(nc_slice(y, 2, t, t + 1));
+    return nc_reshape_2d(y, y->dims[0], B);
+}
+
+
 /* gradients exactly as the chain rule gives them for the formula above:
    dA[j] = v_j.do ; dS[j] = A[j](dA[j] - sum_j A dA) * scale ;
    dq += (k_j + w_r[pi]) dS[j] ; dk_j += q dS[j] ; dw_r[pi] += q dS[j] ;

@@ -178,3 +178,54 @@ def test_profile_variants_match_checker(hosts, name, fused):
         assert M.tensors_close(w_h[k], w_r[k], 1e-5), (name, k, M.rel_l2(w_h[k], w_r[k]))
     hip.close()
     ref.close()
+
+
+@pytest.mark.parametrize("cfg_name,bf16", [("SMALL32", 0), ("C1", 0), ("C1", 1), ("C3S", 0)])
+def test_cached_timestep_logits_are_bit_identical(hosts, cfg_name, bf16):
+    """With width-invariant products, the decoder's one-column evaluations
+    (trf_eval_step) give exactly the logits of the encoder's whole-segment
+    evaluation: what lets a per-timestep decoder follow a whole-segment encoder."""
+    pkg = M.load_pkg()
+    cfg = dict(C3S=dict(n_layer=2, d_model=512, n_head=8, d_inner=2048, d_pos=128, mem_len=64, seg_len=64,
+                        batch_size=8, n_symbols=256, seed=5),
+               # heads of 32 (the cached step needs the single-kernel attention shapes), ragged sizes
+               SMALL32=dict(n_layer=2, d_model=64, n_head=2, d_inner=96, d_pos=13, mem_len=7, seg_len=9,
+                            batch_size=3, n_symbols=40, seed=7),
+               C1=M.C1)[cfg_name]
+    m = pkg.host.Model(hosts[0], pkg.host.make_config(**dict(cfg, use_device=1, fused=1, sgd_opt=M.rmsprop(3e-4))))
+    m.nc.nc_set_matmul_bf16(m.ctx, bf16)
+    m.nc.nc_set_matmul_width_invariant(m.ctx, 1)
+    B, T, V = cfg["batch_size"], cfg["seg_len"], cfg["n_symbols"]
+    syms = M.markov1(B * T * 2, V, seed=31)
+    (tok0, tgt0), (tok1, _) = M.segment_batches(syms, B, T, 2)
+    m.train_step(tok0, tgt0, 3e-4)  # non-trivial weights and a filled memory
+    m.eval(tok1, keep=True)
+    full = m.logits()
+    m.L.trf_eval_end(m.ptr)
+    _, step = m.eval_steps(tok1)
+    m.close()
+    assert step.shape == full.shape
+    assert np.array_equal(step, full)
+
+
+@pytest.mark.parametrize("coder", [0, 2])
+def test_step_decode_round_trip_on_gpu(hosts, coder):
+    """C1 shape, 8 KiB: whole-segment encoder, per-timestep cached decoder."""
+    pkg = M.load_pkg()
+    mode = 1 | 4 | coder
+    n = 4 * 20 * 12 + 7
+    syms = M.markov1(n, 256, seed=99)
+    cfg = dict(M.C1, fused=1, sgd_opt=M.rmsprop(3e-4), use_device=1)
+    enc = pkg.host.Model(hosts[0], pkg.host.make_config(**cfg))
+    data, st = enc.compress(syms, mode)
+    enc.close()
+    dec = pkg.host.Model(hosts[0], pkg.host.make_config(**cfg))
+    back, _ = dec.decompress(data, n, mode)
+    dec.close()
+    assert np.array_equal(back, syms)
+    # the plain replaying decoder reads the same stream
+    dec2 = pkg.host.Model(hosts[0], pkg.host.make_config(**cfg))
+    dec2.nc.nc_set_matmul_width_invariant(dec2.ctx, 1)
+    back2, _ = dec2.decompress(data, n, 1 | coder)
+    dec2.close()
+    assert np.array_equal(back2, syms)

@@ -122,3 +122,38 @@ def test_probabilities_are_causal(H):
         p2 = m.eval(tok2)
         assert np.array_equal(p_full[:t + 1], p2[:t + 1])
     m.close()
+
+
+def test_cached_timestep_evaluation_matches_segment(H):
+    """trf_eval_step (K/V caches, fused entry points) reproduces the columns of
+    the whole-segment evaluation, with a non-empty memory (second segment)."""
+    syms = M.markov1(3 * 8 * 2, 40, seed=21)
+    (tok0, tgt0), (tok1, _) = M.segment_batches(syms, 3, 8, 2)
+    m = _model(H, fused=1, sgd_opt=M.rmsprop(3e-4))
+    m.train_step(tok0, tgt0, 3e-4)  # fills the memory
+    full = m.eval(tok1)
+    full_logits = None
+    step_p, step_l = m.eval_steps(tok1)
+    m.eval(tok1, keep=True)
+    full_logits = m.logits()
+    m.L.trf_eval_end(m.ptr)
+    m.close()
+    assert step_p.shape == full.shape
+    assert M.relerr(step_p, full) <= 1e-6
+    assert M.relerr(step_l, full_logits) <= 1e-6
+
+
+@pytest.mark.parametrize("n", [3 * 8 * 4 + 17, 11])
+@pytest.mark.parametrize("coder", [0, 2])
+def test_step_decode_round_trip(H, n, coder):
+    """Whole-segment encoder, per-timestep cached decoder (NNCP_MODE_STEP_DECODE)."""
+    mode = 1 | 4 | coder
+    syms = M.markov1(n, 40, seed=n + 1)
+    enc = _model(H, fused=1)
+    data, st = enc.compress(syms, mode)
+    enc.close()
+    dec = _model(H, fused=1)
+    out, _ = dec.decompress(data, n, mode)
+    dec.close()
+    assert np.array_equal(out, syms)
+    assert st.n_symbols == n
