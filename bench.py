@@ -193,6 +193,72 @@ def attention_c2(pkg, iters=50):
             "binding_bound": "mfma (39 flop/B > fp32 ridge 20)"}
 
 
+def cdf_c5(pkg, iters=50):
+    """Coder-side probability path at BASELINE configs[4]: fp32 logits for 64
+    streams x 16384 symbols (N(0, 3) plus a Zipf-shaped per-token bias
+    -log(rank) under a seeded rank permutation) -> 16-bit integer CDF, then
+    10^6 uniform 16-bit targets per stream -> symbol index by
+    cumulative-frequency search.  Raw kernel entry points on the null stream,
+    HIP event pair around `iters` launches.  Algorithmic bytes: CDF build
+    4 MiB read + 2 MiB written; lookup 2 B target + 2 B symbol each."""
+    nc = pkg.binding.NC(pkg.binding.HIP_LIB)
+    lib = C.CDLL(pkg.binding.HIP_LIB)
+    hip = C.CDLL("libamdhip64.so")
+    V, n, m = 16384, 64, 1000000
+    rng = np.random.default_rng(5)
+    bias = -np.log(rng.permutation(V) + 1.0)
+    logits = (rng.normal(0, 3, (n, V)) + bias).astype(np.float32)
+    targets = rng.integers(0, 65536, size=(n, m)).astype(np.uint16)
+    d_log, d_t = nc.tensor(logits), nc.tensor(targets)
+    d_cdf = nc.tensor(np.zeros((n, V), np.uint16))
+    d_sym = nc.tensor(np.zeros((n, m), np.uint16))
+    P = [C.c_void_p(nc.lib.nc_tensor_get_ptr(t, None)) for t in (d_log, d_cdf, d_t, d_sym)]
+    i64, i32 = C.c_int64, C.c_int
+
+    def build():
+        return lib.nchip_softmax_cdf16(None, P[0], P[1], i32(V), i64(n))
+
+    def lookup():
+        return lib.nchip_cdf_lookup(None, P[1], P[2], P[3], i32(V), i64(m), i64(n))
+
+    def timed(f, k):
+        e0, e1 = C.c_void_p(), C.c_void_p()
+        hip.hipEventCreate(C.byref(e0))
+        hip.hipEventCreate(C.byref(e1))
+        assert f() == 0
+        hip.hipDeviceSynchronize()
+        hip.hipEventRecord(e0, None)
+        for _ in range(k):
+            f()
+        hip.hipEventRecord(e1, None)
+        hip.hipEventSynchronize(e1)
+        ms = C.c_float()
+        hip.hipEventElapsedTime(C.byref(ms), e0, e1)
+        hip.hipEventDestroy(e0)
+        hip.hipEventDestroy(e1)
+        return ms.value * 1e3 / k
+
+    us_b, us_l = timed(build, iters), timed(lookup, max(1, iters // 5))
+    # the CDF is a function of integers only past the exponential: check it
+    cdf = nc.numpy(d_cdf).astype(np.int64)
+    freq = np.diff(np.concatenate([cdf, np.full((n, 1), 65536)], axis=1), axis=1)
+    sym = nc.numpy(d_sym).astype(np.int64)
+    rows = np.arange(n)[:, None]
+    t64 = targets.astype(np.int64)
+    hi = np.where(sym + 1 < V, np.take_along_axis(cdf, np.minimum(sym + 1, V - 1), axis=1), 65536)
+    ok = bool((cdf[:, 0] == 0).all() and (freq >= 1).all() and (freq.sum(axis=1) == 65536).all()
+              and (cdf[rows, sym] <= t64).all() and (t64 < hi).all())
+    for t in (d_log, d_t, d_cdf, d_sym):
+        nc.free(t)
+    nc.close()
+    b_bytes, l_bytes = n * V * 6, n * m * 4
+    return {"workload": "BASELINE configs[4]: 64 streams x V16384 logits -> cdf16; 1e6 lookups per stream",
+            "us_cdf_build": round(us_b, 2), "cdf_build_GBps": round(b_bytes / us_b / 1e3, 1),
+            "us_lookup": round(us_l, 2), "lookups_per_s": round(n * m / us_l * 1e6, 0),
+            "lookup_GBps": round(l_bytes / us_l / 1e3, 1), "lookup_hbm_frac": round(l_bytes / us_l / 1e3 / 8000, 4),
+            "invariants_ok": ok}
+
+
 def cpu_baseline(pkg, data, n_steps, threads):
     """The CPU checker driving the reference op sequence (whole-segment
     evaluation, float symbol coder: what `nncp --encode_only` does) on the
@@ -218,6 +284,7 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=2, help="0 skips the CPU baseline")
     ap.add_argument("--profile-steps", type=int, default=2)
     ap.add_argument("--attention-iters", type=int, default=50, help="0 skips the isolated attention timing")
+    ap.add_argument("--cdf-iters", type=int, default=50, help="0 skips the coder-side CDF timing")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="first issue one device-to-device copy of this many MiB (a kernel of known "
                          "traffic, to scale FETCH_SIZE / WRITE_SIZE readings of a counter run)")
@@ -285,6 +352,7 @@ def main():
                     "all_gemm_ms_per_step": round(tot_s / args.profile_steps * 1e3, 3)}
     model.close()
     attn = attention_c2(pkg, args.attention_iters) if args.attention_iters else None
+    cdf = cdf_c5(pkg, args.cdf_iters) if args.cdf_iters else None
 
     cpu = None
     if args.cpu_steps:
@@ -309,7 +377,7 @@ def main():
         "kernel_launches_per_step": launches / args.steps,
         "host_seconds": {"eval_and_copy": round(st.t_eval, 4), "code": round(st.t_code, 4),
                          "grad": round(st.t_grad, 4), "update": round(st.t_update, 4)},
-        "roofline": roof, "attention": attn, "cpu_baseline": cpu}))
+        "roofline": roof, "attention": attn, "cdf": cdf, "cpu_baseline": cpu}))
 
 
 if __name__ == "__main__":

@@ -41,72 +41,321 @@ __device__ __forceinline__ unsigned int quant(float x, float mx)
     return (unsigned int)(exp_det(d) * 16777216.0f);
 }
 
-// one block per column; thread t owns the contiguous chunk [t*per, (t+1)*per)
-__global__ __launch_bounds__(TPB) void softmax_cdf16_kernel(const float *logits, uint16_t *cdf, int v)
+// floor(num / den) for num < 2^56, den < 2^41 and a quotient below 2^16: a
+// double-precision estimate (relative error < 2^-50, so at most one off after
+// truncation) corrected by the exact 64-bit remainder.
+__device__ __forceinline__ unsigned int div_floor(unsigned long long num, unsigned long long den, double inv)
 {
-    __shared__ float smax[TPB];
-    __shared__ unsigned long long ssum[TPB];
+    double d = fma((double)(unsigned int)(num >> 32), 4294967296.0, (double)(unsigned int)num);
+    unsigned int q = (unsigned int)(d * inv);
+    long long r = (long long)num - (long long)((unsigned long long)q * den);
+    if (r < 0) q--;
+    else if (r >= (long long)den) q++;
+    return q;
+}
+
+__device__ __forceinline__ unsigned long long wave_scan_incl(unsigned long long v, int lane)
+{
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        unsigned long long o = __shfl_up(v, d, 64);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+
+// One workgroup of NT threads per column (NT == 64: one wave per column, four
+// columns per workgroup).  The column is cut into chunks of 4*NT elements; in
+// a chunk thread t owns the 4 consecutive elements starting at 4*t, so the
+// loads and the uint16 stores of a wave cover one contiguous span, the logits
+// are read once and stay in registers, and the exclusive prefix of an element
+// is (chunks before) + (waves before, via LDS) + (lanes before, via shuffles)
+// + (own earlier elements).  All sums are integers, so their grouping does
+// not change the result.
+template <int NT, int NC, bool KEEP>
+__global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(const float *logits, uint16_t *cdf,
+                                                                        int v, int64_t ncol, int vec)
+{
+    constexpr int NW = NT / 64;
+    constexpr int UNR = KEEP ? NC : 1; // chunk loops stay rolled when chunks are re-read
+    __shared__ float smax[NW];
+    __shared__ unsigned long long swave[NC][NW];
     __shared__ unsigned long long stot;
-    const float *x = logits + (int64_t)blockIdx.x * v;
-    uint16_t *out = cdf + (int64_t)blockIdx.x * v;
-    int t = threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = NT == 64 ? 0 : (int)threadIdx.x >> 6;
+    const int t = NT == 64 ? lane : (int)threadIdx.x;
+    const int64_t col = NT == 64 ? (int64_t)blockIdx.x * 4 + ((int)threadIdx.x >> 6) : (int64_t)blockIdx.x;
+    if (NT == 64 && col >= ncol) return; // whole wave; this shape uses no workgroup barrier
+    const float *x = logits + col * v;
+    uint16_t *out = cdf + col * v;
 
-    float mx = -INFINITY;
-    for (int i = t; i < v; i += TPB) mx = fmaxf(mx, x[i]);
-    smax[t] = mx;
-    __syncthreads();
-    for (int s = TPB / 2; s > 0; s >>= 1) {
-        if (t < s) smax[t] = fmaxf(smax[t], smax[t + s]);
-        __syncthreads();
-    }
-    mx = smax[0];
-
-    int per = (v + TPB - 1) / TPB;
-    int i0 = t * per, i1 = min(v, i0 + per);
-    unsigned long long local = 0;
-    for (int i = i0; i < i1; i++) local += quant(x[i], mx);
-    ssum[t] = local;
-    __syncthreads();
-    // exclusive scan of the 256 chunk totals (integers: order is irrelevant)
-    if (t == 0) {
-        unsigned long long run = 0;
-        for (int k = 0; k < TPB; k++) {
-            unsigned long long c = ssum[k];
-            ssum[k] = run;
-            run += c;
+    // KEEP: the logits stay in registers from the first read on; otherwise
+    // (columns too long for that) each pass reads its chunk again, from L2
+    float xv[KEEP ? NC : 1][4];
+    auto fetch = [&](int c, float (&f)[4]) {
+        int i0 = (c * NT + t) * 4;
+        if (vec && i0 < v) {
+            float4 g = *reinterpret_cast<const float4 *>(x + i0);
+            f[0] = g.x; f[1] = g.y; f[2] = g.z; f[3] = g.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) f[j] = i0 + j < v ? x[i0 + j] : -INFINITY;
         }
-        stot = run;
+    };
+    auto chunk = [&](int c, float (&f)[4]) {
+        if (KEEP) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) f[j] = xv[c][j];
+        } else {
+            fetch(c, f);
+        }
+    };
+    float mx = -INFINITY;
+#pragma unroll UNR
+    for (int c = 0; c < NC; c++) {
+        float f[4];
+        fetch(c, f);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (KEEP) xv[c][j] = f[j];
+            mx = fmaxf(mx, f[j]);
+        }
     }
-    __syncthreads();
-    unsigned long long tot = stot, run = ssum[t];
-    unsigned long long scale = (unsigned long long)(65536 - v);
-    for (int i = i0; i < i1; i++) {
-        out[i] = (uint16_t)(run * scale / tot + (unsigned long long)i);
-        run += quant(x[i], mx);
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+    if (NT > 64) {
+        if (lane == 0) smax[wave] = mx;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < NW; w++) mx = fmaxf(mx, smax[w]);
+    }
+
+    // pass 1: totals per (chunk, wave); the wave-level scan is redone in
+    // pass 2 rather than kept, which holds the register count down
+    unsigned long long wave_tot[NT == 64 ? NC : 1];
+#pragma unroll UNR
+    for (int c = 0; c < NC; c++) {
+        int i0 = (c * NT + t) * 4;
+        unsigned long long s = 0;
+        float f[4];
+        chunk(c, f);
+#pragma unroll
+        for (int j = 0; j < 4; j++) s += i0 + j < v ? quant(f[j], mx) : 0u;
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) s += __shfl_xor(s, d, 64);
+        if (NT == 64) wave_tot[c] = s;
+        if (NT > 64 && lane == 0) swave[c][wave] = s;
+    }
+    unsigned long long tot = 0;
+    if (NT > 64) {
+        __syncthreads();
+        // wave 0 turns the wave totals of each chunk into exclusive prefixes
+        // that run on through the chunks; the grand total goes to stot
+        if (wave == 0) {
+            unsigned long long run = 0;
+#pragma unroll 1
+            for (int c = 0; c < NC; c++) {
+                unsigned long long w = lane < NW ? swave[c][lane] : 0ull;
+                unsigned long long incl = wave_scan_incl(w, lane);
+                if (lane < NW) swave[c][lane] = run + incl - w;
+                run += __shfl(incl, 63, 64);
+            }
+            if (lane == 0) stot = run;
+        }
+        __syncthreads();
+        tot = stot;
+    } else {
+#pragma unroll
+        for (int c = 0; c < NC; c++) tot += wave_tot[c];
+    }
+    const unsigned long long scale = (unsigned long long)(65536 - v);
+    const double inv = 1.0 / (double)tot;
+    unsigned long long chunk_base = 0;
+#pragma unroll UNR
+    for (int c = 0; c < NC; c++) {
+        int i0 = (c * NT + t) * 4;
+        unsigned int q[4];
+        unsigned long long s = 0;
+        float f[4];
+        chunk(c, f);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            q[j] = i0 + j < v ? quant(f[j], mx) : 0u;
+            s += q[j];
+        }
+        unsigned long long run = wave_scan_incl(s, lane) - s;
+        if (NT > 64) {
+            run += swave[c][wave];
+        } else {
+            run += chunk_base;
+            chunk_base += wave_tot[c];
+        }
+        if (i0 >= v) continue;
+        unsigned int o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            o[j] = div_floor(run * scale, tot, inv) + (unsigned int)(i0 + j);
+            run += q[j];
+        }
+        if (vec) {
+            uint2 pk;
+            pk.x = (o[0] & 0xffffu) | (o[1] << 16);
+            pk.y = (o[2] & 0xffffu) | (o[3] << 16);
+            *reinterpret_cast<uint2 *>(out + i0) = pk;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (i0 + j < v) out[i0 + j] = (uint16_t)o[j];
+        }
     }
 }
 
+// Cumulative-frequency search: sym = the index with cdf[sym] <= target <
+// cdf[sym + 1] (cdf[v] = 65536).  The column's CDF is staged in LDS when it
+// fits; each thread then runs four searches side by side, with a fixed trip
+// count of ceil(log2 v) and selects instead of branches, so four LDS reads
+// are in flight per lane (once hi - lo is 1 a further step changes nothing).
+template <bool LDS>
 __global__ __launch_bounds__(TPB) void cdf_lookup_kernel(const uint16_t *cdf, const uint16_t *target,
-                                                         uint16_t *sym, int v, int64_t m, int use_lds)
+                                                         uint16_t *sym, int v, int64_t m, int steps)
 {
-    __shared__ uint16_t sc[16384];
+    __shared__ uint16_t sc[LDS ? 16384 : 1];
     const uint16_t *c = cdf + (int64_t)blockIdx.y * v;
-    if (use_lds) {
+    if (LDS) {
         for (int i = threadIdx.x; i < v; i += TPB) sc[i] = c[i];
         __syncthreads();
     }
     const uint16_t *tp = target + (int64_t)blockIdx.y * m;
     uint16_t *sp = sym + (int64_t)blockIdx.y * m;
-    for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < m; i += (int64_t)gridDim.x * TPB) {
-        unsigned int tv = tp[i];
-        int lo = 0, hi = v; // cdf[lo] <= tv < cdf[hi], with cdf[v] = 65536
-        while (hi - lo > 1) {
-            int mid = (lo + hi) >> 1;
-            unsigned int cv = use_lds ? sc[mid] : c[mid];
-            if (cv <= tv) lo = mid; else hi = mid;
+    const int64_t stride = (int64_t)gridDim.x * TPB;
+    for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < m; i += 4 * stride) {
+        unsigned int tv[4];
+        int lo[4], hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int64_t ij = i + j * stride;
+            tv[j] = tp[ij < m ? ij : i];
+            lo[j] = 0;
+            hi[j] = v;
         }
-        sp[i] = (uint16_t)lo;
+        for (int s = 0; s < steps; s++) {
+            unsigned int cv[4];
+            int mid[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                mid[j] = (lo[j] + hi[j]) >> 1;
+                cv[j] = LDS ? sc[mid[j]] : c[mid[j]];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                bool le = cv[j] <= tv[j];
+                lo[j] = le ? mid[j] : lo[j];
+                hi[j] = le ? hi[j] : mid[j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int64_t ij = i + j * stride;
+            if (ij < m) sp[ij] = (uint16_t)lo[j];
+        }
     }
+}
+
+// Many targets per column: first turn the column's CDF into the full inverse
+// table inv[t] = symbol of target value t (65536 uint16 entries, 128 KiB of
+// LDS; each entry by the same search, read from the cached CDF), after which
+// a lookup is one LDS read.  Entry t depends on the CDF alone, so the result
+// is the one the search gives.
+constexpr int INV_NT = 1024;
+__global__ __launch_bounds__(INV_NT) void cdf_lookup_table_kernel(const uint16_t *cdf, const uint16_t *target,
+                                                                  uint16_t *sym, int v, int64_t m, int steps,
+                                                                  int vec)
+{
+    extern __shared__ __attribute__((aligned(16))) uint16_t inv[];
+    __shared__ uint16_t coarse[INV_NT + 1];
+    const uint16_t *c = cdf + (int64_t)blockIdx.y * v;
+    {   // the symbol of every 64th target value, by the full search
+        int lo = 0, hi = v;
+        unsigned int tv = threadIdx.x * 64;
+        for (int s = 0; s < steps; s++) {
+            int mid = (lo + hi) >> 1;
+            bool le = c[mid] <= tv;
+            lo = le ? mid : lo;
+            hi = le ? hi : mid;
+        }
+        coarse[threadIdx.x] = (uint16_t)lo;
+        if (threadIdx.x == 0) coarse[INV_NT] = (uint16_t)(v - 1);
+    }
+    __syncthreads();
+    // the symbols of target values 64 b .. 64 b + 63 lie between coarse[b] and
+    // coarse[b + 1], at most 65 candidates (every symbol has frequency >= 1):
+    // 7 halvings finish each of them; eight run side by side
+    for (int t0 = threadIdx.x; t0 < 65536; t0 += 8 * INV_NT) {
+        int lo[8], hi[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            int bkt = (t0 + j * INV_NT) >> 6;
+            lo[j] = coarse[bkt];
+            hi[j] = coarse[bkt + 1] + 1;
+        }
+#pragma unroll
+        for (int s = 0; s < 7; s++) {
+            unsigned int cv[8];
+            int mid[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                mid[j] = (lo[j] + hi[j]) >> 1;
+                cv[j] = c[mid[j]];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                bool le = cv[j] <= (unsigned int)(t0 + j * INV_NT);
+                lo[j] = le ? mid[j] : lo[j];
+                hi[j] = le ? hi[j] : mid[j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) inv[t0 + j * INV_NT] = (uint16_t)lo[j];
+    }
+    __syncthreads();
+    const uint16_t *tp = target + (int64_t)blockIdx.y * m;
+    uint16_t *sp = sym + (int64_t)blockIdx.y * m;
+    // this workgroup's share of the column, cut at multiples of 4 targets
+    int64_t quads = (m + 3) >> 2;
+    int64_t per = (quads + gridDim.x - 1) / gridDim.x;
+    int64_t q0 = per * blockIdx.x, q1 = q0 + per < quads ? q0 + per : quads;
+    if (vec) {
+        // four 8-byte loads in flight per lane (index clamped, store guarded)
+        for (int64_t q = q0 + threadIdx.x; q < q1; q += 4 * INV_NT) {
+            uint2 tv[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                int64_t qj = q + j * INV_NT;
+                tv[j] = *reinterpret_cast<const uint2 *>(tp + 4 * (qj < q1 ? qj : q));
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                int64_t qj = q + j * INV_NT;
+                uint2 r;
+                r.x = (unsigned int)inv[tv[j].x & 0xffffu] | ((unsigned int)inv[tv[j].x >> 16] << 16);
+                r.y = (unsigned int)inv[tv[j].y & 0xffffu] | ((unsigned int)inv[tv[j].y >> 16] << 16);
+                if (qj < q1) *reinterpret_cast<uint2 *>(sp + 4 * qj) = r;
+            }
+        }
+    } else {
+        int64_t i1 = 4 * q1 < m ? 4 * q1 : m;
+        for (int64_t i = 4 * q0 + threadIdx.x; i < i1; i += INV_NT) sp[i] = inv[tp[i]];
+    }
+}
+
+bool allow_table_lds()
+{
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(cdf_lookup_table_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 65536 * 2) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return true;
 }
 
 } // namespace
@@ -115,7 +364,19 @@ extern "C" int nchip_softmax_cdf16(void *stream, const float *logits, uint16_t *
 {
     if (n <= 0) return 0;
     if (v < 1 || v > 65535) { fprintf(stderr, "nchip_softmax_cdf16: vocabulary %d outside [1, 65535]\n", v); return -1; }
-    hipLaunchKernelGGL(softmax_cdf16_kernel, dim3((unsigned)n), dim3(TPB), 0, (hipStream_t)stream, logits, cdf, v);
+    hipStream_t st = (hipStream_t)stream;
+    // 16-byte loads and 8-byte stores need every column to start aligned
+    int vec = (v & 3) == 0 && ((uintptr_t)logits & 15) == 0 && ((uintptr_t)cdf & 7) == 0;
+    if (v <= 256)
+        hipLaunchKernelGGL((softmax_cdf16_kernel<64, 1, true>), dim3((unsigned)((n + 3) / 4)), dim3(256), 0, st, logits, cdf, v, n, vec);
+    else if (v <= 1024)
+        hipLaunchKernelGGL((softmax_cdf16_kernel<256, 1, true>), dim3((unsigned)n), dim3(256), 0, st, logits, cdf, v, n, vec);
+    else if (v <= 4096)
+        hipLaunchKernelGGL((softmax_cdf16_kernel<256, 4, true>), dim3((unsigned)n), dim3(256), 0, st, logits, cdf, v, n, vec);
+    else if (v <= 16384)
+        hipLaunchKernelGGL((softmax_cdf16_kernel<1024, 4, true>), dim3((unsigned)n), dim3(1024), 0, st, logits, cdf, v, n, vec);
+    else
+        hipLaunchKernelGGL((softmax_cdf16_kernel<1024, 16, false>), dim3((unsigned)n), dim3(1024), 0, st, logits, cdf, v, n, vec);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { fprintf(stderr, "nchip_softmax_cdf16: %s\n", hipGetErrorString(e)); return -2; }
     return 0;
@@ -126,10 +387,31 @@ extern "C" int nchip_cdf_lookup(void *stream, const uint16_t *cdf, const uint16_
 {
     if (n <= 0 || m <= 0) return 0;
     if (n > 65535) { fprintf(stderr, "nchip_cdf_lookup: too many columns\n"); return -1; }
-    int64_t bx = (m + TPB * 4 - 1) / (TPB * 4);
-    if (bx > 1024) bx = 1024;
-    hipLaunchKernelGGL(cdf_lookup_kernel, dim3((unsigned)bx, (unsigned)n), dim3(TPB), 0, (hipStream_t)stream,
-                       cdf, target, sym, v, m, v <= 16384 ? 1 : 0);
+    // every workgroup of a column stages that column's CDF in LDS first, so
+    // use only as many per column as fill the chip a few times over
+    int steps = 0;
+    while ((1 << steps) < v) steps++;
+    int64_t bx = (m + TPB * 16 - 1) / (TPB * 16);
+    int64_t cap = (4096 + n - 1) / n;
+    if (bx > cap) bx = cap;
+    // the table costs 65536 searches per workgroup: worth it from a few times
+    // that many targets per workgroup on
+    static const bool table_ok = allow_table_lds();
+    if (table_ok && m >= 4 * 65536) {
+        int64_t split = (256 + n - 1) / n; // workgroups per column: one per CU (the table fills its LDS)
+        if (split > m / (2 * 65536)) split = m / (2 * 65536);
+        if (split < 1) split = 1;
+        // 8-byte accesses need every column (m targets apart) to start aligned
+        int vec = (m & 3) == 0 && ((uintptr_t)target & 7) == 0 && ((uintptr_t)sym & 7) == 0;
+        hipLaunchKernelGGL(cdf_lookup_table_kernel, dim3((unsigned)split, (unsigned)n), dim3(INV_NT), 65536 * 2,
+                           (hipStream_t)stream, cdf, target, sym, v, m, steps, vec);
+    } else {
+        dim3 grid((unsigned)bx, (unsigned)n);
+        if (v <= 16384)
+            hipLaunchKernelGGL(cdf_lookup_kernel<true>, grid, dim3(TPB), 0, (hipStream_t)stream, cdf, target, sym, v, m, steps);
+        else
+            hipLaunchKernelGGL(cdf_lookup_kernel<false>, grid, dim3(TPB), 0, (hipStream_t)stream, cdf, target, sym, v, m, steps);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { fprintf(stderr, "nchip_cdf_lookup: %s\n", hipGetErrorString(e)); return -2; }
     return 0;

@@ -130,10 +130,15 @@ def test_cdf16_bit_exact(hip, ref, rng, V, n):
     assert (freq >= 1).all() and (freq.sum(axis=1) == 65536).all()
 
 
-def test_cdf_lookup_bit_exact(hip, ref, rng):
-    V, n, m = 16384, 4, 50000
+# m >= 262144 targets per column takes the inverse-table kernel (vector path
+# when m is a multiple of 4), fewer the per-target search (CDF in LDS up to
+# V 16384, read from memory beyond)
+@pytest.mark.parametrize("V,n,m", [(16384, 4, 50000), (16384, 3, 300000), (1000, 2, 262147),
+                                   (65535, 2, 40000), (65535, 2, 262144), (2, 3, 1000)])
+def test_cdf_lookup_bit_exact(hip, ref, rng, V, n, m):
     x = _adversarial_logits(rng, V, 5)[:n]
     t = rng.integers(0, 65536, size=(n, m)).astype(np.uint16)
+    t[:, :4] = [0, 65535, 1, 65534]
     res = []
     for nc in (hip, ref):
         cdf = nc.nc_soft_max_cdf16(nc.tensor(x))
