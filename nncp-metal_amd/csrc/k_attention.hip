@@ -142,26 +142,35 @@ __global__ __launch_bounds__(TPB) void score_softmax_bwd(ScoreBwdArgs a)
     if (lane == 0) dr[0] = acc;
 }
 
-// db_r[p, h] = b_r_scale * sum_{b,i} dS[j = p-(T-1-i), i, h, b]
-__global__ __launch_bounds__(TPB) void bias_grad_kernel(const float *ds, float *db, int H, int B,
-                                                        int T, int K, float b_r_scale)
+// db_r[p, h] = b_r_scale * sum_{b,i} dS[j = p-(T-1-i), i, h, b], in two steps:
+// workgroup (h, c) sums chunk c of the streams with one thread per p (for a
+// fixed query i consecutive p read consecutive keys j, so the reads of a
+// wavefront are contiguous), then the chunk sums are added in chunk order.
+__global__ __launch_bounds__(TPB) void bias_grad_partial(const float *ds, float *part, int H, int B,
+                                                         int T, int K, int nchunk)
 {
-    __shared__ float sh[TPB];
-    int p = blockIdx.x, h = blockIdx.y;
+    const int h = blockIdx.x, c = blockIdx.y;
+    const int b0 = (int)((int64_t)B * c / nchunk), b1 = (int)((int64_t)B * (c + 1) / nchunk);
+    for (int p = threadIdx.x; p < K; p += TPB) {
+        float acc = 0.0f;
+        const int ilo = max(0, T - 1 - p); // j = p - (T-1-i) >= 0; j < K always holds for p < K
+        for (int b = b0; b < b1; b++) {
+            const float *row = ds + (int64_t)(b * H + h) * T * K + (p - (T - 1));
+#pragma unroll 8
+            for (int i = ilo; i < T; i++) acc += row[(int64_t)i * (K + 1)];
+        }
+        part[((int64_t)c * H + h) * K + p] = acc;
+    }
+}
+
+__global__ __launch_bounds__(TPB) void bias_grad_final(const float *part, float *db, int64_t n, int nchunk,
+                                                       float b_r_scale)
+{
+    int64_t e = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (e >= n) return;
     float acc = 0.0f;
-    for (int e = threadIdx.x; e < B * T; e += TPB) {
-        int i = e % T, b = e / T;
-        int j = p - (T - 1 - i);
-        if (j >= 0 && j < K)
-            acc += ds[((int64_t)(b * H + h) * T + i) * K + j];
-    }
-    sh[threadIdx.x] = acc;
-    __syncthreads();
-    for (int s = TPB / 2; s > 0; s >>= 1) {
-        if ((int)threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) db[(int64_t)h * K + p] = b_r_scale * sh[0];
+    for (int c = 0; c < nchunk; c++) acc += part[(int64_t)c * n + e];
+    db[e] = b_r_scale * acc;
 }
 
 thread_local int g_last_launches = 0;
@@ -280,8 +289,8 @@ extern "C" size_t nchip_relpos_attn_bwd_scratch(int H, int dk, int B, int T, int
 {
     size_t K = (size_t)M + T, BH = (size_t)B * H;
     size_t inner = (size_t)dk * d_pos * H;
-    // dS + drel + per-stream dw_r + reduction temporaries
-    return K * T * BH + (size_t)d_pos * T * BH + inner * B + inner * (B / 8 + 2) + 64;
+    // dS + drel + per-stream dw_r + reduction temporaries + 16 chunk sums of db_r
+    return K * T * BH + (size_t)d_pos * T * BH + inner * B + inner * (B / 8 + 2) + 64 + 16 * K * (size_t)H;
 }
 
 extern "C" int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
@@ -369,10 +378,16 @@ extern "C" int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
     rc |= nchip_gemm2(stream, 0, 1, dv, T, T, 1.0f, dout, ldo * B, ldo, dv,
                       probs + M, K, sK * H, sK, 0.0f, dkv + (int64_t)H * dk, ldkv * B, ldkv, dv, BH, H,
                       nullptr, 0, nullptr, precision, 1, nullptr);
-    if (db_r)
-        hipLaunchKernelGGL(bias_grad_kernel, dim3(K, H), dim3(TPB), 0, st, (const float *)ds, db_r,
-                           H, B, T, K, b_r_scale);
+    if (db_r) {
+        const int nchunk = B < 16 ? B : 16;
+        const int64_t inner = (int64_t)dk * d_pos * H;
+        float *bpart = scratch + sK * BH + sR * BH + inner * B + inner * (B / 8 + 2) + 64; // the last region
+        hipLaunchKernelGGL(bias_grad_partial, dim3(H, nchunk), dim3(TPB), 0, st, (const float *)ds, bpart,
+                           H, B, T, K, nchunk);
+        hipLaunchKernelGGL(bias_grad_final, dim3((unsigned)(((int64_t)H * K + TPB - 1) / TPB)), dim3(TPB), 0, st,
+                           (const float *)bpart, db_r, (int64_t)H * K, nchunk, b_r_scale);
+    }
     if (hipGetLastError() != hipSuccess) return bad("kernel launch failed");
-    g_last_launches = 5 + (M > 0 ? 4 : 0) + (w_r ? 4 : 0) + (db_r ? 1 : 0);
+    g_last_launches = 5 + (M > 0 ? 4 : 0) + (w_r ? 4 : 0) + (db_r ? 2 : 0);
     return rc;
 }

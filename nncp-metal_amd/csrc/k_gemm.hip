@@ -56,6 +56,7 @@ struct GemmArgs {
     float alpha, beta;
     int act;
     int tiles_m, tiles_n;
+    int gm; // tile rows per band of the tile order (see the kernel)
     const NchipGemmProblem *grp; // grouped launch: one problem per table row
     int n_grp;
 };
@@ -280,7 +281,19 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     int ntiles = g.tiles_m * g.tiles_n;
     if (!g.grp && ntiles % NXCD == 0)
         bid = (bid % NXCD) * (ntiles / NXCD) + bid / NXCD;
-    const int tile_m = bid % g.tiles_m, tile_n = bid / g.tiles_m;
+    // Tile order inside an XCD's run: bands of gm tile rows, column by column
+    // inside a band, so the workgroups in flight on one XCD form a block about
+    // as wide as it is tall and share both A and B panels in that XCD's L2.
+    int tile_m, tile_n;
+    if (g.gm > 1) {
+        const int band = g.gm * g.tiles_n, bi = bid / band, first = bi * g.gm;
+        const int rows = min(g.tiles_m - first, g.gm), r = bid - bi * band;
+        tile_m = first + r % rows;
+        tile_n = r / rows;
+    } else {
+        tile_m = bid % g.tiles_m;
+        tile_n = bid / g.tiles_m;
+    }
     const int bz = blockIdx.y;
     const int b = bz / g.ksplit, kz = bz % g.ksplit;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
@@ -607,6 +620,7 @@ struct ProfRec {
 };
 bool g_prof_on = false;
 int g_force_cfg = getenv("NCHIP_GEMM_CFG") ? atoi(getenv("NCHIP_GEMM_CFG")) : 0;
+int g_force_gm = -1;
 std::vector<ProfRec> g_prof;
 
 // With `rec` the kernel's own start / stop timestamps are bound to the record's
@@ -617,6 +631,7 @@ void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
+    g.gm = g_force_gm >= 0 ? g_force_gm : 8;
     dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(64 * WM * WN * KW);
 #define LAUNCH(TA, TB)                                                                                     \
     do {                                                                                                   \
@@ -804,6 +819,11 @@ extern "C" int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, flo
 extern "C" void nchip_gemm_force_config(int cfg)
 {
     g_force_cfg = cfg;
+}
+
+extern "C" void nchip_gemm_force_band(int gm)
+{
+    g_force_gm = gm;
 }
 
 // ---- profiling entry points ---------------------------------------------------

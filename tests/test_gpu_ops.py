@@ -87,7 +87,8 @@ def test_gemm_bf16_variant(hip, ref, rng):
                                  dict(H=3, dk=32, dv=32, B=2, T=7, M=50, d_pos=57, attn_len=57),
                                  dict(H=2, dk=64, dv=64, B=1, T=64, M=64, d_pos=64, attn_len=100),
                                  dict(H=2, dk=64, dv=64, B=2, T=48, M=80, d_pos=128, attn_len=128),
-                                 dict(H=2, dk=64, dv=64, B=2, T=64, M=96, d_pos=160, attn_len=160)])
+                                 dict(H=2, dk=64, dv=64, B=2, T=64, M=96, d_pos=160, attn_len=160),
+                                 dict(H=2, dk=64, dv=64, B=19, T=64, M=192, d_pos=256, attn_len=256)])
 def test_relpos_attention_model_shapes(hip, ref, rng, cfg):
     H, dk, dv, B, T, M, d_pos = (cfg[k] for k in ("H", "dk", "dv", "B", "T", "M", "d_pos"))
     K = M + T
