@@ -114,6 +114,20 @@ int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launch
    choice.  The environment variable NCHIP_GEMM_CFG sets the initial value. */
 void nchip_gemm_force_config(int cfg);
 
+/* Tuning aid: tiles are ordered, inside each XCD's run, in bands of `gm` tile
+   rows (1 = plain column-major tile order; a negative value restores the
+   default of 8). */
+void nchip_gemm_force_band(int gm);
+
+/* bf16 products (precision 1) and where the rounding happens: 0 = inside the
+   tile loader, from the fp32 operands, always; 1 (default) = large unbatched
+   products first write bf16 copies of both operands to a scratch buffer (one
+   streaming pass each) and the tiles load those, half the bytes; 2 = every
+   unbatched bf16 product takes that route (testing aid).  The rounded values
+   and the accumulation order are the same on both routes.  The environment
+   variable NCHIP_GEMM_BF16SRC sets the initial value. */
+void nchip_gemm_bf16_source(int mode);
+
 /* Chooses ksplit for nchip_gemm from the shape alone (never from data). */
 int nchip_gemm_pick_ksplit(int m, int n, int k, int batch);
 

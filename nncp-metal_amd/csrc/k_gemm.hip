@@ -28,6 +28,7 @@
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short shortx8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4))); // a first-class value, unlike the uint4 struct
 
 namespace {
 
@@ -57,6 +58,7 @@ struct GemmArgs {
     int act;
     int tiles_m, tiles_n;
     int gm; // tile rows per band of the tile order (see the kernel)
+    int dbg;
     const NchipGemmProblem *grp; // grouped launch: one problem per table row
     int n_grp;
 };
@@ -232,6 +234,90 @@ struct TileLoaderBf16 {
     }
 };
 
+// Loader for operands that are already bf16 in memory (same column-major
+// layout as the fp32 matrix they were rounded from, padded: the k extent is a
+// whole number of tiles with zeros in the padding, and the allocation runs at
+// least one tile past the last row so reads need no guard).  Same LDS layout
+// as above.  Every load is 16 bytes (8 values):
+//   MAJOR = 1: rows k and k+1 of 8 consecutive columns i -> 8 words, two
+//              16-byte LDS writes;
+//   MAJOR = 0: 8 consecutive k of one column i (row index clamped at the
+//              edge) -> 4 words that already are k pairs, 4 LDS writes.
+template <int BT, int BK, int MAJOR, int NT>
+struct TileLoaderBf16Src {
+    static constexpr int NU = MAJOR ? (BT / 8) * (BK / 2) : BT * (BK / 8); // 16-byte units per tile
+    static constexpr int NV = (NU + NT - 1) / NT;
+    static_assert(NU % 64 == 0 && (NU >= NT ? NU % NT == 0 : true), "whole wavefronts take part or sit out");
+    u32x4 r[NV][MAJOR ? 2 : 1];
+
+    __device__ __forceinline__ static void coords(int v, int t, int &i, int &k)
+    {
+        int idx = t + v * NT;
+        if (MAJOR) { i = (idx % (BT / 8)) * 8; k = (idx / (BT / 8)) * 2; }
+        else       { i = idx / (BK / 8);       k = (idx % (BK / 8)) * 8; }
+    }
+
+    __device__ __forceinline__ void load(const float *pf, int64_t ld, int i0, int k0,
+                                         int imax, int kmax, bool fast, int t)
+    {
+        (void)kmax; (void)fast;
+        const uint16_t *p = reinterpret_cast<const uint16_t *>(pf);
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            if (NU < NT && t >= NU) break;
+            int i, k;
+            coords(v, t, i, k);
+            if (MAJOR) {
+                const uint16_t *src = p + (int64_t)(k0 + k) * ld + (i0 + i);
+                r[v][0] = *reinterpret_cast<const u32x4 *>(src);
+                r[v][1] = *reinterpret_cast<const u32x4 *>(src + ld);
+            } else {
+                int row = i0 + i < imax ? i0 + i : imax - 1;
+                r[v][0] = *reinterpret_cast<const u32x4 *>(p + (int64_t)row * ld + (k0 + k));
+            }
+        }
+    }
+
+    // MAJOR = 1 writes the word-pair layout of TileLoaderBf16 (rows of k pairs,
+    // BT + PAD words each); the two 16-byte halves of a unit go out in an
+    // order that alternates every 4 lanes, so the 8 lanes served together
+    // cover all 32 banks.  MAJOR = 0 keeps k contiguous: row i holds its
+    // BK / 2 words, SQ words apart, and a unit is one 16-byte write.
+    static constexpr int SQ = BK / 2 + 4;
+    __device__ __forceinline__ void store(uint32_t *lds, int t) const
+    {
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            if (NU < NT && t >= NU) break;
+            int i, k;
+            coords(v, t, i, k);
+            if (MAJOR) {
+                const uint32_t a[4] = { r[v][0][0], r[v][0][1], r[v][0][2], r[v][0][3] };
+                const uint32_t b[4] = { r[v][1][0], r[v][1][1], r[v][1][2], r[v][1][3] };
+                uint32_t w[8];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    w[2 * e] = (a[e] & 0xffffu) | (b[e] << 16);
+                    w[2 * e + 1] = (a[e] >> 16) | (b[e] & 0xffff0000u);
+                }
+                const bool hi_first = ((t >> 2) & 1) != 0;
+                uint32_t *dst = lds + (k >> 1) * (BT + PAD) + i;
+                uint32_t f[4], g[4]; // first and second write, chosen word by word (register selects)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    f[e] = hi_first ? w[4 + e] : w[e];
+                    g[e] = hi_first ? w[e] : w[4 + e];
+                }
+                const int o1 = hi_first ? 4 : 0;
+                *reinterpret_cast<u32x4 *>(dst + o1) = u32x4{ f[0], f[1], f[2], f[3] };
+                *reinterpret_cast<u32x4 *>(dst + (4 - o1)) = u32x4{ g[0], g[1], g[2], g[3] };
+            } else {
+                *reinterpret_cast<u32x4 *>(lds + i * SQ + (k >> 1)) = r[v][0];
+            }
+        }
+    }
+};
+
 // KW = 2 doubles the wavefronts of a workgroup without shrinking its tile: the
 // two groups of WM x WN wavefronts share the LDS tiles and split every 32-deep
 // k slab, group 0 taking k%32 < 16 and group 1 the rest; group 1 hands its
@@ -244,10 +330,17 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     constexpr int NT = 64 * WM * WN * KW;                 // threads: KW groups of WM x WN wavefronts
     constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN); // 32x32 MFMA tiles per wavefront
     constexpr int WTM = BM / WM, WTN = BN / WN;           // wavefront tile
-    constexpr int LDS_A = BF16 ? (BK / 2) * (BM + PAD) : BK * (BM + PAD); // in 32-bit words
-    constexpr int LDS_B = BF16 ? (BK / 2) * (BN + PAD) : BK * (BN + PAD);
+    // in 32-bit words; bf16 sources with k contiguous keep rows of BK/2 + 4 words
+    constexpr int SQ = BK / 2 + 4;
+    constexpr int LDS_A = BF16 == 2 && TA ? BM * SQ : (BF16 ? (BK / 2) * (BM + PAD) : BK * (BM + PAD));
+    constexpr int LDS_B = BF16 == 2 && !TB ? BN * SQ : (BF16 ? (BK / 2) * (BN + PAD) : BK * (BN + PAD));
     static_assert(KW == 1 || BM * BN <= 2 * (LDS_A + LDS_B), "accumulator hand-over must fit in the tile buffers");
-    __shared__ __attribute__((aligned(16))) float smem[2 * (LDS_A + LDS_B)];
+    // tile buffers above the 64 KiB a static array may take come from the
+    // launch's dynamic allocation instead
+    constexpr bool BIG_LDS = 2 * (LDS_A + LDS_B) * 4 > 65536;
+    __shared__ __attribute__((aligned(16))) float smem_static[BIG_LDS ? 4 : 2 * (LDS_A + LDS_B)];
+    extern __shared__ __attribute__((aligned(16))) float smem_dynamic[];
+    float *const smem = BIG_LDS ? smem_dynamic : smem_static;
 
     const int t = threadIdx.x, lane = t & 63;
     const int kg = (t >> 6) / (WM * WN), wave = (t >> 6) % (WM * WN);
@@ -305,14 +398,17 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     const float *B = g.B + (int64_t)b_out * g.sb + (int64_t)b_in * g.sb_in;
 
     // fast (vector, unguarded) loads need whole tiles and 16-byte alignment
-    const bool a_full = (m0 + BM <= g.M) && (g.lda % 4 == 0) && (((uintptr_t)A & 15) == 0);
-    const bool b_full = (n0 + BN <= g.N) && (g.ldb % 4 == 0) && (((uintptr_t)B & 15) == 0);
+    // (bf16 sources are padded and aligned by construction: always fast)
+    const bool a_full = BF16 == 2 || ((m0 + BM <= g.M) && (g.lda % 4 == 0) && (((uintptr_t)A & 15) == 0));
+    const bool b_full = BF16 == 2 || ((n0 + BN <= g.N) && (g.ldb % 4 == 0) && (((uintptr_t)B & 15) == 0));
 
     // PF register sets: while tile it is computed, tiles it+1 .. it+PF are landing
     // or in flight, so a load has PF compute phases to arrive.  Two sets are
     // enough on MI355X: four or six measured no faster on any model shape.
-    using LoaderA = std::conditional_t<BF16 != 0, TileLoaderBf16<BM, BK, TA ? 0 : 1, NT>, TileLoader<BM, BK, TA ? 0 : 1, NT>>;
-    using LoaderB = std::conditional_t<BF16 != 0, TileLoaderBf16<BN, BK, TB ? 1 : 0, NT>, TileLoader<BN, BK, TB ? 1 : 0, NT>>;
+    using LoaderA = std::conditional_t<BF16 == 2, TileLoaderBf16Src<BM, BK, TA ? 0 : 1, NT>,
+                    std::conditional_t<BF16 == 1, TileLoaderBf16<BM, BK, TA ? 0 : 1, NT>, TileLoader<BM, BK, TA ? 0 : 1, NT>>>;
+    using LoaderB = std::conditional_t<BF16 == 2, TileLoaderBf16Src<BN, BK, TB ? 1 : 0, NT>,
+                    std::conditional_t<BF16 == 1, TileLoaderBf16<BN, BK, TB ? 1 : 0, NT>, TileLoader<BN, BK, TB ? 1 : 0, NT>>>;
     LoaderA la[PF];
     LoaderB lb[PF];
 
@@ -332,31 +428,9 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     // steady-state loop carries no guarded-load code: the guarded path shares
     // registers with the vector loads and the compiler then serialises every
     // prefetch behind an s_waitcnt vmcnt(0).
-    auto step = [&](int it, int nk, auto fast_tag, auto &la, auto &lb) {
-        constexpr bool FAST = decltype(fast_tag)::value;
-        float *sa = smem + (it & 1) * (LDS_A + LDS_B);
-        float *sb = sa + LDS_A;
-        if constexpr (BF16 != 0) {
-            la.store(reinterpret_cast<uint32_t *>(sa), t);
-            lb.store(reinterpret_cast<uint32_t *>(sb), t);
-        } else {
-            la.store_f32(sa, t);
-            lb.store_f32(sb, t);
-        }
-        __syncthreads();
-        if (FAST || it + PF < nk) {
-            int k0 = kbeg + (it + PF) * BK;
-            bool kf = FAST || (k0 + BK <= kend);
-            const bool second = k0 >= k1; // uniform
-            const float *Ak = second ? A2 : A, *Bk = second ? B2 : B;
-            const int kr = second ? k0 - k1 : k0, ke = second ? kend - k1 : (kend < k1 ? kend : k1);
-            la.load(Ak, g.lda, m0, kr, g.M, ke, FAST || (a_full && kf), t);
-            lb.load(Bk, g.ldb, n0, kr, g.N, ke, FAST || (b_full && kf), t);
-        }
-        // keep the prefetch ahead of the MFMAs: without this fence the
-        // scheduler sinks the global loads below the compute block and their
-        // latency is paid in full at the next LDS write
-        __builtin_amdgcn_sched_barrier(0);
+    // the MFMAs of the tile held in LDS at sa / sb
+    auto compute = [&](const float *sa, const float *sb) {
+        if (g.dbg & 2) return;
         if constexpr (BF16 != 0) {
             // one 32x32x16 MFMA per tile pair per 16 k; group kg takes every KW-th block
             const uint32_t *wa = reinterpret_cast<const uint32_t *>(sa) + (lane >> 5) * 4 * (BM + PAD) + wm * WTM + (lane & 31);
@@ -364,16 +438,26 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 #pragma unroll
             for (int u = 0; u < BK / 16 / KW; u++) {
                 const int row0 = (u * KW + kg) * 8; // word row of this 16-k block
-                uint4 fa[TM], fb[TN];
+                u32x4 fa[TM], fb[TN];
 #pragma unroll
                 for (int j = 0; j < TM; j++) {
-                    const uint32_t *q = wa + row0 * (BM + PAD) + j * 32;
-                    fa[j] = make_uint4(q[0], q[BM + PAD], q[2 * (BM + PAD)], q[3 * (BM + PAD)]);
+                    if constexpr (BF16 == 2 && TA != 0) { // k-contiguous rows: one 16-byte read
+                        fa[j] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const uint32_t *>(sa) +
+                                (wm * WTM + j * 32 + (lane & 31)) * SQ + row0 + (lane >> 5) * 4);
+                    } else {
+                        const uint32_t *q = wa + row0 * (BM + PAD) + j * 32;
+                        fa[j] = u32x4{ q[0], q[BM + PAD], q[2 * (BM + PAD)], q[3 * (BM + PAD)] };
+                    }
                 }
 #pragma unroll
                 for (int i = 0; i < TN; i++) {
-                    const uint32_t *q = wb + row0 * (BN + PAD) + i * 32;
-                    fb[i] = make_uint4(q[0], q[BN + PAD], q[2 * (BN + PAD)], q[3 * (BN + PAD)]);
+                    if constexpr (BF16 == 2 && TB == 0) {
+                        fb[i] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const uint32_t *>(sb) +
+                                (wn * WTN + i * 32 + (lane & 31)) * SQ + row0 + (lane >> 5) * 4);
+                    } else {
+                        const uint32_t *q = wb + row0 * (BN + PAD) + i * 32;
+                        fb[i] = u32x4{ q[0], q[BN + PAD], q[2 * (BN + PAD)], q[3 * (BN + PAD)] };
+                    }
                 }
 #pragma unroll
                 for (int i = 0; i < TN; i++)
@@ -422,11 +506,84 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
         }
     };
 
+    auto step = [&](int it, int nk, auto fast_tag, auto &la, auto &lb) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+        float *sa = smem + (it & 1) * (LDS_A + LDS_B);
+        float *sb = sa + LDS_A;
+        if constexpr (BF16 != 0) {
+            la.store(reinterpret_cast<uint32_t *>(sa), t);
+            lb.store(reinterpret_cast<uint32_t *>(sb), t);
+        } else {
+            la.store_f32(sa, t);
+            lb.store_f32(sb, t);
+        }
+        __syncthreads();
+        if ((FAST || it + PF < nk) && !(g.dbg & 1)) {
+            int k0 = kbeg + (it + PF) * BK;
+            bool kf = FAST || (k0 + BK <= kend);
+            const bool second = k0 >= k1; // uniform
+            const float *Ak = second ? A2 : A, *Bk = second ? B2 : B;
+            const int kr = second ? k0 - k1 : k0, ke = second ? kend - k1 : (kend < k1 ? kend : k1);
+            la.load(Ak, g.lda, m0, kr, g.M, ke, FAST || (a_full && kf), t);
+            lb.load(Bk, g.ldb, n0, kr, g.N, ke, FAST || (b_full && kf), t);
+        }
+        // keep the prefetch ahead of the MFMAs: without this fence the
+        // scheduler sinks the global loads below the compute block and their
+        // latency is paid in full at the next LDS write
+        __builtin_amdgcn_sched_barrier(0);
+        compute(sa, sb);
+    };
+
 #ifdef NCHIP_GEMM_CLOCKS
     long long dbg_c0 = clock64(), dbg_w0 = wall_clock64();
 #endif
-    const int nk = (kend - kbeg + BK - 1) / BK;
+    const int nk = (g.dbg & 4) ? 0 : (kend - kbeg + BK - 1) / BK;
     const int nk_full = (kend - kbeg) / BK; // tiles with a complete k range
+    if constexpr (BF16 == 2) {
+        // bf16 sources: the MFMAs of a tile are short, so the LDS writes of the
+        // next tile go out BEFORE them (into the other buffer, which every
+        // wavefront left at the last barrier) and overlap with them; one
+        // barrier per tile, after the MFMAs.  Register set (i % PF) holds tile
+        // i from its load until that write; it is reloaded with tile i + PF
+        // right after.
+        auto fetch = [&](int tile, auto &la, auto &lb) {
+            const int k0 = kbeg + tile * BK;
+            const bool second = k0 >= k1; // uniform
+            const float *Ak = second ? A2 : A, *Bk = second ? B2 : B;
+            const int kr = second ? k0 - k1 : k0;
+            la.load(Ak, g.lda, m0, kr, g.M, 0, true, t);
+            lb.load(Bk, g.ldb, n0, kr, g.N, 0, true, t);
+        };
+        auto park = [&](int tile, auto &la, auto &lb) {
+            float *sa = smem + (tile & 1) * (LDS_A + LDS_B);
+            la.store(reinterpret_cast<uint32_t *>(sa), t);
+            lb.store(reinterpret_cast<uint32_t *>(sa + LDS_A), t);
+        };
+#pragma unroll
+        for (int j = 0; j < PF; j++)
+            if (j < nk) fetch(j, la[j], lb[j]);
+        if (nk > 0) park(0, la[0], lb[0]);
+        if (PF < nk) fetch(PF, la[0], lb[0]);
+        __syncthreads();
+        for (int it = 0; it < nk; it += PF) {
+#pragma unroll
+            for (int j = 0; j < PF; j++) {
+                const int cur = it + j;
+                if (cur < nk) {
+                    auto &na = la[(j + 1) % PF];
+                    auto &nb = lb[(j + 1) % PF];
+                    if (cur + 1 < nk) {
+                        park(cur + 1, na, nb);
+                        if (cur + 1 + PF < nk && !(g.dbg & 1)) fetch(cur + 1 + PF, na, nb);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    const float *sa = smem + (cur & 1) * (LDS_A + LDS_B);
+                    compute(sa, sa + LDS_A);
+                    __syncthreads();
+                }
+            }
+        }
+    } else {
     int it = 0;
 #pragma unroll
     for (int j = 0; j < PF; j++)
@@ -444,6 +601,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 #pragma unroll
         for (int j = 0; j < PF; j++)
             if (it % PF == j) step(it, nk, std::false_type(), la[j], lb[j]);
+    }
     }
 
 #ifdef NCHIP_GEMM_CLOCKS
@@ -612,6 +770,33 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce(GemmArgs g)
     }
 }
 
+// Rounds a column-major fp32 matrix (rows x cols, leading dimension ld_src) to
+// bf16 (nearest even) in the same layout, padded with zeros to rows_pad x
+// cols_pad (rows_pad a multiple of 8 = the leading dimension of the copy).
+// One thread per 8 consecutive rows of one column.
+__global__ __launch_bounds__(256) void cast_bf16_kernel(const float *src, uint16_t *dst, int rows, int cols,
+                                                        int64_t ld_src, int rows_pad, int cols_pad, int vec)
+{
+    const int units = rows_pad / 8;
+    const int64_t total = (int64_t)units * cols_pad;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+        const int u = (int)(e % units), c = (int)(e / units), r0 = u * 8;
+        float f[8];
+        if (c < cols && vec && r0 + 8 <= rows) {
+            const floatx4 *q = reinterpret_cast<const floatx4 *>(src + (int64_t)c * ld_src + r0);
+            floatx4 a = q[0], b = q[1];
+            f[0] = a[0]; f[1] = a[1]; f[2] = a[2]; f[3] = a[3];
+            f[4] = b[0]; f[5] = b[1]; f[6] = b[2]; f[7] = b[3];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                f[j] = (c < cols && r0 + j < rows) ? src[(int64_t)c * ld_src + r0 + j] : 0.0f;
+        }
+        uint4 w = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
+        *reinterpret_cast<uint4 *>(dst + (int64_t)c * rows_pad + r0) = w;
+    }
+}
+
 // ---- optional per-launch timing (HIP events on the launch stream) ----------
 struct ProfRec {
     hipEvent_t start, stop;
@@ -626,24 +811,95 @@ std::vector<ProfRec> g_prof;
 // With `rec` the kernel's own start / stop timestamps are bound to the record's
 // events (hipExtLaunchKernelGGL), so the measured time is the dispatch alone,
 // as a kernel trace reports it, without the marker packets of hipEventRecord.
+// bytes of the two tile buffer pairs when they exceed what a static array may hold (else 0)
+template <int BM, int BN, int BK, int TA, int TB, int BF16>
+constexpr size_t lds_dynamic_bytes()
+{
+    constexpr int SQ = BK / 2 + 4;
+    constexpr size_t a = BF16 == 2 && TA ? BM * SQ : (BF16 ? (BK / 2) * (BM + PAD) : BK * (BM + PAD));
+    constexpr size_t b = BF16 == 2 && !TB ? BN * SQ : (BF16 ? (BK / 2) * (BN + PAD) : BK * (BN + PAD));
+    constexpr size_t bytes = 2 * (a + b) * sizeof(float);
+    static_assert(bytes <= 160 * 1024, "tile buffers exceed LDS");
+    return bytes > 65536 ? bytes : 0;
+}
+
 template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1, int PF = 2>
 void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     g.gm = g_force_gm >= 0 ? g_force_gm : 8;
+    g.dbg = getenv("NCHIP_GEMM_DBG") ? atoi(getenv("NCHIP_GEMM_DBG")) : 0;
     dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(64 * WM * WN * KW);
 #define LAUNCH(TA, TB)                                                                                     \
     do {                                                                                                   \
-        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>), grid, block, 0, \
+        constexpr size_t dyn = lds_dynamic_bytes<BM, BN, BK, TA, TB, BF16>();                              \
+        if (dyn) {                                                                                         \
+            static const bool ok = hipFuncSetAttribute(                                                    \
+                reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>),     \
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) == hipSuccess;                       \
+            if (!ok) { fprintf(stderr, "nchip_gemm: cannot reserve %zu bytes of LDS\n", dyn); abort(); }  \
+        }                                                                                                  \
+        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>), grid, block, dyn, \
                                        st, rec->start, rec->stop, 0, g);                                   \
-        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>), grid, block, 0, st, g); \
+        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>), grid, block, dyn, st, g); \
     } while (0)
     if (!ta && !tb) LAUNCH(0, 0);
     else if (ta && !tb) LAUNCH(1, 0);
     else if (!ta && tb) LAUNCH(0, 1);
     else LAUNCH(1, 1);
 #undef LAUNCH
+}
+
+// Device scratch for the bf16 copies of one product's operands, one buffer per
+// stream: successive products on a stream reuse it in stream order.  It grows
+// on demand and lives until the process ends.
+struct CastScratch { hipStream_t st; uint16_t *ptr; size_t cap; };
+std::vector<CastScratch> g_cast;
+int g_bf16src = getenv("NCHIP_GEMM_BF16SRC") ? atoi(getenv("NCHIP_GEMM_BF16SRC")) : 1;
+double g_bf16src_min_flops = getenv("NCHIP_GEMM_BF16SRC_FLOPS") ? atof(getenv("NCHIP_GEMM_BF16SRC_FLOPS")) : 8e9;
+
+uint16_t *cast_scratch(hipStream_t st, size_t elems)
+{
+    for (CastScratch &c : g_cast)
+        if (c.st == st) {
+            if (c.cap >= elems) return c.ptr;
+            (void)hipStreamSynchronize(st);
+            (void)hipFree(c.ptr);
+            c.ptr = nullptr; c.cap = 0;
+            size_t cap = elems + elems / 4;
+            if (hipMalloc((void **)&c.ptr, cap * sizeof(uint16_t)) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+            c.cap = cap;
+            return c.ptr;
+        }
+    CastScratch c = { st, nullptr, 0 };
+    if (hipMalloc((void **)&c.ptr, elems * sizeof(uint16_t)) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    c.cap = elems;
+    g_cast.push_back(c);
+    return c.ptr;
+}
+
+constexpr int CAST_SLACK = 512; // elements past a copy that a partial edge tile may read
+
+// copy of a column-major rows x cols operand; k_is_rows says which extent is k
+// (padded to kpad); returns the leading dimension of the copy
+int64_t cast_operand(hipStream_t st, const float *src, int rows, int cols, int64_t ld, bool k_is_rows,
+                     int kpad, uint16_t *dst)
+{
+    const int rows_pad = k_is_rows ? kpad : (rows + 7) / 8 * 8;
+    const int cols_pad = k_is_rows ? cols : kpad;
+    const int vec = (ld % 4 == 0) && (((uintptr_t)src & 15) == 0);
+    int64_t total = (int64_t)(rows_pad / 8) * cols_pad;
+    int nb = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+    hipLaunchKernelGGL(cast_bf16_kernel, dim3(nb), dim3(256), 0, st, src, dst, rows, cols, ld, rows_pad, cols_pad, vec);
+    return rows_pad;
+}
+
+size_t cast_elems(int rows, int cols, bool k_is_rows, int kpad)
+{
+    const size_t rows_pad = k_is_rows ? kpad : (rows + 7) / 8 * 8;
+    const size_t cols_pad = k_is_rows ? cols : kpad;
+    return (rows_pad * cols_pad + CAST_SLACK + 127) / 128 * 128;
 }
 
 } // namespace
@@ -722,7 +978,37 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
         else if (t128x64 >= 256 && m >= 128 && n >= 64) cfg = 4;
         else cfg = 8;
     }
-    if (precision == 1) {
+    // Large bf16 products are bound by operand traffic from L2, not by the MFMA
+    // rate: round both operands to bf16 in memory first (one streaming pass
+    // each) and let the tiles load half the bytes.  The rounded values are
+    // the ones the conversion inside the tile loader would produce, so the
+    // result is the same either way.
+    bool from_bf16 = false;
+    if (precision == 1 && batch == 1 && ksplit == 1 && !invariant &&
+        (g_bf16src == 2 || (g_bf16src == 1 && m >= 128 && n >= 128 && k >= 256 &&
+                            2.0 * m * n * (double)k >= g_bf16src_min_flops))) {
+        const int kpad = (k + 63) / 64 * 64;
+        const size_t ea = cast_elems(ta ? k : m, ta ? m : k, ta != 0, kpad);
+        const size_t eb = cast_elems(tb ? n : k, tb ? k : n, tb == 0, kpad);
+        uint16_t *buf = cast_scratch(st, ea + eb);
+        if (buf) {
+            g.lda = cast_operand(st, A, ta ? k : m, ta ? m : k, lda, ta != 0, kpad, buf);
+            g.ldb = cast_operand(st, B, tb ? n : k, tb ? k : n, ldb, tb == 0, kpad, buf + ea);
+            g.A = reinterpret_cast<const float *>(buf);
+            g.B = reinterpret_cast<const float *>(buf + ea);
+            g.K = kpad; g.kchunk = kpad;
+            from_bf16 = true;
+        }
+    }
+    if (from_bf16) {
+        // 64x64 per wavefront, 64-deep tiles: with enough tiles for two workgroups
+        // per CU four wavefronts each do best; below that, eight wavefronts in
+        // two k groups share one tile
+        const bool four = g_force_cfg == 13 || (g_force_cfg != 11 && g_force_cfg != 7 && t128 >= 512);
+        if (g_force_cfg == 7) launch_tile<128, 128, 32, 4, 2, 2>(st, ta, tb, g, pr);
+        else if (four) launch_tile<128, 128, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+        else launch_tile<128, 128, 64, 2, 2, 2, 2>(st, ta, tb, g, pr);
+    } else if (precision == 1) {
         if (cfg == 7) launch_tile<128, 128, 32, 4, 2, 1>(st, ta, tb, g, pr);
         else if (cfg == 4) launch_tile<128, 64, 32, 4, 2, 1>(st, ta, tb, g, pr);
         else if (cfg == 9) launch_tile<64, 64, 64, 2, 2, 1, 2>(st, ta, tb, g, pr);
@@ -821,6 +1107,14 @@ extern "C" void nchip_gemm_force_config(int cfg)
     g_force_cfg = cfg;
 }
 
+// 0: bf16 products always round their operands inside the tile loader;
+// 1: large ones go through bf16 copies of the operands (default);
+// 2: every unbatched bf16 product does (testing aid)
+extern "C" void nchip_gemm_bf16_source(int mode)
+{
+    g_bf16src = mode;
+}
+
 extern "C" void nchip_gemm_force_band(int gm)
 {
     g_force_gm = gm;
@@ -890,9 +1184,16 @@ extern "C" int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmP
     }
 #define GRP(TA, TB, BF)                                                                                    \
     do {                                                                                                   \
-        if (g_prof_on) hipExtLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, 0, st, \
+        constexpr size_t dyn = lds_dynamic_bytes<128, 128, 32, TA, TB, BF>();                              \
+        if (dyn) {                                                                                         \
+            static const bool ok = hipFuncSetAttribute(                                                    \
+                reinterpret_cast<const void *>(gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>),               \
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) == hipSuccess;                       \
+            if (!ok) { fprintf(stderr, "nchip_gemm_grouped: cannot reserve %zu bytes of LDS\n", dyn); return -2; } \
+        }                                                                                                  \
+        if (g_prof_on) hipExtLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, dyn, st, \
                                              rec.start, rec.stop, 0, g);                                   \
-        else hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, 0, st, g);      \
+        else hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, dyn, st, g);    \
     } while (0)
     if (precision == 1) {
         if (!ta && !tb) GRP(0, 0, 1); else if (ta && !tb) GRP(1, 0, 1); else if (!ta && tb) GRP(0, 1, 1); else GRP(1, 1, 1);

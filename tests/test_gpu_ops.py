@@ -80,6 +80,32 @@ def test_gemm_bf16_variant(hip, ref, rng):
     assert relerr(outs[0], exact) <= 2e-2
 
 
+# bf16 products through bf16 copies of the operands (mode 2 forces that route
+# for any unbatched shape): the rounded values and the accumulation order are
+# those of the 128x128x32 tile kernel rounding inside its loader (config 7),
+# so the two must agree bit for bit; the CPU checker rounds the same way and
+# accumulates in another order.
+@pytest.mark.parametrize("m,n,k", [(256, 384, 512), (130, 70, 100), (1000, 333, 257), (8, 5, 32), (129, 257, 1031)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_gemm_bf16_from_rounded_copies(hip, ref, rng, m, n, k, ta, tb):
+    a = rng.standard_normal((m, k) if ta else (k, m)).astype(np.float32)  # numpy order: (columns, rows)
+    b = rng.standard_normal((k, n) if tb else (n, k)).astype(np.float32)
+    lib = C.CDLL(hip.lib._name)
+    outs = {}
+    for nc, mode in ((hip, 2), (hip, 0), (ref, None)):
+        nc.nc_set_matmul_bf16(nc.ctx, 1)
+        if mode is not None:
+            lib.nchip_gemm_bf16_source(mode)
+            lib.nchip_gemm_force_config(7)
+        x, y = nc.tensor(a), nc.tensor(b)
+        outs[(nc is hip, mode)] = nc.numpy(nc.nc_matmul_add(x, y, None, ta, tb, 1.0), free=True)
+        nc.nc_set_matmul_bf16(nc.ctx, 0)
+    lib.nchip_gemm_bf16_source(1)
+    lib.nchip_gemm_force_config(0)
+    assert np.array_equal(outs[(True, 2)], outs[(True, 0)])
+    assert relerr(outs[(True, 2)], outs[(False, None)]) <= 1e-5
+
+
 @pytest.mark.parametrize("cfg", [dict(H=2, dk=64, dv=64, B=2, T=64, M=64, d_pos=128, attn_len=128),
                                  dict(H=4, dk=32, dv=32, B=3, T=20, M=20, d_pos=40, attn_len=40),
                                  dict(H=2, dk=32, dv=32, B=2, T=32, M=32, d_pos=32, attn_len=48),
