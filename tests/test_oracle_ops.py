@@ -157,3 +157,47 @@ def test_optimisers_closed_form(ref, pkg):
         nc.nc_sgd_opt_set_all(C.byref(nc.plist), None)
         nc.nc_sgd_opt_end(opt)
         nc.close()
+
+
+# ---- coder-side probability path: what the mathematics fixes ---------------------
+def _zipf_logits(rng, n, V):
+    bias = -np.log(rng.permutation(V) + 1.0)
+    return (rng.normal(0, 3, (n, V)) + bias).astype(np.float32)
+
+
+@pytest.mark.parametrize("V,n", [(256, 8), (16384, 3), (2, 4), (1000, 5), (65535, 2)])
+def test_cdf16_invariants_and_accuracy(ref, rng, V, n):
+    """The integer CDF is pinned by what it must be, not by its own formula:
+    starts at 0, every frequency >= 1, total exactly 2^16, and each frequency
+    is 1 + (65536 - V) * softmax within the rounding the construction allows
+    (one floor of a 24-bit quantised exponential per symbol, one floor of the
+    scaled prefix per boundary)."""
+    x = _zipf_logits(rng, n, V)
+    x[0] = 0.0                                  # uniform: every frequency equal up to the floor
+    cdf = ref.numpy(ref.nc_soft_max_cdf16(ref.tensor(x)), free=True).astype(np.int64)
+    assert (cdf[:, 0] == 0).all()
+    freq = np.diff(np.concatenate([cdf, np.full((n, 1), 65536)], axis=1), axis=1)
+    assert (freq >= 1).all() and (freq.sum(axis=1) == 65536).all()
+    x64 = x.astype(np.float64)
+    p = np.exp(np.maximum(x64 - x64.max(axis=1, keepdims=True), -30.0))
+    p /= p.sum(axis=1, keepdims=True)
+    want = 1.0 + (65536 - V) * p
+    # quantising exp to 2^-24 moves a share by < V * 2^-24 relative to the total (the
+    # largest term is 1), each boundary floors once: 2 for the floors + the quantisation
+    slack = 2.0 + (65536 - V) * (V * 2.0 ** -24 + 3e-7)
+    assert np.abs(freq - want).max() <= slack
+    u = freq[0]
+    assert u.max() - u.min() <= 1
+
+
+def test_cdf_lookup_is_the_inverse_of_the_cdf(ref, rng):
+    """searchsorted is an independent statement of 'the symbol whose interval
+    holds the target'."""
+    V, n, m = 4099, 3, 20000
+    cdf_t = ref.nc_soft_max_cdf16(ref.tensor(_zipf_logits(rng, n, V)))
+    cdf = ref.numpy(cdf_t).astype(np.int64)
+    t = rng.integers(0, 65536, size=(n, m)).astype(np.uint16)
+    t[:, :2] = [0, 65535]
+    sym = ref.numpy(ref.nc_cdf_lookup(cdf_t, ref.tensor(t)), free=True).astype(np.int64)
+    for r in range(n):
+        assert np.array_equal(sym[r], np.searchsorted(cdf[r], t[r].astype(np.int64), side="right") - 1)
