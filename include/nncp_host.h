@@ -86,7 +86,21 @@ typedef struct { /* TransformerModelParams + the NNCPModelParams fields it needs
     int fused;      /* 1: trf_eval uses nc_linear / nc_relpos_attention /
                        nc_fused_layer_norm (full-segment evaluation only) */
     int nb_threads;
+    /* retrain (NNCPModelParams, nncp.c:112-113, 153-156): all zero = off, as in
+       the default profile */
+    float dropout_prob, dropout_att_prob; /* used during retrain only */
+    int retrain_period;  /* in symbols; a retrain pass runs between blocks once this many were coded */
+    int retrain_len;     /* length of the retrain buffer, in symbols */
+    int has_retrain_lr;
+    NNCPInterp retrain_lr;
 } NNCPConfig;
+
+typedef struct { /* nncp.c:183-193 */
+    uint16_t *buf;
+    int buf_pos, buf_len; /* next write position; symbols held */
+    int pos;              /* symbols coded since the last retrain pass */
+    int64_t train_step;   /* steps of the retrain schedule (has_retrain_lr) */
+} NNCPRetrainState;
 
 typedef struct NNCPModel NNCPModel;
 
@@ -112,6 +126,11 @@ float trf_eval_gradient(NNCPModel *s, const NCTensor *expected_output);    /* nn
 void trf_reset(NNCPModel *s);                                              /* nncp.c:1195 */
 void trf_update(NNCPModel *s);                                             /* nncp.c:1224 */
 void trf_set_lr(NNCPModel *s, float lr);                                   /* nncp.c:1243 */
+/* dropout on (only if cfg.dropout_prob != 0) / off; while it is on, trf_eval
+   takes the op-by-op path even when cfg.fused is set */
+void trf_set_retrain(NNCPModel *s, int enabled);                           /* nncp.c:1237 */
+NNCPRetrainState *nncp_model_retrain_state(NNCPModel *s);
+void nncp_model_set_train_step(NNCPModel *s, int64_t step);
 /* logits of the last trf_eval (V, B, T|1), borrowed; used by the CDF path */
 NCTensor *trf_last_logits(NNCPModel *s);
 /* Per-timestep evaluation with K/V caches through the fused entry points (the
@@ -151,6 +170,20 @@ typedef struct {
 void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *block_buf,
                         int block_len, int is_decode, int mode, const NNCPInterp *lr,
                         NNCPStats *st);
+
+/* retrain_block (nncp.c:2821-2941): appends the block just coded (encoder) or
+   decoded (decoder) to the retrain buffer; once cfg.retrain_period symbols have
+   gone by since the last pass, resets the memory and trains over the whole
+   buffer again, B streams of buffer_len / B symbols, one segment per step, with
+   dropout on and the rate of cfg.retrain_lr (its own step counter) or of `lr`
+   (the model's counter, which then advances).  Both sides must call it after
+   every block.  No-op when cfg.retrain_period is 0.  st (or NULL) receives the
+   steps and the loss of the pass. */
+void nncp_retrain_block(NNCPModel *s, const uint16_t *block_buf, int block_len,
+                        const NNCPInterp *lr, NNCPStats *st);
+/* symbol idx of a FIFO that holds `size` symbols whose oldest one sits at rpos
+   (nncp.c:2811-2819); 0 before the start */
+int nncp_fifo_symbol(const uint16_t *buf, int rpos, int size, int idx);
 
 /* convenience: whole buffer as one block, in memory; returns the number of
    bytes written (compress) */

@@ -17,6 +17,11 @@ LN_POST, LN_PRE, LN_FINAL, LN_COEF, LN_RMSNORM = 1, 2, 4, 8, 16
 FF_RELU, FF_GELU, FF_GEGLU, FF_GATED_SILU = 0, 1, 2, 3
 
 
+class NNCPInterp(C.Structure):
+    _fields_ = [("n_steps", C.c_int), ("val", C.c_float * 9), ("pos", C.c_int64 * 8),
+                ("decay_power", C.c_float)]
+
+
 class NNCPConfig(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("n_layer", "d_model", "n_head", "d_key", "d_value",
                                        "d_inner", "d_pos", "mem_len")] + \
@@ -25,12 +30,9 @@ class NNCPConfig(C.Structure):
                                        "ln_flags", "ff_act")] + \
                [("init_range", C.c_float), ("embed_mult", C.c_float), ("sgd_opt", B.SGDOptParams)] + \
                [(n, C.c_int) for n in ("batch_size", "seg_len", "n_symbols")] + \
-               [("seed", C.c_uint32), ("use_device", C.c_int), ("fused", C.c_int), ("nb_threads", C.c_int)]
-
-
-class NNCPInterp(C.Structure):
-    _fields_ = [("n_steps", C.c_int), ("val", C.c_float * 9), ("pos", C.c_int64 * 8),
-                ("decay_power", C.c_float)]
+               [("seed", C.c_uint32), ("use_device", C.c_int), ("fused", C.c_int), ("nb_threads", C.c_int)] + \
+               [("dropout_prob", C.c_float), ("dropout_att_prob", C.c_float), ("retrain_period", C.c_int),
+                ("retrain_len", C.c_int), ("has_retrain_lr", C.c_int), ("retrain_lr", NNCPInterp)]
 
 
 class NNCPStats(C.Structure):
@@ -63,6 +65,7 @@ def make_config(**kw):
     cfg = NNCPConfig()
     opt = kw.pop("sgd_opt", None)
     attn = kw.pop("attn_len", None)
+    retrain_lr = kw.pop("retrain_lr", None)
     base = dict(n_layer=4, d_model=256, n_head=8, d_inner=512, d_pos=32, mem_len=32, use_bias=1,
                 use_w_r=1, tied_w_r=1, tied_b_r=1, query_bias=0, ln_flags=LN_POST, ff_act=FF_GELU,
                 init_range=1.0, embed_mult=1.0, batch_size=16, seg_len=32, n_symbols=256, seed=123,
@@ -74,6 +77,9 @@ def make_config(**kw):
         setattr(cfg, k, v)
     for i in range(base["n_layer"]):
         cfg.attn_len[i] = (attn[i] if attn else base["mem_len"] + base["seg_len"])
+    if retrain_lr is not None:
+        cfg.has_retrain_lr = 1
+        cfg.retrain_lr = retrain_lr if isinstance(retrain_lr, NNCPInterp) else constant_lr(retrain_lr)
     cfg.sgd_opt = opt if opt is not None else B.SGDOptParams(
         algo=B.SGD_OPT_ADAM, beta1=0.0, beta2=0.9999, eps=1e-8, gradient_clip=0.1, lr=3e-4)
     return cfg
@@ -113,6 +119,11 @@ class Host:
         L.trf_reset.argtypes = [_P]
         L.trf_update.argtypes = [_P]
         L.trf_set_lr.argtypes = [_P, C.c_float]
+        L.trf_set_retrain.argtypes = [_P, C.c_int]
+        L.nncp_process_block.argtypes = [_P, C.POINTER(NNCPPutBit), C.POINTER(NNCPGetBit), _P, C.c_int, C.c_int,
+                                         C.c_int, C.POINTER(NNCPInterp), C.POINTER(NNCPStats)]
+        L.nncp_retrain_block.argtypes = [_P, _P, C.c_int, C.POINTER(NNCPInterp), C.POINTER(NNCPStats)]
+        L.nncp_fifo_symbol.argtypes = [_P, C.c_int, C.c_int, C.c_int]
         L.trf_last_logits.restype = _P
         L.trf_last_logits.argtypes = [_P]
         L.trf_step_begin.argtypes = [_P]
@@ -258,3 +269,39 @@ class Model:
         self.L.nncp_decompress(self.ptr, data.ctypes.data, data.size, out.ctypes.data, n_syms, mode,
                                C.byref(sched), C.byref(st))
         return out, st
+
+    # -- several blocks through one coder, with the retrain pass between them ----
+    def compress_blocks(self, syms, block_len, mode, lr=3e-4):
+        """The reference's file loop (nncp.c:3375-3460, in memory): blocks of
+        block_len symbols through ONE range coder, nncp_retrain_block after
+        each.  Returns (bytes, coding stats, retrain stats)."""
+        syms = np.ascontiguousarray(syms, dtype=np.uint16)
+        cap = syms.size * 4 + 1024
+        out = np.zeros(cap, dtype=np.uint8)
+        st, rst = NNCPStats(), NNCPStats()
+        sched = constant_lr(lr) if not isinstance(lr, NNCPInterp) else lr
+        pb = NNCPPutBit()
+        self.L.nncp_put_bit_init(C.byref(pb), out.ctypes.data, cap)
+        for pos in range(0, syms.size, block_len):
+            blk = syms[pos:pos + block_len].copy()
+            self.L.nncp_process_block(self.ptr, C.byref(pb), None, blk.ctypes.data, blk.size, 0, mode,
+                                      C.byref(sched), C.byref(st))
+            self.L.nncp_retrain_block(self.ptr, blk.ctypes.data, blk.size, C.byref(sched), C.byref(rst))
+        n = self.L.nncp_put_bit_flush(C.byref(pb))
+        if pb.overflow:
+            raise RuntimeError("output buffer too small")
+        return out[:n].copy(), st, rst
+
+    def decompress_blocks(self, data, n_syms, block_len, mode, lr=3e-4):
+        data = np.ascontiguousarray(data, dtype=np.uint8)
+        out = np.zeros(n_syms, dtype=np.uint16)
+        st, rst = NNCPStats(), NNCPStats()
+        sched = constant_lr(lr) if not isinstance(lr, NNCPInterp) else lr
+        gb = NNCPGetBit()
+        self.L.nncp_get_bit_init(C.byref(gb), data.ctypes.data, data.size)
+        for pos in range(0, n_syms, block_len):
+            blk = out[pos:pos + block_len]
+            self.L.nncp_process_block(self.ptr, None, C.byref(gb), blk.ctypes.data, blk.size, 1, mode,
+                                      C.byref(sched), C.byref(st))
+            self.L.nncp_retrain_block(self.ptr, blk.ctypes.data, blk.size, C.byref(sched), C.byref(rst))
+        return out, st, rst

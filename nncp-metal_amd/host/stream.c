@@ -255,6 +255,77 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
     nc_free_tensor(input);
 }
 
+int nncp_fifo_symbol(const uint16_t *buf, int rpos, int size, int idx) /* nncp.c:2811-2819 */
+{
+    if (idx < 0)
+        return 0;
+    return buf[(rpos + idx) % size];
+}
+
+void nncp_retrain_block(NNCPModel *s, const uint16_t *block_buf, int block_len,
+                        const NNCPInterp *lr, NNCPStats *st)
+{
+    const NNCPConfig *cfg = nncp_model_config(s);
+    NNCPRetrainState *r = nncp_model_retrain_state(s);
+    const int B = cfg->batch_size, T = cfg->seg_len;
+    if (cfg->retrain_period == 0)
+        return;
+    if (cfg->retrain_len <= 0)
+        die_stream("retrain needs a buffer (cfg.retrain_len > 0)");
+    if (!r->buf)
+        r->buf = nc_mallocz(sizeof(r->buf[0]) * cfg->retrain_len);
+    /* append the block, overwriting the oldest symbols (nncp.c:2837-2849) */
+    for (int pos = 0; pos < block_len;) {
+        int l = cfg->retrain_len - r->buf_pos;
+        if (l > block_len - pos)
+            l = block_len - pos;
+        memcpy(r->buf + r->buf_pos, block_buf + pos, sizeof(r->buf[0]) * l);
+        r->buf_pos += l;
+        if (r->buf_pos == cfg->retrain_len)
+            r->buf_pos = 0;
+        pos += l;
+    }
+    r->buf_len = r->buf_len + block_len < cfg->retrain_len ? r->buf_len + block_len : cfg->retrain_len;
+    r->pos += block_len;
+    if (r->pos < cfg->retrain_period)
+        return;
+    r->pos = 0;
+    const int stride = r->buf_len / B; /* nncp.c:2858 */
+    if (stride == 0)
+        return;
+
+    NCDevice *cpu = nncp_model_cpu_device(s);
+    NCTensor *input = nc_new_tensor_2d(cpu, NC_TYPE_I32, B, T);
+    NCTensor *expected = nc_new_tensor_2d(cpu, NC_TYPE_I32, B, T);
+    trf_set_retrain(s, 1);
+    trf_reset(s);
+    /* nncp.c:2882: whole segments while (seg_len + first) * B symbols are held */
+    for (int first = 0; r->buf_len >= (T + first) * B; first += T) {
+        for (int t = 0; t < T; t++)
+            for (int b = 0; b < B; b++) {
+                nc_set1_i32_2d(input, b, t, nncp_fifo_symbol(r->buf, r->buf_pos, r->buf_len, stride * b + first + t - 1));
+                nc_set1_i32_2d(expected, b, t, nncp_fifo_symbol(r->buf, r->buf_pos, r->buf_len, stride * b + first + t));
+            }
+        nc_free_tensor(trf_eval(s, -1, input));
+        const int64_t step = nncp_model_train_step(s);
+        trf_set_lr(s, cfg->has_retrain_lr ? nncp_interp(&cfg->retrain_lr, r->train_step) : nncp_interp(lr, step));
+        float loss = trf_eval_gradient(s, expected);
+        trf_update(s); /* advances the model's step counter */
+        if (cfg->has_retrain_lr) { /* nncp.c:2914-2918 */
+            nncp_model_set_train_step(s, step);
+            r->train_step++;
+        }
+        if (st) {
+            st->loss_bits -= loss / log(2.0);
+            st->n_steps++;
+            st->n_symbols += (int64_t)T * B;
+        }
+    }
+    nc_free_tensor(expected);
+    nc_free_tensor(input);
+    trf_set_retrain(s, 0);
+}
+
 size_t nncp_compress(NNCPModel *s, const uint16_t *syms, int n, uint8_t *out, size_t cap,
                      int mode, const NNCPInterp *lr, NNCPStats *st)
 {

@@ -41,6 +41,10 @@ struct NNCPModel {
     int seq_eval;
     float embed_mult;
     int64_t train_step;
+    /* retrain (nncp.c:183-193, 257-259): dropout is on only inside retrain_block */
+    int dropout_enabled;
+    int fused_now; /* cfg.fused, except while dropout is on (masks sit between the fused steps) */
+    NNCPRetrainState retrain;
 };
 
 static void die(const char *msg)
@@ -102,6 +106,7 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
     s->cpu = nc_new_cpu_device(s->ctx);
     s->dev = c->use_device ? nc_new_cuda_device(s->ctx, 0) : s->cpu;
     s->rnd = nc_rnd_init(s->dev, c->seed);
+    s->fused_now = c->fused;
     if (c->fused)
         nc_set_deferred_weight_grad(s->ctx, 1); /* backward_cb only forwards to sgd_opt_update_var */
     /* trf_init, nncp.c:304-520 */
@@ -171,6 +176,7 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
 
 void nncp_model_free(NNCPModel *s) /* trf_end nncp.c:522-550, nncp_end nncp.c:2802-2809 */
 {
+    nc_free(s->retrain.buf);
     trf_eval_end(s);
     for (int l = 0; l < s->cfg.n_layer; l++) {
         Layer *tl = &s->layers[l];
@@ -226,6 +232,17 @@ const char *nncp_model_param_name(NNCPModel *s, int index)
 /* ---- pieces shared by the evaluation paths ----------------------------------- */
 
 static NCTensor *scalar(NNCPModel *s, float v) { return nc_new_f32(s->dev, v); }
+
+/* nncp.c:290-298: a fresh mask of 0 / 1/(1-prob) from the model's random stream */
+static NCTensor *dropout_mul(NNCPModel *s, NCTensor *x, float prob)
+{
+    NCTensor *mask;
+    if (!s->dropout_enabled || prob == 0)
+        return x;
+    mask = nc_new_tensor_from_tensor_nz(x);
+    nc_tensor_set_dropout(mask, prob, s->rnd);
+    return nc_mul(x, mask);
+}
 
 static NCTensor *layer_norm(NNCPModel *s, NCTensor *x, NCTensor *g, NCTensor *b) /* nncp.c:279-288 */
 {
@@ -306,6 +323,7 @@ static NCTensor *attention_segment_ref(NNCPModel *s, int l, NCTensor *query, NCT
     t0 = nc_mul(t0, scalar(s, 1.0f / sqrtf((float)c->d_key)));
     t0 = nc_masked_fill(t0, nc_dup_tensor(tl->attn_mask), -INFINITY, 0);
     t0 = nc_soft_max(t0);
+    t0 = dropout_mul(s, t0, c->dropout_att_prob); /* nncp.c:797-799 */
     return nc_matmul(value, t0);
 }
 
@@ -401,6 +419,8 @@ static NCTensor *attention_ref(NNCPModel *s, int l, int output_index, NCTensor *
             nc_free_tensor(value0); nc_free_tensor(slot);
         }
     }
+    query = dropout_mul(s, query, c->dropout_prob); /* nncp.c:713-717; none on the keys */
+    value = dropout_mul(s, value, c->dropout_prob);
     key = split_head(key, H);
     query = split_head(query, H);
     value = split_head(value, H);
@@ -412,6 +432,7 @@ static NCTensor *attention_ref(NNCPModel *s, int l, int output_index, NCTensor *
         t0 = attention_timestep_ref(s, l, output_index, query, key, value);
     if (tl->w_o) {
         t0 = nc_matmul(nc_dup_tensor(tl->w_o), concat_head(t0));
+        t0 = dropout_mul(s, t0, c->dropout_prob); /* nncp.c:873-874 */
     } else { /* sum of the heads, nncp.c:875-890 */
         int axis[4] = { 0, 3, 1, 2 };
         t0 = nc_permute(t0, 4, axis);
@@ -456,7 +477,7 @@ static NCTensor *feed_forward(NNCPModel *s, int l, NCTensor *x, NCTensor *res)
     Layer *tl = &s->layers[l];
     NCTensor *t0, *tab[2];
     int act = c->ff_act;
-    if (c->fused && (act == NNCP_FF_GELU || act == NNCP_FF_RELU)) {
+    if (s->fused_now && (act == NNCP_FF_GELU || act == NNCP_FF_RELU)) {
         t0 = nc_linear(nc_dup_tensor(tl->ff1), x, tl->ff_bias1 ? nc_dup_tensor(tl->ff_bias1) : NULL,
                        act == NNCP_FF_GELU ? NC_ACT_GELU : NC_ACT_RELU);
         if (res)
@@ -469,6 +490,7 @@ static NCTensor *feed_forward(NNCPModel *s, int l, NCTensor *x, NCTensor *res)
     t0 = nc_matmul(nc_dup_tensor(tl->ff1), x);
     if (tl->ff_bias1)
         t0 = nc_add(t0, nc_dup_tensor(tl->ff_bias1));
+    t0 = dropout_mul(s, t0, c->dropout_prob); /* before the activation, nncp.c:933-934 */
     switch (act) {
     case NNCP_FF_RELU: t0 = nc_relu(t0); break;
     case NNCP_FF_GELU: t0 = nc_gelu(t0); break;
@@ -485,7 +507,7 @@ static NCTensor *feed_forward(NNCPModel *s, int l, NCTensor *x, NCTensor *res)
     t0 = nc_matmul(nc_dup_tensor(tl->ff2), t0);
     if (tl->ff_bias2)
         t0 = nc_add(t0, nc_dup_tensor(tl->ff_bias2));
-    return t0;
+    return dropout_mul(s, t0, c->dropout_prob); /* nncp.c:973-974 */
 }
 
 static void free_position_tensors(NNCPModel *s)
@@ -502,7 +524,11 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
     int seg_len, B = c->batch_size;
     NCTensor *t0, *x, *output;
 
-    if (c->fused && output_index >= 0)
+    /* dropout masks sit between steps that the fused entry points merge, so a
+       retrain pass goes through the op-by-op sequence */
+    s->fused_now = c->fused && !s->dropout_enabled;
+    const int fused = s->fused_now;
+    if (fused && output_index >= 0)
         die("the fused path evaluates whole segments only (output_index < 0)");
     if (output_index < 0) { /* nncp.c:612-623 */
         t0 = nc_dup_tensor(input);
@@ -517,6 +543,7 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
     t0 = nc_reshape_1d(t0, (size_t)B * seg_len);
     x = nc_get_col(nc_dup_tensor(s->embed), t0);
     x = nc_mul(x, scalar(s, s->embed_mult));
+    x = dropout_mul(s, x, c->dropout_prob); /* nncp.c:631-633 */
 
     for (int l = 0; l < c->n_layer; l++) {
         Layer *tl = &s->layers[l];
@@ -526,12 +553,12 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
         save_layer_input(s, l, output_index, x1, seg_len);
         /* the fused path folds the residual sums (nncp.c:896, 979) into the
            GEMMs that produce their other operand */
-        int fold = c->fused && !(c->ln_flags & NNCP_LN_COEF);
+        int fold = fused && !(c->ln_flags & NNCP_LN_COEF);
         int fold_ff = fold && (c->ff_act == NNCP_FF_GELU || c->ff_act == NNCP_FF_RELU);
         if (fold) {
             t0 = attention_fused(s, l, x1, x);
         } else {
-            t0 = c->fused ? attention_fused(s, l, x1, NULL) : attention_ref(s, l, output_index, x1, seg_len);
+            t0 = fused ? attention_fused(s, l, x1, NULL) : attention_ref(s, l, output_index, x1, seg_len);
             if (c->ln_flags & NNCP_LN_COEF)
                 t0 = nc_mul(t0, nc_dup_tensor(tl->alpha));
             t0 = nc_add(t0, x); /* residual, nncp.c:896 */
@@ -555,8 +582,9 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
     }
     if (c->ln_flags & NNCP_LN_FINAL)
         x = layer_norm(s, x, s->ln_g, s->ln_b);
+    x = dropout_mul(s, x, c->dropout_prob); /* nncp.c:997-999 */
     /* logits and probabilities, nncp.c:1001-1009 */
-    if (c->fused) {
+    if (fused) {
         t0 = nc_linear(nc_dup_tensor(s->embed_out), x, s->out_bias ? nc_dup_tensor(s->out_bias) : NULL, NC_ACT_NONE);
     } else {
         t0 = nc_matmul(nc_dup_tensor(s->embed_out), x);
@@ -570,7 +598,7 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
     if (s->outputs[output_index < 0 ? 0 : output_index])
         die("trf_eval: previous evaluation not consumed (call trf_eval_gradient or trf_eval_end)");
     s->outputs[output_index < 0 ? 0 : output_index] = nc_dup_tensor(output);
-    if (!c->fused && (output_index < 0 || output_index == c->seg_len - 1))
+    if (!fused && (output_index < 0 || output_index == c->seg_len - 1))
         free_position_tensors(s);
     return output;
 }
@@ -598,6 +626,9 @@ void trf_step_begin(NNCPModel *s)
     const NNCPConfig *c = &s->cfg;
     if (!c->fused)
         die("per-timestep cached evaluation needs the fused path (cfg.fused = 1)");
+    if (s->dropout_enabled)
+        die("per-timestep cached evaluation is a decoding path: not during a retrain pass");
+    s->fused_now = 1;
     if (!s->step_kv) {
         s->step_kv = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
         s->step_kvm = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
@@ -784,3 +815,11 @@ void trf_update(NNCPModel *s) /* nncp.c:1224-1235 with mem_update nncp.c:1205-12
 }
 
 void trf_set_lr(NNCPModel *s, float lr) { nc_sgd_opt_set_lr(s->opt, lr); }
+
+void trf_set_retrain(NNCPModel *s, int enabled) /* nncp.c:1237-1241 */
+{
+    s->dropout_enabled = enabled && s->cfg.dropout_prob != 0;
+}
+
+NNCPRetrainState *nncp_model_retrain_state(NNCPModel *s) { return &s->retrain; }
+void nncp_model_set_train_step(NNCPModel *s, int64_t step) { s->train_step = step; }

@@ -157,3 +157,102 @@ def test_step_decode_round_trip(H, n, coder):
     dec.close()
     assert np.array_equal(out, syms)
     assert st.n_symbols == n
+
+
+# ---- retrain passes with dropout (nncp.c:2821-2941, 290-298) ----------------------
+def test_fifo_symbol_is_oldest_first(H):
+    """nncp_fifo_symbol against a plain Python FIFO: index 0 is the oldest symbol
+    held, also after the ring has wrapped; negative indices read 0."""
+    import ctypes as C
+    rng = np.random.default_rng(5)
+    size = 13
+    ring = np.zeros(size, dtype=np.uint16)
+    fifo, pos = [], 0
+    for step in range(40):
+        v = int(rng.integers(1, 1000))
+        ring[pos] = v
+        pos = (pos + 1) % size
+        fifo = (fifo + [v])[-size:]
+        held = len(fifo)
+        # the reference passes (buffer, next write position, symbols held)
+        for idx in {-2, -1, 0, min(1, held - 1), held // 2, held - 1}:
+            want = 0 if idx < 0 else fifo[idx]
+            got = H.lib.nncp_fifo_symbol(ring.ctypes.data_as(C.c_void_p), pos % held, held, idx)
+            assert got == want, (step, idx)
+
+
+@pytest.mark.parametrize("fused", [0, 1])
+@pytest.mark.parametrize("own_lr", [False, True])
+def test_retrain_round_trip(H, fused, own_lr):
+    """Three blocks through one coder with a retrain pass (dropout on) after
+    each: the decoder, replaying the passes on what it decoded, recovers the
+    input and ends with the encoder's weights, bit for bit."""
+    B, T = M.TINY["batch_size"], M.TINY["seg_len"]
+    block = B * T * 3 + 5
+    syms = M.markov1(3 * block - 7, 40, seed=21)
+    kw = dict(fused=fused, sgd_opt=M.rmsprop(), dropout_prob=0.1, dropout_att_prob=0.05,
+              retrain_period=1, retrain_len=2 * block)
+    if own_lr:
+        kw["retrain_lr"] = 1e-4
+    enc = _model(H, **kw)
+    data, st, rst = enc.compress_blocks(syms, block, 1)
+    w_enc, steps_enc = enc.params(), enc.L.nncp_model_train_step(enc.ptr)
+    enc.close()
+    dec = _model(H, **kw)
+    out, _, rst_d = dec.decompress_blocks(data, len(syms), block, 1)
+    w_dec = dec.params()
+    dec.close()
+    assert np.array_equal(out, syms)
+    for k in w_enc:
+        assert np.array_equal(w_enc[k], w_dec[k]), k
+    # passes over 1, 2 and 2 blocks of the buffer, (3 or 6) whole segments each... counted, not assumed:
+    assert rst.n_steps == rst_d.n_steps > 0 and rst.n_symbols == rst.n_steps * B * T
+    coded_steps = st.n_steps
+    assert steps_enc == (coded_steps if own_lr else coded_steps + rst.n_steps)
+
+
+def test_retrain_changes_the_model_and_dropout_is_seeded(H):
+    B, T = M.TINY["batch_size"], M.TINY["seg_len"]
+    block = B * T * 2
+    syms = M.markov1(2 * block, 40, seed=4)
+    res = {}
+    for name, kw in (("plain", {}), ("retrain", dict(retrain_period=1, retrain_len=block)),
+                     ("drop_a", dict(retrain_period=1, retrain_len=block, dropout_prob=0.2)),
+                     ("drop_b", dict(retrain_period=1, retrain_len=block, dropout_prob=0.2))):
+        m = _model(H, sgd_opt=M.rmsprop(), **kw)
+        data, _, rst = m.compress_blocks(syms, block, 1)
+        res[name] = (data.tobytes(), m.get_param("ff1_0"), rst.n_steps)
+        m.close()
+    assert res["plain"][2] == 0 and res["retrain"][2] > 0
+    assert res["plain"][0] != res["retrain"][0]          # the second block is coded by a retrained model
+    assert not np.array_equal(res["retrain"][1], res["drop_a"][1])   # masks act
+    assert res["drop_a"][0] == res["drop_b"][0] and np.array_equal(res["drop_a"][1], res["drop_b"][1])
+
+
+def test_dropout_path_equals_plain_path_at_probability_zero(H):
+    """With dropout_prob = 0 trf_set_retrain(1) changes nothing (nncp.c:1240),
+    in particular a fused model keeps its fused path."""
+    tok = M.markov1(3 * 8, 40, seed=9).astype(np.int32).reshape(8, 3)
+    for fused in (0, 1):
+        m = _model(H, fused=fused)
+        p0 = m.eval(tok)
+        m.L.trf_set_retrain(m.ptr, 1)
+        p1 = m.eval(tok)
+        m.close()
+        assert np.array_equal(p0, p1)
+
+
+def test_dropout_masks_scale_and_rate(H):
+    """Inverted dropout: the expectation of the masked evaluation is the plain
+    one; checked through the mean of the mask itself (0 or 1/(1-p))."""
+    pkg = M.load_pkg()
+    nc = pkg.binding.NC(M.REF_LIB, use_device=False)
+    x = nc.tensor(np.zeros((200, 300), np.float32))
+    rs = nc.lib.nc_rnd_init(None, 77)
+    nc.lib.nc_tensor_set_dropout(x, 0.25, rs)
+    m = nc.numpy(x, free=True)
+    nc.lib.nc_rnd_end(rs)
+    nc.close()
+    vals = np.unique(m)
+    assert len(vals) == 2 and vals[0] == 0 and abs(vals[1] - 1 / 0.75) < 1e-6
+    assert abs((m == 0).mean() - 0.25) < 0.01 and abs(m.mean() - 1.0) < 0.02
