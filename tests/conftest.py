@@ -44,9 +44,15 @@ def ref(pkg):
     nc.close()
 
 
+def hip_lib_path(pkg):
+    """The product library, or - for tests/test_kernels_on_cpu.py, which re-runs the GPU
+    op tests without a GPU - the same sources built for the host (tests/hipcpu)."""
+    return os.environ.get("NNCP_TEST_HIP_LIB") or pkg.binding.HIP_LIB
+
+
 @pytest.fixture()
 def hip(pkg):
-    nc = pkg.binding.NC(pkg.binding.HIP_LIB, use_device=True)
+    nc = pkg.binding.NC(hip_lib_path(pkg), use_device=True)
     yield nc
     nc.close()
 

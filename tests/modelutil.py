@@ -21,7 +21,12 @@ def ref_host():
 
 
 def hip_host():
+    """The product pair of libraries, or - when tests/test_kernels_on_cpu.py re-runs
+    GPU tests without a GPU - the same sources built for the host (tests/hipcpu)."""
     pkg = load_pkg()
+    emu, emu_host = os.environ.get("NNCP_TEST_HIP_LIB"), os.environ.get("NNCP_TEST_HOST_HIP_LIB")
+    if emu and emu_host:
+        return pkg.host.Host(emu_host, emu)
     return pkg.host.Host()
 
 
