@@ -67,3 +67,18 @@ def test_host_tensor_compute_is_refused(emulated):
             "nc.nc_add(a, nc.dup(a))") % (os.path.join(ROOT, "tests"),)
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=emulated)
     assert r.returncode != 0 and "GPU only" in r.stderr
+
+
+def test_random_shapes_stay_in_bounds_and_match(emulated):
+    """Seeded random campaigns through the raw kernel entry points of the CPU build, each
+    operand in an exact-size buffer ending at a guard page: GEMM (layouts, paddings, batches,
+    split-K, fp32 / bf16 / bf16 from copies, forced tile configurations, epilogue options),
+    attention (both generations, backward, single-query step), integer CDF and lookup."""
+    jobs = [("fuzz_gemm.py", "101", "150"), ("fuzz_gemm.py", "102", "150"), ("fuzz_attn.py", "103", "12"),
+            ("fuzz_attn.py", "104", "12"), ("fuzz_cdf.py", "105", "25")]
+    procs = [subprocess.Popen([sys.executable, os.path.join(EMU_DIR, name), seed, count], env=emulated,
+                              stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+             for name, seed, count in jobs]
+    for job, p in zip(jobs, procs):
+        out = p.communicate(timeout=1500)[0]
+        assert p.returncode == 0 and out.strip().startswith("ok:"), (job, out[-3000:])
