@@ -93,7 +93,22 @@ typedef struct { /* TransformerModelParams + the NNCPModelParams fields it needs
     int retrain_len;     /* length of the retrain buffer, in symbols */
     int has_retrain_lr;
     NNCPInterp retrain_lr;
+    /* model class (NNCPModelParams.model_class): 0 = Transformer-XL, the fields
+       above; 1 = LSTM (LSTMParams, nncp.c:124-140), which uses n_layer,
+       batch_size, seg_len, n_symbols, seed, sgd_opt, use_device, nb_threads
+       from above and the fields below */
+    int model_type;
+    int lstm_n_cells, lstm_n_cells2, lstm_n_embed_out; /* n_cells2 >= n_cells: with projection */
+    int lstm_type;                                     /* NNCP_LSTM_* */
+    int lstm_full_connect, lstm_use_layer_norm;
+    float lstm_forget_bias;
 } NNCPConfig;
+
+#define NNCP_MODEL_TRF 0
+#define NNCP_MODEL_LSTM 1
+#define NNCP_LSTM_NORMAL 0  /* nncp.c:117-122 */
+#define NNCP_LSTM_CLAMPED 1
+#define NNCP_LSTM_TIED 2
 
 typedef struct { /* nncp.c:183-193 */
     uint16_t *buf;
@@ -105,6 +120,7 @@ typedef struct { /* nncp.c:183-193 */
 typedef struct NNCPModel NNCPModel;
 
 void nncp_config_default(NNCPConfig *cfg);           /* nncp.c:2471-2513 */
+void nncp_config_default_lstm(NNCPConfig *cfg);      /* the "lstm" profile, nncp.c:2574-2603 */
 NNCPModel *nncp_model_new(const NNCPConfig *cfg);    /* nncp_init + trf_init, nncp.c:2762, 304 */
 void nncp_model_free(NNCPModel *s);                  /* nncp_end + trf_end, nncp.c:2802, 522 */
 const NNCPConfig *nncp_model_config(NNCPModel *s);
@@ -133,6 +149,30 @@ NNCPRetrainState *nncp_model_retrain_state(NNCPModel *s);
 void nncp_model_set_train_step(NNCPModel *s, int64_t step);
 /* logits of the last trf_eval (V, B, T|1), borrowed; used by the CDF path */
 NCTensor *trf_last_logits(NNCPModel *s);
+/* the `lstm` model class (nncp.c:1565-2330: lstm_eval, lstm_eval_gradient, ...),
+   same calling conventions; n_states = seg_len (no overlap), no dropout */
+NCTensor *lstm_eval(NNCPModel *s, int output_index, const NCTensor *input); /* nncp.c:1872 */
+void lstm_eval_end(NNCPModel *s);                                           /* nncp.c:2060 */
+float lstm_eval_gradient(NNCPModel *s, const NCTensor *expected_output);    /* nncp.c:2070 */
+void lstm_reset(NNCPModel *s);                                              /* nncp.c:1859 */
+void lstm_update(NNCPModel *s);                                             /* nncp.c:2136 */
+
+/* NNCPModelClass (nncp.c:49-69): what the block loop calls; trf_* or lstm_* */
+typedef struct {
+    NCTensor *(*eval)(NNCPModel *s, int output_index, const NCTensor *input);
+    void (*eval_end)(NNCPModel *s);
+    float (*eval_gradient)(NNCPModel *s, const NCTensor *expected_output);
+    void (*reset)(NNCPModel *s);
+    void (*update)(NNCPModel *s);
+    void (*set_lr)(NNCPModel *s, float lr);
+    void (*set_retrain)(NNCPModel *s, int enabled);
+    NCTensor *(*last_logits)(NNCPModel *s); /* logits of the last eval, borrowed */
+    /* eval_end for an evaluation that is to leave no trace (the replaying decoder of
+       NNCP_MODE_SEGMENT): also takes back the recurrent state it handed on */
+    void (*eval_discard)(NNCPModel *s);
+} NNCPModelClass;
+const NNCPModelClass *nncp_model_class(NNCPModel *s);
+
 /* Per-timestep evaluation with K/V caches through the fused entry points (the
    decoder's view of a segment, nncp.c:801-863; cfg.fused = 1 and the shapes of
    the single-kernel attention).  trf_step_begin once per segment, then

@@ -32,7 +32,10 @@ class NNCPConfig(C.Structure):
                [(n, C.c_int) for n in ("batch_size", "seg_len", "n_symbols")] + \
                [("seed", C.c_uint32), ("use_device", C.c_int), ("fused", C.c_int), ("nb_threads", C.c_int)] + \
                [("dropout_prob", C.c_float), ("dropout_att_prob", C.c_float), ("retrain_period", C.c_int),
-                ("retrain_len", C.c_int), ("has_retrain_lr", C.c_int), ("retrain_lr", NNCPInterp)]
+                ("retrain_len", C.c_int), ("has_retrain_lr", C.c_int), ("retrain_lr", NNCPInterp)] + \
+               [(n, C.c_int) for n in ("model_type", "lstm_n_cells", "lstm_n_cells2", "lstm_n_embed_out",
+                                       "lstm_type", "lstm_full_connect", "lstm_use_layer_norm")] + \
+               [("lstm_forget_bias", C.c_float)]
 
 
 class NNCPStats(C.Structure):
@@ -50,6 +53,27 @@ class NNCPPutBit(C.Structure):
 class NNCPGetBit(C.Structure):
     _fields_ = [("buf", C.c_void_p), ("buf_len", C.c_size_t), ("idx", C.c_size_t),
                 ("low", C.c_uint32), ("range", C.c_uint32)]
+
+
+MODEL_TRF, MODEL_LSTM = 0, 1
+LSTM_NORMAL, LSTM_CLAMPED, LSTM_TIED = 0, 1, 2
+
+
+def make_lstm_config(**kw):
+    """nncp's "lstm" profile (nncp.c:2574-2603) with overrides."""
+    cfg = NNCPConfig()
+    opt = kw.pop("sgd_opt", None)
+    base = dict(model_type=MODEL_LSTM, n_layer=4, lstm_n_cells=352, lstm_type=LSTM_CLAMPED, lstm_full_connect=1,
+                lstm_use_layer_norm=1, lstm_forget_bias=0.0, batch_size=32, seg_len=20, n_symbols=256, seed=123,
+                use_device=1, nb_threads=1)
+    base.update(kw)
+    base.setdefault("lstm_n_cells2", base["lstm_n_cells"])
+    base.setdefault("lstm_n_embed_out", base["n_layer"])
+    for k, v in base.items():
+        setattr(cfg, k, v)
+    cfg.sgd_opt = opt if opt is not None else B.SGDOptParams(
+        algo=B.SGD_OPT_ADAM, beta1=0.0, beta2=0.9999, eps=1e-10, gradient_clip=0.0, lr=4e-3)
+    return cfg
 
 
 def constant_lr(lr):
@@ -120,6 +144,13 @@ class Host:
         L.trf_update.argtypes = [_P]
         L.trf_set_lr.argtypes = [_P, C.c_float]
         L.trf_set_retrain.argtypes = [_P, C.c_int]
+        L.lstm_eval.restype = _P
+        L.lstm_eval.argtypes = [_P, C.c_int, _P]
+        L.lstm_eval_end.argtypes = [_P]
+        L.lstm_eval_gradient.restype = C.c_float
+        L.lstm_eval_gradient.argtypes = [_P, _P]
+        L.lstm_reset.argtypes = [_P]
+        L.lstm_update.argtypes = [_P]
         L.nncp_process_block.argtypes = [_P, C.POINTER(NNCPPutBit), C.POINTER(NNCPGetBit), _P, C.c_int, C.c_int,
                                          C.c_int, C.POINTER(NNCPInterp), C.POINTER(NNCPStats)]
         L.nncp_retrain_block.argtypes = [_P, _P, C.c_int, C.POINTER(NNCPInterp), C.POINTER(NNCPStats)]
@@ -163,6 +194,11 @@ class Model:
         self.dev = self.L.nncp_model_device(self.ptr)
         self.cpu = self.L.nncp_model_cpu_device(self.ptr)
         self.ctx = self.L.nncp_model_context(self.ptr)
+        # the entry points of the model class in use (trf_* or lstm_*)
+        pre = "lstm" if cfg.model_type == MODEL_LSTM else "trf"
+        self._eval, self._eval_end = getattr(self.L, pre + "_eval"), getattr(self.L, pre + "_eval_end")
+        self._eval_gradient, self._update = getattr(self.L, pre + "_eval_gradient"), getattr(self.L, pre + "_update")
+        self._reset = getattr(self.L, pre + "_reset")
 
     def close(self):
         if self.ptr:
@@ -212,12 +248,12 @@ class Model:
         """tokens: int array (T, B) [numpy order of the (B, T) input tensor].
         Returns the probabilities as numpy (T|1, B, V)."""
         inp = self._host_tensor(np.asarray(tokens, dtype=np.int32))
-        out = self.L.trf_eval(self.ptr, output_index, inp)
+        out = self._eval(self.ptr, output_index, inp)
         self.nc.nc_free_tensor(inp)
         res = self._to_numpy(out)
         self.nc.nc_free_tensor(out)
         if not keep:
-            self.L.trf_eval_end(self.ptr)
+            self._eval_end(self.ptr)
         return res
 
     def logits(self):
@@ -245,10 +281,10 @@ class Model:
         (probabilities, loss in nats summed over the segment)."""
         p = self.eval(tokens, -1, keep=True)
         tgt = self._host_tensor(np.asarray(targets, dtype=np.int32))
-        self.L.trf_set_lr(self.ptr, lr)
-        loss = self.L.trf_eval_gradient(self.ptr, tgt)
+        self.L.trf_set_lr(self.ptr, lr)  # both classes: nc_sgd_opt_set_lr on the model's optimiser
+        loss = self._eval_gradient(self.ptr, tgt)
         self.nc.nc_free_tensor(tgt)
-        self.L.trf_update(self.ptr)
+        self._update(self.ptr)
         return p, -loss
 
     def compress(self, syms, mode, lr=3e-4):

@@ -58,6 +58,7 @@ static void put_symb(BlockView *v, int stream, int pos, int c) /* nncp.c:2956-29
 
 typedef struct {
     NNCPModel *s;
+    const NNCPModelClass *cls;
     NNCPPutBit *pb;
     NNCPGetBit *gb;
     BlockView view;
@@ -79,7 +80,7 @@ static HostDist fetch_dist(Coder *c, NCTensor *output)
     HostDist d;
     memset(&d, 0, sizeof(d));
     if (c->coder == NNCP_CODER_CDF16) {
-        NCTensor *cdf = nc_soft_max_cdf16(nc_dup_tensor(trf_last_logits(c->s)));
+        NCTensor *cdf = nc_soft_max_cdf16(nc_dup_tensor(c->cls->last_logits(c->s)));
         nc_free_tensor(output);
         d.host = nc_tensor_to_cpu_device(cdf);
         d.cdf = nc_tensor_get_ptr(d.host, &d.stride);
@@ -125,7 +126,7 @@ static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int ful
             for (int b = 0; b < B; b++)
                 nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
         t0 = now_s();
-        NCTensor *out = trf_eval(s, -1, input);
+        NCTensor *out = c->cls->eval(s, -1, input);
         HostDist d = fetch_dist(c, out);
         c->st->t_eval += now_s() - t0;
         t0 = now_s();
@@ -161,7 +162,7 @@ static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int ful
         trf_step_end(s);
         if (expected) { /* the graph the encoder differentiated: one whole-segment evaluation */
             t0 = now_s();
-            nc_free_tensor(trf_eval(s, -1, input));
+            nc_free_tensor(c->cls->eval(s, -1, input));
             c->st->t_eval += now_s() - t0;
         }
         return;
@@ -171,7 +172,7 @@ static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int ful
         for (int b = 0; b < B; b++)
             nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
         t0 = now_s();
-        NCTensor *out = trf_eval(s, mode == NNCP_MODE_SEGMENT ? -1 : t, input);
+        NCTensor *out = c->cls->eval(s, mode == NNCP_MODE_SEGMENT ? -1 : t, input);
         HostDist d = fetch_dist(c, out);
         c->st->t_eval += now_s() - t0;
         t0 = now_s();
@@ -186,7 +187,7 @@ static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int ful
         /* replayed segment evaluations are discarded, except the last one of a
            trained segment, whose graph the gradient needs */
         if (mode == NNCP_MODE_SEGMENT && !(expected && t == n_t - 1))
-            trf_eval_end(s);
+            c->cls->eval_discard(s);
     }
     /* decoder in segment mode: the last replay was built once every input of
        the segment was known (the last symbol is a target only), so its graph
@@ -202,11 +203,13 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
     int mode = mode_flags & 1;
     memset(&local, 0, sizeof(local));
     memset(&c, 0, sizeof(c));
-    c.s = s; c.pb = pb; c.gb = gb; c.is_decode = is_decode;
+    c.s = s; c.cls = nncp_model_class(s); c.pb = pb; c.gb = gb; c.is_decode = is_decode;
     c.coder = mode_flags & NNCP_CODER_CDF16;
     if (mode_flags & NNCP_MODE_STEP_DECODE) {
         if (mode != NNCP_MODE_SEGMENT)
             die_stream("NNCP_MODE_STEP_DECODE goes with NNCP_MODE_SEGMENT");
+        if (nncp_model_config(s)->model_type != NNCP_MODEL_TRF)
+            die_stream("NNCP_MODE_STEP_DECODE is a path of the Transformer model class");
         /* both sides: products whose columns do not depend on how many are computed together */
         nc_set_matmul_width_invariant(nncp_model_context(s), 1);
         c.step_decode = is_decode;
@@ -224,18 +227,18 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
     NCDevice *cpu = nncp_model_cpu_device(s);
     NCTensor *input = nc_new_tensor_2d(cpu, NC_TYPE_I32, B, T);
     NCTensor *expected = nc_new_tensor_2d(cpu, NC_TYPE_I32, B, T);
-    trf_reset(s); /* nncp.c:2988 */
+    c.cls->reset(s); /* nncp.c:2988 */
 
     int idx = 0;
     while (idx + T <= c.view.stride) { /* nncp.c:2993 */
         code_segment(&c, mode, idx, T, T, 1, input, expected);
         float rate = nncp_interp(lr, nncp_model_train_step(s)); /* nncp.c:3048-3050 */
-        trf_set_lr(s, rate);
+        c.cls->set_lr(s, rate);
         double t0 = now_s();
-        float loss = trf_eval_gradient(s, expected);
+        float loss = c.cls->eval_gradient(s, expected);
         c.st->t_grad += now_s() - t0;
         t0 = now_s();
-        trf_update(s);
+        c.cls->update(s);
         c.st->t_update += now_s() - t0;
         c.st->loss_bits -= loss / log(2.0);
         c.st->n_steps++;
@@ -248,7 +251,7 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
             for (int b = 0; b < B; b++)
                 nc_set1_i32_2d(input, b, t, 0);
         code_segment(&c, mode, idx, len1, len2, 0, input, NULL);
-        trf_eval_end(s);
+        c.cls->eval_end(s);
         c.st->n_symbols += (int64_t)len2 * B + c.view.rem;
     }
     nc_free_tensor(expected);
@@ -267,6 +270,7 @@ void nncp_retrain_block(NNCPModel *s, const uint16_t *block_buf, int block_len,
 {
     const NNCPConfig *cfg = nncp_model_config(s);
     NNCPRetrainState *r = nncp_model_retrain_state(s);
+    const NNCPModelClass *cls = nncp_model_class(s);
     const int B = cfg->batch_size, T = cfg->seg_len;
     if (cfg->retrain_period == 0)
         return;
@@ -297,8 +301,8 @@ void nncp_retrain_block(NNCPModel *s, const uint16_t *block_buf, int block_len,
     NCDevice *cpu = nncp_model_cpu_device(s);
     NCTensor *input = nc_new_tensor_2d(cpu, NC_TYPE_I32, B, T);
     NCTensor *expected = nc_new_tensor_2d(cpu, NC_TYPE_I32, B, T);
-    trf_set_retrain(s, 1);
-    trf_reset(s);
+    cls->set_retrain(s, 1);
+    cls->reset(s);
     /* nncp.c:2882: whole segments while (seg_len + first) * B symbols are held */
     for (int first = 0; r->buf_len >= (T + first) * B; first += T) {
         for (int t = 0; t < T; t++)
@@ -306,11 +310,11 @@ void nncp_retrain_block(NNCPModel *s, const uint16_t *block_buf, int block_len,
                 nc_set1_i32_2d(input, b, t, nncp_fifo_symbol(r->buf, r->buf_pos, r->buf_len, stride * b + first + t - 1));
                 nc_set1_i32_2d(expected, b, t, nncp_fifo_symbol(r->buf, r->buf_pos, r->buf_len, stride * b + first + t));
             }
-        nc_free_tensor(trf_eval(s, -1, input));
+        nc_free_tensor(cls->eval(s, -1, input));
         const int64_t step = nncp_model_train_step(s);
-        trf_set_lr(s, cfg->has_retrain_lr ? nncp_interp(&cfg->retrain_lr, r->train_step) : nncp_interp(lr, step));
-        float loss = trf_eval_gradient(s, expected);
-        trf_update(s); /* advances the model's step counter */
+        cls->set_lr(s, cfg->has_retrain_lr ? nncp_interp(&cfg->retrain_lr, r->train_step) : nncp_interp(lr, step));
+        float loss = cls->eval_gradient(s, expected);
+        cls->update(s); /* advances the model's step counter */
         if (cfg->has_retrain_lr) { /* nncp.c:2914-2918 */
             nncp_model_set_train_step(s, step);
             r->train_step++;
@@ -323,7 +327,7 @@ void nncp_retrain_block(NNCPModel *s, const uint16_t *block_buf, int block_len,
     }
     nc_free_tensor(expected);
     nc_free_tensor(input);
-    trf_set_retrain(s, 0);
+    cls->set_retrain(s, 0);
 }
 
 size_t nncp_compress(NNCPModel *s, const uint16_t *syms, int n, uint8_t *out, size_t cap,

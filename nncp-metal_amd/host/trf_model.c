@@ -14,38 +14,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
-#include "../../include/nncp_host.h"
-
-typedef struct {
-    NCTensor *w_q, *w_kv, *b_q, *w_o;
-    NCTensor *ff1, *ff2, *ff_bias1, *ff_bias2;
-    NCTensor *w_r, *b_r;
-    NCTensor *ln_g1, *ln_b1, *ln_g2, *ln_b2, *alpha;
-    /* per-timestep evaluation only */
-    NCTensor *mem_key, *mem_value, *tmp_w_r, *tmp_b_r, *attn_mask;
-    NCNode **key_nodes, **kq_nodes, **value_nodes, **va_nodes;
-} Layer;
-
-struct NNCPModel {
-    NNCPConfig cfg;
-    NCContext *ctx;
-    NCDevice *dev, *cpu;
-    NCRNDState *rnd;
-    NCParamList params;
-    Layer *layers;
-    NCTensor *ln_g, *ln_b, *embed, *embed_out, *out_bias;
-    NCTensor **mem_h, **train_h, **outputs;
-    NCTensor **step_kv, **step_kvm; /* per-timestep decoding: K/V of the segment so far, K/V of the memory */
-    NCTensor *logits;
-    NCSGDOptState *opt;
-    int seq_eval;
-    float embed_mult;
-    int64_t train_step;
-    /* retrain (nncp.c:183-193, 257-259): dropout is on only inside retrain_block */
-    int dropout_enabled;
-    int fused_now; /* cfg.fused, except while dropout is on (masks sit between the fused steps) */
-    NNCPRetrainState retrain;
-};
+#include "model_internal.h"
 
 static void die(const char *msg)
 {
@@ -97,6 +66,17 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
     const NNCPConfig *c;
     s->cfg = *cfg;
     c = &s->cfg;
+    if (c->model_type == NNCP_MODEL_LSTM) {
+        /* nncp_init, nncp.c:2770-2779, then lstm_init */
+        s->ctx = nc_context_init(c->nb_threads);
+        s->cpu = nc_new_cpu_device(s->ctx);
+        s->dev = c->use_device ? nc_new_cuda_device(s->ctx, 0) : s->cpu;
+        s->rnd = nc_rnd_init(s->dev, c->seed);
+        s->cls = &nncp_lstm_class;
+        lstm_init(s);
+        return s;
+    }
+    s->cls = &nncp_trf_class;
     if (c->n_layer < 1 || c->n_layer > NNCP_N_LAYER_MAX || c->d_model != c->d_key * c->n_head)
         die("bad configuration (need d_model == d_key * n_head, 1 <= n_layer <= 32)");
     int T = c->seg_len, M = c->mem_len, K = T + M, B = c->batch_size, H = c->n_head, D = c->d_model;
@@ -177,6 +157,13 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
 void nncp_model_free(NNCPModel *s) /* trf_end nncp.c:522-550, nncp_end nncp.c:2802-2809 */
 {
     nc_free(s->retrain.buf);
+    if (s->cfg.model_type == NNCP_MODEL_LSTM) {
+        lstm_end(s);
+        nc_rnd_end(s->rnd);
+        nc_context_end(s->ctx);
+        nc_free(s);
+        return;
+    }
     trf_eval_end(s);
     for (int l = 0; l < s->cfg.n_layer; l++) {
         Layer *tl = &s->layers[l];
@@ -728,7 +715,7 @@ void trf_eval_end(NNCPModel *s) /* nncp.c:1032-1060 */
     s->logits = NULL;
 }
 
-static void backward_cb(void *opaque, NCTensor *yg, NCTensor *get_col_index) /* nncp.c:1078-1096 */
+void nncp_backward_cb(void *opaque, NCTensor *yg, NCTensor *get_col_index) /* nncp.c:1078-1096 */
 {
     sgd_opt_update_var(opaque, yg, get_col_index);
 }
@@ -786,7 +773,7 @@ float trf_eval_gradient(NNCPModel *s, const NCTensor *expected_output1) /* nncp.
     loss = nc_sum(loss);
     ret = nc_get_scalar_f32(loss);
     loss = nc_mul(loss, nc_new_f32(nc_get_tensor_device(loss), -1.0f / (float)(c->seg_len * c->batch_size)));
-    nc_backward(loss, nc_new_f32(s->dev, 1.0f), backward_cb, 0);
+    nc_backward(loss, nc_new_f32(s->dev, 1.0f), nncp_backward_cb, 0);
     nc_free_tensor(loss);
     nc_free_tensor(s->logits);
     s->logits = NULL;
@@ -823,3 +810,10 @@ void trf_set_retrain(NNCPModel *s, int enabled) /* nncp.c:1237-1241 */
 
 NNCPRetrainState *nncp_model_retrain_state(NNCPModel *s) { return &s->retrain; }
 void nncp_model_set_train_step(NNCPModel *s, int64_t step) { s->train_step = step; }
+
+const NNCPModelClass nncp_trf_class = { /* nncp.c:1544-1562 */
+    trf_eval, trf_eval_end, trf_eval_gradient, trf_reset, trf_update, trf_set_lr, trf_set_retrain, trf_last_logits,
+    trf_eval_end, /* no state is handed on before trf_update */
+};
+
+const NNCPModelClass *nncp_model_class(NNCPModel *s) { return s->cls; }

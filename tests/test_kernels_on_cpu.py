@@ -44,17 +44,21 @@ def test_gpu_parity_tests_pass_on_the_cpu_build(emulated):
     256 keys, integer CDF and lookup bit-exactness, optimiser, ...) and a
     model-level subset (training steps against the checker op by op and fused,
     whole-model gradient, cached per-timestep logits bit-identical, a profile
-    variant), with guard pages behind every device buffer."""
+    variant, the retrain pass and the LSTM model class), with guard pages behind every
+    device buffer."""
     ops = _pytest(emulated, ["-n", "5", "tests/test_gpu_ops.py"])
     model = _pytest(emulated, ["-n", "3", "tests/test_gpu_model.py", "-k",
                                "(test_training_steps_match_checker and TINY) or "
                                "(test_cached_timestep_logits_are_bit_identical and SMALL32) or "
                                "test_gradients_match_checker_c1 or "
                                "(test_profile_variants_match_checker and 1-relu_coef)"])
+    new = _pytest(emulated, ["-n", "4", "tests/test_gpu_zz_new_paths.py"])
     out_ops, out_model = ops.communicate(timeout=1500)[0], model.communicate(timeout=1500)[0]
+    out_new = new.communicate(timeout=1500)[0]
     assert ops.returncode == 0, out_ops[-3000:]
     assert model.returncode == 0, out_model[-3000:]
-    assert " passed" in out_ops and " passed" in out_model
+    assert new.returncode == 0, out_new[-3000:]
+    assert " passed" in out_ops and " passed" in out_model and " passed" in out_new and "skipped" not in out_new
 
 
 def test_host_tensor_compute_is_refused(emulated):
