@@ -172,6 +172,8 @@ typedef struct {
     void (*eval_discard)(NNCPModel *s);
 } NNCPModelClass;
 const NNCPModelClass *nncp_model_class(NNCPModel *s);
+/* logits of the last evaluation of either class (V, B, T|1), borrowed */
+NCTensor *nncp_model_last_logits(NNCPModel *s);
 
 /* Per-timestep evaluation with K/V caches through the fused entry points (the
    decoder's view of a segment, nncp.c:801-863; cfg.fused = 1 and the shapes of

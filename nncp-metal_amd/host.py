@@ -156,6 +156,8 @@ class Host:
         L.nncp_retrain_block.argtypes = [_P, _P, C.c_int, C.POINTER(NNCPInterp), C.POINTER(NNCPStats)]
         L.nncp_fifo_symbol.argtypes = [_P, C.c_int, C.c_int, C.c_int]
         L.trf_last_logits.restype = _P
+        L.nncp_model_last_logits.restype = _P
+        L.nncp_model_last_logits.argtypes = [_P]
         L.trf_last_logits.argtypes = [_P]
         L.trf_step_begin.argtypes = [_P]
         L.trf_step_end.argtypes = [_P]
@@ -257,7 +259,7 @@ class Model:
         return res
 
     def logits(self):
-        return self._to_numpy(self.L.trf_last_logits(self.ptr))
+        return self._to_numpy(self.L.nncp_model_last_logits(self.ptr))
 
     def eval_steps(self, tokens):
         """Per-timestep cached evaluation of a whole segment (trf_step_begin +

@@ -817,3 +817,4 @@ const NNCPModelClass nncp_trf_class = { /* nncp.c:1544-1562 */
 };
 
 const NNCPModelClass *nncp_model_class(NNCPModel *s) { return s->cls; }
+NCTensor *nncp_model_last_logits(NNCPModel *s) { return s->cls->last_logits(s); }
