@@ -77,9 +77,13 @@ def test_random_shapes_stay_in_bounds_and_match(emulated):
     """Seeded random campaigns through the raw kernel entry points of the CPU build, each
     operand in an exact-size buffer ending at a guard page: GEMM (layouts, paddings, batches,
     split-K, fp32 / bf16 / bf16 from copies, forced tile configurations, epilogue options),
-    attention (both generations, backward, single-query step), integer CDF and lookup."""
+    attention (both generations, backward, single-query step), integer CDF and lookup; and
+    through the tensor ABI, every op family forward and backward (broadcast forms, reductions,
+    norms, softmax and log-likelihood, slicing / concatenation / permutation, padding, relative
+    shift, embedding gather, linear layers with activations, the optimiser, views and copies)."""
     jobs = [("fuzz_gemm.py", "101", "150"), ("fuzz_gemm.py", "102", "150"), ("fuzz_attn.py", "103", "12"),
-            ("fuzz_attn.py", "104", "12"), ("fuzz_cdf.py", "105", "25")]
+            ("fuzz_attn.py", "104", "12"), ("fuzz_cdf.py", "105", "25"),
+            ("fuzz_ops.py", "106", "800")]
     procs = [subprocess.Popen([sys.executable, os.path.join(EMU_DIR, name), seed, count], env=emulated,
                               stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
              for name, seed, count in jobs]
