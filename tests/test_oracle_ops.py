@@ -201,3 +201,90 @@ def test_cdf_lookup_is_the_inverse_of_the_cdf(ref, rng):
     sym = ref.numpy(ref.nc_cdf_lookup(cdf_t, ref.tensor(t)), free=True).astype(np.int64)
     for r in range(n):
         assert np.array_equal(sym[r], np.searchsorted(cdf[r], t[r].astype(np.int64), side="right") - 1)
+
+
+# ---- against the reference tree's own scalar restatement ------------------------------
+# src/neural/compatibility/cuda_math_compat.c, compiled where it lies into
+# oracle/_ref/libmath_compat_ref.so (softmax :287-332, ReLU :334-348, GELU :350-369,
+# matmul :259-284).  Its tensors are row-major with plain shapes.
+def _compat():
+    import ctypes as C
+    import os
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                        "oracle", "_ref", "libmath_compat_ref.so")
+    if not os.path.exists(path):
+        pytest.skip("oracle/_ref/libmath_compat_ref.so is not built (no reference tree)")
+    lib = C.CDLL(path)
+
+    class T(C.Structure):
+        _fields_ = [("data", C.POINTER(C.c_float)), ("shape", C.POINTER(C.c_size_t)), ("ndim", C.c_size_t),
+                    ("total_size", C.c_size_t), ("requires_grad", C.c_bool), ("is_metal_backed", C.c_bool),
+                    ("metal_buffer", C.c_void_p)]
+    PT = C.POINTER(T)
+    lib.cuda_compat_tensor_create.restype = PT
+    lib.cuda_compat_tensor_create.argtypes = [C.POINTER(C.c_size_t), C.c_size_t, C.c_void_p]
+    lib.cuda_compat_tensor_free.argtypes = [PT]
+    for name, args in (("softmax", [PT, C.c_int, C.c_void_p]), ("relu", [PT, C.c_void_p]),
+                       ("gelu", [PT, C.c_void_p]), ("matmul", [PT, PT, C.c_void_p])):
+        f = getattr(lib, "cuda_compat_" + name)
+        f.restype, f.argtypes = PT, args
+
+    def to(a):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        t = lib.cuda_compat_tensor_create((C.c_size_t * a.ndim)(*a.shape), a.ndim, None)
+        C.memmove(t.contents.data, a.ctypes.data, a.nbytes)
+        return t
+
+    def back(t):
+        shape = [t.contents.shape[i] for i in range(t.contents.ndim)]
+        out = np.ctypeslib.as_array(t.contents.data, shape=(int(np.prod(shape)),)).reshape(shape).copy()
+        lib.cuda_compat_tensor_free(t)
+        return out
+
+    def call(name, *arrays, extra=()):
+        ts = [to(a) for a in arrays]
+        res = getattr(lib, "cuda_compat_" + name)(*ts, *extra, None)
+        assert res, name
+        for t in ts:
+            lib.cuda_compat_tensor_free(t)
+        return back(res)
+    return call
+
+
+def test_softmax_matches_the_reference_restatement(ref, rng):
+    """Same order of operations (row maximum, expf of the difference, left-to-right
+    sum); the checker multiplies by the reciprocal of the sum where the restatement
+    divides, so results agree to the last bit or the one before it, also for long
+    rows and large magnitudes."""
+    call = _compat()
+    for shape, scale in (((7, 256), 3.0), ((3, 16384), 2.0), ((5, 1), 1.0), ((4, 33), 40.0)):
+        x = (rng.standard_normal(shape) * scale).astype(np.float32)
+        want = call("softmax", x, extra=(1,))
+        got = ref.numpy(ref.nc_soft_max(ref.tensor(x)), free=True)
+        assert np.array_equal(got == 0, want == 0), shape
+        nz = want != 0
+        assert (np.abs(got[nz] - want[nz]) <= 2.5e-7 * want[nz]).all(), shape
+
+
+def test_activations_match_the_reference_restatement(ref, rng):
+    """The tanh form of GELU with the constants 0.7978845608 and 0.044715, and ReLU."""
+    call = _compat()
+    x = np.concatenate([rng.standard_normal(4000) * 3, [0.0, -0.0, 1e-20, -30.0, 30.0]]).astype(np.float32)
+    g_want = call("gelu", x)
+    g_got = ref.numpy(ref.nc_gelu(ref.tensor(x)), free=True)
+    assert np.abs(g_got - g_want).max() <= 1e-6 * max(1.0, np.abs(g_want).max())
+    assert np.array_equal(ref.numpy(ref.nc_relu(ref.tensor(x)), free=True), call("relu", x))
+
+
+def test_matmul_matches_the_reference_restatement(ref, rng):
+    """Its row-major (m,k)x(k,n) product against nc_matmul on the same memory read
+    column-major: numpy (n,k) @ numpy (k,m) in the checker's layout."""
+    call = _compat()
+    for m, k, n in ((5, 7, 3), (33, 129, 17), (1, 300, 1)):
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        b = rng.standard_normal((k, n)).astype(np.float32)
+        want = call("matmul", a, b)                        # row-major (m, n)
+        # row-major a (m,k) is the column-major (k,m) matrix a^T; w = b^T (n rows... k cols) likewise
+        got = ref.numpy(ref.nc_matmul(ref.tensor(b), ref.tensor(a)), free=True)
+        assert got.shape == want.shape
+        assert np.abs(got - want).max() <= 2e-6 * np.abs(want).max() * np.sqrt(k)
