@@ -29,6 +29,11 @@ typedef struct { /* arith.h:32-43, in-memory output */
     uint8_t *buf;
     size_t buf_size, idx;
     int overflow;
+    /* optional: a full buffer is handed to sink and reused (the write_func of
+       arith.c:43); without one, bytes past buf_size are dropped and overflow is set */
+    void (*sink)(void *opaque, const uint8_t *buf, size_t n);
+    void *sink_opaque;
+    size_t n_flushed; /* bytes handed to sink so far */
 } NNCPPutBit;
 
 typedef struct { /* arith.h:50-61, in-memory input, zero padded past the end */
@@ -38,8 +43,10 @@ typedef struct { /* arith.h:50-61, in-memory input, zero padded past the end */
 } NNCPGetBit;
 
 void nncp_put_bit_init(NNCPPutBit *s, uint8_t *buf, size_t buf_size);  /* arith.c:43 */
+void nncp_put_bit_set_sink(NNCPPutBit *s, void (*sink)(void *, const uint8_t *, size_t), void *opaque);
 void nncp_put_bit(NNCPPutBit *s, int prob0, int bit);                  /* arith.c:122 */
-size_t nncp_put_bit_flush(NNCPPutBit *s);        /* arith.c:164; returns bytes written */
+size_t nncp_put_bit_flush(NNCPPutBit *s);        /* arith.c:164; returns bytes written (all of
+                                                    them already handed to the sink, if one is set) */
 void nncp_get_bit_init(NNCPGetBit *s, const uint8_t *buf, size_t len); /* arith.c:233 */
 int nncp_get_bit(NNCPGetBit *s, int prob0);                            /* arith.c:259 */
 
@@ -233,6 +240,46 @@ size_t nncp_compress(NNCPModel *s, const uint16_t *syms, int n, uint8_t *out, si
                      int mode, const NNCPInterp *lr, NNCPStats *st);
 void nncp_decompress(NNCPModel *s, const uint8_t *in, size_t len, uint16_t *syms, int n,
                      int mode, const NNCPInterp *lr, NNCPStats *st);
+
+/* ---- file container (encode_file / decode_file, nncp.c:3307-3677) ---------------- */
+/* NNCPModelParams' file-level fields that NNCPConfig does not hold (nncp.c:142-156) */
+typedef struct {
+    NNCPInterp lr, block_len; /* per training step; per file position */
+    int use_bf16;             /* matrix products round their operands to bf16 (nncp --bf16) */
+    int64_t max_size;         /* encoder: truncate the input to this many symbols; -1: no limit */
+    int mode;                 /* NNCP_MODE_* | NNCP_CODER_*; 0 is the reference's stream */
+} NNCPFileParams;
+
+/* nncp_init_params (nncp.c:2464-2636): "default", "enwik8", "enwik9", "lstm",
+   "lstm_fast"; -1 for an unknown name */
+int nncp_profile(NNCPConfig *cfg, NNCPFileParams *fp, const char *profile);
+/* "v0,pos0,v1,...[,p<power>]" (parse_interp_param / dump_interp_param,
+   cp_utils.c:412-470); parse returns -1 on a syntax error, format the length */
+int nncp_parse_interp(NNCPInterp *p, const char *str);
+int nncp_format_interp(char *buf, size_t size, const NNCPInterp *p);
+/* the big-endian header of nncp.c:2662-2760 with the model's own fields
+   (nncp.c:1333-1365, 2198-2211).  write returns the length, 0 if cap is too
+   small.  read returns 0, -1 for an invalid header, -2 for a valid one that
+   asks for an option this build does not have (tied_embed, rot_pos, GRU,
+   n_states != seg_len); cfg.fused, cfg.nb_threads and fp.mode are not part of
+   it (the file loops keep them in the byte that follows). */
+size_t nncp_header_write(uint8_t *buf, size_t cap, const NNCPConfig *cfg, const NNCPFileParams *fp);
+int nncp_header_read(const uint8_t *buf, size_t len, NNCPConfig *cfg, NNCPFileParams *fp, size_t *used);
+/* length of the block that starts at file_pos (nncp.c:3452-3457): the schedule's
+   value rounded down to whole steps of seg_len * batch_size, at least one, at
+   most what remains */
+int nncp_block_len(const NNCPConfig *cfg, const NNCPInterp *sched, int64_t file_pos, int64_t remaining);
+/* Whole files: header, flag byte, 32-bit symbol count, then every block through
+   one range coder with the retrain pass between blocks.  Symbols are bytes, or
+   big-endian 16-bit values when cfg.n_symbols > 256.  No dictionary
+   preprocessor: decode refuses a file written with one.  The decoder takes the
+   model from the file and the device from its caller, as nncp d does.
+   Return 0, or -1 after a message on stderr.  st / retrain_st (or NULL)
+   accumulate the statistics of coding and of the retrain passes. */
+int nncp_encode_file(const char *in_name, const char *out_name, const NNCPConfig *cfg,
+                     const NNCPFileParams *fp, NNCPStats *st, NNCPStats *retrain_st);
+int nncp_decode_file(const char *in_name, const char *out_name, int use_device, int nb_threads,
+                     NNCPStats *st, NNCPStats *retrain_st);
 
 #ifdef __cplusplus
 }

@@ -47,12 +47,18 @@ class NNCPStats(C.Structure):
 class NNCPPutBit(C.Structure):
     _fields_ = [("range", C.c_uint32), ("low", C.c_uint32), ("current_byte", C.c_uint8),
                 ("n_bytes", C.c_uint32), ("buf", C.c_void_p), ("buf_size", C.c_size_t),
-                ("idx", C.c_size_t), ("overflow", C.c_int)]
+                ("idx", C.c_size_t), ("overflow", C.c_int), ("sink", C.c_void_p),
+                ("sink_opaque", C.c_void_p), ("n_flushed", C.c_size_t)]
 
 
 class NNCPGetBit(C.Structure):
     _fields_ = [("buf", C.c_void_p), ("buf_len", C.c_size_t), ("idx", C.c_size_t),
                 ("low", C.c_uint32), ("range", C.c_uint32)]
+
+
+class NNCPFileParams(C.Structure):
+    _fields_ = [("lr", NNCPInterp), ("block_len", NNCPInterp), ("use_bf16", C.c_int),
+                ("max_size", C.c_int64), ("mode", C.c_int)]
 
 
 MODEL_TRF, MODEL_LSTM = 0, 1
@@ -180,11 +186,57 @@ class Host:
         L.nncp_read_sym_cdf.argtypes = [C.POINTER(NNCPGetBit), _P, C.c_int]
         L.nncp_interp.restype = C.c_float
         L.nncp_interp.argtypes = [C.POINTER(NNCPInterp), C.c_int64]
+        L.nncp_profile.argtypes = [C.POINTER(NNCPConfig), C.POINTER(NNCPFileParams), C.c_char_p]
+        L.nncp_parse_interp.argtypes = [C.POINTER(NNCPInterp), C.c_char_p]
+        L.nncp_format_interp.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(NNCPInterp)]
+        L.nncp_header_write.restype = C.c_size_t
+        L.nncp_header_write.argtypes = [_P, C.c_size_t, C.POINTER(NNCPConfig), C.POINTER(NNCPFileParams)]
+        L.nncp_header_read.argtypes = [_P, C.c_size_t, C.POINTER(NNCPConfig), C.POINTER(NNCPFileParams),
+                                       C.POINTER(C.c_size_t)]
+        L.nncp_block_len.argtypes = [C.POINTER(NNCPConfig), C.POINTER(NNCPInterp), C.c_int64, C.c_int64]
+        L.nncp_encode_file.argtypes = [C.c_char_p, C.c_char_p, C.POINTER(NNCPConfig), C.POINTER(NNCPFileParams),
+                                       C.POINTER(NNCPStats), C.POINTER(NNCPStats)]
+        L.nncp_decode_file.argtypes = [C.c_char_p, C.c_char_p, C.c_int, C.c_int, C.POINTER(NNCPStats),
+                                       C.POINTER(NNCPStats)]
+        L.nncp_put_bit_set_sink.argtypes = [C.POINTER(NNCPPutBit), _P, _P]
         # the libnc symbols the host library resolved (same handle namespace)
         self.ncl = C.CDLL(nc_libpath, mode=C.RTLD_LOCAL)
         for name, (res, args) in B._PROTOS.items():
             f = getattr(self.ncl, name)
             f.restype, f.argtypes = res, args
+
+
+def profile(host, name):
+    """(NNCPConfig, NNCPFileParams) of one of nncp's profiles (nncp.c:2464-2636)."""
+    cfg, fp = NNCPConfig(), NNCPFileParams()
+    if host.lib.nncp_profile(C.byref(cfg), C.byref(fp), name.encode()) != 0:
+        raise ValueError("unknown profile: %s" % name)
+    return cfg, fp
+
+
+def file_params(host, lr="3e-4", block_len="500000", use_bf16=0, max_size=-1, mode=0):
+    fp = NNCPFileParams(use_bf16=use_bf16, max_size=max_size, mode=mode)
+    for field, text in (("lr", lr), ("block_len", block_len)):
+        if host.lib.nncp_parse_interp(C.byref(getattr(fp, field)), str(text).encode()) != 0:
+            raise ValueError("bad schedule: %s" % text)
+    return fp
+
+
+def encode_file(host, src, dst, cfg, fp):
+    """nncp c without the preprocessor; returns (coding stats, retrain stats)."""
+    st, rst = NNCPStats(), NNCPStats()
+    if host.lib.nncp_encode_file(os.fsencode(src), os.fsencode(dst), C.byref(cfg), C.byref(fp),
+                                 C.byref(st), C.byref(rst)) != 0:
+        raise RuntimeError("encoding %s failed" % src)
+    return st, rst
+
+
+def decode_file(host, src, dst, use_device=1, nb_threads=1):
+    st, rst = NNCPStats(), NNCPStats()
+    if host.lib.nncp_decode_file(os.fsencode(src), os.fsencode(dst), use_device, nb_threads,
+                                 C.byref(st), C.byref(rst)) != 0:
+        raise RuntimeError("decoding %s failed" % src)
+    return st, rst
 
 
 class Model:

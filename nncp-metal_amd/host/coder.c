@@ -18,6 +18,11 @@
 
 static void emit(NNCPPutBit *s, int v)
 {
+    if (s->idx >= s->buf_size && s->sink && s->buf_size > 0) {
+        s->sink(s->sink_opaque, s->buf, s->idx);
+        s->n_flushed += s->idx;
+        s->idx = 0;
+    }
     if (s->idx < s->buf_size)
         s->buf[s->idx] = (uint8_t)v;
     else
@@ -61,6 +66,12 @@ void nncp_put_bit_init(NNCPPutBit *s, uint8_t *buf, size_t buf_size)
     s->buf_size = buf_size;
 }
 
+void nncp_put_bit_set_sink(NNCPPutBit *s, void (*sink)(void *, const uint8_t *, size_t), void *opaque)
+{
+    s->sink = sink;
+    s->sink_opaque = opaque;
+}
+
 void nncp_put_bit(NNCPPutBit *s, int prob0, int bit)
 {
     uint32_t r0 = (uint32_t)(((uint64_t)s->range * (uint32_t)prob0) >> NNCP_PROB_BITS);
@@ -91,7 +102,12 @@ size_t nncp_put_bit_flush(NNCPPutBit *s)
     shift_out(s, val >> RC_MIN_BITS);
     if (s->n_bytes > 0)
         shift_out(s, 0);
-    return s->idx;
+    if (s->sink) {
+        s->sink(s->sink_opaque, s->buf, s->idx);
+        s->n_flushed += s->idx;
+        s->idx = 0;
+    }
+    return s->n_flushed + s->idx;
 }
 
 static void refill(NNCPGetBit *s) /* arith.c:209-231, zero padding past the end */

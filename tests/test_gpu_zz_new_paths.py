@@ -88,3 +88,28 @@ def test_lstm_training_steps_match_checker_and_stream_round_trips(hosts, variant
         out, _ = dec.decompress(data, n, mode)
         dec.close()
         assert np.array_equal(out, data_syms), mode
+
+
+@pytest.mark.parametrize("stream", ["reference", "fast", "fast_bf16"])
+def test_file_container_round_trip_on_gpu(hosts, tmp_path, stream):
+    """nncp_encode_file / nncp_decode_file with the product library: the decoded file
+    equals the input, and the compressed size is within 0.5 % (bf16: 2 %) of the
+    checker's for the same file and parameters."""
+    hp = M.load_pkg().host
+    n = 200
+    mode = 0 if stream == "reference" else hp.MODE_SEGMENT | hp.CODER_CDF16
+    kw = dict(M.TINY, fused=int(stream != "reference"), sgd_opt=M.rmsprop(), nb_threads=4)
+    syms = M.markov1(n, 40, seed=17)
+    src = str(tmp_path / "in.bin")
+    syms.astype(np.uint8).tofile(src)
+    sizes = []
+    for host, dev in ((hosts[0], 1), (hosts[1], 0)):
+        cfg = hp.make_config(**dict(kw, use_device=dev))
+        fp = hp.file_params(host, "3e-4,8,1e-4", "96,200,120", use_bf16=int(stream == "fast_bf16"), mode=mode)
+        packed, back = str(tmp_path / ("out%d.nncp" % dev)), str(tmp_path / ("back%d.bin" % dev))
+        st, _ = hp.encode_file(host, src, packed, cfg, fp)
+        hp.decode_file(host, packed, back, use_device=dev, nb_threads=4)
+        assert open(back, "rb").read() == open(src, "rb").read()
+        assert st.n_symbols == n
+        sizes.append(os.path.getsize(packed))
+    assert abs(sizes[0] - sizes[1]) <= max(3, (0.02 if stream == "fast_bf16" else 0.005) * sizes[1])
