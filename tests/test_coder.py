@@ -174,3 +174,42 @@ def test_interp_matches_reference(refc, hostc, pkg_mod):
         refc.get_interp_param.argtypes = [C.POINTER(RefInterp), C.c_int64]
         for pos in (0, 1, 999, 1000, 3000, 4999, 5000, 123456):
             assert refc.get_interp_param(C.byref(a), pos) == hostc.lib.nncp_interp(C.byref(b), pos)
+
+
+GOLDEN = os.path.join(ROOT, "tests", "golden", "coder_vectors.npz")
+
+
+def test_coders_reproduce_committed_reference_vectors(hostc, pkg_mod):
+    """The same comparison without the reference tree: tests/golden/coder_vectors.npz holds
+    inputs and the bytes / values that the reference's arith.c and cp_utils.c gave for them
+    (written by tests/golden/make_coder_vectors.py)."""
+    g = np.load(GOLDEN)
+    for kind in ("uniform", "skewed", "carry"):
+        probs, bits = g["rc_%s_prob0" % kind], g["rc_%s_bits" % kind]
+        st, buf = _host_encoder(pkg_mod, hostc, probs.size * 2 + 64)
+        for p, b in zip(probs.tolist(), bits.tolist()):
+            hostc.lib.nncp_put_bit(C.byref(st), p, b)
+        got = buf[:hostc.lib.nncp_put_bit_flush(C.byref(st))].copy()
+        assert np.array_equal(got, g["rc_%s_bytes" % kind]), kind
+        gb = pkg_mod.host.NNCPGetBit()
+        hostc.lib.nncp_get_bit_init(C.byref(gb), got.ctypes.data, got.size)
+        assert [hostc.lib.nncp_get_bit(C.byref(gb), p) for p in probs.tolist()] == bits.tolist(), kind
+    for n_symb in (2, 3, 256, 1000):
+        probs, syms = g["sym_%d_probs" % n_symb], g["sym_%d_syms" % n_symb]
+        st, buf = _host_encoder(pkg_mod, hostc, syms.size * 8 + 64)
+        for p, s in zip(probs, syms.tolist()):
+            hostc.lib.nncp_write_sym(C.byref(st), np.ascontiguousarray(p).ctypes.data, n_symb, s)
+        got = buf[:hostc.lib.nncp_put_bit_flush(C.byref(st))].copy()
+        assert np.array_equal(got, g["sym_%d_bytes" % n_symb]), n_symb
+        gb = pkg_mod.host.NNCPGetBit()
+        hostc.lib.nncp_get_bit_init(C.byref(gb), got.ctypes.data, got.size)
+        for p, s in zip(probs, syms.tolist()):
+            assert hostc.lib.nncp_read_sym(C.byref(gb), np.ascontiguousarray(p).ctypes.data, n_symb) == s
+    for i, power in enumerate(g["interp_power"]):
+        s = pkg_mod.host.NNCPInterp(n_steps=2, decay_power=float(power))
+        for k, v in enumerate(g["interp_val"]):
+            s.val[k] = float(v)
+        for k, v in enumerate(g["interp_pos"]):
+            s.pos[k] = int(v)
+        got = [hostc.lib.nncp_interp(C.byref(s), int(p)) for p in g["interp_at"]]
+        assert np.array_equal(np.array(got, dtype=np.float32), g["interp_out"][i]), power
