@@ -56,3 +56,17 @@ def test_binding_covers_the_link_set_of_the_reference_host():
         lib = ctypes.CDLL(path)
         missing = [n for n in link_set if not hasattr(lib, n)]
         assert not missing, (path, missing)
+
+
+def test_host_library_exports_declared_symbols():
+    """include/nncp_host.h against the host library of the product and of the checker."""
+    text = open(os.path.join(ROOT, "include", "nncp_host.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(nncp_\w+)\s*\(", text)))
+    assert len(names) > 30
+    pkg = load_pkg()
+    ctypes.CDLL(pkg.binding.HIP_LIB, mode=ctypes.RTLD_GLOBAL)
+    for path in (pkg.host.HOST_HIP_LIB, os.path.join(ROOT, "oracle", "libnncp_host_ref.so")):
+        lib = ctypes.CDLL(path)
+        missing = [n for n in names if not hasattr(lib, n)]
+        assert not missing, (path, missing)
