@@ -112,6 +112,8 @@ extern "C" NCContext *nc_context_init(int nb_threads)
     m->grp_staging_cap = 0;
     m->red_staging = nullptr;
     m->red_staging_cap = 0;
+    m->grp_staging_stamp = m->red_staging_stamp = 0;
+    m->sync_count = 0;
     const char *e = getenv("NCHIP_MATMUL_BF16");
     if (e && atoi(e) != 0)
         m->matmul_bf16 = 1;
@@ -159,10 +161,23 @@ extern "C" NCDevice *nc_new_device(NCContext *m, const char *name)
     return &m->cpu;
 }
 
+void nc_stream_wait(NCContext *m)
+{
+    hip_check(hipStreamSynchronize(m->stream), "hipStreamSynchronize");
+    m->sync_count++;
+}
+
+void nc_staging_retire(NCContext *m, void *p, size_t cap, uint64_t stamp)
+{
+    if (!p) return;
+    if (stamp == m->sync_count) nc_stream_wait(m);
+    m->host_pool.put(p, cap);
+}
+
 extern "C" void nc_synchronize(NCDevice *d)
 {
     if (d->ctx->hip_ready)
-        hip_check(hipStreamSynchronize(d->ctx->stream), "hipStreamSynchronize");
+        nc_stream_wait(d->ctx);
 }
 
 extern "C" void nc_prof_dump(void) {}
@@ -492,7 +507,7 @@ extern "C" NCTensor *nc_tensor_to_device(NCTensor *x, NCDevice *d)
         hip_check(hipMemcpyAsync(nc_data(y), nc_data(x), bytes,
                                  d->is_hip ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost, m->stream),
                   "hipMemcpyAsync");
-        hip_check(hipStreamSynchronize(m->stream), "hipStreamSynchronize");
+        nc_stream_wait(m);
     }
     nc_free_tensor(x);
     return y;
@@ -508,7 +523,7 @@ extern "C" NCTensor *nc_tensor_to_cpu_device(NCTensor *x)
     size_t bytes = nc_numel(c) * nc_type_size(c->type);
     if (bytes) {
         hip_check(hipMemcpyAsync(nc_data(y), nc_data(c), bytes, hipMemcpyDeviceToHost, m->stream), "hipMemcpyAsync d2h");
-        hip_check(hipStreamSynchronize(m->stream), "hipStreamSynchronize");
+        nc_stream_wait(m);
     }
     nc_free_tensor(c);
     return y;
@@ -521,7 +536,7 @@ extern "C" float nc_get_scalar_f32(const NCTensor *x) // libnc.h:214 (synchronis
     float v;
     NCContext *m = x->dev->ctx;
     hip_check(hipMemcpyAsync(&v, nc_data(x), sizeof(float), hipMemcpyDeviceToHost, m->stream), "hipMemcpyAsync");
-    hip_check(hipStreamSynchronize(m->stream), "hipStreamSynchronize");
+    nc_stream_wait(m);
     return v;
 }
 
@@ -568,7 +583,7 @@ static void upload_f32(NCTensor *y, const float *host)
     size_t bytes = nc_numel(y) * sizeof(float);
     if (!y->dev->is_hip) { memcpy(nc_data(y), host, bytes); return; }
     hip_check(hipMemcpyAsync(nc_data(y), host, bytes, hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync h2d");
-    hip_check(hipStreamSynchronize(m->stream), "hipStreamSynchronize");
+    nc_stream_wait(m);
 }
 
 // libnc.h:197: uniform in [avg - range, avg + range); generated on the host in
@@ -663,6 +678,7 @@ struct NCSGDOptState {
     std::vector<SGDOptVarState *> vars;
     void *staging = nullptr; // pinned table of the previous update, recycled one update later
     size_t staging_cap = 0;
+    uint64_t staging_stamp = 0;
 };
 
 extern "C" NCSGDOptState *nc_sgd_opt_init(NCContext *m, const SGDOptParams *p)
@@ -674,7 +690,7 @@ extern "C" NCSGDOptState *nc_sgd_opt_init(NCContext *m, const SGDOptParams *p)
 
 extern "C" void nc_sgd_opt_end(NCSGDOptState *s)
 {
-    if (s->staging) s->ctx->host_pool.put(s->staging, s->staging_cap);
+    nc_staging_retire(s->ctx, s->staging, s->staging_cap, s->staging_stamp);
     delete s;
 }
 
@@ -778,8 +794,8 @@ extern "C" void nc_sgd_opt_update(NCSGDOptState *s)
         nc_fatal("optimiser update failed");
     m->launches++;
     // the copy must have read the staging buffer before it is recycled
-    if (s->staging) m->host_pool.put(s->staging, s->staging_cap);
-    s->staging = host; s->staging_cap = hcap;
+    nc_staging_retire(m, s->staging, s->staging_cap, s->staging_stamp);
+    s->staging = host; s->staging_cap = hcap; s->staging_stamp = m->sync_count;
     m->dev_pool.put(dev, dcap); // stream ordered: next user is enqueued after the kernel
     for (SGDOptVarState *vs : s->vars) {
         if (!vs->has_grad) continue;

@@ -85,10 +85,16 @@ struct NCContext {
     std::vector<DeferredReduce> deferred_red;
     std::vector<DeferredTmp> deferred_tmp;    // scratch the partial rows live in
     std::vector<NCTensor *> deferred_keep;    // destination tensors
+    // pinned tables of the last grouped launches; each goes back to the pool
+    // one flush later, and only once the stream has been waited for since its
+    // upload was enqueued (nc_staging_retire)
     void *grp_staging;
     size_t grp_staging_cap;
+    uint64_t grp_staging_stamp;
     void *red_staging;
     size_t red_staging_cap;
+    uint64_t red_staging_stamp;
+    uint64_t sync_count; // completed waits for the stream (nc_stream_wait)
 };
 
 struct NCTensorBuffer {
@@ -155,6 +161,14 @@ static inline hipStream_t nc_stream(const NCTensor *x) { return x->dev->ctx->str
 float *nc_tmp_f32(NCContext *m, size_t n, size_t *cap); // pool scratch; give back with nc_tmp_free
 void nc_tmp_free(NCContext *m, void *p, size_t cap);
 NCTensor *nc_reshape_view(NCTensor *x, int nd, const size_t *dims); // consumes, no graph
+// Every wait for the stream goes through here, so that sync_count tells whether
+// work enqueued at an earlier moment has certainly finished.
+void nc_stream_wait(NCContext *m);
+// Gives a pinned table back to the host pool.  Its upload was enqueued when
+// sync_count read `stamp`; if the stream has not been waited for since (a
+// caller that enqueues step after step without reading anything back), waits
+// first, so the buffer is never rewritten under a copy that has yet to run.
+void nc_staging_retire(NCContext *m, void *p, size_t cap, uint64_t stamp);
 
 // nc_autodiff.cpp
 NCNode *nc_new_node(NCContext *m, int op, int n_args, NCTensor **args);

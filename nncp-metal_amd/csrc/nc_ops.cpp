@@ -1064,9 +1064,9 @@ static void flush_deferred_gemms(NCContext *m)
     if (nchip_gemm_grouped(m->stream, 0, 1, (const NchipGemmProblem *)dev, (int)tab.size(), tiles, m->matmul_bf16, flops))
         nc_fatal("grouped weight-gradient GEMM failed");
     m->launches++;
-    // pinned staging is recycled one flush later (the copy has long run by then)
-    if (m->grp_staging) m->host_pool.put(m->grp_staging, m->grp_staging_cap);
-    m->grp_staging = host; m->grp_staging_cap = hcap;
+    // pinned staging is recycled one flush later, after a wait for the stream
+    nc_staging_retire(m, m->grp_staging, m->grp_staging_cap, m->grp_staging_stamp);
+    m->grp_staging = host; m->grp_staging_cap = hcap; m->grp_staging_stamp = m->sync_count;
     m->dev_pool.put(dev, dcap);
     for (DeferredGemm &d : m->deferred) {
         nc_free_tensor(d.a); nc_free_tensor(d.b); nc_free_tensor(d.c);
@@ -1093,8 +1093,8 @@ static void flush_deferred_sums(NCContext *m)
     hip_check(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync sum table");
     k_reduce_rows_multi(m->stream, (const KReduceRowsEntry *)dev, (int)tab.size(), max_n);
     m->launches++;
-    if (m->red_staging) m->host_pool.put(m->red_staging, m->red_staging_cap);
-    m->red_staging = host; m->red_staging_cap = hcap;
+    nc_staging_retire(m, m->red_staging, m->red_staging_cap, m->red_staging_stamp);
+    m->red_staging = host; m->red_staging_cap = hcap; m->red_staging_stamp = m->sync_count;
     m->dev_pool.put(dev, dcap);
     for (DeferredTmp &t : m->deferred_tmp) nc_tmp_free(m, t.ptr, t.cap);
     for (NCTensor *t : m->deferred_keep) nc_free_tensor(t);
