@@ -159,6 +159,40 @@ def test_optimisers_closed_form(ref, pkg):
         nc.close()
 
 
+def test_optimisers_against_library_routines(ref, pkg):
+    """RMSProp and Adam of the checker against torch.optim (CPU, float64) on a random
+    tensor over several steps with beta1 != 0: a library's statement of the two
+    updates rather than a retyped formula.  torch's Adam divides sqrt(v) by
+    sqrt(1 - beta2^t) before eps is added, as the checker does."""
+    import ctypes as C
+    import torch
+    B = pkg.binding
+    rng = np.random.default_rng(77)
+    w0 = rng.normal(0, 0.5, 257).astype(np.float32)
+    grads = [(rng.normal(0, 1.0, 257) * 10.0 ** rng.integers(-3, 1)).astype(np.float32) for _ in range(6)]
+    for algo, b1 in ((B.SGD_OPT_RMSPROP, 0.0), (B.SGD_OPT_ADAM, 0.9), (B.SGD_OPT_ADAM, 0.0)):
+        nc = B.NC(ref.lib._name, use_device=False)
+        h, p = nc.param(w0.copy())
+        sp = B.SGDOptParams(algo=algo, beta1=b1, beta2=0.99, eps=1e-8, gradient_clip=0.0, lr=3e-3)
+        opt = nc.nc_sgd_opt_init(nc.ctx, C.byref(sp))
+        nc.nc_sgd_opt_set_all(C.byref(nc.plist), opt)
+        tw = torch.tensor(w0.astype(np.float64), requires_grad=True)
+        if algo == B.SGD_OPT_RMSPROP:
+            topt = torch.optim.RMSprop([tw], lr=3e-3, alpha=0.99, eps=1e-8)
+        else:
+            topt = torch.optim.Adam([tw], lr=3e-3, betas=(b1, 0.99), eps=1e-8)
+        for g in grads:
+            nc.sgd_opt_update_var(p, nc.tensor(g), None)
+            nc.nc_sgd_opt_set_lr(opt, 3e-3)
+            nc.nc_sgd_opt_update(opt)
+            tw.grad = torch.tensor(g.astype(np.float64))
+            topt.step()
+            np.testing.assert_allclose(nc.numpy(h.value), tw.detach().numpy(), rtol=2e-5, atol=2e-7)
+        nc.nc_sgd_opt_set_all(C.byref(nc.plist), None)
+        nc.nc_sgd_opt_end(opt)
+        nc.close()
+
+
 # ---- coder-side probability path: what the mathematics fixes ---------------------
 def _zipf_logits(rng, n, V):
     bias = -np.log(rng.permutation(V) + 1.0)
