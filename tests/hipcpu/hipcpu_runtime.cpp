@@ -40,6 +40,11 @@ void (*g_entry)(void *) = nullptr;
 void *g_closure = nullptr;
 void *g_lds = nullptr;
 long g_switches_without_progress = 0;
+/* HIPCPU_ORDER=reverse runs the work-items of a workgroup, and the workgroups of a grid, from
+   the last to the first.  Results must not change: between two barriers every order is one
+   the hardware may choose, so a difference is a missing barrier (or a workgroup that relies
+   on another one of the same launch). */
+const bool g_reverse = getenv("HIPCPU_ORDER") && !strcmp(getenv("HIPCPU_ORDER"), "reverse");
 
 void die(const char *msg)
 {
@@ -122,8 +127,8 @@ void run_block()
     }
     g_switches_without_progress = 0;
     while (g_live > 0) {
-        for (int i = 0; i < g_n && g_live > 0; i++) {
-            Fiber &f = g_fibers[i];
+        for (int k = 0; k < g_n && g_live > 0; k++) {
+            Fiber &f = g_fibers[g_reverse ? g_n - 1 - k : k];
             if (f.done) continue;
             hipcpu_cur = &f.item;
             swapcontext(&g_sched, &f.ctx);
@@ -203,12 +208,13 @@ void hipcpu_launch(dim3 grid, dim3 block, size_t shmem, void (*entry)(void *), v
     g_lds = shmem ? guarded_alloc(shmem) : nullptr;
     hipcpu_block_dim = block;
     hipcpu_grid_dim = grid;
-    for (unsigned z = 0; z < grid.z; z++)
-        for (unsigned y = 0; y < grid.y; y++)
-            for (unsigned x = 0; x < grid.x; x++) {
-                hipcpu_block_idx = dim3(x, y, z);
-                run_block();
-            }
+    const uint64_t n_blocks = (uint64_t)grid.x * grid.y * grid.z;
+    for (uint64_t k = 0; k < n_blocks; k++) {
+        const uint64_t b = g_reverse ? n_blocks - 1 - k : k;
+        hipcpu_block_idx = dim3((unsigned)(b % grid.x), (unsigned)(b / grid.x % grid.y),
+                                (unsigned)(b / ((uint64_t)grid.x * grid.y)));
+        run_block();
+    }
     if (g_lds) guarded_free(g_lds);
     g_lds = nullptr;
 }

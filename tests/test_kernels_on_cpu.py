@@ -63,6 +63,16 @@ def test_gpu_parity_tests_pass_on_the_cpu_build(emulated):
     assert " passed" in out_ops and " passed" in out_model and " passed" in out_new and "skipped" not in out_new
 
 
+def test_results_do_not_depend_on_work_item_order(emulated):
+    """The op-level tests again with the work-items of every workgroup, and the workgroups of
+    every launch, run from the last to the first (HIPCPU_ORDER=reverse).  Between two
+    barriers any order is one the hardware may pick, so a kernel that is missing a barrier
+    (or whose workgroups rely on one another) gives different results here."""
+    p = _pytest(dict(emulated, HIPCPU_ORDER="reverse"), ["-n", "7", "tests/test_gpu_ops.py"])
+    out = p.communicate(timeout=1500)[0]
+    assert p.returncode == 0 and " passed" in out, out[-3000:]
+
+
 def test_host_tensor_compute_is_refused(emulated):
     """No CPU fallback in the product library: compute on a host tensor aborts with a
     message.  (Host-side logic, so it is exercised on the CPU build and not by aborting
