@@ -20,7 +20,6 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(HERE))
 import test_coder as T  # noqa: E402  (structures and the reference encoder wrapper)
-from conftest import REF_LIB  # noqa: E402
 
 
 def range_coder_case(kind, n=4000):
@@ -50,7 +49,6 @@ def symbol_case(n_symb, rows):
 def main():
     if not os.path.exists(T.REF_CODER):
         sys.exit("oracle/_ref/libnncp_coder_ref.so missing: make -C oracle ref")
-    C.CDLL(REF_LIB, mode=C.RTLD_GLOBAL)  # vec_sum_f32 for cp_utils.o
     lib = C.CDLL(T.REF_CODER)
     lib.put_bit_init.argtypes = [C.POINTER(T.RefPutBit), C.POINTER(C.c_uint8), C.c_int, T.WRITE_FUNC, C.c_void_p]
     lib.put_bit.argtypes = [C.POINTER(T.RefPutBit), C.c_int, C.c_int]

@@ -34,7 +34,9 @@ class RefGetBit(C.Structure):  # arith.h:50-61
 def refc():
     if not os.path.exists(REF_CODER):
         pytest.skip("oracle/_ref not built")
-    C.CDLL(REF_LIB, mode=C.RTLD_GLOBAL)  # provides vec_sum_f32 to the reference objects
+    # (vec_sum_f32 comes from the checker library the reference objects were linked against;
+    # nothing is loaded into the global namespace, where it would capture the nc_* calls of
+    # every library loaded later)
     lib = C.CDLL(REF_CODER)
     lib.put_bit_init.argtypes = [C.POINTER(RefPutBit), C.POINTER(C.c_uint8), C.c_int, WRITE_FUNC, C.c_void_p]
     lib.put_bit.argtypes = [C.POINTER(RefPutBit), C.c_int, C.c_int]

@@ -33,7 +33,6 @@ class RefInterp(C.Structure):  # cp_utils.h:62-67
 def refc():
     if not os.path.exists(REF_CODER):
         pytest.skip("oracle/_ref not built")
-    C.CDLL(REF_LIB, mode=C.RTLD_GLOBAL)
     lib = C.CDLL(REF_CODER)
     libc = C.CDLL(None)
     libc.tmpfile.restype = C.c_void_p
