@@ -68,6 +68,12 @@ typedef struct {
     float decay_power;
 } NNCPInterp;
 float nncp_interp(const NNCPInterp *p, int64_t pos);
+/* The address of nc_context_init as the calls of this library resolve it.  A loader that
+   holds the libnc it meant to pair with this library compares it with that library's own
+   symbol: a libnc that sits in the process-wide namespace (RTLD_GLOBAL, LD_PRELOAD) is found
+   first by the dynamic linker and would otherwise take the calls unnoticed.  (No
+   counterpart in the reference, which links one libnc statically into one executable.) */
+const void *nncp_bound_libnc(void);
 
 /* ---- Transformer-XL model ------------------------------------------------------ */
 #define NNCP_LN_POST (1 << 0)    /* nncp.c:74-78 */

@@ -201,6 +201,11 @@ class Host:
         L.nncp_put_bit_set_sink.argtypes = [C.POINTER(NNCPPutBit), _P, _P]
         # the libnc symbols the host library resolved (same handle namespace)
         self.ncl = C.CDLL(nc_libpath, mode=C.RTLD_LOCAL)
+        # the tensor calls of the host code must land in that very library (and not in another
+        # libnc that some earlier load put into the process-wide namespace)
+        L.nncp_bound_libnc.restype = _P
+        if L.nncp_bound_libnc() != C.cast(self.ncl.nc_context_init, _P).value:
+            raise RuntimeError("%s is bound to another libnc than %s" % (libpath, nc_libpath))
         for name, (res, args) in B._PROTOS.items():
             f = getattr(self.ncl, name)
             f.restype, f.argtypes = res, args

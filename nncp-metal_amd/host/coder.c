@@ -215,6 +215,11 @@ int nncp_read_sym_cdf(NNCPGetBit *gb, const uint16_t *cdf, int n_symb)
 }
 
 /* cp_utils.c:380-410 */
+const void *nncp_bound_libnc(void)
+{
+    return (const void *)&nc_context_init;
+}
+
 float nncp_interp(const NNCPInterp *p, int64_t pos)
 {
     for (int i = 0; i < p->n_steps; i++) {

@@ -69,3 +69,21 @@ def test_host_library_exports_declared_symbols():
         lib = ctypes.CDLL(path)
         missing = [n for n in names if not hasattr(lib, n)]
         assert not missing, (path, missing)
+
+
+def test_host_loader_refuses_a_host_library_bound_to_another_libnc():
+    """With the checker in the process-wide namespace the dynamic linker would hand its nc_*
+    functions to the product's host library (a GPU run would then silently compute on the
+    CPU): Host() must notice and refuse.  Run in a child process, whose namespace it spoils."""
+    import subprocess
+    import sys
+    code = ("import sys, ctypes; sys.path.insert(0, %r); from conftest import load_pkg, REF_LIB;"
+            "pkg = load_pkg(); ctypes.CDLL(REF_LIB, mode=ctypes.RTLD_GLOBAL)\n"
+            "try:\n    pkg.host.Host()\nexcept RuntimeError as e:\n    print('refused:', e); sys.exit(0)\n"
+            "sys.exit(1)") % (os.path.join(ROOT, "tests"),)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+    assert r.returncode == 0 and "bound to another libnc" in r.stdout, r.stdout + r.stderr
+    # and the plain pairing loads
+    pkg = load_pkg()
+    pkg.host.Host()
+    pkg.host.Host(os.path.join(ROOT, "oracle", "libnncp_host_ref.so"), os.path.join(ROOT, "oracle", "libnc_ref.so"))
