@@ -113,3 +113,34 @@ def test_file_container_round_trip_on_gpu(hosts, tmp_path, stream):
         assert st.n_symbols == n
         sizes.append(os.path.getsize(packed))
     assert abs(sizes[0] - sizes[1]) <= max(3, (0.02 if stream == "fast_bf16" else 0.005) * sizes[1])
+
+
+@pytest.mark.parametrize("source", [0, 2])
+def test_bf16_operand_rounding_is_bitwise_the_checkers(source):
+    """A * I with the bf16 switch on returns the rounded operand itself: the kernels' rounding
+    (inside the tile loader, source 0, and in the streaming cast pass, source 2) must be the
+    checker's round-to-nearest-even bit for bit - ties, values next to ties, subnormals."""
+    import ctypes as C
+    from conftest import REF_LIB, hip_lib_path
+    pkg = M.load_pkg()
+    rng = np.random.default_rng(12)
+    vals = (rng.standard_normal(2000) * 10.0 ** rng.integers(-30, 30, 2000)).astype(np.float32)
+    ties = (rng.integers(0, 1 << 31, 1000, dtype=np.int64).astype(np.uint32) & np.uint32(0xFFFF0000)) | np.uint32(0x8000)
+    bits = np.concatenate([vals.view(np.uint32), ties, ties - np.uint32(1), ties + np.uint32(1),
+                           np.array([1, 0x8000, 0x18000, 0x7FFFFF], dtype=np.uint32)])
+    a = bits.view(np.float32)
+    a = a[np.isfinite(a) & (np.abs(a) < 1e38)]
+    a = a[: a.size // 64 * 64].reshape(-1, 64)
+    eye = np.eye(64, dtype=np.float32)
+    outs = []
+    lib = C.CDLL(hip_lib_path(pkg))
+    for path, dev in ((hip_lib_path(pkg), True), (REF_LIB, False)):
+        nc = pkg.binding.NC(path, use_device=dev)
+        nc.nc_set_matmul_bf16(nc.ctx, 1)
+        if dev:
+            lib.nchip_gemm_bf16_source(source)
+        outs.append(nc.numpy(nc.nc_matmul(nc.tensor(eye), nc.tensor(a)), free=True))
+        nc.nc_set_matmul_bf16(nc.ctx, 0)
+        nc.close()
+    lib.nchip_gemm_bf16_source(1)
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))

@@ -193,6 +193,35 @@ def test_optimisers_against_library_routines(ref, pkg):
         nc.close()
 
 
+def test_bf16_operand_rounding_is_round_to_nearest_even(ref):
+    """The operand rounding of the bf16 variant, read off as A * I with the switch on
+    (products with 1 and sums with 0 are exact), against torch's float32 -> bfloat16
+    conversion bit for bit: random values over many binades, exact ties to either side,
+    values one unit off a tie, subnormals, signed zeros, the largest finite value."""
+    import torch
+    rng = np.random.default_rng(12)
+    vals = (rng.standard_normal(4000) * 10.0 ** rng.integers(-30, 30, 4000)).astype(np.float32)
+    bits = rng.integers(0, 1 << 31, 3000, dtype=np.int64).astype(np.uint32)
+    ties = (bits & np.uint32(0xFFFF0000)) | np.uint32(0x8000)               # exactly halfway
+    near = np.concatenate([ties - np.uint32(1), ties + np.uint32(1)])
+    special = np.array([0x00000001, 0x00008000, 0x00018000, 0x007FFFFF, 0x80000000, 0x7F7F0000, 0x7F7F7FFF],
+                       dtype=np.uint32)
+    allbits = np.concatenate([vals.view(np.uint32), ties, near, special, ties | np.uint32(0x80000000)])
+    a = allbits.view(np.float32)
+    a = a[np.isfinite(a)]
+    a = a[: a.size // 8 * 8].reshape(-1, 8)                                 # libnc (8, n): 8 rows
+    eye = np.eye(8, dtype=np.float32)
+    ref.nc_set_matmul_bf16(ref.ctx, 1)
+    got = ref.numpy(ref.nc_matmul(ref.tensor(eye), ref.tensor(a)), free=True)
+    ref.nc_set_matmul_bf16(ref.ctx, 0)
+    want = torch.from_numpy(a.copy()).to(torch.bfloat16).to(torch.float32).numpy()
+    finite = np.isfinite(want)                                              # a rounding that overflows: not a GEMM input
+    assert finite.mean() > 0.99
+    nz = finite & (want != 0)                                               # -0 * 1 + 0 * 0 ... sums to +0
+    assert np.array_equal(got[nz].view(np.uint32), want[nz].view(np.uint32))
+    assert not got[finite & (want == 0)].any()
+
+
 # ---- coder-side probability path: what the mathematics fixes ---------------------
 def _zipf_logits(rng, n, V):
     bias = -np.log(rng.permutation(V) + 1.0)
