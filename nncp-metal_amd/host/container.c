@@ -202,6 +202,52 @@ static int get_sgd_opt(Cur *c, SGDOptParams *p)
     return 0;
 }
 
+static int finite_interp(const NNCPInterp *p)
+{
+    for (int i = 0; i <= p->n_steps; i++)
+        if (!isfinite(p->val[i]))
+            return 0;
+    return isfinite(p->decay_power);
+}
+
+/* A header comes from a file: sizes that would divide by zero, index outside a table or make
+   the model constructor give up (which ends the process) are refused here instead. */
+static int config_is_sane(const NNCPConfig *c, const NNCPFileParams *fp)
+{
+    if (c->batch_size < 1 || c->seg_len < 1 || c->n_symbols < 2 || c->n_layer < 1 || c->n_layer > NNCP_N_LAYER_MAX)
+        return 0;
+    if (!finite_interp(&fp->lr) || !finite_interp(&fp->block_len) || fp->block_len.val[0] < 1.0f)
+        return 0;
+    if (c->retrain_period < 0 || (c->retrain_period != 0 && c->retrain_len < 1))
+        return 0;
+    if (c->has_retrain_lr && !finite_interp(&c->retrain_lr))
+        return 0;
+    if (c->sgd_opt.algo != SGD_OPT_BASIC &&
+        !(isfinite(c->sgd_opt.u.adam.beta1) && isfinite(c->sgd_opt.u.adam.beta2) &&
+          isfinite(c->sgd_opt.u.adam.eps) && isfinite(c->sgd_opt.u.adam.gradient_clip)))
+        return 0;
+    if (c->model_type == NNCP_MODEL_TRF) {
+        if (c->n_head < 1 || c->d_key < 1 || c->d_value < 1 || c->d_inner < 1 ||
+            (c->use_w_r && c->d_pos < 1))
+            return 0;
+        for (int i = 0; i < c->n_layer; i++)
+            if (c->attn_len[i] < 1)
+                return 0;
+        if (c->ff_act > NNCP_FF_GATED_SILU ||
+            (c->ln_flags & ~(NNCP_LN_POST | NNCP_LN_PRE | NNCP_LN_FINAL | NNCP_LN_COEF | NNCP_LN_RMSNORM)))
+            return 0;
+        if (!isfinite(c->init_range) || !isfinite(c->embed_mult) || !isfinite(c->dropout_prob) ||
+            !isfinite(c->dropout_att_prob) || c->dropout_prob < 0 || c->dropout_prob >= 1 ||
+            c->dropout_att_prob < 0 || c->dropout_att_prob >= 1)
+            return 0;
+    } else {
+        if (c->lstm_n_cells < 1 || c->lstm_n_embed_out < 1 || c->lstm_n_embed_out > c->n_layer ||
+            !isfinite(c->lstm_forget_bias))
+            return 0;
+    }
+    return 1;
+}
+
 size_t nncp_header_write(uint8_t *buf, size_t cap, const NNCPConfig *c, const NNCPFileParams *fp)
 {
     Cur k = { buf, NULL, 0, cap, 0 };
@@ -343,7 +389,7 @@ int nncp_header_read(const uint8_t *buf, size_t len, NNCPConfig *c, NNCPFilePara
     } else {
         return -1;
     }
-    if (k.bad)
+    if (k.bad || !config_is_sane(c, fp))
         return -1;
     c->sgd_opt.lr = fp->lr.val[0];
     if (used)
@@ -360,10 +406,16 @@ int nncp_block_len(const NNCPConfig *c, const NNCPInterp *sched, int64_t file_po
     return n > remaining ? (int)remaining : n;
 }
 
+typedef struct {
+    FILE *f;
+    int failed;
+} FileSink;
+
 static void file_sink(void *opaque, const uint8_t *buf, size_t n)
 {
-    if (fwrite(buf, 1, n, (FILE *)opaque) != n)
-        perror("nncp_host: write");
+    FileSink *k = opaque;
+    if (!k->failed && fwrite(buf, 1, n, k->f) != n)
+        k->failed = 1;
 }
 
 static void add_stats(NNCPStats *to, const NNCPStats *from)
@@ -407,6 +459,10 @@ int nncp_encode_file(const char *in_name, const char *out_name, const NNCPConfig
     if (!st) st = &dummy;
     if (!retrain_st) retrain_st = &dummy2;
     n = nncp_header_write(head, sizeof(head) - 5, c, fp);
+    if (n == 0) {
+        fclose(f); fclose(fo);
+        return fail("header does not fit", out_name);
+    }
     head[n++] = (uint8_t)((fp->mode & 7) << 1 | (c->fused != 0) << 4); /* bit 0: no preprocessing */
     fseeko(f, 0, SEEK_END);
     file_len = ftello(f) >> symb_shift;
@@ -419,11 +475,11 @@ int nncp_encode_file(const char *in_name, const char *out_name, const NNCPConfig
     }
     head[n++] = (uint8_t)(file_len >> 24); head[n++] = (uint8_t)(file_len >> 16);
     head[n++] = (uint8_t)(file_len >> 8); head[n++] = (uint8_t)file_len;
-    fwrite(head, 1, n, fo);
+    FileSink sink = { fo, fwrite(head, 1, n, fo) != n };
 
     arith_buf = malloc(ARITH_BUF_LEN);
     nncp_put_bit_init(&pb, arith_buf, ARITH_BUF_LEN);
-    nncp_put_bit_set_sink(&pb, file_sink, fo);
+    nncp_put_bit_set_sink(&pb, file_sink, &sink);
     NNCPModel *s = model_for_file(c, fp);
     int rc = 0;
     while (pos < file_len) {
@@ -465,7 +521,7 @@ int nncp_encode_file(const char *in_name, const char *out_name, const NNCPConfig
     nncp_model_free(s);
     free(block);
     free(arith_buf);
-    if (fclose(fo) != 0)
+    if (fclose(fo) != 0 || sink.failed)
         rc = fail("write error", out_name);
     fclose(f);
     return rc;

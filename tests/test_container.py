@@ -246,6 +246,18 @@ def test_header_rejects_what_it_cannot_hold(H, pkg):
     assert read(good[:tied_embed] + b"\x01" + good[tied_embed + 1:]) == -2
     assert read(good[:tied_embed + 6] + b"\x01" + good[tied_embed + 7:]) == -2      # rot_pos
     assert read(good[:off_model] + b"\x07" + good[off_model + 1:]) == -1            # unknown model id
+    # sizes a model cannot be built from (they would divide by zero or end the process in the
+    # model constructor) make the header invalid
+    assert read(good[:8] + b"\x00\x00" + good[10:]) == -1                           # batch_size 0
+    assert read(good[:10] + b"\x00\x00" + good[12:]) == -1                          # seg_len 0
+    assert read(good[:12] + b"\x00\x01" + good[14:]) == -1                          # one symbol
+    assert read(good[:off_model + 1] + b"\x00" + good[off_model + 2:]) == -1         # no layers
+    assert read(good[:off_model + 2] + b"\x00" + good[off_model + 3:]) == -1         # no heads
+    assert read(good[:off_model + 3] + b"\x00\x00" + good[off_model + 5:]) == -1    # d_key 0
+    ff_act = tied_embed + 8 + 8
+    assert good[ff_act] == hp.FF_GELU and read(good[:ff_act] + b"\x09" + good[ff_act + 1:]) == -1
+    nan = b"\x7f\xc0\x00\x00"
+    assert read(good[:ff_act - 8] + nan + good[ff_act - 4:]) == -1                   # init_range NaN
     assert H.lib.nncp_header_write(C.create_string_buffer(20), 20, C.byref(cfg), C.byref(fp)) == 0
     # this build's RMSProp travels as algorithm 16 with Adam's four fields
     cfg.sgd_opt = M.rmsprop()
