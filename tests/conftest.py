@@ -30,6 +30,16 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_runtest_setup(item):
+    """Names every GPU test on the real stderr, flushed, before it touches the card: if a run
+    ends without a report, the last such line says which case was on the GPU."""
+    if item.get_closest_marker("gpu") is not None:
+        capture = item.config.pluginmanager.getplugin("capturemanager")
+        with capture.global_and_fixture_disabled():   # past pytest's capture of file descriptor 2
+            sys.stderr.write("[gpu] %s\n" % item.nodeid)
+            sys.stderr.flush()
+
+
 @pytest.fixture(scope="session")
 def pkg():
     return load_pkg()
