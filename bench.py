@@ -98,6 +98,12 @@ def bigram_zipf_dirichlet(n, n_symbols=16384, seed=2025, alpha=0.1, keep=256):
     return out
 
 
+def say(what):
+    """Progress on stderr, flushed before the step it names starts (stdout carries the one
+    JSON line only)."""
+    print("[bench] " + what, file=sys.stderr, flush=True)
+
+
 def init_weights(model, seed=99, sigma=0.02):
     """N(0, sigma) for every matrix, 1 for LayerNorm gains, 0 for biases."""
     rng = np.random.default_rng(seed)
@@ -324,14 +330,17 @@ def main_c4(args):
     mode = H.MODE_SEGMENT | H.CODER_CDF16
     pos = 0
     if args.warmup:
+        say("C4 %s: %d warm-up steps" % (args.variant, args.warmup))
         run_block(model, H, data[pos:pos + args.warmup * per_step], mode)
         pos += args.warmup * per_step
+    say("C4 %s: %d timed steps" % (args.variant, args.steps))
     l0 = model.nc.nc_get_launch_count(model.ctx)
     sec, nbytes, st = run_block(model, H, data[pos:pos + args.steps * per_step], mode)
     launches = model.nc.nc_get_launch_count(model.ctx) - l0
     pos += args.steps * per_step
     roof = None
     if args.profile_steps:
+        say("C4 %s: %d steps with per-launch GEMM events" % (args.variant, args.profile_steps))
         rows = gemm_profile(model, H, data[pos:pos + args.profile_steps * per_step], mode, pkg.binding.HIP_LIB)
         if rows:
             dom = max(rows, key=lambda r: r["seconds"])
@@ -412,8 +421,10 @@ def main():
 
     pos = 0
     if args.warmup:
+        say("C3 %s: %d warm-up steps" % (args.variant, args.warmup))
         run_block(model, H, data[pos:pos + args.warmup * per_step], mode)
         pos += args.warmup * per_step
+    say("C3 %s: %d timed steps" % (args.variant, args.steps))
     l0 = model.nc.nc_get_launch_count(model.ctx)
     sec, nbytes, st = run_block(model, H, data[pos:pos + args.steps * per_step], mode)
     launches = model.nc.nc_get_launch_count(model.ctx) - l0
@@ -422,6 +433,7 @@ def main():
 
     roof = None
     if args.profile_steps:
+        say("C3 %s: %d steps with per-launch GEMM events" % (args.variant, args.profile_steps))
         rows = gemm_profile(model, H, data[pos:pos + args.profile_steps * per_step], mode,
                             pkg.binding.HIP_LIB)
         if rows:
@@ -439,12 +451,18 @@ def main():
                     "all_gemm_tflops": round(tot_f / tot_s / 1e12, 3),
                     "all_gemm_ms_per_step": round(tot_s / args.profile_steps * 1e3, 3)}
     model.close()
-    attn = attention_c2(pkg, args.attention_iters) if args.attention_iters else None
-    cdf = cdf_c5(pkg, args.cdf_iters) if args.cdf_iters else None
+    attn = cdf = None
+    if args.attention_iters:
+        say("isolated attention, B32 H8 d64 T64 K128, %d forward+backward pairs" % args.attention_iters)
+        attn = attention_c2(pkg, args.attention_iters)
+    if args.cdf_iters:
+        say("coder-side CDF path, 64 x 16384 logits, %d iterations" % args.cdf_iters)
+        cdf = cdf_c5(pkg, args.cdf_iters)
 
     cpu = None
     if args.cpu_steps:
         threads = min(os.cpu_count() or 1, 16)
+        say("CPU checker, %d steps on %d threads" % (args.cpu_steps, threads))
         v = cpu_baseline(pkg, data, args.cpu_steps, threads)
         cpu = {"value": round(v, 1), "unit": "symbols/s", "cores": threads, "kind": "port",
                "sample": "first %d steps (%d symbols) of the same workload, CPU checker driving the "
