@@ -20,12 +20,13 @@ def _model(H, **kw):
     return pkg.host.Model(H, pkg.host.make_config(**base))
 
 
-@pytest.mark.parametrize("n", [3 * 8 * 5, 3 * 8 * 4 + 17, 11, 3 * 8 - 1])
+@pytest.mark.parametrize("n", [3 * 8 * 5, 3 * 8 * 4 + 17, 11, 3 * 8 - 1, 0, 1, 2])
 @pytest.mark.parametrize("mode", [0, 1, 2, 3])
 def test_stream_round_trip(H, n, mode):
     """encode -> decode identity incl. block_len % B != 0, a tail shorter than
-    a segment and a block shorter than one segment; all four mode/coder pairs."""
-    syms = M.markov1(n, 40, seed=n)
+    a segment, a block shorter than one segment, fewer symbols than streams and
+    the empty block; all four mode/coder pairs."""
+    syms = M.markov1(max(n, 1), 40, seed=n)[:n]
     enc = _model(H)
     data, st = enc.compress(syms, mode)
     enc.close()
