@@ -144,3 +144,46 @@ def test_bf16_operand_rounding_is_bitwise_the_checkers(source):
         nc.close()
     lib.nchip_gemm_bf16_source(1)
     assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+
+
+def _fast_stream_properties(host, cfg, syms, variant):
+    """Two encodings give the same bytes; the replaying decoder and the cached per-timestep
+    decoder both return the input."""
+    hp = M.load_pkg().host
+    n = len(syms)
+
+    def model():
+        m = hp.Model(host, hp.make_config(**cfg))
+        m.nc.nc_set_matmul_bf16(m.ctx, int(variant == "bf16"))
+        return m
+    for mode in (hp.MODE_SEGMENT | hp.CODER_CDF16, hp.MODE_SEGMENT | hp.MODE_STEP_DECODE | hp.CODER_CDF16):
+        streams = []
+        for _ in range(2):
+            enc = model()
+            data, st = enc.compress(syms, mode)
+            enc.close()
+            streams.append(data)
+        assert np.array_equal(streams[0], streams[1]), mode
+        assert st.n_symbols == n and 0 < len(streams[0]) < 2 * n, mode
+        dec = model()
+        back, _ = dec.decompress(streams[0], n, mode)
+        dec.close()
+        assert np.array_equal(back, syms), mode
+
+
+@pytest.mark.parametrize("variant", ["fp32", "bf16"])
+def test_fast_stream_properties_small(hosts, variant):
+    # heads of 32: the cached per-timestep decoder needs the single-kernel attention shapes
+    cfg = dict(n_layer=2, d_model=64, n_head=2, d_inner=96, d_pos=13, mem_len=7, seg_len=9, batch_size=3,
+               n_symbols=40, seed=7, fused=1, sgd_opt=M.rmsprop(3e-4), use_device=1)
+    _fast_stream_properties(hosts[0], cfg, M.markov1(3 * 9 * 3 + 3 * 2 + 1, 40, seed=5), variant)
+
+
+@pytest.mark.parametrize("variant", ["fp32", "bf16"])
+def test_full_size_c3_stream_round_trip_on_gpu(hosts, variant):
+    """The headline configuration at its real size (12 layers, d_model 512, 8 x 64, d_ff 2048,
+    64 + 64 keys, 32 streams, bytes): three trained segments and a ragged tail through the fast
+    stream, checked through properties that do not depend on the size."""
+    cfg = dict(n_layer=12, d_model=512, n_head=8, d_inner=2048, d_pos=128, mem_len=64, seg_len=64,
+               batch_size=32, n_symbols=256, seed=123, fused=1, sgd_opt=M.rmsprop(3e-4), use_device=1)
+    _fast_stream_properties(hosts[0], cfg, M.markov1(32 * 64 * 3 + 32 * 5 + 7, 256, seed=2024), variant)

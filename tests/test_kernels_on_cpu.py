@@ -53,8 +53,10 @@ def test_gpu_parity_tests_pass_on_the_cpu_build(emulated):
                                "test_gradients_match_checker_c1 or "
                                "(test_profile_variants_match_checker and 1-relu_coef)"])
     # (of the three file-container cases one runs here: fibers make the others minutes long)
+    # (and the full-size round trip is hours of fibers: it waits for the GPU)
     new = _pytest(emulated, ["-n", "4", "tests/test_gpu_zz_new_paths.py", "-k",
-                             "not (file_container and (reference or bf16))"])
+                             "not (file_container and (reference or bf16)) and not full_size and "
+                             "not (properties_small and bf16)"])
     out_ops, out_model = ops.communicate(timeout=1500)[0], model.communicate(timeout=1500)[0]
     out_new = new.communicate(timeout=1500)[0]
     assert ops.returncode == 0, out_ops[-3000:]
