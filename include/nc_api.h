@@ -233,6 +233,9 @@ NCTensor *nc_matmul_add(NCTensor *w, NCTensor *x, NCTensor *c, BOOL w_trans,
 NCTensor *nc_matmul(NCTensor *w, NCTensor *x);                         /* libnc.h:373 */
 NCTensor *nc_get_col(NCTensor *w, NCTensor *x);                        /* libnc.h:375 */
 NCTensor *nc_soft_max(NCTensor *x);                                    /* libnc.h:382 */
+/* max(soft_max[i] * mult, 1) converted to int32 (floor), 0 <= mult <= 2^32; the integer
+   CDF for the coder is nc_soft_max_cdf16 (nc_ext.h), which adds the exact total */
+NCTensor *nc_soft_max_int(NCTensor *x, float mult);                    /* libnc.h:383-384 */
 NCTensor *nc_indexed_log(NCTensor *x, NCTensor *eout);                 /* libnc.h:388 */
 NCTensor *nc_layer_norm(NCTensor *x, float eps);                       /* libnc.h:389 */
 NCTensor *nc_rms_norm(NCTensor *x, float eps);                         /* libnc.h:390 */

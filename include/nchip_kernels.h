@@ -243,6 +243,10 @@ int nchip_opt_update_multi(void *stream, int algo, const NchipOptTensor *dev_tab
 /* logits (v, n) f32 -> cdf (v, n) u16 as specified in nc_ext.h
    (nc_soft_max_cdf16); bit-identical to the CPU checker. */
 int nchip_softmax_cdf16(void *stream, const float *logits, uint16_t *cdf, int v, int64_t n);
+/* Integer probabilities per column (nc_soft_max_int, libnc.h:383-384): out[i] =
+   max(floor(q[i] * mult / sum q), 1) as int32, q the 24-bit integer exponentials of the CDF
+   above; 0 <= mult <= 2^32; bit-identical to the CPU checker. */
+int nchip_softmax_int(void *stream, const float *logits, int32_t *out, int v, int64_t n, float mult);
 /* sym[i, c] = largest s with cdf[s, c] <= target[i, c]; targets (m, n). */
 int nchip_cdf_lookup(void *stream, const uint16_t *cdf, const uint16_t *target,
                      uint16_t *sym, int v, int64_t m, int64_t n);

@@ -358,7 +358,57 @@ bool allow_table_lds()
     return true;
 }
 
+// Integer probabilities of libnc's nc_soft_max_int: y[i] = max(floor(q[i] * mult / Q), 1)
+// with the same 24-bit integer exponentials q and their exact sum Q as the CDF above.
+// q[i] * mult is exact in double (25 + 24 significant bits), the division is the one
+// correctly rounded IEEE operation, so the CPU checker computes the same integers.  One
+// workgroup per column, three passes over the column (maximum, sum, values): the second and
+// third read it from cache.  Not on the coder's path (nncp.c does not call it).
+__global__ __launch_bounds__(TPB) void softmax_int_kernel(const float *logits, int32_t *out, int v, float mult)
+{
+    __shared__ float s_max[TPB];
+    __shared__ unsigned long long s_sum[TPB];
+    const float *x = logits + (int64_t)blockIdx.x * v;
+    int32_t *y = out + (int64_t)blockIdx.x * v;
+    const int t = threadIdx.x;
+    float mx = x[0];
+    for (int i = t; i < v; i += TPB) mx = x[i] > mx ? x[i] : mx;
+    s_max[t] = mx;
+    __syncthreads();
+    for (int d = TPB / 2; d > 0; d >>= 1) {
+        if (t < d) s_max[t] = s_max[t + d] > s_max[t] ? s_max[t + d] : s_max[t];
+        __syncthreads();
+    }
+    mx = s_max[0];
+    unsigned long long tot = 0;
+    for (int i = t; i < v; i += TPB) tot += quant(x[i], mx);
+    s_sum[t] = tot;
+    __syncthreads();
+    for (int d = TPB / 2; d > 0; d >>= 1) {
+        if (t < d) s_sum[t] += s_sum[t + d];
+        __syncthreads();
+    }
+    const double q_total = (double)s_sum[0], m = (double)mult;
+    for (int i = t; i < v; i += TPB) {
+        double p = (double)quant(x[i], mx) * m / q_total;
+        y[i] = p >= 2147483647.0 ? 2147483647 : (p >= 1.0 ? (int32_t)p : 1);
+    }
+}
+
 } // namespace
+
+extern "C" int nchip_softmax_int(void *stream, const float *logits, int32_t *out, int v, int64_t n, float mult)
+{
+    if (n <= 0) return 0;
+    if (v < 1 || n > 0x7fffffff || !(mult >= 0.0f) || mult > 4294967296.0f) {
+        fprintf(stderr, "nchip_softmax_int: v %d, n %lld or mult %g outside what the kernel takes\n", v, (long long)n, (double)mult);
+        return -1;
+    }
+    hipLaunchKernelGGL(softmax_int_kernel, dim3((unsigned)n), dim3(TPB), 0, (hipStream_t)stream, logits, out, v, mult);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { fprintf(stderr, "nchip_softmax_int: %s\n", hipGetErrorString(e)); return -2; }
+    return 0;
+}
 
 extern "C" int nchip_softmax_cdf16(void *stream, const float *logits, uint16_t *cdf, int v, int64_t n)
 {

@@ -999,6 +999,19 @@ extern "C" NCTensor *nc_soft_max_cdf16(NCTensor *logits)
     return y;
 }
 
+extern "C" NCTensor *nc_soft_max_int(NCTensor *x, float mult) // libnc.h:383-384
+{
+    x = nc_contig(x);
+    need_f32(x, "nc_soft_max_int");
+    size_t v = x->dims[0];
+    NCTensor *y = nc_alloc(x->dev, NC_TYPE_I32, x->n_dims, x->dims, false);
+    if (nchip_softmax_int(nc_stream(x), nc_f32(x), (int32_t *)nc_data(y), (int)v, (int64_t)(nc_numel(x) / v), mult))
+        nc_fatal("nc_soft_max_int failed");
+    LAUNCHED(x);
+    nc_free_tensor(x);
+    return y;
+}
+
 extern "C" NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets)
 {
     cdf = nc_contig(cdf); targets = nc_contig(targets);

@@ -303,6 +303,45 @@ NCTensor *nc_soft_max_cdf16(NCTensor *logits)
     return y;
 }
 
+/* libnc.h:383-384, "max(soft_max[i] * mult, 1) converted to int32".  Build-defined where the
+   header is silent: the probabilities are the 24-bit integer exponentials of the CDF above over
+   their exact sum, and the conversion is a floor; q * mult is exact in double and the division
+   is one correctly rounded operation, so the GPU kernel computes the same integers. */
+NCTensor *nc_soft_max_int(NCTensor *x, float mult)
+{
+    NCTensor *y;
+    size_t V, cols;
+    x = nc_contig(x);
+    if (x->type != NC_TYPE_F32 || x->n_dims < 1)
+        nc_fatal("soft_max_int: f32 input expected");
+    if (!(mult >= 0.0f) || mult > 4294967296.0f)
+        nc_fatal("soft_max_int: mult %g outside [0, 2^32]", (double)mult);
+    V = x->dims[0];
+    cols = nc_numel(x) / V;
+    y = nc_alloc(x->dev, NC_TYPE_I32, x->n_dims, x->dims, 0);
+    for (size_t c = 0; c < cols; c++) {
+        const float *in = nc_f32(x) + c * V;
+        int32_t *out = (int32_t *)y->buf->data + c * V;
+        float mx = in[0];
+        uint64_t tot = 0;
+        for (size_t i = 1; i < V; i++)
+            mx = in[i] > mx ? in[i] : mx;
+        for (size_t i = 0; i < V; i++) {
+            float d = in[i] - mx;
+            d = d < -30.0f ? -30.0f : d;
+            tot += (uint32_t)(nc_exp_det(d) * 16777216.0f);
+        }
+        for (size_t i = 0; i < V; i++) {
+            float d = in[i] - mx;
+            d = d < -30.0f ? -30.0f : d;
+            double p = (double)(uint32_t)(nc_exp_det(d) * 16777216.0f) * (double)mult / (double)tot;
+            out[i] = p >= 2147483647.0 ? 2147483647 : (p >= 1.0 ? (int32_t)p : 1);
+        }
+    }
+    nc_free_tensor(x);
+    return y;
+}
+
 NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets)
 {
     NCTensor *y;

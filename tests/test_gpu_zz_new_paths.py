@@ -187,3 +187,20 @@ def test_full_size_c3_stream_round_trip_on_gpu(hosts, variant):
     cfg = dict(n_layer=12, d_model=512, n_head=8, d_inner=2048, d_pos=128, mem_len=64, seg_len=64,
                batch_size=32, n_symbols=256, seed=123, fused=1, sgd_opt=M.rmsprop(3e-4), use_device=1)
     _fast_stream_properties(hosts[0], cfg, M.markov1(32 * 64 * 3 + 32 * 5 + 7, 256, seed=2024), variant)
+
+
+@pytest.mark.parametrize("V,n", [(256, 64), (16384, 5), (3, 7), (1000, 33), (1, 4), (65535, 2)])
+def test_soft_max_int_bit_exact(V, n):
+    """nc_soft_max_int of the product against the checker, integer for integer."""
+    from conftest import REF_LIB, hip_lib_path
+    pkg = M.load_pkg()
+    rng = np.random.default_rng(V)
+    x = (rng.normal(0, 3, (n, V)) - np.log(rng.permutation(V) + 1.0)).astype(np.float32)
+    x[0, : min(V, 4)] = [-1e30, 80.0, -80.0, 0.0][: min(V, 4)]       # clamped tail, dominant symbol
+    for mult in (65536.0, 1000.5, 2.0 ** 31, 0.0):
+        outs = []
+        for path, dev in ((hip_lib_path(pkg), True), (REF_LIB, False)):
+            nc = pkg.binding.NC(path, use_device=dev)
+            outs.append(nc.numpy(nc.nc_soft_max_int(nc.tensor(x), mult), free=True))
+            nc.close()
+        assert outs[0].dtype == np.int32 and np.array_equal(outs[0], outs[1]), mult

@@ -228,6 +228,26 @@ def _zipf_logits(rng, n, V):
     return (rng.normal(0, 3, (n, V)) + bias).astype(np.float32)
 
 
+@pytest.mark.parametrize("V,n", [(256, 6), (16384, 2), (1, 3), (3, 5), (1000, 4)])
+@pytest.mark.parametrize("mult", [65536.0, 1000.5, 2.0 ** 31, 1.0])
+def test_soft_max_int_against_float64_softmax(ref, rng, V, n, mult):
+    """nc_soft_max_int (libnc.h:383-384), "max(soft_max[i] * mult, 1) converted to int32", pinned
+    by what it must be: int32, never below 1, ordered like the logits, and the float64 softmax
+    times mult to within one unit plus the accuracy of the exponentials it is built from
+    (24-bit fixed point relative to the column's largest, each rounded down: 2^-23 of the
+    largest entry absolute, 2^-20 relative, and V * 2^-24 relative from the V floors in the sum)."""
+    x = _zipf_logits(rng, n, V)
+    y = ref.numpy(ref.nc_soft_max_int(ref.tensor(x), mult), free=True)
+    assert y.dtype == np.int32 and y.shape == x.shape and (y >= 1).all()
+    p = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
+    p /= p.sum(axis=1, keepdims=True)
+    want = np.maximum(p * mult, 1.0)
+    assert (np.abs(y - want) <= 1.0 + want * (2.0 ** -20 + V * 2.0 ** -24)
+            + mult * p.max(axis=1, keepdims=True) * 2.0 ** -23).all()
+    order = np.argsort(x, axis=1, kind="stable")
+    assert (np.diff(np.take_along_axis(y, order, axis=1), axis=1) >= 0).all()
+
+
 @pytest.mark.parametrize("V,n", [(256, 8), (16384, 3), (2, 4), (1000, 5), (65535, 2)])
 def test_cdf16_invariants_and_accuracy(ref, rng, V, n):
     """The integer CDF is pinned by what it must be, not by its own formula:
