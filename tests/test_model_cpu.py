@@ -257,3 +257,29 @@ def test_dropout_masks_scale_and_rate(H):
     vals = np.unique(m)
     assert len(vals) == 2 and vals[0] == 0 and abs(vals[1] - 1 / 0.75) < 1e-6
     assert abs((m == 0).mean() - 0.25) < 0.01 and abs(m.mean() - 1.0) < 0.02
+
+
+def test_c1_prefix_reference_and_fast_streams_agree_in_size(H):
+    """BASELINE config 1 (2 layers, d_model 128, 4 x 32, d_ff 512, T = M = 20, batch 4, RMSProp
+    3e-4) on a prefix of its order-1 Markov bytes: the reference-faithful stream (one evaluation
+    per timestep, float symbol coder, cp_utils.c:299-323) and the fast stream (whole-segment
+    evaluation, 16-bit integer CDF) both round-trip, and their sizes agree within 0.5 %.  (On the
+    full 64 KiB both come to 55 719 bytes, 6.80 bits per symbol, after 819 steps and a 4-symbol
+    tail; that run takes two minutes on the checker and is not repeated here.)"""
+    pkg = M.load_pkg()
+    hp = pkg.host
+    n = 4 * 20 * 25 + 13
+    syms = M.markov1(65536, 256, seed=1234)[:n]
+    sizes = {}
+    for name, mode, fused in (("reference", 0, 0), ("fast", hp.MODE_SEGMENT | hp.CODER_CDF16, 1)):
+        cfg = dict(M.C1, use_device=0, nb_threads=4, fused=fused, sgd_opt=M.rmsprop(3e-4))
+        enc = hp.Model(H, hp.make_config(**cfg))
+        data, st = enc.compress(syms, mode)
+        enc.close()
+        assert st.n_steps == 25 and st.n_symbols == n
+        dec = hp.Model(H, hp.make_config(**cfg))
+        back, _ = dec.decompress(data, n, mode)
+        dec.close()
+        assert np.array_equal(back, syms), name
+        sizes[name] = len(data)
+    assert abs(sizes["fast"] - sizes["reference"]) <= 0.005 * sizes["reference"], sizes
