@@ -204,3 +204,28 @@ def test_soft_max_int_bit_exact(V, n):
             outs.append(nc.numpy(nc.nc_soft_max_int(nc.tensor(x), mult), free=True))
             nc.close()
         assert outs[0].dtype == np.int32 and np.array_equal(outs[0], outs[1]), mult
+
+
+@pytest.mark.parametrize("cfg_name", ["TINY", "C1"])
+def test_training_100_steps_match_checker(hosts, cfg_name):
+    """The 1e-5 bar after 1, 10 and 100 steps of the fused path (probabilities, loss, every
+    parameter tensor).  On the CPU build of the kernels the small configuration stays at 6e-7
+    over all 100 steps; too long to repeat there in every test run."""
+    pkg = M.load_pkg()
+    cfg = getattr(M, cfg_name)
+    hip = pkg.host.Model(hosts[0], pkg.host.make_config(**dict(cfg, use_device=1, fused=1, sgd_opt=M.rmsprop(3e-4))))
+    ref = pkg.host.Model(hosts[1], pkg.host.make_config(**dict(cfg, use_device=0, nb_threads=8, fused=1,
+                                                               sgd_opt=M.rmsprop(3e-4))))
+    B, T, V = cfg["batch_size"], cfg["seg_len"], cfg["n_symbols"]
+    syms = M.markov1(B * T * 100, V, seed=77)
+    for step, (tok, tgt) in enumerate(M.segment_batches(syms, B, T, 100), 1):
+        ph, lh = hip.train_step(tok, tgt, 3e-4)
+        pr, lr_ = ref.train_step(tok, tgt, 3e-4)
+        if step in (1, 10, 100):
+            assert M.relerr(ph, pr) <= 1e-5, step
+            assert abs(lh - lr_) <= 1e-5 * abs(lr_), step
+            w_h, w_r = hip.params(), ref.params()
+            for k in w_r:
+                assert M.tensors_close(w_h[k], w_r[k], 1e-5), (step, k, M.rel_l2(w_h[k], w_r[k]))
+    hip.close()
+    ref.close()
