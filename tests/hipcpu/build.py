@@ -39,7 +39,19 @@ def _compile(name):
     return obj
 
 
-def build(jobs=8):
+def up_to_date():
+    """The library is newer than everything it is built from."""
+    if not os.path.exists(OUT):
+        return False
+    inc = os.path.join(ROOT, "include")
+    deps = [os.path.join(d, f) for d in (CSRC, inc, HERE, os.path.join(HERE, "hip")) for f in os.listdir(d)
+            if f.endswith((".hip", ".cpp", ".h", ".py"))]
+    return os.path.getmtime(OUT) > max(os.path.getmtime(f) for f in deps)
+
+
+def build(jobs=8, force=False):
+    if not force and up_to_date():
+        return OUT
     os.makedirs(BUILD, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(_compile, SOURCES))
@@ -56,4 +68,4 @@ def build(jobs=8):
 
 
 if __name__ == "__main__":
-    print(build())
+    print(build(force=True))

@@ -1,9 +1,10 @@
-"""GPU side of the paths written after the last GPU run: the retrain pass
-(nncp_retrain_block, dropout) and the LSTM model class - the same host C code as
-on the CPU checker, linked against libnc_hip.so.  They have run on the CPU build
-of the kernels (tests/test_kernels_on_cpu.py sets NNCP_TEST_HIP_LIB) but not yet
-on an MI355X, so without that variable they are skipped.  Collected after the
-other GPU tests (file name)."""
+"""GPU tests written after the last GPU run: the retrain pass (nncp_retrain_block, dropout),
+the LSTM model class and the file container - the same host C code as on the CPU checker,
+linked against libnc_hip.so - the bitwise bf16 operand rounding, nc_soft_max_int, the 1e-5
+bar after 100 steps and the round trip of the headline configuration at its full size.  They
+have run on the CPU build of the kernels (tests/test_kernels_on_cpu.py sets NNCP_TEST_HIP_LIB;
+the two long ones only in a small form) but not yet on an MI355X, so without that variable they
+are skipped.  Collected after the other GPU tests (file name)."""
 import os
 
 import numpy as np
@@ -176,7 +177,7 @@ def test_fast_stream_properties_small(hosts, variant):
     # heads of 32: the cached per-timestep decoder needs the single-kernel attention shapes
     cfg = dict(n_layer=2, d_model=64, n_head=2, d_inner=96, d_pos=13, mem_len=7, seg_len=9, batch_size=3,
                n_symbols=40, seed=7, fused=1, sgd_opt=M.rmsprop(3e-4), use_device=1)
-    _fast_stream_properties(hosts[0], cfg, M.markov1(3 * 9 * 3 + 3 * 2 + 1, 40, seed=5), variant)
+    _fast_stream_properties(hosts[0], cfg, M.markov1(3 * 9 * 2 + 3 * 2 + 1, 40, seed=5), variant)
 
 
 @pytest.mark.parametrize("variant", ["fp32", "bf16"])

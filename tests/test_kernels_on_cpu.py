@@ -26,7 +26,8 @@ def emulated():
         hipcpu_build.build()
     finally:
         sys.path.remove(EMU_DIR)
-    r = subprocess.run(["make", "-B", "LIBNC_DIR=../../tests/hipcpu", "LIBNC=nc_hipcpu", "OUT=" + EMU_HOST,
+    # (rebuilt only when a source is newer; a stale library cannot pass for a fresh one)
+    r = subprocess.run(["make", "LIBNC_DIR=../../tests/hipcpu", "LIBNC=nc_hipcpu", "OUT=" + EMU_HOST,
                         "RPATH=$$ORIGIN"], cwd=os.path.join(ROOT, "nncp-metal_amd", "host"),
                        capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
@@ -46,15 +47,15 @@ def test_gpu_parity_tests_pass_on_the_cpu_build(emulated):
     whole-model gradient, cached per-timestep logits bit-identical, a profile
     variant, the retrain pass, the LSTM model class and a file through the container), with
     guard pages behind every device buffer."""
-    ops = _pytest(emulated, ["-n", "5", "tests/test_gpu_ops.py"])
-    model = _pytest(emulated, ["-n", "3", "tests/test_gpu_model.py", "-k",
+    ops = _pytest(emulated, ["-n", "4", "tests/test_gpu_ops.py"])
+    model = _pytest(emulated, ["-n", "2", "tests/test_gpu_model.py", "-k",
                                "(test_training_steps_match_checker and TINY) or "
                                "(test_cached_timestep_logits_are_bit_identical and SMALL32) or "
                                "test_gradients_match_checker_c1 or "
                                "(test_profile_variants_match_checker and 1-relu_coef)"])
     # (of the three file-container cases one runs here: fibers make the others minutes long)
     # (and the full-size round trip is hours of fibers: it waits for the GPU)
-    new = _pytest(emulated, ["-n", "4", "tests/test_gpu_zz_new_paths.py", "-k",
+    new = _pytest(emulated, ["-n", "6", "tests/test_gpu_zz_new_paths.py", "-k",
                              "not (file_container and (reference or bf16)) and not full_size and "
                              "not (properties_small and bf16) and not 100_steps"])
     out_ops, out_model = ops.communicate(timeout=1500)[0], model.communicate(timeout=1500)[0]
