@@ -286,6 +286,14 @@ class Model:
         C.memmove(self.nc.nc_tensor_get_ptr(x, None), arr.ctypes.data, arr.nbytes)
         return x
 
+    def _symbols(self, a):
+        """Token ids as int32, refused when one lies outside the alphabet: on the device they
+        index the embedding table and the probability columns unchecked."""
+        a = np.asarray(a, dtype=np.int32)
+        if a.size and (a.min() < 0 or a.max() >= self.cfg.n_symbols):
+            raise ValueError("symbol outside [0, %d)" % self.cfg.n_symbols)
+        return a
+
     def param_names(self):
         n = self.L.nncp_model_param_count(self.ptr)
         return [self.L.nncp_model_param_name(self.ptr, i).decode() for i in range(n)]
@@ -306,7 +314,7 @@ class Model:
     def eval(self, tokens, output_index=-1, keep=False):
         """tokens: int array (T, B) [numpy order of the (B, T) input tensor].
         Returns the probabilities as numpy (T|1, B, V)."""
-        inp = self._host_tensor(np.asarray(tokens, dtype=np.int32))
+        inp = self._host_tensor(self._symbols(tokens))
         out = self._eval(self.ptr, output_index, inp)
         self.nc.nc_free_tensor(inp)
         res = self._to_numpy(out)
@@ -322,7 +330,7 @@ class Model:
         """Per-timestep cached evaluation of a whole segment (trf_step_begin +
         trf_eval_step for every position).  Returns (probabilities (T, B, V),
         logits (T, B, V)) assembled from the single-column results."""
-        tokens = np.asarray(tokens, dtype=np.int32)
+        tokens = self._symbols(tokens)
         inp = self._host_tensor(tokens)
         self.L.trf_step_begin(self.ptr)
         probs, logits = [], []
@@ -339,7 +347,7 @@ class Model:
         """One full-segment evaluation + gradient + update; returns
         (probabilities, loss in nats summed over the segment)."""
         p = self.eval(tokens, -1, keep=True)
-        tgt = self._host_tensor(np.asarray(targets, dtype=np.int32))
+        tgt = self._host_tensor(self._symbols(targets))
         self.L.trf_set_lr(self.ptr, lr)  # both classes: nc_sgd_opt_set_lr on the model's optimiser
         loss = self._eval_gradient(self.ptr, tgt)
         self.nc.nc_free_tensor(tgt)

@@ -218,6 +218,13 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
 
     const NNCPConfig *cfg = nncp_model_config(s);
     int B = cfg->batch_size, T = cfg->seg_len;
+    /* symbols index the embedding table and the probability columns on the device, where
+       nothing checks them: an encoder refuses a block that holds one outside the alphabet
+       (a decoder only ever produces symbols below n_symbols) */
+    if (!is_decode)
+        for (int i = 0; i < block_len; i++)
+            if (block_buf[i] >= cfg->n_symbols)
+                die_stream("a symbol of the block lies outside the model's alphabet");
     c.n_symbols = cfg->n_symbols;
     c.B = B;
     c.view.rbuf = block_buf; c.view.wbuf = block_buf;

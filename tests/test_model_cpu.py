@@ -2,6 +2,8 @@
 round-trips, per-timestep and whole-segment evaluation agree (nncp.c's
 seq_eval invariant), the fused entry points reproduce the op-by-op path, and
 the whole-model gradient matches a directional finite difference."""
+import os
+
 import numpy as np
 import pytest
 
@@ -283,3 +285,23 @@ def test_c1_prefix_reference_and_fast_streams_agree_in_size(H):
         assert np.array_equal(back, syms), name
         sizes[name] = len(data)
     assert abs(sizes["fast"] - sizes["reference"]) <= 0.005 * sizes["reference"], sizes
+
+
+def test_symbols_outside_the_alphabet_are_refused_on_the_host(H):
+    """Symbols index device tables unchecked, so the host turns them away first: the Python
+    layer raises, the C block loop ends the process with a message (checked in a child)."""
+    import subprocess
+    import sys
+    m = _model(H)
+    bad = np.zeros((8, 3), dtype=np.int32)
+    bad[2, 1] = 40                                     # alphabet of TINY is 0..39
+    with pytest.raises(ValueError):
+        m.eval(bad)
+    with pytest.raises(ValueError):
+        m.train_step(np.zeros((8, 3), dtype=np.int32), bad, 3e-4)
+    m.close()
+    code = ("import sys; sys.path.insert(0, %r); import numpy as np, modelutil as M\n"
+            "pkg = M.load_pkg(); m = pkg.host.Model(M.ref_host(), pkg.host.make_config(**dict(M.TINY, use_device=0)))\n"
+            "m.compress(np.array([1, 2, 40, 3], dtype=np.uint16), 0)") % (os.path.dirname(os.path.abspath(__file__)),)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+    assert r.returncode != 0 and "outside the model's alphabet" in r.stderr
