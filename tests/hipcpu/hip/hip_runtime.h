@@ -10,6 +10,14 @@
  * from hipMalloc / hipHostMalloc and the dynamic LDS of a launch sit against guard
  * pages, so an out-of-range access raises SIGSEGV at the faulting statement.  The three
  * MFMA instructions the kernels use are computed from their documented lane layouts.
+ *
+ * The stream is asynchronous as on the GPU: kernel launches and asynchronous copies
+ * between hipMalloc / hipHostMalloc blocks are queued (kernel arguments by value) and
+ * carried out in order as late as the API allows - at the next wait (stream, device,
+ * event), blocking copy, copy to pageable memory or free.  Host code that rewrites or
+ * recycles a pinned buffer before the work that reads it has run, or reads results
+ * without waiting, therefore misbehaves here as it may on the GPU.  HIPCPU_SYNC=1 runs
+ * every operation at once instead.
  */
 #ifndef HIPCPU_RUNTIME_H
 #define HIPCPU_RUNTIME_H
@@ -20,6 +28,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <functional>
 #include <tuple>
 #include <type_traits>
 #include <utility>
@@ -86,18 +95,24 @@ static inline hipError_t hipGetDeviceCount(int *n) { *n = 1; return hipSuccess; 
 static inline hipError_t hipStreamCreate(hipStream_t *s) { *s = (hipStream_t)0x1; return hipSuccess; }
 static inline hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned) { *s = (hipStream_t)0x1; return hipSuccess; }
 static inline hipError_t hipStreamDestroy(hipStream_t) { return hipSuccess; }
-static inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
-static inline hipError_t hipDeviceSynchronize(void) { return hipSuccess; }
+extern "C" hipError_t hipcpu_memcpy_async(void *d, const void *s, size_t n);
+extern "C" void hipcpu_flush_copies(void);
+static inline hipError_t hipStreamSynchronize(hipStream_t) { hipcpu_flush_copies(); return hipSuccess; }
+static inline hipError_t hipDeviceSynchronize(void) { hipcpu_flush_copies(); return hipSuccess; }
 static inline hipError_t hipMemcpyAsync(void *d, const void *s, size_t n, hipMemcpyKind, hipStream_t)
 {
+    return hipcpu_memcpy_async(d, s, n);
+}
+static inline hipError_t hipMemcpy(void *d, const void *s, size_t n, hipMemcpyKind)
+{
+    hipcpu_flush_copies();
     memmove(d, s, n);
     return hipSuccess;
 }
-static inline hipError_t hipMemcpy(void *d, const void *s, size_t n, hipMemcpyKind) { memmove(d, s, n); return hipSuccess; }
 static inline hipError_t hipEventCreate(hipEvent_t *e) { *e = nullptr; return hipSuccess; }
 static inline hipError_t hipEventDestroy(hipEvent_t) { return hipSuccess; }
 static inline hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
-static inline hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
+static inline hipError_t hipEventSynchronize(hipEvent_t) { hipcpu_flush_copies(); return hipSuccess; }
 static inline hipError_t hipEventElapsedTime(float *ms, hipEvent_t, hipEvent_t) { *ms = 1e-3f; return hipSuccess; }
 static inline hipError_t hipFuncSetAttribute(const void *, hipFuncAttribute, int) { return hipSuccess; }
 
@@ -105,14 +120,19 @@ static inline hipError_t hipFuncSetAttribute(const void *, hipFuncAttribute, int
 template <typename F, typename Tuple, size_t... I>
 static void hipcpu_apply(F f, Tuple &t, std::index_sequence<I...>) { f(std::get<I>(t)...); }
 
+void hipcpu_enqueue(std::function<void()> op);
+
 template <typename F, typename... A>
 static void hipcpu_launch_impl(F kernel, dim3 grid, dim3 block, size_t shmem, A... args)
 {
-    struct Closure { F k; std::tuple<A...> a; } c{ kernel, std::tuple<A...>(args...) };
-    hipcpu_launch(grid, block, shmem, [](void *p) {
-        Closure *q = (Closure *)p;
-        hipcpu_apply(q->k, q->a, std::index_sequence_for<A...>());
-    }, &c);
+    struct Closure { F k; std::tuple<A...> a; };
+    Closure c{ kernel, std::tuple<A...>(args...) };
+    hipcpu_enqueue([c, grid, block, shmem]() mutable {
+        hipcpu_launch(grid, block, shmem, [](void *p) {
+            Closure *q = (Closure *)p;
+            hipcpu_apply(q->k, q->a, std::index_sequence_for<A...>());
+        }, &c);
+    });
 }
 #define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...) \
     hipcpu_launch_impl(kernel, dim3(grid), dim3(block), (size_t)(shmem), ##__VA_ARGS__)

@@ -6,6 +6,7 @@
 #include <sys/mman.h>
 #include <ucontext.h>
 #include <unistd.h>
+#include <functional>
 #include <map>
 #include <vector>
 
@@ -73,9 +74,33 @@ void *guarded_alloc(size_t n)
     return p;
 }
 
+/* ---- the stream: a queue of launches and copies, drained at the waits ---------------------- */
+std::vector<std::function<void()>> g_queue;
+bool g_draining = false;
+const bool g_sync = getenv("HIPCPU_SYNC") && atoi(getenv("HIPCPU_SYNC")) != 0;
+
+bool in_runtime_block(const void *q)
+{
+    auto it = g_allocs.upper_bound(const_cast<void *>(q));
+    if (it == g_allocs.begin()) return false;
+    --it;
+    const char *end = (const char *)it->second.map + it->second.map_len - PAGE;
+    return (const char *)q >= (const char *)it->first && (const char *)q < end;
+}
+
+void flush_copies()
+{
+    if (g_draining) return;
+    g_draining = true;
+    for (size_t i = 0; i < g_queue.size(); i++) g_queue[i]();
+    g_queue.clear();
+    g_draining = false;
+}
+
 void guarded_free(void *p)
 {
     if (!p) return;
+    flush_copies(); /* the runtime waits for the device before it releases memory */
     auto it = g_allocs.find(p);
     if (it == g_allocs.end()) die("free of a pointer that hipMalloc did not return");
     munmap(it->second.map, it->second.map_len);
@@ -225,7 +250,27 @@ hipError_t hipMalloc(void **p, size_t n)
     return *p ? hipSuccess : hipErrorOutOfMemory;
 }
 hipError_t hipFree(void *p) { guarded_free(p); return hipSuccess; }
-hipError_t hipHostMalloc(void **p, size_t n, unsigned) { return hipMalloc(p, n); }
-hipError_t hipHostFree(void *p) { return hipFree(p); }
+void hipcpu_flush_copies(void) { flush_copies(); }
+hipError_t hipcpu_memcpy_async(void *d, const void *s, size_t n)
+{
+    if (in_runtime_block(d) && in_runtime_block(s)) {
+        hipcpu_enqueue([d, s, n]() { memmove(d, s, n); });
+    } else if (in_runtime_block(d)) {
+        /* pageable source: staged before the call returns, written in stream order */
+        std::vector<char> staged((const char *)s, (const char *)s + n);
+        hipcpu_enqueue([d, staged]() { memcpy(d, staged.data(), staged.size()); });
+    } else {
+        flush_copies(); /* pageable destination: the call waits */
+        memmove(d, s, n);
+    }
+    return hipSuccess;
+}
 
 } // extern "C"
+
+void hipcpu_enqueue(std::function<void()> op)
+{
+    if (g_sync || g_draining) { op(); return; }
+    g_queue.push_back(std::move(op));
+    if (g_queue.size() >= 100000) flush_copies();
+}

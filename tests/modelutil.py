@@ -101,3 +101,43 @@ def tensors_close(a, b, tol=1e-5, max_factor=30, outliers=1e-4):
     n_out = int((d > max_factor * tol).sum())
     return (rel_l2(a, b) <= tol and d.max() <= 4 * max_factor * tol
             and n_out <= max(1, int(outliers * d.size)))
+
+
+def float64_trajectory(cfg, w0, batches, snapshots, lr=3e-4, beta2=0.99, eps=1e-8, threads=None):
+    """The same RMSProp training steps evaluated in float64 by the torch statement of
+    tests/test_model_torch.py (index-level formulas, autograd gradients), from the weights
+    w0 and an empty memory.  Returns ([(probabilities (T, B, V), loss summed over the
+    segment)], {step: {name: weights}}).  It is the arbiter where two fp32 evaluations differ
+    by more than the bar: fp32 rounding noise, amplified by the sign-like RMSProp update of
+    small gradients, is then measured on both sides against it."""
+    import torch
+    from test_model_torch import _torch_step
+    if threads:
+        torch.set_num_threads(threads)
+    cfg = dict(cfg)
+    cfg.setdefault("attn_len", [cfg["mem_len"] + cfg["seg_len"]] * cfg["n_layer"])
+    B, T, D = cfg["batch_size"], cfg["seg_len"], cfg["d_model"]
+    w = {k: torch.tensor(v.astype(np.float64), requires_grad=True) for k, v in w0.items()}
+    v2 = {k: torch.zeros_like(t) for k, t in w.items()}
+    mem = [torch.zeros(B, cfg["mem_len"], D, dtype=torch.float64) for _ in range(cfg["n_layer"])]
+    steps, weights = [], {}
+    for step, (tok, tgt) in enumerate(batches, 1):
+        probs, nll, inputs = _torch_step(w, cfg, tok, tgt, mem)
+        nll.backward()
+        with torch.no_grad():
+            for k in w:
+                g = w[k].grad
+                v2[k] = beta2 * v2[k] + (1 - beta2) * g * g
+                w[k] -= lr * g / (v2[k].sqrt() + eps)
+                w[k].grad = None
+        mem = [torch.cat([m[:, T:], x.detach().transpose(0, 1)], dim=1) for m, x in zip(mem, inputs)]
+        steps.append((probs.detach().numpy(), nll.item() * B * T))
+        if step in snapshots:
+            weights[step] = {k: t.detach().numpy().copy() for k, t in w.items()}
+    return steps, weights
+
+
+def within_or_no_worse(err, yardstick, tol, factor=3.0):
+    """err <= tol, or - where the reference's own fp32 arithmetic is further than tol from the
+    float64 evaluation - err within `factor` of that yardstick: the same order of rounding noise."""
+    return err <= max(tol, factor * yardstick)

@@ -4,19 +4,18 @@ of nc_relpos_attention (nncp.c:763-800) under a change of variables done on the 
     q' = q + u,   w_r[:, d_pos-1-d, h] = R[d],   b_r[K-1-d, h] = (v_h - u_h).R[d],  b_r_scale = 1
 and its gradients follow by the chain rule (du = sum dq' - dv,  dv_h = sum_d db_r[K-1-d, h] R[d]).
 Checked on the CPU checker against a torch float64 statement of the classic form with autograd;
-the GPU kernels are compared with the checker through the same entry point elsewhere."""
+the GPU kernels go through the same comparison at the size of the isolated-attention
+configuration (32 streams, 8 heads of 64, 64 queries against 64 + 64 keys)."""
 import math
 
 import numpy as np
+import pytest
 import torch
 
 import cases
 
-H, DK, B, T, MEM = 2, 8, 2, 6, 6
-K = T + MEM
 
-
-def _table():
+def _table(K, DK):
     d = np.arange(K, dtype=np.float64)[:, None]
     inv = 1.0 / 10000 ** (np.arange(0, DK, 2) / DK)
     r = np.zeros((K, DK))
@@ -24,14 +23,15 @@ def _table():
     return r  # R[d], d = distance from the key to the query
 
 
-def test_classic_txl_attention_through_the_relpos_entry_point(ref):
+def _classic_against_torch(nc, H, DK, B, T, MEM, sigma, sigma_uv, tol):
+    K = T + MEM
     rng = np.random.default_rng(21)
-    q = rng.normal(0, 0.5, (T, B, H, DK))
-    kv = rng.normal(0, 0.5, (T, B, 2 * H * DK))
-    kvm = rng.normal(0, 0.5, (MEM, B, 2 * H * DK))
-    u, v = rng.normal(0, 0.3, (H, DK)), rng.normal(0, 0.3, (H, DK))
+    q = rng.normal(0, sigma, (T, B, H, DK))
+    kv = rng.normal(0, sigma, (T, B, 2 * H * DK))
+    kvm = rng.normal(0, sigma, (MEM, B, 2 * H * DK))
+    u, v = rng.normal(0, sigma_uv, (H, DK)), rng.normal(0, sigma_uv, (H, DK))
     weight = rng.normal(0, 1, (T, B, H * DK))
-    R = _table()
+    R = _table(K, DK)
 
     # --- classic form in torch ---------------------------------------------------
     tq, tkv, tkvm, tu, tv = (torch.tensor(a, requires_grad=True) for a in (q, kv, kvm, u, v))
@@ -53,11 +53,11 @@ def test_classic_txl_attention_through_the_relpos_entry_point(ref):
     b_r = np.einsum("hd,pd->hp", v - u, R)[:, ::-1].copy()         # column K-1-d holds distance d
     arrays = [a.astype(np.float32) for a in ((q + u).reshape(T, B, H * DK), kv, kvm, w_r, b_r)]
     case = cases.Case("classic", None,
-                      lambda nc, q_, kv_, kvm_, w_, b_: nc.nc_relpos_attention(q_, kv_, kvm_, w_, b_, H, DK, K, 1.0),
+                      lambda nc_, q_, kv_, kvm_, w_, b_: nc_.nc_relpos_attention(q_, kv_, kvm_, w_, b_, H, DK, K, 1.0),
                       None)
-    out, (dq, dkv, dkvm, dw_r, db_r) = case.run(ref, arrays, weight)
+    out, (dq, dkv, dkvm, dw_r, db_r) = case.run(nc, arrays, weight)
 
-    def close(a, b, tol=2e-5):
+    def close(a, b):
         return np.abs(a - b).max() <= tol * max(np.abs(b).max(), 1e-30)
     assert close(out, out_t.detach().numpy())
     assert close(dq.reshape(T, B, H, DK), tq.grad.numpy())
@@ -67,3 +67,14 @@ def test_classic_txl_attention_through_the_relpos_entry_point(ref):
     du = dq.reshape(T, B, H, DK).astype(np.float64).sum(axis=(0, 1)) - dv
     assert close(dv, tv.grad.numpy())
     assert close(du, tu.grad.numpy())
+
+
+def test_classic_txl_attention_through_the_relpos_entry_point(ref):
+    _classic_against_torch(ref, H=2, DK=8, B=2, T=6, MEM=6, sigma=0.5, sigma_uv=0.3, tol=2e-5)
+
+
+@pytest.mark.gpu
+def test_classic_txl_attention_on_gpu_at_the_isolated_attention_size(hip):
+    """Q, K, V ~ N(0, 1/64), u, v ~ N(0, 0.02), upstream gradient ~ N(0, 1): the single-kernel
+    forward and backward against torch float64 autograd of the classic form, 1e-5."""
+    _classic_against_torch(hip, H=8, DK=64, B=32, T=64, MEM=64, sigma=0.125, sigma_uv=0.02, tol=1e-5)

@@ -206,6 +206,15 @@ def test_cached_timestep_logits_are_bit_identical(hosts, cfg_name, bf16):
     m.close()
     assert step.shape == full.shape
     assert np.array_equal(step, full)
+    # and they are the checker's whole-segment logits for the same weights and memory
+    ref = pkg.host.Model(hosts[1], pkg.host.make_config(**dict(cfg, use_device=0, nb_threads=8, fused=1,
+                                                               sgd_opt=M.rmsprop(3e-4))))
+    ref.train_step(tok0, tgt0, 3e-4)
+    ref.eval(tok1, keep=True)
+    ref_logits = ref.logits()
+    ref.L.trf_eval_end(ref.ptr)
+    ref.close()
+    assert M.relerr(step, ref_logits) <= (2e-2 if bf16 else 1e-5)
 
 
 @pytest.mark.parametrize("coder", [0, 2])
