@@ -208,6 +208,12 @@ int nchip_softmax_bwd(void *stream, const float *y, const float *g, float *dx, i
 /* y[c] = log p[idx[c], c]; fused gradient dlogits = g[c]*(onehot - p)
    (libnc.h:385-388; nncp.c:1170). */
 int nchip_indexed_log(void *stream, const float *p, const int32_t *idx, float *y, int v, int64_t n);
+/* nchip_indexed_log and nchip_get_col index a table with the caller's data.  An index outside
+   [0, v) reads nothing - the result is 0 - and raises a flag in pinned host memory.
+   nchip_index_error() returns that flag and clears it; it is meaningful after a wait for the
+   stream the kernels ran on (nc_synchronize and every other wait of the tensor library check
+   it and end the process with a message, as libnc does on misuse). */
+int nchip_index_error(void);
 int nchip_nll_bwd(void *stream, const float *p, const int32_t *idx, const float *g,
                   float *dlogits, int v, int64_t n, int fused);
 

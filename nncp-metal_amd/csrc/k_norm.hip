@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
+#include <mutex>
 #include "../../include/nchip_kernels.h"
 
 namespace {
@@ -213,10 +215,16 @@ __global__ __launch_bounds__(TPB) void softmax_bwd_kernel(const float *y, const 
     for (int i = lane; i < v; i += 64) dx[c * v + i] = yc[i] * (gc[i] - s);
 }
 
-__global__ void indexed_log_kernel(const float *p, const int32_t *idx, float *y, int v, int64_t n)
+// Indices come from the caller's data: one outside [0, v) reads nothing (the result is 0)
+// and raises the flag, a word of pinned host memory that the host looks at after a wait.
+__global__ void indexed_log_kernel(const float *p, const int32_t *idx, float *y, int v, int64_t n, int *bad)
 {
     int64_t c = (int64_t)blockIdx.x * TPB + threadIdx.x;
-    if (c < n) y[c] = logf(p[c * v + idx[c]]);
+    if (c >= n) return;
+    const int s = idx[c];
+    const bool ok = (unsigned)s < (unsigned)v;
+    y[c] = ok ? logf(p[c * v + s]) : 0.0f;
+    if (!ok) *bad = 1;
 }
 
 __global__ void nll_bwd_kernel(const float *p, const int32_t *idx, const float *g, float *dl,
@@ -233,12 +241,15 @@ __global__ void nll_bwd_kernel(const float *p, const int32_t *idx, const float *
     }
 }
 
-__global__ void get_col_kernel(const float *w, const int32_t *idx, float *y, int d, int64_t total)
+__global__ void get_col_kernel(const float *w, const int32_t *idx, float *y, int d, int v, int64_t total, int *bad)
 {
     for (int64_t e = (int64_t)blockIdx.x * TPB + threadIdx.x; e < total; e += (int64_t)gridDim.x * TPB) {
         int64_t c = e / d;
         int i = (int)(e % d);
-        y[e] = w[(int64_t)idx[c] * d + i];
+        const int s = idx[c];
+        const bool ok = (unsigned)s < (unsigned)v;
+        y[e] = ok ? w[(int64_t)s * d + i] : 0.0f;
+        if (!ok && i == 0) *bad = 1;
     }
 }
 
@@ -461,10 +472,38 @@ int nchip_softmax_bwd(void *stream, const float *y, const float *g, float *dx, i
     return check("nchip_softmax_bwd");
 }
 
+// The out-of-range flag: one int of pinned host memory per process, written by the kernels
+// that index a table with caller data, read (and cleared) by nchip_index_error().
+static int *index_flag()
+{
+    static int *flag = nullptr;
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!flag) {
+        void *p = nullptr;
+        if (hipHostMalloc(&p, 64, hipHostMallocDefault) != hipSuccess || !p) {
+            fprintf(stderr, "nchip: cannot allocate the index error flag\n");
+            abort();
+        }
+        flag = (int *)p;
+        *flag = 0;
+    }
+    return flag;
+}
+
+int nchip_index_error(void)
+{
+    int *f = index_flag();
+    const int v = *(volatile int *)f;
+    *(volatile int *)f = 0;
+    return v;
+}
+
 int nchip_indexed_log(void *stream, const float *p, const int32_t *idx, float *y, int v, int64_t n)
 {
     if (n <= 0) return 0;
-    hipLaunchKernelGGL(indexed_log_kernel, dim3(grid_for(n, 1 << 20)), dim3(TPB), 0, (hipStream_t)stream, p, idx, y, v, n);
+    hipLaunchKernelGGL(indexed_log_kernel, dim3(grid_for(n, 1 << 20)), dim3(TPB), 0, (hipStream_t)stream, p, idx, y, v, n,
+                       index_flag());
     return check("nchip_indexed_log");
 }
 
@@ -478,9 +517,9 @@ int nchip_nll_bwd(void *stream, const float *p, const int32_t *idx, const float 
 
 int nchip_get_col(void *stream, const float *w, const int32_t *idx, float *y, int d, int v, int64_t n)
 {
-    (void)v;
     if (n <= 0) return 0;
-    hipLaunchKernelGGL(get_col_kernel, dim3(grid_for(n * d)), dim3(TPB), 0, (hipStream_t)stream, w, idx, y, d, n * d);
+    hipLaunchKernelGGL(get_col_kernel, dim3(grid_for(n * d)), dim3(TPB), 0, (hipStream_t)stream, w, idx, y, d, v, n * d,
+                       index_flag());
     return check("nchip_get_col");
 }
 

@@ -165,6 +165,8 @@ void nc_stream_wait(NCContext *m)
 {
     hip_check(hipStreamSynchronize(m->stream), "hipStreamSynchronize");
     m->sync_count++;
+    if (nchip_index_error())
+        nc_fatal("a token index outside its table reached nc_get_col or nc_indexed_log");
 }
 
 void nc_staging_retire(NCContext *m, void *p, size_t cap, uint64_t stamp)
@@ -741,6 +743,9 @@ extern "C" void sgd_opt_update_var(void *opaque, NCTensor *yg, NCTensor *get_col
         vs->has_grad = true;
     } else {
         need_dev(yg, "sgd_opt_update_var");
+        // a second gradient before the update (accumulation): with deferred weight gradients
+        // yg, or the gradient kept from the first pass, may still wait for the grouped launch
+        nc_flush_deferred(nc_ctx(yg));
         NCTensor *sum = nc_alloc_like(yg);
         k_binary_prefix(nc_stream(yg), KB_ADD, nc_f32(vs->g), nc_f32(yg), nc_f32(sum), (int64_t)vs->n, (int64_t)vs->n);
         nc_ctx(yg)->launches++;

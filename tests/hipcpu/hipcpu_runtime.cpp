@@ -250,6 +250,8 @@ hipError_t hipMalloc(void **p, size_t n)
     return *p ? hipSuccess : hipErrorOutOfMemory;
 }
 hipError_t hipFree(void *p) { guarded_free(p); return hipSuccess; }
+hipError_t hipHostMalloc(void **p, size_t n, unsigned) { return hipMalloc(p, n); }
+hipError_t hipHostFree(void *p) { return hipFree(p); }
 void hipcpu_flush_copies(void) { flush_copies(); }
 hipError_t hipcpu_memcpy_async(void *d, const void *s, size_t n)
 {

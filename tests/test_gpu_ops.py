@@ -197,6 +197,35 @@ def test_optimiser_step(hip, ref, rng, pkg, algo):
     assert relerr(res[0], res[1]) <= 1e-6
 
 
+def test_two_gradients_before_one_update_with_deferred_weight_gradients(hip, rng, pkg):
+    """Gradient accumulation (two nc_backward passes, one nc_sgd_opt_update) while the weight
+    gradients of a pass are deferred to one grouped launch at its end: the second pass must
+    add to a gradient that has been written.  Plain SGD with lr = 1 exposes the sum."""
+    B = pkg.binding
+    w0 = rng.standard_normal((30, 40)).astype(np.float32)          # (m = 40, k = 30) in libnc order
+    x = rng.standard_normal((16, 30)).astype(np.float32)
+    up = [rng.standard_normal((16, 40)).astype(np.float32) for _ in range(2)]
+    nc = B.NC(hip.lib._name, use_device=True)
+    nc.nc_set_deferred_weight_grad(nc.ctx, 1)
+    h, p = nc.param(w0)
+    sp = B.SGDOptParams(algo=B.SGD_OPT_BASIC, lr=1.0)
+    opt = nc.nc_sgd_opt_init(nc.ctx, C.byref(sp))
+    nc.nc_sgd_opt_set_all(C.byref(nc.plist), opt)
+    forward = C.cast(nc.lib.sgd_opt_update_var, B.PARAM_UPDATE_FUNC)
+    for u in up:
+        y = nc.nc_matmul(nc.dup(h.value), nc.tensor(x))
+        loss = nc.nc_sum(nc.nc_mul(y, nc.tensor(u)))
+        nc.lib.nc_backward(loss, nc.nc_new_f32(nc.dev, 1.0), forward, 0)
+        nc.free(loss)
+    nc.nc_sgd_opt_update(opt)
+    w1 = nc.numpy(h.value)
+    nc.nc_sgd_opt_set_all(C.byref(nc.plist), None)
+    nc.nc_sgd_opt_end(opt)
+    nc.close()
+    grad = x.astype(np.float64).T @ (up[0].astype(np.float64) + up[1])     # numpy (k, m): dW[m, k] = sum_n dY[m, n] X[k, n]
+    assert relerr(w0 - w1, grad) <= 1e-5
+
+
 def test_views_and_copies_on_device(hip, rng):
     x = rng.standard_normal((6, 2, 3)).astype(np.float32)
     t = hip.tensor(x)

@@ -88,6 +88,30 @@ def test_host_tensor_compute_is_refused(emulated):
     assert r.returncode != 0 and "GPU only" in r.stderr
 
 
+def test_token_outside_the_table_reads_nothing_and_ends_the_process_at_the_next_wait(emulated):
+    """nc_get_col with an index >= the number of columns (and a negative one): the kernel reads
+    nothing out of range (the guard pages of this build would end the process with SIGSEGV), the
+    column comes out as zeros and the next wait ends the process with a message.  Through the
+    raw entry point the flag is returned by nchip_index_error()."""
+    code = ("import sys, os, ctypes as C; sys.path.insert(0, %r); from conftest import load_pkg; import numpy as np;"
+            "B = load_pkg().binding; path = os.environ['NNCP_TEST_HIP_LIB']; nc = B.NC(path, use_device=True);"
+            "lib = C.CDLL(path);"
+            "w = nc.tensor(np.ones((5, 8), np.float32)); idx = nc.tensor(np.array([1, %s, 4], np.int32));"
+            "y = nc.tensor(np.full((3, 8), 7.0, np.float32)); nc.nc_synchronize(nc.dev);"
+            "p = lambda t: C.c_void_p(nc.lib.nc_tensor_get_ptr(t, None));"
+            "assert lib.nchip_get_col(None, p(w), p(idx), p(y), 8, 5, C.c_int64(3)) == 0;"
+            "lib.hipcpu_flush_copies();"
+            "print('flag', lib.nchip_index_error(), lib.nchip_index_error());"
+            "out = np.ctypeslib.as_array(C.cast(p(y), C.POINTER(C.c_float)), (3, 8));"
+            "print('rows', out[0, 0], out[1].any(), out[2, 0]); sys.stdout.flush();"
+            "z = nc.nc_get_col(w, idx); nc.numpy(z)")
+    for bad in ("5", "-1"):
+        r = subprocess.run([sys.executable, "-c", code % (os.path.join(ROOT, "tests"), bad)],
+                           capture_output=True, text=True, env=emulated)
+        assert "flag 1 0" in r.stdout and "rows 1.0 False 1.0" in r.stdout, (r.stdout, r.stderr[-2000:])
+        assert r.returncode != 0 and "outside its table" in r.stderr, r.stderr[-2000:]
+
+
 def test_random_shapes_stay_in_bounds_and_match(emulated):
     """Seeded random campaigns through the raw kernel entry points of the CPU build, each
     operand in an exact-size buffer ending at a guard page: GEMM (layouts, paddings, batches,
