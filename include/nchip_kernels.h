@@ -200,6 +200,22 @@ int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float 
                    const float *w, float *dx, const float *dx_add, float *dw, float *db,
                    float *partial, int d, int64_t n, int avg);
 
+/* nchip_norm_bwd for callers that cannot allocate device memory (code under HIP graph
+   capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+   reference.  Same arguments without `partial`: the partial dw / db rows go to a buffer the
+   library itself holds in device memory, nchip_norm_bwd_static_capacity() floats (8 MiB)
+   per GPU for the life of the process, and the call allocates nothing.  (d, n) must satisfy
+   nchip_norm_bwd_rows(d, n) * 2 * d <= that capacity - true for every n when d is 128, 256,
+   512 or 1024, and for d <= 32768 otherwise - else the call returns -3 with a message and
+   launches nothing.  The stream must belong to the current device.  All calls on one GPU
+   share the buffer: calls that may overlap there (different streams, different threads)
+   race; calls on one stream are ordered and safe.  Results are bit-identical to
+   nchip_norm_bwd. */
+size_t nchip_norm_bwd_static_capacity(void);
+int nchip_norm_bwd_static(void *stream, const float *g, const float *xhat, const float *rstd,
+                          const float *w, float *dx, const float *dx_add, float *dw, float *db,
+                          int d, int64_t n, int avg);
+
 /* softmax over axis 0 of (v, n) and its backward dx = y*(g - sum(g*y))
    (libnc.h:382; nncp.c:796, 1008). */
 int nchip_softmax_fwd(void *stream, const float *x, float *y, int v, int64_t n);

@@ -10,6 +10,13 @@
 #include <mutex>
 #include "../../include/nchip_kernels.h"
 
+// Scratch of nchip_norm_bwd_static: the partial dw / db rows of the norm backward, held by the
+// library itself so that the call allocates nothing.  In host code this name is only a
+// handle for hipGetSymbolAddress: every GPU holds its own copy at its own address, looked up
+// once per device (static_scratch_of_current_device) and passed to the kernels as a pointer.
+constexpr size_t NORM_STATIC_SCRATCH_FLOATS = (size_t)2 << 20; // 8 MiB
+static __device__ __align__(256) float scratch[NORM_STATIC_SCRATCH_FLOATS];
+
 namespace {
 
 constexpr int TPB = 256;
@@ -456,6 +463,53 @@ int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float 
                                (const float *)partial, dw, db, d, rows);
     }
     return check("nchip_norm_bwd");
+}
+
+size_t nchip_norm_bwd_static_capacity(void) { return NORM_STATIC_SCRATCH_FLOATS; }
+
+// device address of `scratch` on the current device, looked up once per device
+static float *static_scratch_of_current_device()
+{
+    constexpr int MAX_DEVICES = 64;
+    static float *ptr_of[MAX_DEVICES];
+    static std::mutex mu;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        fprintf(stderr, "nchip_norm_bwd_static: no current device (%s)\n", hipGetErrorString(e));
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr_of[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            fprintf(stderr, "nchip_norm_bwd_static: hipGetSymbolAddress failed on device %d: %s\n", dev,
+                    hipGetErrorString(e));
+            return nullptr;
+        }
+        ptr_of[dev] = (float *)p;
+    }
+    return ptr_of[dev];
+}
+
+int nchip_norm_bwd_static(void *stream, const float *g, const float *xhat, const float *rstd, const float *w,
+                          float *dx, const float *dx_add, float *dw, float *db, int d, int64_t n, int avg)
+{
+    if (n <= 0 || d <= 0) return 0;
+    const size_t need = (size_t)nchip_norm_bwd_rows(d, n) * 2 * (size_t)d;
+    if (need > NORM_STATIC_SCRATCH_FLOATS) {
+        fprintf(stderr, "nchip_norm_bwd_static: (d = %d, n = %lld) needs %zu floats of scratch, the library's "
+                        "buffer holds %zu; use nchip_norm_bwd with a buffer of the caller\n",
+                d, (long long)n, need, (size_t)NORM_STATIC_SCRATCH_FLOATS);
+        return -3;
+    }
+    float *partial = nullptr;
+    if (dw || db) { // every partial row that is summed is written first: nothing has to start at zero
+        partial = static_scratch_of_current_device();
+        if (!partial) return -4;
+    }
+    return nchip_norm_bwd(stream, g, xhat, rstd, w, dx, dx_add, dw, db, partial, d, n, avg);
 }
 
 int nchip_softmax_fwd(void *stream, const float *x, float *y, int v, int64_t n)

@@ -38,6 +38,8 @@
 #define __host__
 #define __forceinline__ inline __attribute__((always_inline))
 #define __launch_bounds__(...)
+#define __align__(n) __attribute__((aligned(n)))
+#define HIP_SYMBOL(x) (x)
 #define __shared__ static
 
 typedef void *hipStream_t;
@@ -91,6 +93,8 @@ hipError_t hipHostFree(void *p);
 static inline hipError_t hipGetLastError(void) { return hipSuccess; }
 static inline const char *hipGetErrorString(hipError_t) { return "hipcpu"; }
 static inline hipError_t hipSetDevice(int) { return hipSuccess; }
+static inline hipError_t hipGetDevice(int *d) { *d = 0; return hipSuccess; }
+static inline hipError_t hipGetSymbolAddress(void **p, const void *symbol) { *p = const_cast<void *>(symbol); return hipSuccess; }
 static inline hipError_t hipGetDeviceCount(int *n) { *n = 1; return hipSuccess; }
 static inline hipError_t hipStreamCreate(hipStream_t *s) { *s = (hipStream_t)0x1; return hipSuccess; }
 static inline hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned) { *s = (hipStream_t)0x1; return hipSuccess; }
