@@ -4,10 +4,15 @@
  * TEST INFRASTRUCTURE ONLY (CPU checker + timed CPU baseline).  The reference
  * ships libnc as a header only (libnc.h); what each function must do is taken
  * from that header's comments and from how nncp.c uses it (cited per function).
- * Behaviour the header does not fix (RNG stream, Adam details, vec_sum_f32
- * order) is defined here and marked "build-defined": parity unpinned for:
- * nc_tensor_set_rnd_unif, nc_tensor_set_dropout, nc_sgd_opt_update
- * (bias correction / clip semantics), vec_sum_f32 order.
+ * Behaviour the header does not fix is defined here and marked "build-defined".
+ * What each such function computes is pinned by tests (the random fills against
+ * an independent statement of Marsaglia's xorwow and the uniform law, the
+ * optimisers against torch.optim in float64, vec_sum_f32 as a left-to-right
+ * sum); that libnc's own choice is the same one cannot be known from the
+ * header, so against libnc itself parity stays unpinned for:
+ * nc_tensor_set_rnd_unif, nc_tensor_set_dropout (which generator and stream),
+ * nc_sgd_opt_update (bias correction / clip semantics), vec_sum_f32 order.
+ * nc_cmul (rotary position embedding) is not implemented on either side.
  */
 #include <stdarg.h>
 #include <stdio.h>

@@ -226,6 +226,27 @@ def test_two_gradients_before_one_update_with_deferred_weight_gradients(hip, rng
     assert relerr(w0 - w1, grad) <= 1e-5
 
 
+def test_random_fills_are_the_checkers_bit_for_bit(hip, ref):
+    """nc_tensor_set_rnd_unif and nc_tensor_set_dropout (libnc.h:195-201): same seed, same
+    tensors from both libraries, across several calls on one generator state."""
+    outs = []
+    for nc in (hip, ref):
+        rs = nc.lib.nc_rnd_init(nc.dev, 321)
+        got = []
+        for shape, avg, width in (((64, 48), 0.0, 0.0625), ((1000,), 1.0, 2.0)):
+            t = nc.tensor(np.zeros(shape, np.float32))
+            nc.lib.nc_tensor_set_rnd_unif(t, avg, width, rs)
+            got.append(nc.numpy(t, free=True))
+        t = nc.tensor(np.zeros((50, 30), np.float32))
+        nc.lib.nc_tensor_set_dropout(t, 0.3, rs)
+        got.append(nc.numpy(t, free=True))
+        nc.lib.nc_rnd_end(rs)
+        outs.append(got)
+    for a, b in zip(*outs):
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.ptp(outs[0][0]) > 0.1 and set(np.unique(outs[0][2])) == {0.0, np.float32(1 / 0.7)}
+
+
 def test_views_and_copies_on_device(hip, rng):
     x = rng.standard_normal((6, 2, 3)).astype(np.float32)
     t = hip.tensor(x)

@@ -371,3 +371,55 @@ def test_matmul_matches_the_reference_restatement(ref, rng):
         got = ref.numpy(ref.nc_matmul(ref.tensor(b), ref.tensor(a)), free=True)
         assert got.shape == want.shape
         assert np.abs(got - want).max() <= 2e-6 * np.abs(want).max() * np.sqrt(k)
+
+
+def _xorwow_stream(seed, n):
+    """Marsaglia's xorwow ("Xorshift RNGs", 2003, section 3.1) from the paper's own starting state,
+    the seed folded into x and d, 16 outputs discarded: the stream the build defines for libnc's
+    RNDState (libnc.h:584-589 names exactly these six words)."""
+    mask = 0xFFFFFFFF
+    x, y, z, w, v = (123456789 ^ seed) & mask, 362436069, 521288629, 88675123, 5783321
+    d = (6615241 + seed * 2654435761) & mask
+    out = []
+    for i in range(n + 16):
+        t = x ^ (x >> 2)
+        x, y, z, w = y, z, w, v
+        v = ((v ^ (v << 4)) ^ (t ^ (t << 1))) & mask
+        d = (d + 362437) & mask
+        if i >= 16:
+            out.append((d + v) & mask)
+    return np.array(out, dtype=np.uint64)
+
+
+def test_rnd_unif_is_the_xorwow_stream_and_uniform(ref):
+    """nc_tensor_set_rnd_unif (libnc.h:195-200): the stream against an independent statement of
+    the published generator, value for value; range [avg - range, avg + range) and moments of the
+    uniform law; a Kolmogorov-Smirnov test; equal seeds give equal tensors, other seeds do not; a
+    second call continues the stream."""
+    from scipy import stats
+    n = 200000
+
+    def draw(seed, avg, rng_, count=n, calls=1):
+        rs = ref.lib.nc_rnd_init(None, seed)
+        outs = []
+        for _ in range(calls):
+            t = ref.tensor(np.zeros(count, np.float32))
+            ref.lib.nc_tensor_set_rnd_unif(t, avg, rng_, rs)
+            outs.append(ref.numpy(t, free=True))
+        ref.lib.nc_rnd_end(rs)
+        return outs if calls > 1 else outs[0]
+
+    for seed in (0, 123, 0xDEADBEEF):
+        u = (_xorwow_stream(seed, 1000) >> np.uint64(8)).astype(np.float32) * np.float32(1.0 / 16777216.0)
+        expect = np.float32(0.25) + np.float32(0.5) * (np.float32(2.0) * u - np.float32(1.0))
+        assert np.array_equal(draw(seed, 0.25, 0.5, 1000), expect), seed
+    a = draw(123, 1.5, 0.25)
+    assert a.min() >= 1.25 and a.max() < 1.75
+    assert abs(a.mean() - 1.5) < 4 * 0.25 / np.sqrt(3 * n)                 # 4 sigma of the sample mean
+    assert abs(a.var() - 0.25 ** 2 / 3) < 0.01 * 0.25 ** 2 / 3
+    assert stats.kstest((a - 1.25) / 0.5, "uniform").pvalue > 1e-3
+    assert abs(np.corrcoef(a[:-1], a[1:])[0, 1]) < 0.01                  # no lag-1 correlation
+    assert np.array_equal(a, draw(123, 1.5, 0.25))
+    assert not np.array_equal(a, draw(124, 1.5, 0.25))
+    first, second = draw(9, 0.0, 1.0, 500, calls=2)
+    assert np.array_equal(np.concatenate([first, second]), draw(9, 0.0, 1.0, 1000))
