@@ -30,6 +30,7 @@
 #include <math.h>
 #include <stdint.h>
 #include "k_internal.h"
+#include "k_addrspace.h"
 
 namespace {
 
@@ -69,7 +70,7 @@ __device__ __forceinline__ void fetch_rows(floatx4_t (&v)[ROWS * (DK / 4) / 256]
         // always load (from a clamped, valid row) and select afterwards: a load
         // under a divergent branch would be waited for before the next is issued
         int rc = row < rows_valid ? row : rows_valid - 1;
-        floatx4_t x = *reinterpret_cast<const floatx4_t *>(src(rc < 0 ? 0 : rc) + c);
+        floatx4_t x = *as_global(reinterpret_cast<const floatx4_t *>(src(rc < 0 ? 0 : rc) + c));
         v[it] = row < rows_valid ? x : floatx4_t{ 0, 0, 0, 0 };
     }
 }

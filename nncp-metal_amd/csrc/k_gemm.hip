@@ -24,12 +24,14 @@
 #include <type_traits>
 #include <vector>
 #include "../../include/nchip_kernels.h"
+#include "k_addrspace.h"
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short shortx8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4))); // a first-class value, unlike the uint4 struct
 
+// (operand loads and result stores go through global-address-space pointers: k_addrspace.h)
 namespace {
 
 constexpr int KALIGN = 16; // split-K chunk granularity
@@ -98,11 +100,26 @@ __device__ __forceinline__ unsigned short f32_to_bf16(float f)
 // MAJOR = 1: the tile's long axis (m or n) is contiguous in memory
 //            (A with ta = 0, B with tb = 1);  element (i, k) at p[i + k*ld].
 // MAJOR = 0: k is contiguous (A with ta = 1, B with tb = 0); (i, k) at p[k + i*ld].
+//
+// A k-contiguous tile is fetched row by row: BK / 4 consecutive lanes take one
+// row's BK floats (whole 128-byte lines when BK = 32), so a wavefront touches
+// 64 * 4 / BK rows instead of 64 - one cache line per lane was what bound these
+// tiles.  Its LDS rows are BT + 1 floats apart (FPAD_K): the four transposing
+// writes of a lane then fall on banks 4*(k/4) + e + i, distinct over the 32
+// lanes served together.
+constexpr int FPAD_K = 1;
 template <int BT, int BK, int MAJOR, int NT>
 struct TileLoader {
     static constexpr int NV = BT * BK / 4 / NT; // float4 per thread
+    static constexpr int RS = BT + (MAJOR ? PAD : FPAD_K); // LDS row stride
     static_assert(NV >= 1 && NV * NT * 4 == BT * BK, "tile must divide evenly over the threads");
     floatx4 r[NV];
+
+    __device__ __forceinline__ static void coords(int idx, int &i, int &k)
+    {
+        if (MAJOR) { i = (idx % (BT / 4)) * 4; k = idx / (BT / 4); }
+        else       { i = idx / (BK / 4);       k = (idx % (BK / 4)) * 4; }
+    }
 
     __device__ __forceinline__ void load(const float *p, int64_t ld, int i0, int k0,
                                          int imax, int kmax, bool fast, int t)
@@ -111,12 +128,11 @@ struct TileLoader {
         for (int v = 0; v < NV; v++) {
             int idx = t + v * NT;
             int i, k;
-            if (MAJOR) { i = (idx % (BT / 4)) * 4; k = idx / (BT / 4); }
-            else       { i = idx % BT;             k = (idx / BT) * 4; }
+            coords(idx, i, k);
             if (fast) {
                 const float *src = MAJOR ? p + (int64_t)(k0 + k) * ld + (i0 + i)
                                          : p + (int64_t)(i0 + i) * ld + (k0 + k);
-                r[v] = *reinterpret_cast<const floatx4 *>(src);
+                r[v] = *as_global(reinterpret_cast<const floatx4 *>(src));
             } else {
                 floatx4 tmp;
 #pragma unroll
@@ -124,8 +140,8 @@ struct TileLoader {
                     int ii = MAJOR ? i + e : i, kk = MAJOR ? k : k + e;
                     float val = 0.0f;
                     if (i0 + ii < imax && k0 + kk < kmax)
-                        val = MAJOR ? p[(int64_t)(k0 + kk) * ld + (i0 + ii)]
-                                    : p[(int64_t)(i0 + ii) * ld + (k0 + kk)];
+                        val = MAJOR ? as_global(p)[(int64_t)(k0 + kk) * ld + (i0 + ii)]
+                                    : as_global(p)[(int64_t)(i0 + ii) * ld + (k0 + kk)];
                     tmp[e] = val;
                 }
                 r[v] = tmp;
@@ -133,20 +149,19 @@ struct TileLoader {
         }
     }
 
-    // fp32 LDS tile: rows are k, BT + PAD floats each
+    // fp32 LDS tile: rows are k, RS floats each
     __device__ __forceinline__ void store_f32(float *lds, int t) const
     {
 #pragma unroll
         for (int v = 0; v < NV; v++) {
-            int idx = t + v * NT;
+            int i, k;
+            coords(t + v * NT, i, k);
             if (MAJOR) {
-                int i = (idx % (BT / 4)) * 4, k = idx / (BT / 4);
-                *reinterpret_cast<floatx4 *>(lds + k * (BT + PAD) + i) = r[v];
+                *reinterpret_cast<floatx4 *>(lds + k * RS + i) = r[v];
             } else {
-                int i = idx % BT, k = (idx / BT) * 4;
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    lds[(k + e) * (BT + PAD) + i] = r[v][e];
+                    lds[(k + e) * RS + i] = r[v][e];
             }
         }
     }
@@ -195,11 +210,11 @@ struct TileLoaderBf16 {
             if (fast) {
                 if (MAJOR) {
                     const float *src = p + (int64_t)(k0 + k) * ld + (i0 + i);
-                    floatx2_t a = *reinterpret_cast<const floatx2_t *>(src);
-                    floatx2_t b = *reinterpret_cast<const floatx2_t *>(src + ld);
+                    floatx2_t a = *as_global(reinterpret_cast<const floatx2_t *>(src));
+                    floatx2_t b = *as_global(reinterpret_cast<const floatx2_t *>(src + ld));
                     r[v] = floatx4{ a[0], a[1], b[0], b[1] };
                 } else {
-                    r[v] = *reinterpret_cast<const floatx4 *>(p + (int64_t)(i0 + i) * ld + (k0 + k));
+                    r[v] = *as_global(reinterpret_cast<const floatx4 *>(p + (int64_t)(i0 + i) * ld + (k0 + k)));
                 }
             } else {
                 floatx4 tmp;
@@ -208,8 +223,8 @@ struct TileLoaderBf16 {
                     int ii = MAJOR ? i + (e & 1) : i, kk = MAJOR ? k + (e >> 1) : k + e;
                     float val = 0.0f;
                     if (i0 + ii < imax && k0 + kk < kmax)
-                        val = MAJOR ? p[(int64_t)(k0 + kk) * ld + (i0 + ii)]
-                                    : p[(int64_t)(i0 + ii) * ld + (k0 + kk)];
+                        val = MAJOR ? as_global(p)[(int64_t)(k0 + kk) * ld + (i0 + ii)]
+                                    : as_global(p)[(int64_t)(i0 + ii) * ld + (k0 + kk)];
                     tmp[e] = val;
                 }
                 r[v] = tmp;
@@ -269,11 +284,11 @@ struct TileLoaderBf16Src {
             coords(v, t, i, k);
             if (MAJOR) {
                 const uint16_t *src = p + (int64_t)(k0 + k) * ld + (i0 + i);
-                r[v][0] = *reinterpret_cast<const u32x4 *>(src);
-                r[v][1] = *reinterpret_cast<const u32x4 *>(src + ld);
+                r[v][0] = *as_global(reinterpret_cast<const u32x4 *>(src));
+                r[v][1] = *as_global(reinterpret_cast<const u32x4 *>(src + ld));
             } else {
                 int row = i0 + i < imax ? i0 + i : imax - 1;
-                r[v][0] = *reinterpret_cast<const u32x4 *>(p + (int64_t)row * ld + (k0 + k));
+                r[v][0] = *as_global(reinterpret_cast<const u32x4 *>(p + (int64_t)row * ld + (k0 + k)));
             }
         }
     }
@@ -322,7 +337,7 @@ struct TileLoaderBf16Src {
 // two groups of WM x WN wavefronts share the LDS tiles and split every 32-deep
 // k slab, group 0 taking k%32 < 16 and group 1 the rest; group 1 hands its
 // accumulators over through LDS at the end (C = chain0 + chain1, fixed order).
-template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16, int KW = 1, int PF = 2>
+template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2)>
 __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 {
     GemmArgs g = g0;
@@ -332,8 +347,10 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     constexpr int WTM = BM / WM, WTN = BN / WN;           // wavefront tile
     // in 32-bit words; bf16 sources with k contiguous keep rows of BK/2 + 4 words
     constexpr int SQ = BK / 2 + 4;
-    constexpr int LDS_A = BF16 == 2 && TA ? BM * SQ : (BF16 ? (BK / 2) * (BM + PAD) : BK * (BM + PAD));
-    constexpr int LDS_B = BF16 == 2 && !TB ? BN * SQ : (BF16 ? (BK / 2) * (BN + PAD) : BK * (BN + PAD));
+    // fp32 row strides of the LDS tiles (see TileLoader)
+    constexpr int RSA = BM + (TA ? FPAD_K : PAD), RSB = BN + (TB ? PAD : FPAD_K);
+    constexpr int LDS_A = BF16 == 2 && TA ? BM * SQ : (BF16 ? (BK / 2) * (BM + PAD) : BK * RSA);
+    constexpr int LDS_B = BF16 == 2 && !TB ? BN * SQ : (BF16 ? (BK / 2) * (BN + PAD) : BK * RSB);
     static_assert(KW == 1 || BM * BN <= 2 * (LDS_A + LDS_B), "accumulator hand-over must fit in the tile buffers");
     // tile buffers above the 64 KiB a static array may take come from the
     // launch's dynamic allocation instead
@@ -430,7 +447,6 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     // prefetch behind an s_waitcnt vmcnt(0).
     // the MFMAs of the tile held in LDS at sa / sb
     auto compute = [&](const float *sa, const float *sb) {
-        if (g.dbg & 2) return;
         if constexpr (BF16 != 0) {
             // one 32x32x16 MFMA per tile pair per 16 k; group kg takes every KW-th block
             const uint32_t *wa = reinterpret_cast<const uint32_t *>(sa) + (lane >> 5) * 4 * (BM + PAD) + wm * WTM + (lane & 31);
@@ -469,39 +485,41 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
                             acc[i][j], 0, 0, 0);
             }
         } else {
-            // fragments of k-step u+1 are fetched while the MFMAs of u run.
-            // LDS row of step u: 2u (KW = 1), or the u-th pair of this group's
-            // half of each 32-deep slab (KW = 2)
+            // The k-steps of a tile go in chunks of CH: the fragments of chunk c+1 are read
+            // from LDS (into the other half of fa / fb) before the MFMAs of chunk c are issued,
+            // and a scheduling fence keeps them there - left alone, the scheduler sinks every
+            // read next to its use and each MFMA pair then waits a full LDS round trip.
+            // LDS row of step u: 2u (KW = 1), or the u-th pair of this group's half of each
+            // 32-deep slab (KW = 2).
             constexpr int NSTEP = BK / 2 / KW;
             auto krow = [](int u) { return KW == 1 ? 2 * u : (u >> 3) * 32 + 2 * (u & 7); };
-            // FD-1 k-steps of fragments are in flight ahead of the MFMAs: with one
-            // 32x32 tile per wavefront a k-step is a single 64-cycle MFMA, shorter
-            // than an LDS round trip
-            constexpr int FD = NSTEP < 4 ? NSTEP : 4;
-            float fa[FD][TM], fb[FD][TN];
-            const float *pa = sa + ((lane >> 5) + kg * 16) * (BM + PAD) + wm * WTM + (lane & 31);
-            const float *pb = sb + ((lane >> 5) + kg * 16) * (BN + PAD) + wn * WTN + (lane & 31);
+            constexpr int CH = NSTEP < 4 ? NSTEP : 4, NCH = NSTEP / CH;
+            static_assert(NSTEP % CH == 0, "whole chunks");
+            float fa[2][CH][TM], fb[2][CH][TN];
+            const float *pa = sa + ((lane >> 5) + kg * 16) * RSA + wm * WTM + (lane & 31);
+            const float *pb = sb + ((lane >> 5) + kg * 16) * RSB + wn * WTN + (lane & 31);
+            auto fetch_chunk = [&](int c, int buf) {
 #pragma unroll
-            for (int u = 0; u < FD - 1; u++) {
+                for (int u = 0; u < CH; u++) {
 #pragma unroll
-                for (int j = 0; j < TM; j++) fa[u][j] = pa[krow(u) * (BM + PAD) + j * 32];
+                    for (int j = 0; j < TM; j++) fa[buf][u][j] = pa[krow(c * CH + u) * RSA + j * 32];
 #pragma unroll
-                for (int i = 0; i < TN; i++) fb[u][i] = pb[krow(u) * (BN + PAD) + i * 32];
-            }
-#pragma unroll
-            for (int u = 0; u < NSTEP; u++) {
-                const int cur = u % FD, nxt = (u + FD - 1) % FD;
-                if (u + FD - 1 < NSTEP) {
-#pragma unroll
-                    for (int j = 0; j < TM; j++) fa[nxt][j] = pa[krow(u + FD - 1) * (BM + PAD) + j * 32];
-#pragma unroll
-                    for (int i = 0; i < TN; i++) fb[nxt][i] = pb[krow(u + FD - 1) * (BN + PAD) + i * 32];
+                    for (int i = 0; i < TN; i++) fb[buf][u][i] = pb[krow(c * CH + u) * RSB + i * 32];
                 }
+            };
+            fetch_chunk(0, 0);
 #pragma unroll
-                for (int i = 0; i < TN; i++)
+            for (int c = 0; c < NCH; c++) {
+                if (c + 1 < NCH) fetch_chunk(c + 1, (c + 1) & 1);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int j = 0; j < TM; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[cur][i], fa[cur][j], acc[i][j], 0, 0, 0);
+                for (int u = 0; u < CH; u++)
+#pragma unroll
+                    for (int i = 0; i < TN; i++)
+#pragma unroll
+                        for (int j = 0; j < TM; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[c & 1][u][i], fa[c & 1][u][j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
@@ -518,7 +536,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
             lb.store_f32(sb, t);
         }
         __syncthreads();
-        if ((FAST || it + PF < nk) && !(g.dbg & 1)) {
+        if (FAST || it + PF < nk) {
             int k0 = kbeg + (it + PF) * BK;
             bool kf = FAST || (k0 + BK <= kend);
             const bool second = k0 >= k1; // uniform
@@ -537,66 +555,90 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 #ifdef NCHIP_GEMM_CLOCKS
     long long dbg_c0 = clock64(), dbg_w0 = wall_clock64();
 #endif
-    const int nk = (g.dbg & 4) ? 0 : (kend - kbeg + BK - 1) / BK;
+    const int nk = (kend - kbeg + BK - 1) / BK;
     const int nk_full = (kend - kbeg) / BK; // tiles with a complete k range
-    if constexpr (BF16 == 2) {
-        // bf16 sources: the MFMAs of a tile are short, so the LDS writes of the
-        // next tile go out BEFORE them (into the other buffer, which every
+    if constexpr (SA != 0) {
+        // Store-ahead order: the LDS writes of the next tile go out BEFORE the
+        // MFMAs of the current one (into the other buffer, which every
         // wavefront left at the last barrier) and overlap with them; one
         // barrier per tile, after the MFMAs.  Register set (i % PF) holds tile
         // i from its load until that write; it is reloaded with tile i + PF
         // right after.
-        auto fetch = [&](int tile, auto &la, auto &lb) {
+        auto fetch = [&](int tile, auto fast_tag, auto &la, auto &lb) {
+            constexpr bool FAST = decltype(fast_tag)::value;
             const int k0 = kbeg + tile * BK;
+            const bool kf = FAST || (k0 + BK <= kend);
             const bool second = k0 >= k1; // uniform
             const float *Ak = second ? A2 : A, *Bk = second ? B2 : B;
-            const int kr = second ? k0 - k1 : k0;
-            la.load(Ak, g.lda, m0, kr, g.M, 0, true, t);
-            lb.load(Bk, g.ldb, n0, kr, g.N, 0, true, t);
+            const int kr = second ? k0 - k1 : k0, ke = second ? kend - k1 : (kend < k1 ? kend : k1);
+            la.load(Ak, g.lda, m0, kr, g.M, ke, FAST || (a_full && kf), t);
+            lb.load(Bk, g.ldb, n0, kr, g.N, ke, FAST || (b_full && kf), t);
         };
         auto park = [&](int tile, auto &la, auto &lb) {
             float *sa = smem + (tile & 1) * (LDS_A + LDS_B);
-            la.store(reinterpret_cast<uint32_t *>(sa), t);
-            lb.store(reinterpret_cast<uint32_t *>(sa + LDS_A), t);
+            if constexpr (BF16 != 0) {
+                la.store(reinterpret_cast<uint32_t *>(sa), t);
+                lb.store(reinterpret_cast<uint32_t *>(sa + LDS_A), t);
+            } else {
+                la.store_f32(sa, t);
+                lb.store_f32(sa + LDS_A, t);
+            }
+        };
+        auto body = [&](int cur, auto fast_tag, auto &na, auto &nb) {
+            constexpr bool FAST = decltype(fast_tag)::value;
+            if (FAST || cur + 1 < nk) {
+                park(cur + 1, na, nb);
+                if (FAST || cur + 1 + PF < nk) fetch(cur + 1 + PF, fast_tag, na, nb);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const float *sa = smem + (cur & 1) * (LDS_A + LDS_B);
+            compute(sa, sa + LDS_A);
+            __syncthreads();
         };
 #pragma unroll
         for (int j = 0; j < PF; j++)
-            if (j < nk) fetch(j, la[j], lb[j]);
+            if (j < nk) fetch(j, std::false_type(), la[j], lb[j]);
         if (nk > 0) park(0, la[0], lb[0]);
-        if (PF < nk) fetch(PF, la[0], lb[0]);
+        if (PF < nk) fetch(PF, std::false_type(), la[0], lb[0]);
         __syncthreads();
-        for (int it = 0; it < nk; it += PF) {
+        int it = 0;
+        if (a_full && b_full) // steady state: every tile fetched here is complete
+            for (; it + 2 * PF < nk_full; it += PF) {
 #pragma unroll
-            for (int j = 0; j < PF; j++) {
-                const int cur = it + j;
-                if (cur < nk) {
-                    auto &na = la[(j + 1) % PF];
-                    auto &nb = lb[(j + 1) % PF];
-                    if (cur + 1 < nk) {
-                        park(cur + 1, na, nb);
-                        if (cur + 1 + PF < nk && !(g.dbg & 1)) fetch(cur + 1 + PF, na, nb);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                    const float *sa = smem + (cur & 1) * (LDS_A + LDS_B);
-                    compute(sa, sa + LDS_A);
-                    __syncthreads();
-                }
+                for (int j = 0; j < PF; j++) body(it + j, std::true_type(), la[(j + 1) % PF], lb[(j + 1) % PF]);
             }
+        for (; it < nk; it += PF) {
+#pragma unroll
+            for (int j = 0; j < PF; j++)
+                if (it + j < nk) body(it + j, std::false_type(), la[(j + 1) % PF], lb[(j + 1) % PF]);
         }
     } else {
     int it = 0;
+    if (a_full && b_full && 2 * PF - 1 < nk_full) {
+        // steady state: tiles it+PF .. it+2PF-1 are complete, unguarded vector loads.  The
+        // first PF tiles are fetched by the same straight-line vector loads as inside the
+        // loop: the compiler then sees one and the same sequence of outstanding loads on
+        // entry and on the back edge and waits for the oldest register set only
+        // (s_waitcnt vmcnt(n)) instead of for everything in flight.
 #pragma unroll
-    for (int j = 0; j < PF; j++)
-        if (j < nk) {
-            bool kf = nk_full > j;
-            la[j].load(A, g.lda, m0, kbeg + j * BK, g.M, kend, a_full && kf, t);
-            lb[j].load(B, g.ldb, n0, kbeg + j * BK, g.N, kend, b_full && kf, t);
+        for (int j = 0; j < PF; j++) {
+            la[j].load(A, g.lda, m0, kbeg + j * BK, g.M, kend, true, t);
+            lb[j].load(B, g.ldb, n0, kbeg + j * BK, g.N, kend, true, t);
+            __builtin_amdgcn_sched_barrier(0); // oldest tile first, as on the back edge
         }
-    if (a_full && b_full) // steady state: tiles it+PF .. it+2PF-1 are complete, unguarded vector loads
         for (; it + 2 * PF - 1 < nk_full; it += PF) {
 #pragma unroll
             for (int j = 0; j < PF; j++) step(it + j, nk, std::true_type(), la[j], lb[j]);
         }
+    } else {
+#pragma unroll
+        for (int j = 0; j < PF; j++)
+            if (j < nk) {
+                bool kf = nk_full > j;
+                la[j].load(A, g.lda, m0, kbeg + j * BK, g.M, kend, a_full && kf, t);
+                lb[j].load(B, g.ldb, n0, kbeg + j * BK, g.N, kend, b_full && kf, t);
+            }
+    }
     for (; it < nk; it++) { // edge tiles and the k tail (it is a multiple of PF when the loop starts)
 #pragma unroll
         for (int j = 0; j < PF; j++)
@@ -642,7 +684,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     const int mm_base = m0 + wm * WTM + (lane & 31);
     const int nn_base = n0 + wn * WTN + (lane >> 5) * 4;
     if (g.ksplit > 1) {
-        float *ws = g.ws + ((int64_t)(kz * g.batch + b)) * g.M * g.N;
+        float NCHIP_GLOBAL *ws = as_global(g.ws + ((int64_t)(kz * g.batch + b)) * g.M * g.N);
 #pragma unroll
         for (int i = 0; i < TN; i++)
 #pragma unroll
@@ -659,16 +701,16 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
         return;
     }
     const int64_t coff = (int64_t)b_out * g.sc + (int64_t)b_in * g.sc_in;
-    float *C = g.C + coff;
-    float *P = g.pre ? g.pre + coff : nullptr;
-    const float *Radd = g.add ? g.add + coff : nullptr;
+    float NCHIP_GLOBAL *C = as_global(g.C + coff);
+    float NCHIP_GLOBAL *P = g.pre ? as_global(g.pre + coff) : nullptr;
+    const float NCHIP_GLOBAL *Radd = g.add ? as_global(g.add + coff) : nullptr;
     // The 16 values of a 32x32 accumulator tile go to 16 columns of C.  Everything
     // read here (addend, beta*C) is fetched for all 16 first, so the loads are in
     // flight together, and the uniform option tests are hoisted out of the
     // element loop: a branch per element with a load behind it costs one memory
     // round trip each.
     const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N); // uniform
-    const float *Dp = g.dpre ? g.dpre + coff : nullptr;
+    const float NCHIP_GLOBAL *Dp = g.dpre ? as_global(g.dpre + coff) : nullptr;
     const bool plain = !g.bias && !P && !Radd && !Dp && g.beta == 0.0f && g.act == NCHIP_ACT_NONE;
 #pragma unroll
     for (int i = 0; i < TN; i++)
@@ -677,7 +719,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
             const int m = mm_base + j * 32;
             const int nb = nn_base + i * 32;
             if (!full && m >= g.M) continue;
-            float *Cp = C + (int64_t)nb * g.ldc + m; // element r lives at Cp + nofs(r)*ldc
+            float NCHIP_GLOBAL *Cp = C + (int64_t)nb * g.ldc + m; // element r lives at Cp + nofs(r)*ldc
             auto nofs = [](int r) { return (r >> 2) * 8 + (r & 3); };
             if (plain && full) {
 #pragma unroll
@@ -691,7 +733,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 #pragma unroll
             for (int r = 0; r < 16; r++) extra[r] = 0.0f;
             if (Radd) {
-                const float *Ap = Radd + (int64_t)nb * g.ldc + m;
+                const float NCHIP_GLOBAL *Ap = Radd + (int64_t)nb * g.ldc + m;
 #pragma unroll
                 for (int r = 0; r < 16; r++) extra[r] = ok[r] ? Ap[(int64_t)nofs(r) * g.ldc] : 0.0f;
             }
@@ -701,7 +743,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 #pragma unroll
                 for (int r = 0; r < 16; r++) prev[r] = ok[r] ? Cp[(int64_t)nofs(r) * g.ldc] : 0.0f;
             }
-            const float bv = g.bias ? g.bias[m] : 0.0f;
+            const float bv = g.bias ? as_global(g.bias)[m] : 0.0f;
             float v[16];
 #pragma unroll
             for (int r = 0; r < 16; r++) {
@@ -710,7 +752,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
                 v[r] += bv;
             }
             if (P) {
-                float *Pp = P + (int64_t)nb * g.ldc + m;
+                float NCHIP_GLOBAL *Pp = P + (int64_t)nb * g.ldc + m;
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                     if (ok[r]) Pp[(int64_t)nofs(r) * g.ldc] = v[r];
@@ -723,7 +765,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
                 for (int r = 0; r < 16; r++) v[r] = v[r] > 0.0f ? v[r] : 0.0f;
             }
             if (Dp) { // gradient through an activation: times act'(pre-activation)
-                const float *Dq = Dp + (int64_t)nb * g.ldc + m;
+                const float NCHIP_GLOBAL *Dq = Dp + (int64_t)nb * g.ldc + m;
                 float pz[16];
 #pragma unroll
                 for (int r = 0; r < 16; r++) pz[r] = ok[r] ? Dq[(int64_t)nofs(r) * g.ldc] : 0.0f;
@@ -816,33 +858,33 @@ template <int BM, int BN, int BK, int TA, int TB, int BF16>
 constexpr size_t lds_dynamic_bytes()
 {
     constexpr int SQ = BK / 2 + 4;
-    constexpr size_t a = BF16 == 2 && TA ? BM * SQ : (BF16 ? (BK / 2) * (BM + PAD) : BK * (BM + PAD));
-    constexpr size_t b = BF16 == 2 && !TB ? BN * SQ : (BF16 ? (BK / 2) * (BN + PAD) : BK * (BN + PAD));
+    constexpr size_t a = BF16 == 2 && TA ? BM * SQ : (BF16 ? (BK / 2) * (BM + PAD) : BK * (BM + (TA ? FPAD_K : PAD)));
+    constexpr size_t b = BF16 == 2 && !TB ? BN * SQ : (BF16 ? (BK / 2) * (BN + PAD) : BK * (BN + (TB ? PAD : FPAD_K)));
     constexpr size_t bytes = 2 * (a + b) * sizeof(float);
     static_assert(bytes <= 160 * 1024, "tile buffers exceed LDS");
     return bytes > 65536 ? bytes : 0;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1, int PF = 2>
+template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2)>
 void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     g.gm = g_force_gm >= 0 ? g_force_gm : 8;
-    g.dbg = getenv("NCHIP_GEMM_DBG") ? atoi(getenv("NCHIP_GEMM_DBG")) : 0;
+    g.dbg = 0;
     dim3 grid(g.tiles_m * g.tiles_n, g.batch * g.ksplit), block(64 * WM * WN * KW);
 #define LAUNCH(TA, TB)                                                                                     \
     do {                                                                                                   \
         constexpr size_t dyn = lds_dynamic_bytes<BM, BN, BK, TA, TB, BF16>();                              \
         if (dyn) {                                                                                         \
             static const bool ok = hipFuncSetAttribute(                                                    \
-                reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>),     \
+                reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA>),     \
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) == hipSuccess;                       \
             if (!ok) { fprintf(stderr, "nchip_gemm: cannot reserve %zu bytes of LDS\n", dyn); abort(); }  \
         }                                                                                                  \
-        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>), grid, block, dyn, \
+        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA>), grid, block, dyn, \
                                        st, rec->start, rec->stop, 0, g);                                   \
-        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF>), grid, block, dyn, st, g); \
+        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA>), grid, block, dyn, st, g); \
     } while (0)
     if (!ta && !tb) LAUNCH(0, 0);
     else if (ta && !tb) LAUNCH(1, 0);
@@ -970,13 +1012,13 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     // workgroup (64x64x32, two k groups of 4 wavefronts); once
     // 128x64 tiles still give >= 256 workgroups, 8 wavefronts of 32x32 on a
     // 128x64x32 tile win; very large problems use 128x128x32 with 8 wavefronts.
-    int cfg = invariant ? 8 : g_force_cfg; // tuning aid: 0 = choose from the shape
+    int cfg = invariant ? 10 : g_force_cfg; // tuning aid: 0 = choose from the shape
     int64_t nb = (int64_t)batch * ksplit;
     int64_t t128x64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64) * nb;
     if (!cfg) {
         if (t128 >= 512 && m >= 128 && n >= 128) cfg = 7;
         else if (t128x64 >= 256 && m >= 128 && n >= 64) cfg = 4;
-        else cfg = 8;
+        else cfg = 10; // 64x64x32, two k groups, four register sets of tiles in flight
     }
     // Large bf16 products are bound by operand traffic from L2, not by the MFMA
     // rate: round both operands to bf16 in memory first (one streaming pass
@@ -1031,13 +1073,11 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
         launch_tile<64, 64, 64, 2, 2, 0, 2>(st, ta, tb, g, pr);
     } else if (cfg == 10) {
         launch_tile<64, 64, 32, 2, 2, 0, 2, 4>(st, ta, tb, g, pr);
-
-
     } else {
         launch_tile<64, 64, 16, 2, 2, 0>(st, ta, tb, g, pr);
     }
     if (g_prof_on) {
-        int tile = cfg == 7 ? 2 : (cfg == 4 ? 1 : (cfg == 8 ? 3 : 0));
+        int tile = cfg == 7 ? 2 : (cfg == 4 ? 1 : ((cfg == 8 || cfg == 10) ? 3 : 0));
         rec.variant = tile * 8 + (ta ? 4 : 0) + (tb ? 2 : 0) + (precision == 1 ? 1 : 0);
         g_prof.push_back(rec);
     }
@@ -1182,25 +1222,27 @@ extern "C" int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmP
         rec.variant = 2 * 8 + (ta ? 4 : 0) + (tb ? 2 : 0) + (precision == 1 ? 1 : 0);
         rec.flops = total_flops;
     }
-#define GRP(TA, TB, BF)                                                                                    \
+#define GRP2(TA, TB, BF, SAV)                                                                                  \
     do {                                                                                                   \
         constexpr size_t dyn = lds_dynamic_bytes<128, 128, 32, TA, TB, BF>();                              \
         if (dyn) {                                                                                         \
             static const bool ok = hipFuncSetAttribute(                                                    \
-                reinterpret_cast<const void *>(gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>),               \
+                reinterpret_cast<const void *>(gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV>),               \
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) == hipSuccess;                       \
             if (!ok) { fprintf(stderr, "nchip_gemm_grouped: cannot reserve %zu bytes of LDS\n", dyn); return -2; } \
         }                                                                                                  \
-        if (g_prof_on) hipExtLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, dyn, st, \
+        if (g_prof_on) hipExtLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV>), grid, block, dyn, st, \
                                              rec.start, rec.stop, 0, g);                                   \
-        else hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF>), grid, block, dyn, st, g);    \
+        else hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV>), grid, block, dyn, st, g);    \
     } while (0)
+#define GRP(TA, TB, BF) GRP2(TA, TB, BF, (BF == 2))
     if (precision == 1) {
         if (!ta && !tb) GRP(0, 0, 1); else if (ta && !tb) GRP(1, 0, 1); else if (!ta && tb) GRP(0, 1, 1); else GRP(1, 1, 1);
     } else {
         if (!ta && !tb) GRP(0, 0, 0); else if (ta && !tb) GRP(1, 0, 0); else if (!ta && tb) GRP(0, 1, 0); else GRP(1, 1, 0);
     }
 #undef GRP
+#undef GRP2
     if (g_prof_on) g_prof.push_back(rec);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

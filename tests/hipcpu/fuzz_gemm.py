@@ -21,6 +21,7 @@ def dev(arr):
     C.memmove(p, arr.ctypes.data, arr.nbytes)
     return p
 def back(p, n):
+    lib.hipcpu_flush_copies()  # the stand-in runs queued launches at a wait
     out = np.empty(n, np.float32); C.memmove(out.ctypes.data, p, n * 4); return out
 def bf16r(x):
     u = x.astype(np.float32).view(np.uint32).astype(np.uint64)
