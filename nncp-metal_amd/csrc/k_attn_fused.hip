@@ -56,9 +56,11 @@ __device__ __forceinline__ void wave_lds_sync()
 
 // Staging of a [ROWS][DK + 4] LDS tile from global rows of DK floats, split in
 // two so that the loads of every tile are in flight before the first LDS store
-// waits on one: fetch_rows issues the float4 loads (rows >= rows_valid read as
-// zero), put_rows stores the whole tile.  src(row) is the row address; src(0)
-// must be readable even when rows_valid is 0.
+// waits on one: fetch_rows only issues the float4 loads (rows >= rows_valid read
+// a clamped, valid row), put_rows zeroes those rows and stores the whole tile.
+// Nothing touches a loaded register between the two - a select right after the
+// load would be scheduled early and wait for everything in flight.  src(row) is
+// the row address; src(0) must be readable even when rows_valid is 0.
 template <int DK, int ROWS, typename F>
 __device__ __forceinline__ void fetch_rows(floatx4_t (&v)[ROWS * (DK / 4) / 256], int rows_valid, F src)
 {
@@ -67,23 +69,20 @@ __device__ __forceinline__ void fetch_rows(floatx4_t (&v)[ROWS * (DK / 4) / 256]
     for (int it = 0; it < ROWS * C4 / 256; it++) {
         int idx = threadIdx.x + it * 256;
         int row = idx / C4, c = (idx % C4) * 4;
-        // always load (from a clamped, valid row) and select afterwards: a load
-        // under a divergent branch would be waited for before the next is issued
         int rc = row < rows_valid ? row : rows_valid - 1;
-        floatx4_t x = *as_global(reinterpret_cast<const floatx4_t *>(src(rc < 0 ? 0 : rc) + c));
-        v[it] = row < rows_valid ? x : floatx4_t{ 0, 0, 0, 0 };
+        v[it] = *as_global(reinterpret_cast<const floatx4_t *>(src(rc < 0 ? 0 : rc) + c));
     }
 }
 
 template <int DK, int ROWS>
-__device__ __forceinline__ void put_rows(float *dst, const floatx4_t (&v)[ROWS * (DK / 4) / 256])
+__device__ __forceinline__ void put_rows(float *dst, const floatx4_t (&v)[ROWS * (DK / 4) / 256], int rows_valid)
 {
     constexpr int RS = DK + 4, C4 = DK / 4;
 #pragma unroll
     for (int it = 0; it < ROWS * C4 / 256; it++) {
         int idx = threadIdx.x + it * 256;
         int row = idx / C4, c = (idx % C4) * 4;
-        *reinterpret_cast<floatx4_t *>(dst + row * RS + c) = v[it];
+        *reinterpret_cast<floatx4_t *>(dst + row * RS + c) = row < rows_valid ? v[it] : floatx4_t{ 0, 0, 0, 0 };
     }
 }
 
@@ -130,7 +129,11 @@ struct FwdLayout {
                          r = v + KR * RS, b = r + 4 * 16 * FA_RSTRIDE, floats = b + FA_NB;
 };
 
-template <int DK, int NT>
+// VEC: K is a multiple of 4, so a lane's four probabilities of a key tile move as one 16-byte
+// access; otherwise four clamped 4-byte accesses.  A compile-time choice keeps the loads and
+// stores straight-line: with both forms behind a run-time branch the compiler waits for
+// everything in flight (s_waitcnt vmcnt(0)) after each one.
+template <int DK, int NT, bool VEC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
 {
@@ -150,8 +153,13 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
     const bool has_w = a.w_r != nullptr;
     PHASE_MARK(0);
 
-    // All global loads are issued up front; each tile is parked in LDS just
-    // before the phase that needs it, so K and V arrive under the rel phase.
+    // All global loads are issued up front, in the order they are waited for (a wait for one
+    // load is a wait for every older one): the bias row, Q and the position vectors for the
+    // rel phase, then K and V, which arrive under that phase.
+    const float bias_t = (a.b_r && t < a.K) ? as_global(a.b_r)[(int64_t)h * a.K + t] : 0.0f;
+    // position vectors of this head (without them: no valid row, the clamped reads hit q)
+    const float *w_base = has_w ? a.w_r + (int64_t)h * a.d_pos * DK : a.q;
+    const int n_w = has_w ? a.d_pos : 0;
     floatx4_t vq[FA_TMAX * (DK / 4) / 256], vw[KR * (DK / 4) / 256], vk[KR * (DK / 4) / 256],
         vv[KR * (DK / 4) / 256];
     {
@@ -164,13 +172,13 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
         fetch_rows<DK, FA_TMAX>(vq, a.T, [&](int r) {
             return a.q + (int64_t)h * DK + a.ldq * (b + (a.q_only >= 0 ? 0 : (int64_t)a.B * r));
         });
-        fetch_rows<DK, KR>(vw, has_w ? a.d_pos : 0, [&](int r) { return has_w ? a.w_r + ((int64_t)h * a.d_pos + r) * DK : a.q; });
+        fetch_rows<DK, KR>(vw, n_w, [&](int r) { return w_base + (int64_t)r * DK; });
         fetch_rows<DK, KR>(vk, a.K, kvrow);
         fetch_rows<DK, KR>(vv, a.K, [&](int r) { return kvrow(r) + (int64_t)a.H * DK; });
     }
-    if (t < FA_NB) Bs[t] = (a.b_r && t < a.K) ? a.b_r[(int64_t)h * a.K + t] * (a.b_r_scale * a.scale) : 0.0f;
-    put_rows<DK, FA_TMAX>(Qs, vq);
-    put_rows<DK, KR>(Ws, vw);
+    if (t < FA_NB) Bs[t] = bias_t * (a.b_r_scale * a.scale);
+    put_rows<DK, FA_TMAX>(Qs, vq, a.T);
+    put_rows<DK, KR>(Ws, vw, n_w);
     __syncthreads();
     PHASE_MARK(1);
 
@@ -195,7 +203,8 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
         }
         wave_lds_sync();
     }
-    put_rows<DK, KR>(Ks, vk);
+    put_rows<DK, KR>(Ks, vk, a.K);
+    put_rows<DK, KR>(Vs, vv, a.K); // (its own region: parked here, while no store is in flight behind it)
     __syncthreads();
     PHASE_MARK(2);
 
@@ -258,14 +267,15 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
         for (int r = 0; r < 4; r++) sc[jt][r] *= inv;
 
     if (a.probs && i < a.T) {
-        float *pc = a.probs + (((int64_t)b * a.H + h) * a.T + i) * a.K;
-        const bool vec = (a.K & 3) == 0;
+        float NCHIP_GLOBAL *pc = as_global(a.probs) + (((int64_t)b * a.H + h) * a.T + i) * a.K;
 #pragma unroll
         for (int jt = 0; jt < NT; jt++) {
             int j0 = jt * 16 + 4 * g;
-            if (vec && j0 < a.K) {
-                floatx4_t v = { sc[jt][0], sc[jt][1], sc[jt][2], sc[jt][3] };
-                *reinterpret_cast<floatx4_t *>(pc + j0) = v;
+            if (VEC) {
+                if (j0 < a.K) {
+                    floatx4_t v = { sc[jt][0], sc[jt][1], sc[jt][2], sc[jt][3] };
+                    *reinterpret_cast<floatx4_t NCHIP_GLOBAL *>(pc + j0) = v;
+                }
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; r++)
@@ -273,8 +283,6 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
             }
         }
     }
-    put_rows<DK, KR>(Vs, vv);
-    __syncthreads();
     PHASE_MARK(4);
 
     // O = V P: the ND feature tiles are independent accumulation chains
@@ -296,9 +304,9 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
         if (a.q_only >= 0 ? i == a.q_only : i < a.T) {
 #pragma unroll
             for (int dt = 0; dt < ND; dt++) {
-                float *o = a.out + (int64_t)h * DK + dt * 16 + 4 * g +
-                           a.ldo * (b + (a.q_only >= 0 ? 0 : (int64_t)a.B * i));
-                *reinterpret_cast<floatx4_t *>(o) = acc[dt];
+                float NCHIP_GLOBAL *o = as_global(a.out) + (int64_t)h * DK + dt * 16 + 4 * g +
+                                        a.ldo * (b + (a.q_only >= 0 ? 0 : (int64_t)a.B * i));
+                *reinterpret_cast<floatx4_t NCHIP_GLOBAL *>(o) = acc[dt];
             }
         }
     }
@@ -316,7 +324,7 @@ struct BwdLayout {
     static constexpr int red = o;                          // db_r halves, over dO once it is dead
 };
 
-template <int DK, int NT>
+template <int DK, int NT, bool VEC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void relpos_attn_bwd_fused(FusedAttnBwdArgs a)
 {
@@ -338,9 +346,12 @@ void relpos_attn_bwd_fused(FusedAttnBwdArgs a)
 
     // every global load is issued up front, in the order the phases need the
     // tiles; each tile is parked in LDS just before its first use
+    const float *w_base = has_w ? a.w_r + (int64_t)h * a.d_pos * DK : a.q;
+    const int n_w = has_w ? a.d_pos : 0;
     floatx4_t vq[FA_TMAX * (DK / 4) / 256], vo[FA_TMAX * (DK / 4) / 256], vw[KR * (DK / 4) / 256],
         vk[KR * (DK / 4) / 256], vv[KR * (DK / 4) / 256];
     float p[NT][4], ds[NT][4];
+    floatx4_t praw[NT];
     {
         auto kvrow = [&](int r) {
             return (r < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * r)
@@ -348,34 +359,33 @@ void relpos_attn_bwd_fused(FusedAttnBwdArgs a)
         };
         fetch_rows<DK, FA_TMAX>(vo, a.T, [&](int r) { return a.dout + (int64_t)h * DK + a.ldo * (b + (int64_t)a.B * r); });
         fetch_rows<DK, KR>(vv, a.K, [&](int r) { return kvrow(r) + (int64_t)a.H * DK; });
-        const float *pc = a.probs + (((int64_t)b * a.H + h) * a.T + (i < a.T ? i : 0)) * a.K;
-        const bool vec = (a.K & 3) == 0;
+        const float NCHIP_GLOBAL *pc = as_global(a.probs) + (((int64_t)b * a.H + h) * a.T + (i < a.T ? i : 0)) * a.K;
 #pragma unroll
-        for (int jt = 0; jt < NT; jt++) {
-            floatx4_t pv = { 0, 0, 0, 0 };
+        for (int jt = 0; jt < NT; jt++) { // unconditional loads from clamped addresses; masked at first use
             int j0 = jt * 16 + 4 * g;
-            if (vec) { // unconditional load from a clamped address, then select
-                floatx4_t x = *reinterpret_cast<const floatx4_t *>(pc + (j0 < a.K ? j0 : 0));
-                if (i < a.T && j0 < a.K) pv = x;
-            } else if (i < a.T) {
+            if (VEC) {
+                praw[jt] = *reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(pc + (j0 < a.K ? j0 : 0));
+            } else {
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (j0 + r < a.K) pv[r] = pc[j0 + r];
+                for (int r = 0; r < 4; r++) praw[jt][r] = pc[j0 + r < a.K ? j0 + r : 0];
             }
-#pragma unroll
-            for (int r = 0; r < 4; r++) p[jt][r] = pv[r];
         }
         fetch_rows<DK, KR>(vk, a.K, kvrow);
-        fetch_rows<DK, KR>(vw, has_w ? a.d_pos : 0, [&](int r) { return has_w ? a.w_r + ((int64_t)h * a.d_pos + r) * DK : a.q; });
+        fetch_rows<DK, KR>(vw, n_w, [&](int r) { return w_base + (int64_t)r * DK; });
         fetch_rows<DK, FA_TMAX>(vq, a.T, [&](int r) { return a.q + (int64_t)h * DK + a.ldq * (b + (int64_t)a.B * r); });
     }
-    put_rows<DK, FA_TMAX>(Os, vo);
-    put_rows<DK, KR>(Vs, vv);
+    put_rows<DK, FA_TMAX>(Os, vo, a.T);
+    put_rows<DK, KR>(Vs, vv, a.K);
     __syncthreads();
     PHASE_MARK(1);
 
     // dA = V^T dO, then dS = P (dA - colsum(P dA)) / sqrt(dk)
     {
+#pragma unroll
+        for (int jt = 0; jt < NT; jt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                p[jt][r] = (i < a.T && jt * 16 + 4 * g + r < a.K) ? praw[jt][r] : 0.0f;
         float dof[NS];
 #pragma unroll
         for (int s = 0; s < NS; s++) dof[s] = Os[i * RS + 4 * s + g];
@@ -403,9 +413,9 @@ void relpos_attn_bwd_fused(FusedAttnBwdArgs a)
             for (int r = 0; r < 4; r++) ds[jt][r] = p[jt][r] * (ds[jt][r] - dot) * a.scale; // masked: p = 0
     }
     PHASE_MARK(2);
-    put_rows<DK, KR>(Ks, vk);
-    put_rows<DK, KR>(Ws, vw);
-    put_rows<DK, FA_TMAX>(Qs, vq);
+    put_rows<DK, KR>(Ks, vk, a.K);
+    put_rows<DK, KR>(Ws, vw, n_w);
+    put_rows<DK, FA_TMAX>(Qs, vq, a.T);
     __syncthreads(); // K, w_r, Q visible; every wavefront is done with V: its space becomes the dRel strip
     PHASE_MARK(3);
 
@@ -623,26 +633,42 @@ bool allow_lds(KernelT kern, size_t bytes)
     return true;
 }
 
-template <int DK, int NT>
-int launch_fwd(hipStream_t st, const FusedAttnFwdArgs &a)
+template <int DK, int NT, bool VEC>
+int launch_fwd_v(hipStream_t st, const FusedAttnFwdArgs &a)
 {
     constexpr size_t bytes = sizeof(float) * FwdLayout<DK, NT>::floats;
     static_assert(bytes <= 160 * 1024, "forward tiles exceed LDS");
-    static const bool ok = allow_lds(relpos_attn_fwd_fused<DK, NT>, bytes);
+    static const bool ok = allow_lds(relpos_attn_fwd_fused<DK, NT, VEC>, bytes);
     if (!ok) return -1;
-    hipLaunchKernelGGL((relpos_attn_fwd_fused<DK, NT>), dim3(a.B * a.H), dim3(256), bytes, st, a);
+    hipLaunchKernelGGL((relpos_attn_fwd_fused<DK, NT, VEC>), dim3(a.B * a.H), dim3(256), bytes, st, a);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// 16-byte accesses to a column of probabilities need K % 4 == 0 and an aligned base
+template <typename Args>
+bool probs_vec(const Args &a) { return (a.K & 3) == 0 && (((uintptr_t)a.probs) & 15) == 0; }
+
+template <int DK, int NT>
+int launch_fwd(hipStream_t st, const FusedAttnFwdArgs &a)
+{
+    return probs_vec(a) ? launch_fwd_v<DK, NT, true>(st, a) : launch_fwd_v<DK, NT, false>(st, a);
+}
+
+template <int DK, int NT, bool VEC>
+int launch_bwd_v(hipStream_t st, const FusedAttnBwdArgs &a)
+{
+    constexpr size_t bytes = sizeof(float) * BwdLayout<DK, NT>::floats;
+    static_assert(bytes <= 160 * 1024, "backward tiles exceed LDS");
+    static const bool ok = allow_lds(relpos_attn_bwd_fused<DK, NT, VEC>, bytes);
+    if (!ok) return -1;
+    hipLaunchKernelGGL((relpos_attn_bwd_fused<DK, NT, VEC>), dim3(a.B * a.H), dim3(256), bytes, st, a);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 template <int DK, int NT>
 int launch_bwd(hipStream_t st, const FusedAttnBwdArgs &a)
 {
-    constexpr size_t bytes = sizeof(float) * BwdLayout<DK, NT>::floats;
-    static_assert(bytes <= 160 * 1024, "backward tiles exceed LDS");
-    static const bool ok = allow_lds(relpos_attn_bwd_fused<DK, NT>, bytes);
-    if (!ok) return -1;
-    hipLaunchKernelGGL((relpos_attn_bwd_fused<DK, NT>), dim3(a.B * a.H), dim3(256), bytes, st, a);
-    return hipGetLastError() == hipSuccess ? 0 : -1;
+    return probs_vec(a) ? launch_bwd_v<DK, NT, true>(st, a) : launch_bwd_v<DK, NT, false>(st, a);
 }
 
 } // namespace
