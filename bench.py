@@ -98,6 +98,18 @@ def bigram_zipf_dirichlet(n, n_symbols=16384, seed=2025, alpha=0.1, keep=256):
     return out
 
 
+def hip_runtime():
+    """The HIP runtime instance that libnc_hip.so itself is linked to (already mapped into this
+    process), and not whichever file the loader would pick for the bare name: with a second
+    copy of the runtime in the process (a wheel that bundles one), events and waits issued
+    through the wrong instance would not order with the library's kernels."""
+    for line in open("/proc/self/maps"):
+        path = line.split()[-1]
+        if "libamdhip64" in os.path.basename(path):
+            return C.CDLL(path)
+    return C.CDLL("libamdhip64.so")
+
+
 def say(what):
     """Progress on stderr, flushed before the step it names starts (stdout carries the one
     JSON line only)."""
@@ -161,7 +173,7 @@ def attention_c2(pkg, iters=50):
     dQ,dK,dV out = 72 MiB; dense flops 11 GEMM-likes x 268 M = 2.95 G."""
     nc = pkg.binding.NC(pkg.binding.HIP_LIB)
     lib = C.CDLL(pkg.binding.HIP_LIB)
-    hip = C.CDLL("libamdhip64.so")
+    hip = hip_runtime()
     B, Hh, dk, T, M = 32, 8, 64, 64, 64
     K, d_pos = M + T, M + T
     rng = np.random.default_rng(0)
@@ -240,7 +252,7 @@ def cdf_c5(pkg, iters=50):
     4 MiB read + 2 MiB written; lookup 2 B target + 2 B symbol each."""
     nc = pkg.binding.NC(pkg.binding.HIP_LIB)
     lib = C.CDLL(pkg.binding.HIP_LIB)
-    hip = C.CDLL("libamdhip64.so")
+    hip = hip_runtime()
     V, n, m = 16384, 64, 1000000
     rng = np.random.default_rng(5)
     bias = -np.log(rng.permutation(V) + 1.0)
@@ -407,7 +419,7 @@ def main():
     mode = H.MODE_SEGMENT | H.CODER_CDF16
 
     if args.calibrate_copy_mib:
-        hip = C.CDLL("libamdhip64.so")
+        hip = hip_runtime()
         nbytes_cal = args.calibrate_copy_mib << 20
         src, dst = C.c_void_p(), C.c_void_p()
         assert hip.hipMalloc(C.byref(src), C.c_size_t(nbytes_cal)) == 0

@@ -104,6 +104,12 @@ int nc_set_deferred_weight_grad(NCContext *m, int enable);
 /* Number of kernel launches issued so far (0 in libnc_ref.so). */
 int64_t nc_get_launch_count(NCContext *m);
 
+/* The stream (a hipStream_t) on which this context enqueues all its device work, for callers
+   that mix the raw kernel entry points of nchip_kernels.h with tensor calls: work they
+   enqueue on it runs in order with the library's own, and nc_synchronize() waits for it.
+   NULL before the device exists and in libnc_ref.so. */
+void *nc_context_stream(NCContext *m);
+
 #ifdef __cplusplus
 }
 #endif

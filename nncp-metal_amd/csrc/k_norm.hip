@@ -60,6 +60,43 @@ __global__ __launch_bounds__(TPB) void norm_fwd_kernel(const float *x, const flo
     }
 }
 
+// d = 64*NV: the column is read once and stays in registers (the generic kernel walks it
+// three times, each pass waiting for memory: with a few thousand columns that latency is
+// the whole run time).  Same per-lane summation order, so the results are the same.
+template <int NV>
+__global__ __launch_bounds__(TPB) void norm_fwd_reg(const float *x, const float *w, const float *b,
+                                                    float *y, float *xhat, float *rstd,
+                                                    int64_t n, float eps, int avg)
+{
+    constexpr int D = 64 * NV;
+    const int lane = threadIdx.x & 63;
+    const int64_t c = (int64_t)blockIdx.x * WPB + (threadIdx.x >> 6);
+    if (c >= n) return;
+    const float *xc = x + c * D;
+    float xv[NV], wv[NV], bv[NV];
+#pragma unroll
+    for (int v = 0; v < NV; v++) xv[v] = xc[lane + 64 * v];
+    if (w) {
+#pragma unroll
+        for (int v = 0; v < NV; v++) { wv[v] = w[lane + 64 * v]; bv[v] = b[lane + 64 * v]; }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; v++) s += xv[v];
+    const float mean = avg ? wave_sum(s) / (float)D : 0.0f;
+    float q = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; v++) { float t = xv[v] - mean; q += t * t; }
+    const float r = 1.0f / sqrtf(wave_sum(q) / (float)D + eps);
+    if (lane == 0) rstd[c] = r;
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const float h = (xv[v] - mean) * r;
+        if (xhat) xhat[c * D + lane + 64 * v] = h;
+        y[c * D + lane + 64 * v] = w ? h * wv[v] + bv[v] : h;
+    }
+}
+
 // dx = rstd * (gh - mean(gh) - xhat * mean(gh * xhat)),  gh = g * w
 __global__ __launch_bounds__(TPB) void norm_bwd_dx_kernel(const float *g, const float *xhat,
                                                           const float *rstd, const float *w,
@@ -400,8 +437,15 @@ int nchip_norm_fwd(void *stream, const float *x, const float *w, const float *b,
 {
     if (n <= 0 || d <= 0) return 0;
     if ((w == nullptr) != (b == nullptr)) { fprintf(stderr, "nchip_norm_fwd: w and b go together\n"); return -1; }
-    hipLaunchKernelGGL(norm_fwd_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, (hipStream_t)stream,
-                       x, w, b, y, xhat, rstd, d, n, eps, avg);
+    const dim3 grid((unsigned)((n + WPB - 1) / WPB));
+#define NORM_FWD(NV) hipLaunchKernelGGL(norm_fwd_reg<NV>, grid, dim3(TPB), 0, (hipStream_t)stream, x, w, b, y, xhat, rstd, n, eps, avg)
+    if (d == 128) NORM_FWD(2);
+    else if (d == 256) NORM_FWD(4);
+    else if (d == 512) NORM_FWD(8);
+    else if (d == 1024) NORM_FWD(16);
+    else
+        hipLaunchKernelGGL(norm_fwd_kernel, grid, dim3(TPB), 0, (hipStream_t)stream, x, w, b, y, xhat, rstd, d, n, eps, avg);
+#undef NORM_FWD
     return check("nchip_norm_fwd");
 }
 

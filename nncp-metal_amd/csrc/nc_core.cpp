@@ -200,6 +200,8 @@ extern "C" int nc_set_matmul_bf16(NCContext *m, int enable)
 
 extern "C" int64_t nc_get_launch_count(NCContext *m) { return m->launches; }
 
+extern "C" void *nc_context_stream(NCContext *m) { return m->hip_ready ? (void *)m->stream : nullptr; }
+
 extern "C" int nc_set_deferred_weight_grad(NCContext *m, int enable)
 {
     int old = m->defer_wgrad;

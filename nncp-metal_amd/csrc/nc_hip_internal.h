@@ -62,6 +62,17 @@ struct DeferredReduce {
     const NCNode *param;
 };
 struct DeferredTmp { float *ptr; size_t cap; };
+// A parameter used by several nodes of one graph (position vectors and biases tied over the
+// layers): every use leaves its partial rows to a first-level sum into one row of `stage`
+// (one row per use, in the order the backward pass reaches them), and a second-level sum
+// over those rows gives the gradient tensor that the first use handed to the graph.
+struct DeferredShared {
+    const NCNode *param;
+    float *stage;
+    size_t cap;
+    NCTensor *dst;
+    int n, uses, next;
+};
 
 #define NC_BW_ARGS 8 // node arguments for which nc_backward offers the existing gradient
 
@@ -81,6 +92,7 @@ struct NCContext {
     // (bw_prev) and whether the node's backward folded them in (bw_used)
     NCTensor *bw_prev[NC_BW_ARGS];
     bool bw_used[NC_BW_ARGS];
+    std::vector<DeferredShared> deferred_shared;
     std::vector<DeferredGemm> deferred;
     std::vector<DeferredReduce> deferred_red;
     std::vector<DeferredTmp> deferred_tmp;    // scratch the partial rows live in

@@ -84,6 +84,9 @@ static NCTensor *dev_binary(int op, const NCTensor *a, const NCTensor *b)
 // sums g (consumed) down to `target` (each target dim equals g's or is 1/missing)
 static void defer_sum(NCContext *m, const float *src, NCTensor *dst, int rows, int64_t stride, int n,
                       const NCNode *param);
+bool nc_can_defer_shared_sum(const NCContext *m, const NCNode *parent);
+static NCTensor *defer_shared_sum(NCContext *m, const float *src, NCTensor *like, int rows, int64_t stride,
+                                  const NCNode *param);
 
 // defer_param: the parameter node the result is the gradient of, when its
 // final sum over partial rows may wait for the end of nc_backward
@@ -955,8 +958,12 @@ static void attn_bw(NCNode *nd, NCTensor *g, NCTensor **ga)
     NCTensor *dbr = nd->ia[4] ? new_f32(q, 2, bd) : nullptr;
     size_t cap;
     float *scratch = nc_tmp_f32(m, nchip_relpos_attn_bwd_scratch(a.H, a.dk, a.B, a.T, a.M, a.d_pos), &cap);
-    const int keep = (dwr || dbr) && (!dwr || nc_can_defer_sum(m, nd->parents[3])) &&
-                     (!dbr || nc_can_defer_sum(m, nd->parents[4]));
+    // per-stream partials may be summed late when the gradients go straight to parameters:
+    // used once (one sum), or shared by several attention nodes (two-level sum)
+    const bool once = (!dwr || nc_can_defer_sum(m, nd->parents[3])) && (!dbr || nc_can_defer_sum(m, nd->parents[4]));
+    const bool shared = (!dwr || nc_can_defer_shared_sum(m, nd->parents[3])) &&
+                        (!dbr || nc_can_defer_shared_sum(m, nd->parents[4]));
+    const int keep = (dwr || dbr) && (once || shared);
     int rc = nchip_relpos_attn_bwd(m->stream, nc_f32(q), (int64_t)q->dims[0], nc_f32(kv),
                                    kvm ? nc_f32(kvm) : nullptr, (int64_t)kv->dims[0],
                                    w_r ? nc_f32(w_r) : nullptr, nc_f32(probs), nc_f32(gc),
@@ -968,8 +975,13 @@ static void attn_bw(NCNode *nd, NCTensor *g, NCTensor **ga)
     if (rc == 1) {
         // per-stream dw_r / db_r partials stay in scratch until the batched sum
         const int64_t n_w = dwr ? (int64_t)nc_numel(dwr) : 0, n_b = dbr ? (int64_t)nc_numel(dbr) : 0;
-        if (dwr) defer_sum(m, scratch, dwr, a.B, n_w, (int)n_w, nd->parents[3]);
-        if (dbr) defer_sum(m, scratch + n_w * a.B, dbr, a.B, n_b, (int)n_b, nd->parents[4]);
+        if (once) {
+            if (dwr) defer_sum(m, scratch, dwr, a.B, n_w, (int)n_w, nd->parents[3]);
+            if (dbr) defer_sum(m, scratch + n_w * a.B, dbr, a.B, n_b, (int)n_b, nd->parents[4]);
+        } else {
+            if (dwr) { NCTensor *t = defer_shared_sum(m, scratch, dwr, a.B, n_w, nd->parents[3]); nc_free_tensor(dwr); dwr = t; }
+            if (dbr) { NCTensor *t = defer_shared_sum(m, scratch + n_w * a.B, dbr, a.B, n_b, nd->parents[4]); nc_free_tensor(dbr); dbr = t; }
+        }
         DeferredTmp dt = { scratch, cap };
         m->deferred_tmp.push_back(dt);
     } else {
@@ -1088,6 +1100,21 @@ static void flush_deferred_gemms(NCContext *m)
     m->deferred.clear();
 }
 
+// one launch over a table of row sums; the pinned copy of the table is retired one launch later
+static void launch_row_sums(NCContext *m, const std::vector<KReduceRowsEntry> &tab, int max_n)
+{
+    size_t bytes = tab.size() * sizeof(KReduceRowsEntry), hcap, dcap;
+    void *host = m->host_pool.get(bytes, &hcap);
+    void *dev = m->dev_pool.get(bytes, &dcap);
+    memcpy(host, tab.data(), bytes);
+    hip_check(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync sum table");
+    k_reduce_rows_multi(m->stream, (const KReduceRowsEntry *)dev, (int)tab.size(), max_n);
+    m->launches++;
+    nc_staging_retire(m, m->red_staging, m->red_staging_cap, m->red_staging_stamp);
+    m->red_staging = host; m->red_staging_cap = hcap; m->red_staging_stamp = m->sync_count;
+    m->dev_pool.put(dev, dcap);
+}
+
 static void flush_deferred_sums(NCContext *m)
 {
     if (m->deferred_red.empty()) return;
@@ -1099,16 +1126,22 @@ static void flush_deferred_sums(NCContext *m)
         if (d.n > max_n) max_n = d.n;
         tab.push_back(e);
     }
-    size_t bytes = tab.size() * sizeof(KReduceRowsEntry), hcap, dcap;
-    void *host = m->host_pool.get(bytes, &hcap);
-    void *dev = m->dev_pool.get(bytes, &dcap);
-    memcpy(host, tab.data(), bytes);
-    hip_check(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync sum table");
-    k_reduce_rows_multi(m->stream, (const KReduceRowsEntry *)dev, (int)tab.size(), max_n);
-    m->launches++;
-    nc_staging_retire(m, m->red_staging, m->red_staging_cap, m->red_staging_stamp);
-    m->red_staging = host; m->red_staging_cap = hcap; m->red_staging_stamp = m->sync_count;
-    m->dev_pool.put(dev, dcap);
+    launch_row_sums(m, tab, max_n);
+    if (!m->deferred_shared.empty()) {
+        // second level: the rows of each shared parameter's stage (one per use that was
+        // reached, in that order) into its gradient tensor
+        tab.clear();
+        max_n = 0;
+        for (DeferredShared &d : m->deferred_shared) {
+            KReduceRowsEntry e;
+            e.src = d.stage; e.dst = nc_f32(d.dst); e.stride = d.n; e.rows = d.next; e.n = d.n;
+            if (d.n > max_n) max_n = d.n;
+            tab.push_back(e);
+        }
+        launch_row_sums(m, tab, max_n);
+        for (DeferredShared &d : m->deferred_shared) { nc_tmp_free(m, d.stage, d.cap); nc_free_tensor(d.dst); }
+        m->deferred_shared.clear();
+    }
     for (DeferredTmp &t : m->deferred_tmp) nc_tmp_free(m, t.ptr, t.cap);
     for (NCTensor *t : m->deferred_keep) nc_free_tensor(t);
     m->deferred_red.clear(); m->deferred_tmp.clear(); m->deferred_keep.clear();
@@ -1130,6 +1163,8 @@ bool nc_has_deferred(const NCContext *m, const NCNode *param)
         if (e.param == param) return true;
     for (const DeferredReduce &e : m->deferred_red)
         if (e.param == param) return true;
+    for (const DeferredShared &e : m->deferred_shared)
+        if (e.param == param) return true;
     return false;
 }
 
@@ -1146,6 +1181,39 @@ static void defer_sum(NCContext *m, const float *src, NCTensor *dst, int rows, i
     d.src = src; d.dst = nc_f32(dst); d.rows = rows; d.stride = stride; d.n = n; d.param = param;
     m->deferred_red.push_back(d);
     m->deferred_keep.push_back(nc_dup_tensor(dst));
+}
+
+// a gradient that goes straight to a parameter with several uses in this graph
+bool nc_can_defer_shared_sum(const NCContext *m, const NCNode *parent)
+{
+    return m->defer_wgrad && parent && parent->op == OP_PARAM && parent->consumers > 1;
+}
+
+// One use's partial rows of a shared parameter.  Returns the tensor to hand to the graph: the
+// gradient tensor itself at the first use, nullptr afterwards (the same tensor gets the total).
+static NCTensor *defer_shared_sum(NCContext *m, const float *src, NCTensor *like, int rows, int64_t stride,
+                                  const NCNode *param)
+{
+    const int n = (int)nc_numel(like);
+    DeferredShared *d = nullptr;
+    for (DeferredShared &e : m->deferred_shared)
+        if (e.param == param) d = &e;
+    NCTensor *ret = nullptr;
+    if (!d) {
+        DeferredShared e;
+        e.param = param; e.n = n; e.uses = param->consumers; e.next = 0;
+        e.stage = nc_tmp_f32(m, (size_t)e.uses * n, &e.cap);
+        e.dst = nc_alloc_like(like);
+        m->deferred_shared.push_back(e);
+        d = &m->deferred_shared.back();
+        ret = nc_dup_tensor(d->dst);
+    }
+    if (d->n != n || d->next >= d->uses) nc_fatal("shared gradient sum: unexpected use of a parameter");
+    DeferredReduce r;
+    r.src = src; r.dst = d->stage + (size_t)d->next * n; r.rows = rows; r.stride = stride; r.n = n; r.param = param;
+    m->deferred_red.push_back(r);
+    d->next++;
+    return ret;
 }
 
 // ---- backward dispatch --------------------------------------------------------

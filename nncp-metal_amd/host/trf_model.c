@@ -259,6 +259,14 @@ static NCTensor *concat_head(NCTensor *x) /* nncp.c:569-579 */
 /* store layer input into train_h (whole segment or one timestep), nncp.c:647-657 */
 static void save_layer_input(NNCPModel *s, int l, int output_index, NCTensor *x, int seg_len)
 {
+    if (s->fused_now && output_index < 0) {
+        /* whole segment on the fused path: train_h keeps the layer input itself (a view
+           of its storage outside the graph) instead of a copy of it */
+        NCTensor *v = nc_slice_alias(x, 1, 0, (size_t)s->cfg.batch_size * seg_len);
+        nc_free_tensor(s->train_h[l]);
+        s->train_h[l] = nc_reshape_3d(v, s->cfg.d_model, s->cfg.batch_size, seg_len);
+        return;
+    }
     NCTensor *dst = output_index < 0 ? nc_dup_tensor(s->train_h[l])
                                      : nc_slice_alias(s->train_h[l], 2, output_index, output_index + 1);
     NCTensor *src = nc_reshape_3d(nc_dup_tensor(x), s->cfg.d_model, s->cfg.batch_size, seg_len);
@@ -794,6 +802,12 @@ void trf_update(NNCPModel *s) /* nncp.c:1224-1235 with mem_update nncp.c:1205-12
         if (M > T) {
             nc_tensor_copy_slice(s->mem_h[l], s->mem_h[l], 2, 0, M - T, T);
             nc_tensor_copy_slice(s->mem_h[l], s->train_h[l], 2, M - T, M, 0);
+        } else if (M == T) {
+            /* the memory becomes exactly the saved layer inputs: the two tensors trade
+               places (train_h is rewritten in full before it is read again) */
+            NCTensor *tmp = s->mem_h[l];
+            s->mem_h[l] = s->train_h[l];
+            s->train_h[l] = tmp;
         } else {
             nc_tensor_copy_slice(s->mem_h[l], s->train_h[l], 2, 0, M, T - M);
         }

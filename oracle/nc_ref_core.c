@@ -78,6 +78,7 @@ void nc_synchronize(NCDevice *d) { (void)d; }
 void nc_prof_dump(void) {}
 int nc_set_matmul_bf16(NCContext *m, int enable);
 int64_t nc_get_launch_count(NCContext *m) { (void)m; return 0; }
+void *nc_context_stream(NCContext *m) { (void)m; return NULL; }
 int nc_set_deferred_weight_grad(NCContext *m, int enable) { (void)m; (void)enable; return 0; }
 int nc_set_matmul_width_invariant(NCContext *m, int enable) { (void)m; (void)enable; return 0; }
 

