@@ -32,18 +32,32 @@ C3 = dict(n_layer=12, d_model=512, n_head=8, d_inner=2048, d_pos=128, mem_len=64
 PEAK_TFLOPS = {"fp32": 157.3, "bf16": 2500.0}
 
 
-# HBM-side bytes per launch (read + written) of the GEMM instantiations at this
-# workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
-# scaled by a 256 MiB copy (--calibrate-copy-mib); a counter run cannot be
-# taken from inside the timed run, so the measured values are carried here.
-# The summary under profiles/ (c3_fp32_hbm_traffic_pmc.txt) holds the readings.
-MEASURED_TRAFFIC_BYTES = {
-    "gemm_kernel<64,64,32,2,2,1,0,0,2>": 28.12e6 + 4.19e6,
-    "gemm_kernel<64,64,32,2,2,0,0,0,2>": 27.69e6 + 4.14e6,
-    "gemm_kernel<128,64,32,4,2,0,0,0>": 26.88e6 + 16.78e6,
-    "gemm_kernel<128,64,32,4,2,1,0,0>": 38.04e6 + 16.78e6,
-    "gemm_kernel<128,128,32,4,2,0,1,0>": 3255.31e6 + 151.52e6,
-}
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def measured_traffic(kernel, summary="c3_fp32_hbm_traffic_pmc.txt"):
+    """HBM-side bytes per launch (read + written) of a kernel instantiation, from the committed
+    rocprofv3 summary (FETCH_SIZE / WRITE_SIZE runs of this script, scaled by a device copy of
+    known size; a counter run cannot be taken from inside the timed run).  The summary's rows
+    are `<kernel name> <launches> <FETCH KiB> <WRITE KiB> <read MB> <write MB>`; names are
+    compared without blanks and by prefix, because the event records name a kernel by its
+    leading template arguments only.  None when the summary does not hold the kernel."""
+    path = os.path.join(PROFILES, summary)
+    if not os.path.exists(path):
+        return None
+    want = kernel.replace(" ", "").rstrip(">")
+    for line in open(path):
+        parts = line.rsplit(None, 5)
+        if len(parts) != 6:
+            continue
+        name = parts[0].replace(" ", "")
+        try:
+            read_mb, write_mb = float(parts[4]), float(parts[5])
+        except ValueError:
+            continue
+        if name.startswith(want):
+            return (read_mb + write_mb) * 1e6
+    return None
 
 
 def markov3_dirichlet(n, seed=2024, alpha=0.05, n_symbols=256):
@@ -324,6 +338,47 @@ def cpu_baseline(pkg, data, n_steps, threads):
     return n / sec
 
 
+def decode_c3(pkg, data, n_segments, variant):
+    """Decoding rate of the same workload: n_segments trained segments encoded by the
+    whole-segment encoder, then decoded by the per-timestep decoder with K/V caches
+    (NNCP_MODE_STEP_DECODE; it evaluates one token column per timestep and replays the
+    training step once per segment) - timed, and checked to return the input."""
+    H = pkg.host
+    opt = pkg.binding.SGDOptParams(algo=pkg.binding.SGD_OPT_RMSPROP, beta2=0.99, eps=1e-8, lr=3e-4)
+    per_step = C3["batch_size"] * C3["seg_len"]
+    syms = np.ascontiguousarray(data[:n_segments * per_step])
+    mode = H.MODE_SEGMENT | H.MODE_STEP_DECODE | H.CODER_CDF16
+
+    def model():
+        m = H.Model(H.Host(), H.make_config(**dict(C3, use_device=1, fused=1, sgd_opt=opt)))
+        init_weights(m)
+        m.nc.nc_set_matmul_bf16(m.ctx, 1 if variant == "bf16" else 0)
+        return m
+    enc = model()
+    stream = np.zeros(syms.size * 4 + 4096, dtype=np.uint8)
+    st = H.NNCPStats()
+    sched = H.constant_lr(3e-4)
+    enc.nc.nc_synchronize(enc.dev)
+    t0 = time.perf_counter()
+    n = enc.L.nncp_compress(enc.ptr, syms.ctypes.data, syms.size, stream.ctypes.data, stream.size, mode,
+                            C.byref(sched), C.byref(st))
+    enc.nc.nc_synchronize(enc.dev)
+    t_enc = time.perf_counter() - t0
+    enc.close()
+    dec = model()
+    out = np.zeros(syms.size, dtype=np.uint16)
+    dec.nc.nc_synchronize(dec.dev)
+    t0 = time.perf_counter()
+    dec.L.nncp_decompress(dec.ptr, stream.ctypes.data, n, out.ctypes.data, syms.size, mode, C.byref(sched), C.byref(st))
+    dec.nc.nc_synchronize(dec.dev)
+    sec = time.perf_counter() - t0
+    dec.close()
+    return {"value": round(syms.size / sec, 1), "unit": "symbols/s", "ms_per_segment": round(sec / n_segments * 1e3, 2),
+            "segments": n_segments, "decoder": "per-timestep with K/V caches + one training step per segment",
+            "encode_ms_per_segment_same_mode": round(t_enc / n_segments * 1e3, 2),
+            "round_trip_ok": bool(np.array_equal(out, syms))}
+
+
 def main_c4(args):
     """BASELINE configs[3] (not the headline metric; `--workload c4`): 20 layers,
     d_model 1024, 16 heads x 64, d_ff 4096, 64 + 192 keys, batch 64, V 16384,
@@ -388,7 +443,11 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--variant", choices=["fp32", "bf16"], default="fp32")
-    ap.add_argument("--cpu-steps", type=int, default=2, help="0 skips the CPU baseline")
+    ap.add_argument("--also", default="bf16", help="further variants measured after the headline one and "
+                                                   "reported under `variants` (comma separated, empty for none)")
+    ap.add_argument("--cpu-steps", type=int, default=4, help="0 skips the CPU baseline")
+    ap.add_argument("--cpu-single-steps", type=int, default=1, help="steps of the single-thread CPU baseline (0 skips it)")
+    ap.add_argument("--decode-segments", type=int, default=2, help="segments decoded for the `decode` object (0 skips it)")
     ap.add_argument("--profile-steps", type=int, default=2)
     ap.add_argument("--attention-iters", type=int, default=50, help="0 skips the isolated attention timing")
     ap.add_argument("--cdf-iters", type=int, default=50, help="0 skips the coder-side CDF timing")
@@ -410,12 +469,8 @@ def main():
     B, T = C3["batch_size"], C3["seg_len"]
     per_step = B * T
     total_steps = args.warmup + args.steps + args.profile_steps
-    data = markov3_dirichlet(max(total_steps, args.cpu_steps) * per_step)
-
+    data = markov3_dirichlet(max(total_steps, args.cpu_steps, args.decode_segments) * per_step)
     opt = pkg.binding.SGDOptParams(algo=pkg.binding.SGD_OPT_RMSPROP, beta2=0.99, eps=1e-8, lr=3e-4)
-    model = H.Model(H.Host(), H.make_config(**dict(C3, use_device=1, fused=1, sgd_opt=opt)))
-    init_weights(model)
-    model.nc.nc_set_matmul_bf16(model.ctx, 1 if args.variant == "bf16" else 0)
     mode = H.MODE_SEGMENT | H.CODER_CDF16
 
     if args.calibrate_copy_mib:
@@ -431,48 +486,71 @@ def main():
         hip.hipFree(src)
         hip.hipFree(dst)
 
-    pos = 0
-    if args.warmup:
-        say("C3 %s: %d warm-up steps" % (args.variant, args.warmup))
-        run_block(model, H, data[pos:pos + args.warmup * per_step], mode)
-        pos += args.warmup * per_step
-    say("C3 %s: %d timed steps" % (args.variant, args.steps))
-    l0 = model.nc.nc_get_launch_count(model.ctx)
-    sec, nbytes, st = run_block(model, H, data[pos:pos + args.steps * per_step], mode)
-    launches = model.nc.nc_get_launch_count(model.ctx) - l0
-    pos += args.steps * per_step
-    value = args.steps * per_step / sec
+    def measure(variant):
+        """warm-up, the timed steps and the per-launch GEMM timing of one arithmetic variant"""
+        model = H.Model(H.Host(), H.make_config(**dict(C3, use_device=1, fused=1, sgd_opt=opt)))
+        init_weights(model)
+        model.nc.nc_set_matmul_bf16(model.ctx, 1 if variant == "bf16" else 0)
+        pos = 0
+        if args.warmup:
+            say("C3 %s: %d warm-up steps" % (variant, args.warmup))
+            run_block(model, H, data[pos:pos + args.warmup * per_step], mode)
+            pos += args.warmup * per_step
+        say("C3 %s: %d timed steps" % (variant, args.steps))
+        l0 = model.nc.nc_get_launch_count(model.ctx)
+        sec, nbytes, st = run_block(model, H, data[pos:pos + args.steps * per_step], mode)
+        launches = model.nc.nc_get_launch_count(model.ctx) - l0
+        pos += args.steps * per_step
+        roof = None
+        if args.profile_steps:
+            say("C3 %s: %d steps with per-launch GEMM events" % (variant, args.profile_steps))
+            rows = gemm_profile(model, H, data[pos:pos + args.profile_steps * per_step], mode,
+                                pkg.binding.HIP_LIB)
+            if rows:
+                dom = max(rows, key=lambda r: r["seconds"])
+                achieved = dom["flops"] / dom["seconds"] / 1e12
+                peak = PEAK_TFLOPS[variant]
+                tot_f = sum(r["flops"] for r in rows)
+                tot_s = sum(r["seconds"] for r in rows)
+                roof = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 3),
+                        "peak": peak, "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
+                        "traffic": measured_traffic(dom["kernel"]) if variant == "fp32" else None,
+                        "launches_per_step": dom["launches"] / args.profile_steps,
+                        "avg_launch_us": round(dom["seconds"] / dom["launches"] * 1e6, 2),
+                        "flops_per_launch": dom["flops"] / dom["launches"],
+                        "all_gemm_tflops": round(tot_f / tot_s / 1e12, 3),
+                        "all_gemm_ms_per_step": round(tot_s / args.profile_steps * 1e3, 3)}
+        model.close()
+        return {"value": round(args.steps * per_step / sec, 1), "ms_per_step": round(sec / args.steps * 1e3, 3),
+                "dtype": "f32" if variant == "fp32" else "bf16-in/f32-acc",
+                "bits_per_symbol": round(nbytes * 8 / (args.steps * per_step), 4),
+                "kernel_launches_per_step": launches / args.steps,
+                "host_seconds": {"eval_and_copy": round(st.t_eval, 4), "code": round(st.t_code, 4),
+                                 "grad": round(st.t_grad, 4), "update": round(st.t_update, 4)},
+                "roofline": roof}
 
-    roof = None
-    if args.profile_steps:
-        say("C3 %s: %d steps with per-launch GEMM events" % (args.variant, args.profile_steps))
-        rows = gemm_profile(model, H, data[pos:pos + args.profile_steps * per_step], mode,
-                            pkg.binding.HIP_LIB)
-        if rows:
-            dom = max(rows, key=lambda r: r["seconds"])
-            achieved = dom["flops"] / dom["seconds"] / 1e12
-            peak = PEAK_TFLOPS[args.variant]
-            tot_f = sum(r["flops"] for r in rows)
-            tot_s = sum(r["seconds"] for r in rows)
-            roof = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 3),
-                    "peak": peak, "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
-                    "traffic": MEASURED_TRAFFIC_BYTES.get(dom["kernel"]) if args.variant == "fp32" else None,
-                    "launches_per_step": dom["launches"] / args.profile_steps,
-                    "avg_launch_us": round(dom["seconds"] / dom["launches"] * 1e6, 2),
-                    "flops_per_launch": dom["flops"] / dom["launches"],
-                    "all_gemm_tflops": round(tot_f / tot_s / 1e12, 3),
-                    "all_gemm_ms_per_step": round(tot_s / args.profile_steps * 1e3, 3)}
-    model.close()
-    attn = cdf = None
+    head = measure(args.variant)
+    variants = {args.variant: {k: head[k] for k in ("value", "ms_per_step", "dtype", "bits_per_symbol")}}
+    for v in args.also.split(","):
+        if v and v != args.variant:
+            r = measure(v)
+            variants[v] = {k: r[k] for k in ("value", "ms_per_step", "dtype", "bits_per_symbol")}
+            variants[v]["all_gemm_tflops"] = r["roofline"]["all_gemm_tflops"] if r["roofline"] else None
+
+    attn = cdf = dec = None
     if args.attention_iters:
         say("isolated attention, B32 H8 d64 T64 K128, %d forward+backward pairs" % args.attention_iters)
         attn = attention_c2(pkg, args.attention_iters)
     if args.cdf_iters:
         say("coder-side CDF path, 64 x 16384 logits, %d iterations" % args.cdf_iters)
         cdf = cdf_c5(pkg, args.cdf_iters)
+    if args.decode_segments:
+        say("decoding %d segments with the per-timestep decoder" % args.decode_segments)
+        dec = decode_c3(pkg, data, args.decode_segments, args.variant)
 
     cpu = None
     if args.cpu_steps:
+        # the box's CPU share for one GPU is 16 threads, whatever the machine shows
         threads = min(os.cpu_count() or 1, 16)
         say("CPU checker, %d steps on %d threads" % (args.cpu_steps, threads))
         v = cpu_baseline(pkg, data, args.cpu_steps, threads)
@@ -480,22 +558,27 @@ def main():
                "sample": "first %d steps (%d symbols) of the same workload, CPU checker driving the "
                          "reference op sequence, whole-segment evaluation, float symbol coder"
                          % (args.cpu_steps, args.cpu_steps * per_step)}
+        if args.cpu_single_steps:
+            say("CPU checker, %d step(s) on 1 thread" % args.cpu_single_steps)
+            v1 = cpu_baseline(pkg, data, args.cpu_single_steps, 1)
+            cpu["single_thread"] = {"value": round(v1, 1), "cores": 1,
+                                    "sample": "first %d step(s)" % args.cpu_single_steps}
 
     print(json.dumps({
         "metric": "symbols/sec compressed (train+code) 12L d512",
-        "value": round(value, 1), "unit": "symbols/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(sec / args.steps * 1e3, 3),
+        "value": head["value"], "unit": "symbols/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if args.variant == "fp32" else "bf16-in/f32-acc", "data": "synthetic",
+        "dtype": head["dtype"], "data": "synthetic",
         "config": {"workload": "BASELINE configs[2]: 12L d512 8x64 ff2048 T64 M64 B32 V256, RMSProp, "
                                "order-3 Markov Dirichlet(0.05) prefix, weights N(0,0.02)",
                    "symbols_per_step": per_step, "coder": "gpu cdf16 + host range coder",
                    "variant": args.variant},
-        "bits_per_symbol": round(nbytes * 8 / (args.steps * per_step), 4),
-        "kernel_launches_per_step": launches / args.steps,
-        "host_seconds": {"eval_and_copy": round(st.t_eval, 4), "code": round(st.t_code, 4),
-                         "grad": round(st.t_grad, 4), "update": round(st.t_update, 4)},
-        "roofline": roof, "attention": attn, "cdf": cdf, "cpu_baseline": cpu}))
+        "bits_per_symbol": head["bits_per_symbol"],
+        "kernel_launches_per_step": head["kernel_launches_per_step"],
+        "host_seconds": head["host_seconds"],
+        "roofline": head["roofline"], "variants": variants, "attention": attn, "cdf": cdf, "decode": dec,
+        "cpu_baseline": cpu}))
 
 
 if __name__ == "__main__":
