@@ -114,6 +114,13 @@ int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launch
    choice.  The environment variable NCHIP_GEMM_CFG sets the initial value. */
 void nchip_gemm_force_config(int cfg);
 
+/* Testing aid: width-invariant fp32 products (NCHIP_GEMM_WIDTH_INVARIANT) with at most 64
+   columns, untransposed operands and beta = 0 run a register-streaming kernel that issues the
+   tile kernel's MFMA sequence without its LDS pipeline (the decoder's per-timestep products);
+   0 sends them through the tile kernel again, 1 (default) restores the choice.  The results
+   are the same bits either way. */
+void nchip_gemm_few_columns_kernel(int on);
+
 /* Tuning aid: tiles are ordered, inside each XCD's run, in bands of `gm` tile
    rows (1 = plain column-major tile order; a negative value restores the
    default of 8). */

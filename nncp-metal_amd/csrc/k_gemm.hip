@@ -333,14 +333,195 @@ struct TileLoaderBf16Src {
     }
 };
 
+// Epilogue of one 32x32 accumulator tile: acc[r] is C[m][nb + (r/4)*8 + r%4] (nb already
+// holds the lane's (lane/32)*4).  The 16 values go to 16 columns of C.  Everything read here
+// (addend, beta*C) is fetched for all 16 first, so the loads are in flight together, and the
+// uniform option tests sit outside the element loops: a branch per element with a load
+// behind it costs one memory round trip each.  Every product kernel ends in this function,
+// so kernels that feed it the same accumulators write the same bits.
+__device__ __forceinline__ void epilogue_tile(const GemmArgs &g, const floatx16 &acc, int m, int nb,
+                                              float NCHIP_GLOBAL *C, float NCHIP_GLOBAL *P,
+                                              const float NCHIP_GLOBAL *Radd, const float NCHIP_GLOBAL *Dp,
+                                              bool full, bool plain)
+{
+    if (!full && m >= g.M) return;
+    float NCHIP_GLOBAL *Cp = C + (int64_t)nb * g.ldc + m; // element r lives at Cp + nofs(r)*ldc
+    auto nofs = [](int r) { return (r >> 2) * 8 + (r & 3); };
+    if (plain && full) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) Cp[(int64_t)nofs(r) * g.ldc] = g.alpha * acc[r];
+        return;
+    }
+    bool ok[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) ok[r] = full || nb + nofs(r) < g.N;
+    float extra[16]; // beta*C + addend
+#pragma unroll
+    for (int r = 0; r < 16; r++) extra[r] = 0.0f;
+    if (Radd) {
+        const float NCHIP_GLOBAL *Ap = Radd + (int64_t)nb * g.ldc + m;
+#pragma unroll
+        for (int r = 0; r < 16; r++) extra[r] = ok[r] ? Ap[(int64_t)nofs(r) * g.ldc] : 0.0f;
+    }
+    float prev[16];
+    const bool has_beta = g.beta != 0.0f;
+    if (has_beta) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) prev[r] = ok[r] ? Cp[(int64_t)nofs(r) * g.ldc] : 0.0f;
+    }
+    const float bv = g.bias ? as_global(g.bias)[m] : 0.0f;
+    float v[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        v[r] = g.alpha * acc[r];
+        if (has_beta) v[r] += g.beta * prev[r];
+        v[r] += bv;
+    }
+    if (P) {
+        float NCHIP_GLOBAL *Pp = P + (int64_t)nb * g.ldc + m;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            if (ok[r]) Pp[(int64_t)nofs(r) * g.ldc] = v[r];
+    }
+    if (g.act == NCHIP_ACT_GELU) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) v[r] = gelu_tanh(v[r]);
+    } else if (g.act == NCHIP_ACT_RELU) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) v[r] = v[r] > 0.0f ? v[r] : 0.0f;
+    }
+    if (Dp) { // gradient through an activation: times act'(pre-activation)
+        const float NCHIP_GLOBAL *Dq = Dp + (int64_t)nb * g.ldc + m;
+        float pz[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) pz[r] = ok[r] ? Dq[(int64_t)nofs(r) * g.ldc] : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) v[r] = (v[r] + extra[r]) * act_grad(pz[r], g.dact);
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r];
+        return;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+        if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r] + extra[r];
+}
+
+// Product with a few token columns for the width-invariant class: C (M x N, 32 columns per
+// workgroup column) = A (M x K, m contiguous, M a multiple of 32) * B (K x N, k contiguous),
+// fp32, K a multiple of 32, operand columns 16-byte aligned.  Per output element it issues
+// exactly the MFMA sequence of the four-chain 64x64x32 tile kernel (gemm_kernel with
+// NACC = 2: chain c takes k%32 in [8c, 8c+8), two k per v_mfma_f32_32x32x2_f32 in increasing
+// order; C = (c0 + c1) + (c2 + c3); the same epilogue), so its columns are bit-identical to
+// those of a wide product.  What differs is the plumbing.  A workgroup is one 32-row tile
+// and its four wavefronts are the four chains, one per SIMD: the product then runs at the
+// speed of one dependent MFMA chain of K/8 instructions, the least this arithmetic allows
+// on one CU.  There is nothing to share between wavefronts, so the k loop has no barrier:
+// a wavefront fetches its 8 k of every slab with ONE 16-byte load per lane and operand
+// (8 x 32 rows of A, 32 columns x 8 k of B), PFD slabs ahead - at 2 microseconds of
+// latency and 256 cycles of MFMA per slab the loads of 16 slabs must be in flight - and
+// turns them into MFMA fragments through a private corner of LDS (in order within a
+// wavefront, so a write followed by a read needs no barrier).  Columns past the edge read
+// a clamped address and are never stored.
+template <int PFD>
+__global__ __launch_bounds__(256) void gemm_skinny_nn(GemmArgs g)
+{
+    static_assert(PFD % 2 == 0, "fragment registers alternate by slab parity");
+    constexpr int AST = 36, BST = 12; // row strides of the staged slabs: A [8 k][32 m], B [32 n][8 k]
+    __shared__ __attribute__((aligned(16))) float stage[4][8 * AST + 32 * BST];
+    __shared__ float red[3][16 * 64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int m0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
+    const int kh = lane >> 5;
+    const int ak = lane >> 3, am = (lane & 7) * 4; // this lane's k row and first of four rows m of the A slab
+    const int bn = lane >> 1, bk = (lane & 1) * 4; // this lane's column and first of four k of the B slab
+    const int bcol = n0 + bn < g.N ? n0 + bn : g.N - 1;
+    const floatx4 NCHIP_GLOBAL *Ag = reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(
+        as_global(g.A) + (int64_t)(8 * w + ak) * g.lda + m0 + am);
+    const floatx4 NCHIP_GLOBAL *Bg = reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(
+        as_global(g.B) + (int64_t)bcol * g.ldb + 8 * w + bk);
+    const int64_t a_step = 8 * g.lda; // 32 k rows, in 16-byte units
+    float *As = stage[w], *Bs = As + 8 * AST;
+    floatx4 *aw = reinterpret_cast<floatx4 *>(As + ak * AST + am);
+    floatx4 *bw = reinterpret_cast<floatx4 *>(Bs + bn * BST + bk);
+    const float *ar = As + kh * AST + (lane & 31); // MFMA step s reads k = 2s + kh
+    const float *br = Bs + (lane & 31) * BST + kh;
+    const int nslab = g.K / 32;
+    floatx4 ra[PFD], rb[PFD];
+    // (register sets and fragment sets are passed by reference: every index below is a
+    // constant once the loops are unrolled, so the arrays stay in registers)
+    auto load = [&](floatx4 &a, floatx4 &b, int slab) {
+        slab = slab < nslab ? slab : nslab - 1; // past the end: the last slab again, never used
+        a = Ag[slab * a_step];
+        b = Bg[slab * 8];
+    };
+    float fa[2][4], fb[2][4];
+    auto stage_slab = [&](const floatx4 &a, const floatx4 &b, float (&xa)[4], float (&xb)[4]) { // registers -> LDS -> fragments
+        *aw = a;
+        *bw = b;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int s4 = 0; s4 < 4; s4++) {
+            xa[s4] = ar[2 * s4 * AST];
+            xb[s4] = br[2 * s4];
+        }
+        __builtin_amdgcn_wave_barrier();
+    };
+#pragma unroll
+    for (int j = 0; j < PFD; j++) {
+        load(ra[j], rb[j], j);
+        __builtin_amdgcn_sched_barrier(0); // oldest slab first, as on the back edge
+    }
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+    stage_slab(ra[0], rb[0], fa[0], fb[0]);
+    load(ra[0], rb[0], PFD);
+    for (int slab0 = 0; slab0 < nslab; slab0 += PFD) {
+#pragma unroll
+        for (int j = 0; j < PFD; j++) {
+            // fragments of the next slab while the MFMAs of this one run
+            stage_slab(ra[(j + 1) % PFD], rb[(j + 1) % PFD], fa[(j + 1) & 1], fb[(j + 1) & 1]);
+            load(ra[(j + 1) % PFD], rb[(j + 1) % PFD], slab0 + j + 1 + PFD);
+            __builtin_amdgcn_sched_barrier(0);
+            if (slab0 + j < nslab) { // uniform
+#pragma unroll
+                for (int s4 = 0; s4 < 4; s4++)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j & 1][s4], fa[j & 1][s4], acc, 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (w > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) red[w - 1][r * 64 + lane] = acc[r];
+    }
+    __syncthreads();
+    if (w > 0) return;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = (acc[r] + red[0][r * 64 + lane]) + (red[1][r * 64 + lane] + red[2][r * 64 + lane]);
+    const bool full = n0 + 32 <= g.N;
+    float NCHIP_GLOBAL *P = g.pre ? as_global(g.pre) : nullptr;
+    const float NCHIP_GLOBAL *Radd = g.add ? as_global(g.add) : nullptr;
+    const float NCHIP_GLOBAL *Dp = g.dpre ? as_global(g.dpre) : nullptr;
+    const bool plain = !g.bias && !P && !Radd && !Dp && g.beta == 0.0f && g.act == NCHIP_ACT_NONE;
+    epilogue_tile(g, acc, m0 + (lane & 31), n0 + kh * 4, as_global(g.C), P, Radd, Dp, full, plain);
+}
+
 // KW = 2 doubles the wavefronts of a workgroup without shrinking its tile: the
 // two groups of WM x WN wavefronts share the LDS tiles and split every 32-deep
 // k slab, group 0 taking k%32 < 16 and group 1 the rest; group 1 hands its
 // accumulators over through LDS at the end (C = chain0 + chain1, fixed order).
-template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2)>
+// NACC = 2 (the width-invariant class): each k group keeps two accumulator sets and gives
+// the first four MFMA steps of every 32-deep slab to one, the last four to the other, so a
+// product is four chains - chain c takes k%32 in [8c, 8c+8) - summed as (c0 + c1) + (c2 + c3).
+// The products are the same; the order of the additions is what a kernel with four
+// wavefronts per row tile can reproduce (gemm_skinny_nn).
+template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2), int NACC = 1>
 __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 {
     GemmArgs g = g0;
+    static_assert(NACC == 1 || (NACC == 2 && BF16 == 0 && KW == 2 && BK == 32), "two accumulator sets: fp32 64-wide class only");
     static_assert(KW == 1 || (KW == 2 && BK % 32 == 0), "k groups split 32-deep slabs");
     constexpr int NT = 64 * WM * WN * KW;                 // threads: KW groups of WM x WN wavefronts
     constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN); // 32x32 MFMA tiles per wavefront
@@ -429,14 +610,14 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     LoaderA la[PF];
     LoaderB lb[PF];
 
-    floatx16 acc[TN][TM];
+    floatx16 acc[TN][TM], acc2[TN][TM]; // acc2: second chain of a k group (NACC = 2)
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
         for (int j = 0; j < TM; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++)
-                acc[i][j][r] = 0.0f;
+                acc[i][j][r] = acc2[i][j][r] = 0.0f;
 
     // One pipeline step: write the register set holding tile `it` to LDS buffer
     // it&1, barrier, refill that set with tile it+PF (when there is one), then
@@ -517,8 +698,12 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 #pragma unroll
                     for (int i = 0; i < TN; i++)
 #pragma unroll
-                        for (int j = 0; j < TM; j++)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[c & 1][u][i], fa[c & 1][u][j], acc[i][j], 0, 0, 0);
+                        for (int j = 0; j < TM; j++) {
+                            if (NACC == 2 && (c & 1)) // steps 4..7 of the slab: the group's second chain
+                                acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[c & 1][u][i], fa[c & 1][u][j], acc2[i][j], 0, 0, 0);
+                            else
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[c & 1][u][i], fa[c & 1][u][j], acc[i][j], 0, 0, 0);
+                        }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -656,6 +841,15 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
         g_gemm_clk[5 + 3 * blockIdx.x] = wall_clock64();  // end of the k loop
     }
 #endif
+    if constexpr (NACC == 2) {
+        static_assert(NACC == 1 || (BK / 2 / KW == 8), "chunks of four steps: one chunk per chain");
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int j = 0; j < TM; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] += acc2[i][j][r];
+    }
     if (KW == 2) {
         // group 1 parks its accumulators in LDS (the tiles are dead), group 0 adds them
         __syncthreads();
@@ -704,11 +898,6 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     float NCHIP_GLOBAL *C = as_global(g.C + coff);
     float NCHIP_GLOBAL *P = g.pre ? as_global(g.pre + coff) : nullptr;
     const float NCHIP_GLOBAL *Radd = g.add ? as_global(g.add + coff) : nullptr;
-    // The 16 values of a 32x32 accumulator tile go to 16 columns of C.  Everything
-    // read here (addend, beta*C) is fetched for all 16 first, so the loads are in
-    // flight together, and the uniform option tests are hoisted out of the
-    // element loop: a branch per element with a load behind it costs one memory
-    // round trip each.
     const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N); // uniform
     const float NCHIP_GLOBAL *Dp = g.dpre ? as_global(g.dpre + coff) : nullptr;
     const bool plain = !g.bias && !P && !Radd && !Dp && g.beta == 0.0f && g.act == NCHIP_ACT_NONE;
@@ -716,69 +905,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     for (int i = 0; i < TN; i++)
 #pragma unroll
         for (int j = 0; j < TM; j++) {
-            const int m = mm_base + j * 32;
-            const int nb = nn_base + i * 32;
-            if (!full && m >= g.M) continue;
-            float NCHIP_GLOBAL *Cp = C + (int64_t)nb * g.ldc + m; // element r lives at Cp + nofs(r)*ldc
-            auto nofs = [](int r) { return (r >> 2) * 8 + (r & 3); };
-            if (plain && full) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) Cp[(int64_t)nofs(r) * g.ldc] = g.alpha * acc[i][j][r];
-                continue;
-            }
-            bool ok[16];
-#pragma unroll
-            for (int r = 0; r < 16; r++) ok[r] = full || nb + nofs(r) < g.N;
-            float extra[16]; // beta*C + addend
-#pragma unroll
-            for (int r = 0; r < 16; r++) extra[r] = 0.0f;
-            if (Radd) {
-                const float NCHIP_GLOBAL *Ap = Radd + (int64_t)nb * g.ldc + m;
-#pragma unroll
-                for (int r = 0; r < 16; r++) extra[r] = ok[r] ? Ap[(int64_t)nofs(r) * g.ldc] : 0.0f;
-            }
-            float prev[16];
-            const bool has_beta = g.beta != 0.0f;
-            if (has_beta) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) prev[r] = ok[r] ? Cp[(int64_t)nofs(r) * g.ldc] : 0.0f;
-            }
-            const float bv = g.bias ? as_global(g.bias)[m] : 0.0f;
-            float v[16];
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                v[r] = g.alpha * acc[i][j][r];
-                if (has_beta) v[r] += g.beta * prev[r];
-                v[r] += bv;
-            }
-            if (P) {
-                float NCHIP_GLOBAL *Pp = P + (int64_t)nb * g.ldc + m;
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                    if (ok[r]) Pp[(int64_t)nofs(r) * g.ldc] = v[r];
-            }
-            if (g.act == NCHIP_ACT_GELU) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) v[r] = gelu_tanh(v[r]);
-            } else if (g.act == NCHIP_ACT_RELU) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) v[r] = v[r] > 0.0f ? v[r] : 0.0f;
-            }
-            if (Dp) { // gradient through an activation: times act'(pre-activation)
-                const float NCHIP_GLOBAL *Dq = Dp + (int64_t)nb * g.ldc + m;
-                float pz[16];
-#pragma unroll
-                for (int r = 0; r < 16; r++) pz[r] = ok[r] ? Dq[(int64_t)nofs(r) * g.ldc] : 0.0f;
-#pragma unroll
-                for (int r = 0; r < 16; r++) v[r] = (v[r] + extra[r]) * act_grad(pz[r], g.dact);
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                    if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r];
-                continue;
-            }
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r] + extra[r];
+            epilogue_tile(g, acc[i][j], mm_base + j * 32, nn_base + i * 32, C, P, Radd, Dp, full, plain);
         }
 #ifdef NCHIP_GEMM_CLOCKS
     if (g_gemm_clk && blockIdx.y == 0 && t == 0) g_gemm_clk[6 + 3 * blockIdx.x] = wall_clock64(); // stores issued
@@ -847,6 +974,7 @@ struct ProfRec {
 };
 bool g_prof_on = false;
 int g_force_cfg = getenv("NCHIP_GEMM_CFG") ? atoi(getenv("NCHIP_GEMM_CFG")) : 0;
+int g_skinny = 1; // width-invariant products with <= 64 columns take the register-streaming kernel
 int g_force_gm = -1;
 std::vector<ProfRec> g_prof;
 
@@ -865,7 +993,7 @@ constexpr size_t lds_dynamic_bytes()
     return bytes > 65536 ? bytes : 0;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2)>
+template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2), int NACC = 1>
 void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
@@ -878,13 +1006,13 @@ void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
         constexpr size_t dyn = lds_dynamic_bytes<BM, BN, BK, TA, TB, BF16>();                              \
         if (dyn) {                                                                                         \
             static const bool ok = hipFuncSetAttribute(                                                    \
-                reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA>),     \
+                reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA, NACC>),     \
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) == hipSuccess;                       \
             if (!ok) { fprintf(stderr, "nchip_gemm: cannot reserve %zu bytes of LDS\n", dyn); abort(); }  \
         }                                                                                                  \
-        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA>), grid, block, dyn, \
+        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA, NACC>), grid, block, dyn, \
                                        st, rec->start, rec->stop, 0, g);                                   \
-        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA>), grid, block, dyn, st, g); \
+        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA, NACC>), grid, block, dyn, st, g); \
     } while (0)
     if (!ta && !tb) LAUNCH(0, 0);
     else if (ta && !tb) LAUNCH(1, 0);
@@ -1007,12 +1135,23 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
         rec.flops = 2.0 * m * n * (double)k * batch;
     }
     ProfRec *pr = g_prof_on ? &rec : nullptr;
+    if (invariant && g_skinny && !ta && !tb && batch == 1 && precision == 0 && n <= 64 && k >= 32 && k % 32 == 0 &&
+        m % 32 == 0 && lda % 4 == 0 && ldb % 4 == 0 && (((uintptr_t)A | (uintptr_t)B) & 15) == 0 && beta == 0.0f && !g_prof_on) {
+        // a few token columns: the same arithmetic without the tile pipeline
+        hipLaunchKernelGGL(gemm_skinny_nn<16>, dim3(m / 32, (n + 31) / 32), dim3(256), 0, st, g);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            fprintf(stderr, "nchip_gemm: launch failed: %s\n", hipGetErrorString(e));
+            return -2;
+        }
+        return 0;
+    }
     // Tile configuration from the shape alone.  Measured on MI355X (fp32):
     // small outputs want the most workgroups and the most wavefronts per
     // workgroup (64x64x32, two k groups of 4 wavefronts); once
     // 128x64 tiles still give >= 256 workgroups, 8 wavefronts of 32x32 on a
     // 128x64x32 tile win; very large problems use 128x128x32 with 8 wavefronts.
-    int cfg = invariant ? 10 : g_force_cfg; // tuning aid: 0 = choose from the shape
+    int cfg = invariant ? 30 : g_force_cfg; // tuning aid: 0 = choose from the shape
     int64_t nb = (int64_t)batch * ksplit;
     int64_t t128x64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64) * nb;
     if (!cfg) {
@@ -1073,11 +1212,13 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
         launch_tile<64, 64, 64, 2, 2, 0, 2>(st, ta, tb, g, pr);
     } else if (cfg == 10) {
         launch_tile<64, 64, 32, 2, 2, 0, 2, 4>(st, ta, tb, g, pr);
+    } else if (cfg == 30) { // the width-invariant class: four chains per element
+        launch_tile<64, 64, 32, 2, 2, 0, 2, 4, 0, 2>(st, ta, tb, g, pr);
     } else {
         launch_tile<64, 64, 16, 2, 2, 0>(st, ta, tb, g, pr);
     }
     if (g_prof_on) {
-        int tile = cfg == 7 ? 2 : (cfg == 4 ? 1 : ((cfg == 8 || cfg == 10) ? 3 : 0));
+        int tile = cfg == 7 ? 2 : (cfg == 4 ? 1 : ((cfg == 8 || cfg == 10 || cfg == 30) ? 3 : 0));
         rec.variant = tile * 8 + (ta ? 4 : 0) + (tb ? 2 : 0) + (precision == 1 ? 1 : 0);
         g_prof.push_back(rec);
     }
@@ -1145,6 +1286,13 @@ extern "C" int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, flo
 extern "C" void nchip_gemm_force_config(int cfg)
 {
     g_force_cfg = cfg;
+}
+
+// testing aid: 0 sends width-invariant products of a few columns through the tile
+// kernel again (same bits, by construction: the tests compare the two)
+extern "C" void nchip_gemm_few_columns_kernel(int on)
+{
+    g_skinny = on;
 }
 
 // 0: bf16 products always round their operands inside the tile loader;

@@ -66,6 +66,42 @@ def test_gemm_columns_do_not_depend_on_batch_width(hip, rng):
     assert np.array_equal(full, again)
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 512, 32), (2048, 512, 32), (512, 2048, 32), (256, 512, 32), (100, 70, 7),
+                                   (64, 33, 33), (130, 1, 64), (1024, 96, 40)])
+def test_few_column_products_are_the_wide_products_columns(hip, rng, m, k, n):
+    """Width-invariant mode: a product with a few token columns (the decoder's per-timestep
+    shape, which takes the register-streaming kernel) equals, bit for bit, the same product
+    through the tile kernel and the matching columns of a wide product, with every epilogue
+    option the forward pass uses (bias, GELU, residual addend)."""
+    lib = C.CDLL(hip.lib._name)
+    w = rng.standard_normal((k, m)).astype(np.float32)
+    wide = rng.standard_normal((200 + n, k)).astype(np.float32)
+    bias = rng.standard_normal(m).astype(np.float32)
+    res = rng.standard_normal((200 + n, m)).astype(np.float32)
+    NC_ACT_NONE, NC_ACT_GELU = 0, 1
+
+    def products(x, r):
+        outs = [hip.numpy(hip.nc_matmul(hip.tensor(w), hip.tensor(x)), free=True),
+                hip.numpy(hip.nc_linear(hip.tensor(w), hip.tensor(x), hip.tensor(bias), NC_ACT_GELU), free=True),
+                hip.numpy(hip.nc_linear_add(hip.tensor(w), hip.tensor(x), hip.tensor(bias), NC_ACT_NONE, hip.tensor(r)), free=True),
+                hip.numpy(hip.nc_matmul_add(hip.tensor(w), hip.tensor(x), hip.tensor(r), 0, 0, 1.0), free=True)]
+        return outs
+    hip.nc_set_matmul_width_invariant(hip.ctx, 1)
+    try:
+        whole = products(wide, res)
+        few = products(wide[150:150 + n], res[150:150 + n])
+        lib.nchip_gemm_few_columns_kernel(0)
+        few_tiles = products(wide[150:150 + n], res[150:150 + n])
+    finally:
+        lib.nchip_gemm_few_columns_kernel(1)
+        hip.nc_set_matmul_width_invariant(hip.ctx, 0)
+    for a, b, c in zip(whole, few, few_tiles):
+        assert np.array_equal(a[150:150 + n], b)
+        assert np.array_equal(b, c)
+    ref64 = wide[150:150 + n].astype(np.float64) @ w.astype(np.float64)
+    assert relerr(few[0], ref64) <= TOL
+
+
 def test_gemm_bf16_variant(hip, ref, rng):
     w = rng.standard_normal((256, 320)).astype(np.float32)
     x = rng.standard_normal((200, 256)).astype(np.float32)
