@@ -120,11 +120,15 @@ extern "C" NCContext *nc_context_init(int nb_threads)
     return m;
 }
 
+static void staging_reclaim(NCContext *m);
+
 extern "C" void nc_context_end(NCContext *m)
 {
     if (!m) return;
     if (m->hip_ready) {
         (void)hipStreamSynchronize(m->stream);
+        m->sync_count++;
+        staging_reclaim(m);
         m->dev_pool.release_all();
         m->host_pool.release_all();
         (void)hipStreamDestroy(m->stream);
@@ -161,19 +165,39 @@ extern "C" NCDevice *nc_new_device(NCContext *m, const char *name)
     return &m->cpu;
 }
 
+// pinned tables whose upload the stream has consumed (a wait has happened since it was
+// enqueued) go back to the host pool
+static void staging_reclaim(NCContext *m)
+{
+    size_t kept = 0;
+    for (const StagingRetired &r : m->staging_retired) {
+        if (r.stamp < m->sync_count) m->host_pool.put(r.p, r.cap);
+        else m->staging_retired[kept++] = r;
+    }
+    m->staging_retired.resize(kept);
+}
+
 void nc_stream_wait(NCContext *m)
 {
     hip_check(hipStreamSynchronize(m->stream), "hipStreamSynchronize");
     m->sync_count++;
+    staging_reclaim(m);
     if (nchip_index_error())
         nc_fatal("a token index outside its table reached nc_get_col or nc_indexed_log");
 }
 
+// A pinned table that an asynchronous upload reads may be rewritten only after the stream
+// has executed that upload.  The host runs ahead of the stream, so "enough later launches
+// were issued" says nothing: the buffer waits in a list until the stream has been waited for
+// at least once since the upload was enqueued (stamp = the wait count at that moment).
+// No wait is forced here - a training step waits twice on its own (distributions to the
+// host, loss) - unless the list grows long.
 void nc_staging_retire(NCContext *m, void *p, size_t cap, uint64_t stamp)
 {
     if (!p) return;
-    if (stamp == m->sync_count) nc_stream_wait(m);
-    m->host_pool.put(p, cap);
+    m->staging_retired.push_back(StagingRetired{ p, cap, stamp });
+    if (m->staging_retired.size() > 64) nc_stream_wait(m);
+    else staging_reclaim(m);
 }
 
 extern "C" void nc_synchronize(NCDevice *d)

@@ -76,6 +76,9 @@ struct DeferredShared {
 
 #define NC_BW_ARGS 8 // node arguments for which nc_backward offers the existing gradient
 
+// a pinned table that was released while its upload may still be queued
+struct StagingRetired { void *p; size_t cap; uint64_t stamp; };
+
 struct NCContext {
     int nb_threads;
     NCDevice cpu, hip;
@@ -100,6 +103,7 @@ struct NCContext {
     // pinned tables of the last grouped launches; each goes back to the pool
     // one flush later, and only once the stream has been waited for since its
     // upload was enqueued (nc_staging_retire)
+    std::vector<StagingRetired> staging_retired; // released tables the stream may still read
     void *grp_staging;
     size_t grp_staging_cap;
     uint64_t grp_staging_stamp;

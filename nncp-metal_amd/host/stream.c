@@ -112,6 +112,42 @@ static int symbol_is_coded(int t, int stream, int len2, int rem, int full)
     return full || t < len2 || (t == len2 && stream < rem); /* nncp.c:3099-3100 */
 }
 
+/* The encoder's whole-segment evaluation in two halves.  The first fills the input (and the
+   training targets: the encoder knows its symbols before it codes them), evaluates the
+   segment and brings the distributions to the host; the second feeds them to the
+   arithmetic coder.  Between the two a caller may queue the training step, whose kernels
+   then run while the host codes (nncp.c:3024-3050 does the same work in sequence: eval,
+   code, train; the bytes and the weights do not depend on the order of the last two). */
+static HostDist encode_segment_eval(Coder *c, int idx, int n_t, int len2, int full,
+                                    NCTensor *input, NCTensor *expected)
+{
+    int B = c->B;
+    for (int t = 0; t < n_t; t++)
+        for (int b = 0; b < B; b++) {
+            nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
+            if (expected && symbol_is_coded(t, b, len2, c->view.rem, full))
+                nc_set1_i32_2d(expected, b, t, get_symb(&c->view, b, idx + t));
+        }
+    double t0 = now_s();
+    NCTensor *out = c->cls->eval(c->s, -1, input);
+    HostDist d = fetch_dist(c, out);
+    c->st->t_eval += now_s() - t0;
+    return d;
+}
+
+static void encode_segment_emit(Coder *c, HostDist *d, int idx, int n_t, int len2, int full)
+{
+    int B = c->B;
+    double t0 = now_s();
+    for (int t = 0; t < n_t; t++)
+        for (int b = 0; b < B; b++)
+            if (symbol_is_coded(t, b, len2, c->view.rem, full))
+                code_symbol(c, d, (size_t)t * B + b, b, idx + t);
+    c->st->t_code += now_s() - t0;
+    nc_free_tensor(d->host);
+    d->host = NULL;
+}
+
 /* One segment starting at block position idx: n_t timesteps are coded (T for a
    full segment, fewer in the tail).  Fills `expected` when training follows. */
 static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int full,
@@ -122,22 +158,8 @@ static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int ful
     double t0;
     if (mode == NNCP_MODE_SEGMENT && !c->is_decode) {
         /* nncp.c:3024-3046 */
-        for (int t = 0; t < n_t; t++)
-            for (int b = 0; b < B; b++)
-                nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
-        t0 = now_s();
-        NCTensor *out = c->cls->eval(s, -1, input);
-        HostDist d = fetch_dist(c, out);
-        c->st->t_eval += now_s() - t0;
-        t0 = now_s();
-        for (int t = 0; t < n_t; t++)
-            for (int b = 0; b < B; b++)
-                if (symbol_is_coded(t, b, len2, c->view.rem, full)) {
-                    int sym = code_symbol(c, &d, (size_t)t * B + b, b, idx + t);
-                    if (expected) nc_set1_i32_2d(expected, b, t, sym);
-                }
-        c->st->t_code += now_s() - t0;
-        nc_free_tensor(d.host);
+        HostDist d = encode_segment_eval(c, idx, n_t, len2, full, input, expected);
+        encode_segment_emit(c, &d, idx, n_t, len2, full);
         return;
     }
     if (mode == NNCP_MODE_SEGMENT && c->step_decode) {
@@ -237,8 +259,13 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
     c.cls->reset(s); /* nncp.c:2988 */
 
     int idx = 0;
+    const int overlap = mode == NNCP_MODE_SEGMENT && !is_decode; /* code while the training kernels run */
     while (idx + T <= c.view.stride) { /* nncp.c:2993 */
-        code_segment(&c, mode, idx, T, T, 1, input, expected);
+        HostDist pending = { 0 };
+        if (overlap)
+            pending = encode_segment_eval(&c, idx, T, T, 1, input, expected);
+        else
+            code_segment(&c, mode, idx, T, T, 1, input, expected);
         float rate = nncp_interp(lr, nncp_model_train_step(s)); /* nncp.c:3048-3050 */
         c.cls->set_lr(s, rate);
         double t0 = now_s();
@@ -247,6 +274,8 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
         t0 = now_s();
         c.cls->update(s);
         c.st->t_update += now_s() - t0;
+        if (overlap)
+            encode_segment_emit(&c, &pending, idx, T, T, 1);
         c.st->loss_bits -= loss / log(2.0);
         c.st->n_steps++;
         c.st->n_symbols += (int64_t)T * B;

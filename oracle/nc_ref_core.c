@@ -60,6 +60,9 @@ NCContext *nc_context_init(int nb_threads)
     omp_set_num_threads(m->nb_threads);
     m->cpu = nc_mallocz(sizeof(NCDevice));
     m->cpu->ctx = m;
+    /* the bf16 operand emulation is one switch for the whole checker: a new context starts
+       in fp32, as a context of the product does, whatever an earlier one left behind */
+    nc_set_matmul_bf16(m, 0);
     return m;
 }
 
