@@ -266,6 +266,19 @@ __attribute__((format(printf, 3, 4))) NCParam *
 nc_new_param(NCParamList *pl, NCTensor **pval, const char *fmt, ...);  /* libnc.h:521 */
 void nc_param_list_end(NCParamList *pl);                               /* libnc.h:522 */
 size_t nc_get_param_count(NCParamList *pl);                            /* libnc.h:525 */
+NCParam *nc_find_param(NCParamList *pl, const char *name);             /* libnc.h:524 */
+/* parameter files (libnc's own layout is not published: the layout is this library's,
+   stated in csrc/nc_params_io.cpp; a file written by one build of this library is read by
+   another, on either device) */
+void nc_save_param_header(FILE *f, const char *config);                /* libnc.h:528 */
+void nc_save_param(FILE *f, const NCTensor *v1, const char *name);     /* libnc.h:529 */
+void nc_save_coefs(NCParamList *pl, const char *filename);             /* libnc.h:530 */
+char *nc_load_param_header(FILE *f);                                   /* libnc.h:533 */
+NCTensor *nc_load_param(NCContext *m, FILE *f, char *name,
+                        size_t name_size);                             /* libnc.h:535 */
+void nc_load_coefs(NCParamList *pl, const char *filename);             /* libnc.h:536 */
+void nc_update_param(NCParamList *pl, const char *name,
+                     const NCTensor *v);                               /* libnc.h:580 */
 NCSGDOptState *nc_sgd_opt_init(NCContext *m, const SGDOptParams *p);   /* libnc.h:561 */
 void nc_sgd_opt_end(NCSGDOptState *s);                                 /* libnc.h:562 */
 void sgd_opt_update_var(void *opaque, NCTensor *yg,

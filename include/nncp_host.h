@@ -146,6 +146,11 @@ NCTensor **nncp_model_param(NNCPModel *s, const char *name);
 int nncp_model_param_count(NNCPModel *s);
 const char *nncp_model_param_name(NNCPModel *s, int index);
 int64_t nncp_model_train_step(NNCPModel *s);
+/* every registered parameter to / from a parameter file (nc_save_coefs / nc_load_coefs,
+   libnc.h:530, 536; the file named by --load_coefs, nncp.c:3761).  Loading needs a model of
+   the same configuration: names, shapes and types must match. */
+void nncp_model_save_coefs(NNCPModel *s, const char *filename);
+void nncp_model_load_coefs(NNCPModel *s, const char *filename);
 
 /* the `trf` model class (nncp.c:1544-1562); input/expected are (B, T) i32
    host tensors, borrowed; trf_eval returns an owned (V, B, T|1) tensor */

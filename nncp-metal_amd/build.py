@@ -14,7 +14,7 @@ SOURCES = {
     "k_gemm.hip": [], "k_elementwise.hip": [], "k_norm.hip": [], "k_attention.hip": [], "k_attn_fused.hip": [],
     # bit-exact integer-CDF path: no contraction, no reassociation
     "k_cdf.hip": ["-ffp-contract=off"],
-    "nc_core.cpp": ["-x", "hip"], "nc_autodiff.cpp": ["-x", "hip"],
+    "nc_core.cpp": ["-x", "hip"], "nc_autodiff.cpp": ["-x", "hip"], "nc_params_io.cpp": ["-x", "hip"],
     "nc_ops.cpp": ["-x", "hip", "-ffp-contract=off"],
 }
 

@@ -517,7 +517,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_nn(GemmArgs g)
 // product is four chains - chain c takes k%32 in [8c, 8c+8) - summed as (c0 + c1) + (c2 + c3).
 // The products are the same; the order of the additions is what a kernel with four
 // wavefronts per row tile can reproduce (gemm_skinny_nn).
-template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2), int NACC = 1>
+template <int BM, int BN, int BK, int WM, int WN, int TA, int TB, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2), int NACC = 1, int FRAG = 0>
 __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 {
     GemmArgs g = g0;
@@ -688,6 +688,37 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
                     for (int i = 0; i < TN; i++) fb[buf][u][i] = pb[krow(c * CH + u) * RSB + i * 32];
                 }
             };
+            if constexpr (FRAG == 1) {
+                // rolling window instead of chunks: the fragments of step u+3 are read while
+                // the MFMAs of step u run, and the scheduler is left to place them (wavefronts
+                // that own two or more accumulator tiles have enough MFMA time per step)
+                static_assert(NACC == 1, "the rolling window feeds one accumulator set");
+                constexpr int FD = NSTEP < 4 ? NSTEP : 4;
+                float ga[FD][TM], gb[FD][TN];
+#pragma unroll
+                for (int u = 0; u < FD - 1; u++) {
+#pragma unroll
+                    for (int j = 0; j < TM; j++) ga[u][j] = pa[krow(u) * RSA + j * 32];
+#pragma unroll
+                    for (int i = 0; i < TN; i++) gb[u][i] = pb[krow(u) * RSB + i * 32];
+                }
+#pragma unroll
+                for (int u = 0; u < NSTEP; u++) {
+                    const int cur = u % FD, nxt = (u + FD - 1) % FD;
+                    if (u + FD - 1 < NSTEP) {
+#pragma unroll
+                        for (int j = 0; j < TM; j++) ga[nxt][j] = pa[krow(u + FD - 1) * RSA + j * 32];
+#pragma unroll
+                        for (int i = 0; i < TN; i++) gb[nxt][i] = pb[krow(u + FD - 1) * RSB + i * 32];
+                    }
+#pragma unroll
+                    for (int i = 0; i < TN; i++)
+#pragma unroll
+                        for (int j = 0; j < TM; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(gb[cur][i], ga[cur][j], acc[i][j], 0, 0, 0);
+                }
+                return;
+            }
             fetch_chunk(0, 0);
 #pragma unroll
             for (int c = 0; c < NCH; c++) {
@@ -993,7 +1024,7 @@ constexpr size_t lds_dynamic_bytes()
     return bytes > 65536 ? bytes : 0;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2), int NACC = 1>
+template <int BM, int BN, int BK, int WM, int WN, int BF16, int KW = 1, int PF = 2, int SA = (BF16 == 2), int NACC = 1, int FRAG = 0>
 void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
@@ -1006,13 +1037,13 @@ void launch_tile(hipStream_t st, int ta, int tb, GemmArgs &g, ProfRec *rec)
         constexpr size_t dyn = lds_dynamic_bytes<BM, BN, BK, TA, TB, BF16>();                              \
         if (dyn) {                                                                                         \
             static const bool ok = hipFuncSetAttribute(                                                    \
-                reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA, NACC>),     \
+                reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA, NACC, FRAG>),     \
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) == hipSuccess;                       \
             if (!ok) { fprintf(stderr, "nchip_gemm: cannot reserve %zu bytes of LDS\n", dyn); abort(); }  \
         }                                                                                                  \
-        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA, NACC>), grid, block, dyn, \
+        if (rec) hipExtLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA, NACC, FRAG>), grid, block, dyn, \
                                        st, rec->start, rec->stop, 0, g);                                   \
-        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA, NACC>), grid, block, dyn, st, g); \
+        else hipLaunchKernelGGL((gemm_kernel<BM, BN, BK, WM, WN, TA, TB, BF16, KW, PF, SA, NACC, FRAG>), grid, block, dyn, st, g); \
     } while (0)
     if (!ta && !tb) LAUNCH(0, 0);
     else if (ta && !tb) LAUNCH(1, 0);
@@ -1205,7 +1236,7 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     } else if (cfg == 6) {
         launch_tile<64, 128, 16, 2, 2, 0>(st, ta, tb, g, pr);
     } else if (cfg == 7) {
-        launch_tile<128, 128, 32, 4, 2, 0>(st, ta, tb, g, pr);
+        launch_tile<128, 128, 32, 4, 2, 0, 1, 2, 0, 1, 1>(st, ta, tb, g, pr); // rolling fragment window: two accumulator tiles per wavefront
     } else if (cfg == 8) {
         launch_tile<64, 64, 32, 2, 2, 0, 2>(st, ta, tb, g, pr);
     } else if (cfg == 9) {
@@ -1375,13 +1406,13 @@ extern "C" int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmP
         constexpr size_t dyn = lds_dynamic_bytes<128, 128, 32, TA, TB, BF>();                              \
         if (dyn) {                                                                                         \
             static const bool ok = hipFuncSetAttribute(                                                    \
-                reinterpret_cast<const void *>(gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV>),               \
+                reinterpret_cast<const void *>(gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV, 1, (BF == 0)>),               \
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) == hipSuccess;                       \
             if (!ok) { fprintf(stderr, "nchip_gemm_grouped: cannot reserve %zu bytes of LDS\n", dyn); return -2; } \
         }                                                                                                  \
-        if (g_prof_on) hipExtLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV>), grid, block, dyn, st, \
+        if (g_prof_on) hipExtLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV, 1, (BF == 0)>), grid, block, dyn, st, \
                                              rec.start, rec.stop, 0, g);                                   \
-        else hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV>), grid, block, dyn, st, g);    \
+        else hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV, 1, (BF == 0)>), grid, block, dyn, st, g);    \
     } while (0)
 #define GRP(TA, TB, BF) GRP2(TA, TB, BF, (BF == 2))
     if (precision == 1) {

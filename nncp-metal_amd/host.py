@@ -139,6 +139,9 @@ class Host:
         L.nncp_model_param_count.argtypes = [_P]
         L.nncp_model_param_name.restype = C.c_char_p
         L.nncp_model_param_name.argtypes = [_P, C.c_int]
+        for n in ("nncp_model_save_coefs", "nncp_model_load_coefs"):
+            getattr(L, n).restype = None
+            getattr(L, n).argtypes = [_P, C.c_char_p]
         L.nncp_model_train_step.restype = C.c_int64
         L.nncp_model_train_step.argtypes = [_P]
         L.trf_eval.restype = _P
@@ -309,6 +312,15 @@ class Model:
 
     def params(self):
         return {n: self.get_param(n) for n in self.param_names()}
+
+    def save_coefs(self, path):
+        """Every parameter to a parameter file (nc_save_coefs, libnc.h:530)."""
+        self.L.nncp_model_save_coefs(self.ptr, os.fsencode(path))
+
+    def load_coefs(self, path):
+        """Parameters from a file written by save_coefs of a model of the same
+        configuration, on either library (nc_load_coefs, libnc.h:536)."""
+        self.L.nncp_model_load_coefs(self.ptr, os.fsencode(path))
 
     # -- the model class ---------------------------------------------------
     def eval(self, tokens, output_index=-1, keep=False):

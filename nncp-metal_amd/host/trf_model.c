@@ -216,6 +216,11 @@ const char *nncp_model_param_name(NNCPModel *s, int index)
     return NULL;
 }
 
+/* parameter files: what --load_coefs names (nncp.c:3149, 3761; its use at nncp.c:3439-3442 and
+   3604-3607 is compiled out in the reference, the calls are libnc.h:530, 536) */
+void nncp_model_save_coefs(NNCPModel *s, const char *filename) { nc_save_coefs(&s->params, filename); }
+void nncp_model_load_coefs(NNCPModel *s, const char *filename) { nc_load_coefs(&s->params, filename); }
+
 /* ---- pieces shared by the evaluation paths ----------------------------------- */
 
 static NCTensor *scalar(NNCPModel *s, float v) { return nc_new_f32(s->dev, v); }

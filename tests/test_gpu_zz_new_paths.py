@@ -204,6 +204,39 @@ def test_soft_max_int_bit_exact(V, n):
         assert outs[0].dtype == np.int32 and np.array_equal(outs[0], outs[1]), mult
 
 
+def test_parameter_files_cross_between_the_gpu_and_the_checker(hosts, tmp_path):
+    """nc_save_coefs / nc_load_coefs (libnc.h:530, 536): parameters trained on the GPU, saved by
+    the product library and loaded by the checker's own reader are the same bits, and so the
+    other way round (the two libraries implement the file layout separately); the loaded GPU
+    model then evaluates like the model that was saved."""
+    pkg = M.load_pkg()
+    cfg = dict(M.TINY, fused=1, sgd_opt=M.rmsprop(3e-3))
+    B, T = cfg["batch_size"], cfg["seg_len"]
+    syms = M.markov1(B * T * 4, cfg["n_symbols"], seed=5)
+    batches = list(M.segment_batches(syms, B, T, 4))
+    gpu = pkg.host.Model(hosts[0], pkg.host.make_config(**dict(cfg, use_device=1)))
+    for tok, tgt in batches[:3]:
+        gpu.train_step(tok, tgt, 3e-3)
+    gpu.save_coefs(str(tmp_path / "from_gpu.bin"))
+    ref = pkg.host.Model(hosts[1], pkg.host.make_config(**dict(cfg, seed=7, use_device=0, nb_threads=2)))
+    ref.load_coefs(str(tmp_path / "from_gpu.bin"))
+    for n in gpu.param_names():
+        assert np.array_equal(gpu.get_param(n), ref.get_param(n)), n
+    ref.save_coefs(str(tmp_path / "from_checker.bin"))
+    assert (tmp_path / "from_checker.bin").read_bytes() == (tmp_path / "from_gpu.bin").read_bytes()
+    gpu2 = pkg.host.Model(hosts[0], pkg.host.make_config(**dict(cfg, seed=8, use_device=1)))
+    gpu2.load_coefs(str(tmp_path / "from_checker.bin"))
+    tok, tgt = batches[3]
+    p1 = gpu.eval(tok)       # the memory of both models is empty for gpu2 only: compare a fresh segment
+    gpu.close()
+    gpu3 = pkg.host.Model(hosts[0], pkg.host.make_config(**dict(cfg, seed=9, use_device=1)))
+    gpu3.load_coefs(str(tmp_path / "from_gpu.bin"))
+    assert np.array_equal(gpu2.eval(tok), gpu3.eval(tok))
+    assert p1.shape == (T, B, cfg["n_symbols"])
+    for m in (ref, gpu2, gpu3):
+        m.close()
+
+
 @pytest.mark.parametrize("cfg_name", ["TINY", "C1"])
 def test_training_100_steps_match_checker(hosts, cfg_name):
     """The 1e-5 bar after 1, 10 and 100 steps of the fused path (probabilities, loss, every
