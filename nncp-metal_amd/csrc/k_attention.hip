@@ -271,7 +271,7 @@ extern "C" int nchip_relpos_attn_fwd_step(void *stream, const float *q, int64_t 
     if (!q || !kv || !out || (M > 0 && !kvm)) return bad("null pointer");
     if (t < 0 || t >= T) return bad("query position outside the segment");
     const int K = M + T;
-    if (!k_attn_fused_shape_ok(dk, dv, T, K, d_pos, w_r != nullptr) || ldq % 4 || ldkv % 4 || ldo % 4 ||
+    if (!k_attn_fused_step_ok(dk, dv, T, K, d_pos, w_r != nullptr) || ldq % 4 || ldkv % 4 || ldo % 4 ||
         !al16(q) || !al16(kv) || (kvm && !al16(kvm)) || (w_r && !al16(w_r)) || !al16(out))
         return bad("single-query attention needs the single-kernel shapes (d_head 32/64, T <= 64, K <= 128)");
     FusedAttnFwdArgs a;

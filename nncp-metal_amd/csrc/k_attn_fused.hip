@@ -189,17 +189,30 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
 
     float *Rw = Rs + (w * 16 + il) * FA_RSTRIDE; // this lane's column of rel
     {
-        float af[2][NS];
-        load_afrag<NS>(af[0], Ws + il * RS + g);
+        // two position tiles at a time: their accumulation chains alternate in the MFMA
+        // pipe (a dependent MFMA waits about twice its own issue time for its predecessor)
+        static_assert(NT % 2 == 0, "tiles are taken in pairs");
+        float af[2][2][NS];
+        load_afrag<NS>(af[0][0], Ws + il * RS + g);
+        load_afrag<NS>(af[0][1], Ws + (16 + il) * RS + g);
 #pragma unroll
-        for (int pt = 0; pt < NT; pt++) {
-            if (pt + 1 < NT) load_afrag<NS>(af[(pt + 1) & 1], Ws + ((pt + 1) * 16 + il) * RS + g);
+        for (int pp = 0; pp < NT / 2; pp++) {
+            if (pp + 1 < NT / 2) {
+                load_afrag<NS>(af[(pp + 1) & 1][0], Ws + ((2 * pp + 2) * 16 + il) * RS + g);
+                load_afrag<NS>(af[(pp + 1) & 1][1], Ws + ((2 * pp + 3) * 16 + il) * RS + g);
+            }
             PIPELINE_FENCE();
-            floatx4_t acc = { 0, 0, 0, 0 };
+            floatx4_t acc0 = { 0, 0, 0, 0 }, acc1 = { 0, 0, 0, 0 };
 #pragma unroll
-            for (int s = 0; s < NS; s++) acc = mfma16(af[pt & 1][s], qf[s], acc);
+            for (int s = 0; s < NS; s++) {
+                acc0 = mfma16(af[pp & 1][0][s], qf[s], acc0);
+                acc1 = mfma16(af[pp & 1][1][s], qf[s], acc1);
+            }
 #pragma unroll
-            for (int r = 0; r < 4; r++) Rw[pt * 16 + 4 * g + r] = acc[r];
+            for (int r = 0; r < 4; r++) {
+                Rw[(2 * pp) * 16 + 4 * g + r] = acc0[r];
+                Rw[(2 * pp + 1) * 16 + 4 * g + r] = acc1[r];
+            }
         }
         wave_lds_sync();
     }
@@ -215,34 +228,47 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
         const int pbase = a.d_pos - 1 - dbase;  // its rel row before clamping
         const int pmax = a.d_pos - 1;
         const unsigned dlim = i < a.T ? (unsigned)a.attn_len : 0u;
-        float af[2][NS];
-        load_afrag<NS>(af[0], Ks + il * RS + g);
+        float af[2][2][NS]; // key tiles in pairs, as the position tiles above
+        load_afrag<NS>(af[0][0], Ks + il * RS + g);
+        load_afrag<NS>(af[0][1], Ks + (16 + il) * RS + g);
 #pragma unroll
-        for (int jt = 0; jt < NT; jt++) {
-            if (jt + 1 < NT) load_afrag<NS>(af[(jt + 1) & 1], Ks + ((jt + 1) * 16 + il) * RS + g);
+        for (int jp = 0; jp < NT / 2; jp++) {
+            if (jp + 1 < NT / 2) {
+                load_afrag<NS>(af[(jp + 1) & 1][0], Ks + ((2 * jp + 2) * 16 + il) * RS + g);
+                load_afrag<NS>(af[(jp + 1) & 1][1], Ks + ((2 * jp + 3) * 16 + il) * RS + g);
+            }
             PIPELINE_FENCE();
             // shifted rel and bias of the 4 keys of this lane: loaded unconditionally
             // (clamped / padded, always inside the arrays) and selected afterwards
-            float relv[4], bv[4];
+            float relv[2][4], bv[2][4];
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                int delta = dbase - (jt * 16 + r);
-                int pi = pbase + (jt * 16 + r); // d_pos-1-delta
-                pi = pi < 0 ? 0 : (pi > pmax ? pmax : pi);
-                relv[r] = Rw[pi];
-                bv[r] = Bs[(a.K - 1 - delta) & (FA_NB - 1)];
+            for (int e = 0; e < 2; e++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int jt = 2 * jp + e;
+                    int delta = dbase - (jt * 16 + r);
+                    int pi = pbase + (jt * 16 + r); // d_pos-1-delta
+                    pi = pi < 0 ? 0 : (pi > pmax ? pmax : pi);
+                    relv[e][r] = Rw[pi];
+                    bv[e][r] = Bs[(a.K - 1 - delta) & (FA_NB - 1)];
+                }
+            floatx4_t acc[2] = { { 0, 0, 0, 0 }, { 0, 0, 0, 0 } };
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                acc[0] = mfma16(af[jp & 1][0][s], qf[s], acc[0]);
+                acc[1] = mfma16(af[jp & 1][1][s], qf[s], acc[1]);
             }
-            floatx4_t acc = { 0, 0, 0, 0 };
 #pragma unroll
-            for (int s = 0; s < NS; s++) acc = mfma16(af[jt & 1][s], qf[s], acc);
+            for (int e = 0; e < 2; e++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                // key j < K is implied: delta >= 0 > i - T for a real column
-                unsigned delta = (unsigned)(dbase - (jt * 16 + r));
-                float v = delta < dlim ? acc[r] + relv[r] + bv[r] : -INFINITY;
-                sc[jt][r] = v;
-                mx = fmaxf(mx, v);
-            }
+                for (int r = 0; r < 4; r++) {
+                    // key j < K is implied: delta >= 0 > i - T for a real column
+                    const int jt = 2 * jp + e;
+                    unsigned delta = (unsigned)(dbase - (jt * 16 + r));
+                    float v = delta < dlim ? acc[e][r] + relv[e][r] + bv[e][r] : -INFINITY;
+                    sc[jt][r] = v;
+                    mx = fmaxf(mx, v);
+                }
         }
     }
     PHASE_MARK(3);
@@ -389,21 +415,30 @@ void relpos_attn_bwd_fused(FusedAttnBwdArgs a)
         float dof[NS];
 #pragma unroll
         for (int s = 0; s < NS; s++) dof[s] = Os[i * RS + 4 * s + g];
-        float af[2][NS];
-        load_afrag<NS>(af[0], Vs + il * RS + g);
+        float af[2][2][NS]; // key tiles in pairs: two accumulation chains alternate in the MFMA pipe
+        load_afrag<NS>(af[0][0], Vs + il * RS + g);
+        load_afrag<NS>(af[0][1], Vs + (16 + il) * RS + g);
         float dot = 0.0f;
 #pragma unroll
-        for (int jt = 0; jt < NT; jt++) {
-            if (jt + 1 < NT) load_afrag<NS>(af[(jt + 1) & 1], Vs + ((jt + 1) * 16 + il) * RS + g);
-            PIPELINE_FENCE();
-            floatx4_t acc = { 0, 0, 0, 0 };
-#pragma unroll
-            for (int s = 0; s < NS; s++) acc = mfma16(af[jt & 1][s], dof[s], acc);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                ds[jt][r] = acc[r];
-                dot += p[jt][r] * acc[r];
+        for (int jp = 0; jp < NT / 2; jp++) {
+            if (jp + 1 < NT / 2) {
+                load_afrag<NS>(af[(jp + 1) & 1][0], Vs + ((2 * jp + 2) * 16 + il) * RS + g);
+                load_afrag<NS>(af[(jp + 1) & 1][1], Vs + ((2 * jp + 3) * 16 + il) * RS + g);
             }
+            PIPELINE_FENCE();
+            floatx4_t acc[2] = { { 0, 0, 0, 0 }, { 0, 0, 0, 0 } };
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                acc[0] = mfma16(af[jp & 1][0][s], dof[s], acc[0]);
+                acc[1] = mfma16(af[jp & 1][1][s], dof[s], acc[1]);
+            }
+#pragma unroll
+            for (int e = 0; e < 2; e++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) { // (the sum keeps its key order)
+                    ds[2 * jp + e][r] = acc[e][r];
+                    dot += p[2 * jp + e][r] * acc[e][r];
+                }
         }
         dot += __shfl_xor(dot, 16, 64);
         dot += __shfl_xor(dot, 32, 64);
@@ -622,6 +657,494 @@ __global__ __launch_bounds__(256) void attn_param_grad_reduce(const float *dwp, 
     *dst = acc;
 }
 
+// ---- more than 128 keys: the same arithmetic with the key / position axis in chunks ------
+// Up to 320 keys and relative positions (NTT 16-key tiles, a multiple of 4).  Q, the rel
+// strips and the bias row stay in LDS for the whole kernel; w_r, K and V pass through ONE
+// staging tile of 128 rows, chunk after chunk (global -> registers two chunks ahead ->
+// LDS), two barriers per chunk.  A column's scores for all keys live in registers
+// (NTT x 4 per lane), so the softmax is the one-pass softmax of the kernels above: maximum
+// and sum over all keys, no running rescale.
+template <int NTT>
+struct TiledDims {
+    static_assert(NTT % 4 == 0 && NTT > 8 && NTT <= 20, "12, 16 or 20 key tiles");
+    static constexpr int NCH = (NTT + 7) / 8;       // chunks of up to 8 tiles
+    static constexpr int KP = NTT * 16;             // padded key / position count
+    static constexpr int RST = KP + 3;              // rel strip row
+    static constexpr int NB = 1024;                 // bias row incl. every index a masked key can form
+    static constexpr int tiles_of(int c) { return NTT - 8 * c < 8 ? NTT - 8 * c : 8; }
+};
+
+template <int DK, int NTT>
+struct FwdTiledLayout {
+    using D = TiledDims<NTT>;
+    static constexpr int RS = DK + 4;
+    static constexpr int q = 0, st = q + FA_TMAX * RS, r = st + 128 * RS, b = r + 4 * 16 * D::RST,
+                         floats = b + D::NB;
+};
+
+template <int DK, int NTT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void relpos_attn_fwd_tiled(FusedAttnFwdArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    using L = FwdTiledLayout<DK, NTT>;
+    using D = TiledDims<NTT>;
+    constexpr int RS = DK + 4, NS = DK / 4, ND = DK / 16, NCH = D::NCH, RST = D::RST, NI = 3 * NCH;
+    float *Qs = lds + L::q, *Ss = lds + L::st, *Rs = lds + L::r, *Bs = lds + L::b;
+
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int b = blockIdx.x % a.B, h = blockIdx.x / a.B;
+    const int il = lane & 15, g = lane >> 4;
+    const int i = 16 * w + il;
+    const bool has_w = a.w_r != nullptr;
+    const float *w_base = has_w ? a.w_r + (int64_t)h * a.d_pos * DK : a.q;
+    const int n_w = has_w ? a.d_pos : 0;
+    auto kvrow = [&](int r) {
+        return (r < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * r)
+                        : a.kv + a.ldkv * (b + (int64_t)a.B * (r - a.M))) + (int64_t)h * DK;
+    };
+    // staging items in the order they are used: position chunks, key chunks, value chunks
+    floatx4_t vq[FA_TMAX * (DK / 4) / 256], vs[2][128 * (DK / 4) / 256];
+    auto rows_of = [&](int item) { // valid rows of the item's chunk
+        const int c = item % NCH, total = item < NCH ? n_w : a.K;
+        const int left = total - 128 * c;
+        return left < 0 ? 0 : (left > 128 ? 128 : left);
+    };
+    auto fetch = [&](int item, floatx4_t (&v)[128 * (DK / 4) / 256]) {
+        const int c = item % NCH, kind = item / NCH, nv = rows_of(item);
+        if (kind == 0) fetch_rows<DK, 128>(v, nv, [&](int r) { return w_base + (int64_t)(nv ? r + 128 * c : 0) * DK; });
+        else if (kind == 1) fetch_rows<DK, 128>(v, nv, [&](int r) { return kvrow(nv ? r + 128 * c : 0); });
+        else fetch_rows<DK, 128>(v, nv, [&](int r) { return kvrow(nv ? r + 128 * c : 0) + (int64_t)a.H * DK; });
+    };
+    for (int e = t; e < D::NB; e += 256)
+        Bs[e] = (a.b_r && e < a.K) ? as_global(a.b_r)[(int64_t)h * a.K + e] * (a.b_r_scale * a.scale) : 0.0f;
+    fetch_rows<DK, FA_TMAX>(vq, a.T, [&](int r) { return a.q + (int64_t)h * DK + a.ldq * (b + (int64_t)a.B * r); });
+    fetch(0, vs[0]);
+    fetch(1, vs[1]);
+    put_rows<DK, FA_TMAX>(Qs, vq, a.T);
+
+    float qf[NS];
+    float *Rw = Rs + (w * 16 + il) * RST; // this lane's column of rel
+    float sc[NTT][4];
+    float mx = -INFINITY;
+    floatx4_t oacc[ND];
+#pragma unroll
+    for (int dt = 0; dt < ND; dt++) oacc[dt] = floatx4_t{ 0, 0, 0, 0 };
+    const int dbase = i + a.M - 4 * g;      // delta of key 4g of tile 0
+    const int pbase = a.d_pos - 1 - dbase;  // its rel row before clamping
+    const int pmax = a.d_pos - 1;
+    const unsigned dlim = i < a.T ? (unsigned)a.attn_len : 0u;
+
+#pragma unroll
+    for (int item = 0; item < NI; item++) {
+        const int c = item % NCH, kind = item / NCH;
+        constexpr int dummy = 0; (void)dummy;
+        if (item > 0) __syncthreads(); // every wavefront has left the staging tile
+        put_rows<DK, 128>(Ss, vs[item & 1], rows_of(item));
+        if (item + 2 < NI) fetch(item + 2, vs[item & 1]);
+        __syncthreads();
+        if (item == 0) {
+#pragma unroll
+            for (int s = 0; s < NS; s++) qf[s] = Qs[i * RS + 4 * s + g] * a.scale; // 1/sqrt(dk) folded in
+        }
+        const int nt = D::tiles_of(c);
+        if (kind == 0) {
+            // rel = w_r^T q for the positions of this chunk -> strip
+            float af[2][NS];
+            load_afrag<NS>(af[0], Ss + il * RS + g);
+#pragma unroll
+            for (int pt = 0; pt < 8; pt++) {
+                if (pt >= nt) break;
+                if (pt + 1 < nt) load_afrag<NS>(af[(pt + 1) & 1], Ss + ((pt + 1) * 16 + il) * RS + g);
+                PIPELINE_FENCE();
+                floatx4_t acc = { 0, 0, 0, 0 };
+#pragma unroll
+                for (int s = 0; s < NS; s++) acc = mfma16(af[pt & 1][s], qf[s], acc);
+#pragma unroll
+                for (int r = 0; r < 4; r++) Rw[(8 * c + pt) * 16 + 4 * g + r] = acc[r];
+            }
+            if (c == NCH - 1) wave_lds_sync();
+        } else if (kind == 1) {
+            float af[2][NS];
+            load_afrag<NS>(af[0], Ss + il * RS + g);
+#pragma unroll
+            for (int jl = 0; jl < 8; jl++) {
+                if (jl >= nt) break;
+                const int jt = 8 * c + jl;
+                if (jl + 1 < nt) load_afrag<NS>(af[(jl + 1) & 1], Ss + ((jl + 1) * 16 + il) * RS + g);
+                PIPELINE_FENCE();
+                float relv[4], bv[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    int delta = dbase - (jt * 16 + r);
+                    int pi = pbase + (jt * 16 + r); // d_pos-1-delta
+                    pi = pi < 0 ? 0 : (pi > pmax ? pmax : pi);
+                    relv[r] = Rw[pi];
+                    bv[r] = Bs[(a.K - 1 - delta) & (D::NB - 1)];
+                }
+                floatx4_t acc = { 0, 0, 0, 0 };
+#pragma unroll
+                for (int s = 0; s < NS; s++) acc = mfma16(af[jl & 1][s], qf[s], acc);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    unsigned delta = (unsigned)(dbase - (jt * 16 + r));
+                    float v = delta < dlim ? acc[r] + relv[r] + bv[r] : -INFINITY;
+                    sc[jt][r] = v;
+                    mx = fmaxf(mx, v);
+                }
+            }
+            if (c == NCH - 1) {
+                // softmax over all keys of the column (lanes l, l^16, l^32, l^48 share it)
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                if (mx == -INFINITY) mx = 0.0f; // padding column
+                float sum = 0.0f;
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float e = __expf(sc[jt][r] - mx); // exp(-inf) = 0 for masked keys
+                        sc[jt][r] = e;
+                        sum += e;
+                    }
+                sum += __shfl_xor(sum, 16, 64);
+                sum += __shfl_xor(sum, 32, 64);
+                float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) sc[jt][r] *= inv;
+                if (a.probs && i < a.T) {
+                    float NCHIP_GLOBAL *pc = as_global(a.probs) + (((int64_t)b * a.H + h) * a.T + i) * a.K;
+#pragma unroll
+                    for (int jt = 0; jt < NTT; jt++) {
+                        int j0 = jt * 16 + 4 * g;
+                        if (j0 < a.K) { // K is a multiple of 4: whole quads
+                            floatx4_t v = { sc[jt][0], sc[jt][1], sc[jt][2], sc[jt][3] };
+                            *reinterpret_cast<floatx4_t NCHIP_GLOBAL *>(pc + j0) = v;
+                        }
+                    }
+                }
+            }
+        } else {
+            // O += V P over the keys of this chunk
+            float vf[2][ND][4];
+            load_tokfrag<ND, RS>(vf[0], Ss, 0, g, il);
+#pragma unroll
+            for (int jl = 0; jl < 8; jl++) {
+                if (jl >= nt) break;
+                const int jt = 8 * c + jl;
+                if (jl + 1 < nt) load_tokfrag<ND, RS>(vf[(jl + 1) & 1], Ss, jl + 1, g, il);
+                PIPELINE_FENCE();
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int dt = 0; dt < ND; dt++) oacc[dt] = mfma16(vf[jl & 1][dt][r], sc[jt][r], oacc[dt]);
+            }
+        }
+    }
+    if (i < a.T) {
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++) {
+            float NCHIP_GLOBAL *o = as_global(a.out) + (int64_t)h * DK + dt * 16 + 4 * g + a.ldo * (b + (int64_t)a.B * i);
+            *reinterpret_cast<floatx4_t NCHIP_GLOBAL *>(o) = oacc[dt];
+        }
+    }
+}
+
+template <int DK, int NTT>
+struct BwdTiledLayout {
+    using D = TiledDims<NTT>;
+    static constexpr int RS = DK + 4;
+    static_assert(2 * 64 * FA_PSTRIDE <= 128 * RS, "the transposed P / dS tiles of 64 keys fit in the staging tile");
+    static constexpr int q = 0, o = q + FA_TMAX * RS, st = o + FA_TMAX * RS, r = st + 128 * RS,
+                         floats = r + FA_TMAX * D::RST;
+};
+
+// Backward for more than 128 keys.  dO, Q and the dRel strip stay in LDS; V, K and w_r pass
+// through the staging tile in chunks of 128 rows (dA, then dq), and P^T / dS^T are parked
+// in the same tile 64 keys at a time for dK, dV and the db_r diagonals.  The probabilities
+// and dS of a column for all keys live in registers.
+template <int DK, int NTT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void relpos_attn_bwd_tiled(FusedAttnBwdArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    using L = BwdTiledLayout<DK, NTT>;
+    using D = TiledDims<NTT>;
+    constexpr int RS = DK + 4, NS = DK / 4, ND = DK / 16, NCH = D::NCH, RST = D::RST, NI = 3 * NCH, PS = FA_PSTRIDE;
+    constexpr int NSQ = FA_TMAX / 4, KP = D::KP;
+    float *Qs = lds + L::q, *Os = lds + L::o, *Ss = lds + L::st, *Rs = lds + L::r;
+    float *Pt = Ss, *St = Ss + 64 * PS; // [64 keys][PS] each
+
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int b = blockIdx.x % a.B, h = blockIdx.x / a.B;
+    const bool has_w = a.w_r != nullptr;
+    const int il = lane & 15, g = lane >> 4;
+    const int i = 16 * w + il;
+    const float *w_base = has_w ? a.w_r + (int64_t)h * a.d_pos * DK : a.q;
+    const int n_w = has_w ? a.d_pos : 0;
+    auto kvrow = [&](int r) {
+        return (r < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * r)
+                        : a.kv + a.ldkv * (b + (int64_t)a.B * (r - a.M))) + (int64_t)h * DK;
+    };
+    // staging items: value chunks (dA), key chunks (dq), position chunks (dq)
+    floatx4_t vq[FA_TMAX * (DK / 4) / 256], vo[FA_TMAX * (DK / 4) / 256], vs[2][128 * (DK / 4) / 256];
+    auto rows_of = [&](int item) {
+        const int c = item % NCH, total = item < 2 * NCH ? a.K : n_w;
+        const int left = total - 128 * c;
+        return left < 0 ? 0 : (left > 128 ? 128 : left);
+    };
+    auto fetch = [&](int item, floatx4_t (&v)[128 * (DK / 4) / 256]) {
+        const int c = item % NCH, kind = item / NCH, nv = rows_of(item);
+        if (kind == 0) fetch_rows<DK, 128>(v, nv, [&](int r) { return kvrow(nv ? r + 128 * c : 0) + (int64_t)a.H * DK; });
+        else if (kind == 1) fetch_rows<DK, 128>(v, nv, [&](int r) { return kvrow(nv ? r + 128 * c : 0); });
+        else fetch_rows<DK, 128>(v, nv, [&](int r) { return w_base + (int64_t)(nv ? r + 128 * c : 0) * DK; });
+    };
+    float p[NTT][4], ds[NTT][4];
+    fetch_rows<DK, FA_TMAX>(vo, a.T, [&](int r) { return a.dout + (int64_t)h * DK + a.ldo * (b + (int64_t)a.B * r); });
+    fetch(0, vs[0]);
+    {
+        const float NCHIP_GLOBAL *pc = as_global(a.probs) + (((int64_t)b * a.H + h) * a.T + (i < a.T ? i : 0)) * a.K;
+#pragma unroll
+        for (int jt = 0; jt < NTT; jt++) { // unconditional loads from clamped addresses; masked at first use
+            int j0 = jt * 16 + 4 * g;
+            floatx4_t v = *reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(pc + (j0 < a.K ? j0 : 0));
+#pragma unroll
+            for (int r = 0; r < 4; r++) p[jt][r] = v[r];
+        }
+    }
+    fetch(1, vs[1]);
+    fetch_rows<DK, FA_TMAX>(vq, a.T, [&](int r) { return a.q + (int64_t)h * DK + a.ldq * (b + (int64_t)a.B * r); });
+    put_rows<DK, FA_TMAX>(Os, vo, a.T);
+    put_rows<DK, FA_TMAX>(Qs, vq, a.T);
+
+    float dof[NS];
+    float dot = 0.0f;
+    float *Rw = Rs + i * RST;
+    floatx4_t dqa[ND];
+#pragma unroll
+    for (int dt = 0; dt < ND; dt++) dqa[dt] = floatx4_t{ 0, 0, 0, 0 };
+
+#pragma unroll
+    for (int item = 0; item < NI; item++) {
+        const int c = item % NCH, kind = item / NCH;
+        if (item > 0) __syncthreads(); // every wavefront has left the staging tile
+        put_rows<DK, 128>(Ss, vs[item & 1], rows_of(item));
+        if (item + 2 < NI) fetch(item + 2, vs[item & 1]);
+        __syncthreads();
+        const int nt = D::tiles_of(c);
+        if (kind == 0) {
+            if (item == 0) {
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        p[jt][r] = (i < a.T && jt * 16 + 4 * g + r < a.K) ? p[jt][r] : 0.0f;
+#pragma unroll
+                for (int s = 0; s < NS; s++) dof[s] = Os[i * RS + 4 * s + g];
+            }
+            // dA = V^T dO for the keys of this chunk
+            float af[2][NS];
+            load_afrag<NS>(af[0], Ss + il * RS + g);
+#pragma unroll
+            for (int jl = 0; jl < 8; jl++) {
+                if (jl >= nt) break;
+                const int jt = 8 * c + jl;
+                if (jl + 1 < nt) load_afrag<NS>(af[(jl + 1) & 1], Ss + ((jl + 1) * 16 + il) * RS + g);
+                PIPELINE_FENCE();
+                floatx4_t acc = { 0, 0, 0, 0 };
+#pragma unroll
+                for (int s = 0; s < NS; s++) acc = mfma16(af[jl & 1][s], dof[s], acc);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    ds[jt][r] = acc[r];
+                    dot += p[jt][r] * acc[r];
+                }
+            }
+            if (c == NCH - 1) {
+                // dS = P (dA - colsum(P dA)) / sqrt(dk), then its rel-shift adjoint into the strip
+                dot += __shfl_xor(dot, 16, 64);
+                dot += __shfl_xor(dot, 32, 64);
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) ds[jt][r] = p[jt][r] * (ds[jt][r] - dot) * a.scale; // masked: p = 0
+                for (int pp = g; pp < KP; pp += 4) Rw[pp] = 0.0f;
+                wave_lds_sync();
+                const int dbase = i + a.M - 4 * g, pbase = a.d_pos - 1 - dbase;
+                const unsigned dlim = (i < a.T && has_w) ? (unsigned)a.attn_len : 0u;
+                float acc0 = 0.0f;
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        unsigned delta = (unsigned)(dbase - (jt * 16 + r));
+                        int pi = pbase + (jt * 16 + r);
+                        // rows >= 1 receive exactly one key; row 0 collects the far keys;
+                        // masked keys go to a dump slot past the strip (never read)
+                        const bool on = delta < dlim;
+                        Rw[(on && pi >= 1) ? pi : RST - 1] = ds[jt][r];
+                        acc0 += (on && pi < 1) ? ds[jt][r] : 0.0f;
+                    }
+                acc0 += __shfl_xor(acc0, 16, 64);
+                acc0 += __shfl_xor(acc0, 32, 64);
+                if (g == 0) Rw[0] = acc0;
+                wave_lds_sync();
+            }
+        } else {
+            // dq += K dS (kind 1) or w_r dRel (kind 2) over the rows of this chunk
+            float kf[2][ND][4], rf[2][4];
+            load_tokfrag<ND, RS>(kf[0], Ss, 0, g, il);
+            if (kind == 2) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) rf[0][r] = Rw[(8 * c) * 16 + 4 * g + r];
+            }
+#pragma unroll
+            for (int jl = 0; jl < 8; jl++) {
+                if (jl >= nt) break;
+                const int jt = 8 * c + jl;
+                if (jl + 1 < nt) {
+                    load_tokfrag<ND, RS>(kf[(jl + 1) & 1], Ss, jl + 1, g, il);
+                    if (kind == 2) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) rf[(jl + 1) & 1][r] = Rw[(jt + 1) * 16 + 4 * g + r];
+                    }
+                }
+                PIPELINE_FENCE();
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int dt = 0; dt < ND; dt++)
+                        dqa[dt] = mfma16(kf[jl & 1][dt][r], kind == 1 ? ds[jt][r] : rf[jl & 1][r], dqa[dt]);
+            }
+        }
+    }
+    if (i < a.T) {
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++) {
+            float *o = a.dq + (int64_t)h * DK + dt * 16 + 4 * g + a.ldq * (b + (int64_t)a.B * i);
+            *reinterpret_cast<floatx4_t *>(o) = dqa[dt];
+        }
+    }
+
+    // the contraction now runs over the query index; k-slot g of step s is
+    // query 16*(s/4) + 4g + s%4, which keeps the Q / dO reads conflict-free
+    auto load_qd = [&](float (&f)[ND], const float *base, int s) {
+        int iq = 16 * (s >> 2) + 4 * g + (s & 3);
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++) f[dt] = base[iq * RS + dt * 16 + il];
+    };
+    // dK = Q dS^T, dV = dO P^T, 64 keys at a time: wavefront w owns key tile 4*hc + w;
+    // db_r: thread t sums the diagonals delta = t and t + 256 over the parked keys
+    float dbacc[2] = { 0.0f, 0.0f };
+#pragma unroll
+    for (int hc = 0; hc < NTT / 4; hc++) {
+        __syncthreads(); // the staging tile (or the previous 64 keys) is dead
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int jl = e * 16 + 4 * g + r;
+                Pt[jl * PS + i] = p[4 * hc + e][r];
+                St[jl * PS + i] = ds[4 * hc + e][r];
+            }
+        __syncthreads();
+        {
+            float sb[NSQ], pb[NSQ];
+#pragma unroll
+            for (int s = 0; s < NSQ; s++) {
+                int iq = 16 * (s >> 2) + 4 * g + (s & 3);
+                sb[s] = St[(w * 16 + il) * PS + iq];
+                pb[s] = Pt[(w * 16 + il) * PS + iq];
+            }
+            floatx4_t ak[ND], av[ND];
+#pragma unroll
+            for (int dt = 0; dt < ND; dt++) { ak[dt] = floatx4_t{ 0, 0, 0, 0 }; av[dt] = floatx4_t{ 0, 0, 0, 0 }; }
+            float qa[2][ND], oa[2][ND];
+            load_qd(qa[0], Qs, 0);
+            load_qd(oa[0], Os, 0);
+#pragma unroll
+            for (int s = 0; s < NSQ; s++) {
+                if (s + 1 < NSQ) { load_qd(qa[(s + 1) & 1], Qs, s + 1); load_qd(oa[(s + 1) & 1], Os, s + 1); }
+                PIPELINE_FENCE();
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++) {
+                    ak[dt] = mfma16(qa[s & 1][dt], sb[s], ak[dt]);
+                    av[dt] = mfma16(oa[s & 1][dt], pb[s], av[dt]);
+                }
+            }
+            const int j = (4 * hc + w) * 16 + il;
+            if (j < a.K) {
+                float *dst = (j < a.M ? a.dkvm + a.ldkv * (b + (int64_t)a.B * j)
+                                      : a.dkv + a.ldkv * (b + (int64_t)a.B * (j - a.M))) + (int64_t)h * DK;
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++) {
+                    *reinterpret_cast<floatx4_t *>(dst + dt * 16 + 4 * g) = ak[dt];
+                    *reinterpret_cast<floatx4_t *>(dst + (int64_t)a.H * DK + dt * 16 + 4 * g) = av[dt];
+                }
+            }
+        }
+        if (a.dbp) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int delta = t + 256 * u;
+                // keys 64*hc .. 64*hc+63 of diagonal delta belong to queries lo .. lo+63
+                const int lo = delta - a.M + 64 * hc;
+                float acc = 0.0f;
+#pragma unroll 8
+                for (int q8 = 0; q8 < 64; q8++) {
+                    const int iq = lo + q8;
+                    const bool on = delta < a.K && iq >= 0 && iq < a.T && 64 * hc + q8 < a.K;
+                    float v = St[(on ? q8 : 0) * PS + (on ? iq : 0)];
+                    acc += on ? v : 0.0f;
+                }
+                dbacc[u] += acc;
+            }
+        }
+    }
+    // dw_r partial of this (stream, head): Q dRel^T, wavefront w owns position tiles w, w+4, ...
+    if (has_w) {
+        float *dwz = a.dwp + ((int64_t)b * a.H + h) * a.d_pos * DK;
+#pragma unroll
+        for (int u = 0; u < NTT / 4; u++) {
+            const int pt = w + 4 * u;
+            float rb[NSQ];
+#pragma unroll
+            for (int s = 0; s < NSQ; s++) {
+                int iq = 16 * (s >> 2) + 4 * g + (s & 3);
+                rb[s] = Rs[iq * RST + pt * 16 + il];
+            }
+            floatx4_t acc[ND];
+#pragma unroll
+            for (int dt = 0; dt < ND; dt++) acc[dt] = floatx4_t{ 0, 0, 0, 0 };
+            float qa[2][ND];
+            load_qd(qa[0], Qs, 0);
+#pragma unroll
+            for (int s = 0; s < NSQ; s++) {
+                if (s + 1 < NSQ) load_qd(qa[(s + 1) & 1], Qs, s + 1);
+                PIPELINE_FENCE();
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++) acc[dt] = mfma16(qa[s & 1][dt], rb[s], acc[dt]);
+            }
+            const int pp = pt * 16 + il;
+            if (pp < a.d_pos) {
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++)
+                    *reinterpret_cast<floatx4_t *>(dwz + (int64_t)pp * DK + dt * 16 + 4 * g) = acc[dt];
+            }
+        }
+    }
+    if (a.dbp) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int delta = t + 256 * u;
+            if (delta < a.K)
+                a.dbp[((int64_t)b * a.H + h) * a.K + (a.K - 1 - delta)] = a.b_r_scale * dbacc[u];
+        }
+    }
+}
+
 template <typename KernelT>
 bool allow_lds(KernelT kern, size_t bytes)
 {
@@ -671,15 +1194,57 @@ int launch_bwd(hipStream_t st, const FusedAttnBwdArgs &a)
     return probs_vec(a) ? launch_bwd_v<DK, NT, true>(st, a) : launch_bwd_v<DK, NT, false>(st, a);
 }
 
+template <int DK, int NTT>
+int launch_fwd_tiled(hipStream_t st, const FusedAttnFwdArgs &a)
+{
+    constexpr size_t bytes = sizeof(float) * FwdTiledLayout<DK, NTT>::floats;
+    static_assert(bytes <= 160 * 1024, "forward tiles exceed LDS");
+    static const bool ok = allow_lds(relpos_attn_fwd_tiled<DK, NTT>, bytes);
+    if (!ok) return -1;
+    hipLaunchKernelGGL((relpos_attn_fwd_tiled<DK, NTT>), dim3(a.B * a.H), dim3(256), bytes, st, a);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <int DK, int NTT>
+int launch_bwd_tiled(hipStream_t st, const FusedAttnBwdArgs &a)
+{
+    constexpr size_t bytes = sizeof(float) * BwdTiledLayout<DK, NTT>::floats;
+    static_assert(bytes <= 160 * 1024, "backward tiles exceed LDS");
+    static const bool ok = allow_lds(relpos_attn_bwd_tiled<DK, NTT>, bytes);
+    if (!ok) return -1;
+    hipLaunchKernelGGL((relpos_attn_bwd_tiled<DK, NTT>), dim3(a.B * a.H), dim3(256), bytes, st, a);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// 16-key tiles the chunked kernels need for K keys and d_pos positions (0: not their shape)
+int tiled_ntt(int K, int d_pos)
+{
+    const int need = K > d_pos ? K : d_pos;
+    const int ntt = ((need + 15) / 16 + 3) / 4 * 4;
+    return (need > 128 && ntt <= 20 && (K & 3) == 0) ? ntt : 0;
+}
+
 } // namespace
 
-bool k_attn_fused_shape_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr)
+bool k_attn_fused_step_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr)
 {
     return dk == dv && (dk == 64 || dk == 32) && T <= FA_TMAX && K <= 128 && (!has_wr || d_pos <= 128);
 }
 
+bool k_attn_fused_shape_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr)
+{
+    if (k_attn_fused_step_ok(dk, dv, T, K, d_pos, has_wr)) return true;
+    return dk == 64 && dv == 64 && T <= FA_TMAX && tiled_ntt(K, has_wr ? d_pos : 1) != 0;
+}
+
 int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk)
 {
+    if (const int ntt = (a.K > 128 || a.d_pos > 128) ? tiled_ntt(a.K, a.d_pos) : 0) {
+        if (dk != 64 || a.q_only >= 0 || !a.probs || !probs_vec(a)) return -1;
+        return ntt == 12 ? launch_fwd_tiled<64, 12>(st, a) : ntt == 16 ? launch_fwd_tiled<64, 16>(st, a)
+                                                                      : launch_fwd_tiled<64, 20>(st, a);
+    }
+    if (a.K > 128 || a.d_pos > 128) return -1;
     const bool small = a.K <= 64 && a.d_pos <= 64;
     if (dk == 64) return small ? launch_fwd<64, 4>(st, a) : launch_fwd<64, 8>(st, a);
     return small ? launch_fwd<32, 4>(st, a) : launch_fwd<32, 8>(st, a);
@@ -689,7 +1254,14 @@ int k_attn_fused_bwd(hipStream_t st, const FusedAttnBwdArgs &a, int dk, float *d
                      int64_t n_w, int64_t n_b, int *launches, bool keep_partials)
 {
     const bool small = a.K <= 64 && a.d_pos <= 64;
-    int rc = dk == 64 ? (small ? launch_bwd<64, 4>(st, a) : launch_bwd<64, 8>(st, a))
+    int rc;
+    if (a.K > 128 || a.d_pos > 128) {
+        const int ntt = tiled_ntt(a.K, a.d_pos);
+        if (!ntt || dk != 64 || !probs_vec(a)) return -1;
+        rc = ntt == 12 ? launch_bwd_tiled<64, 12>(st, a) : ntt == 16 ? launch_bwd_tiled<64, 16>(st, a)
+                                                                    : launch_bwd_tiled<64, 20>(st, a);
+    } else
+        rc = dk == 64 ? (small ? launch_bwd<64, 4>(st, a) : launch_bwd<64, 8>(st, a))
                       : (small ? launch_bwd<32, 4>(st, a) : launch_bwd<32, 8>(st, a));
     if (rc) return rc;
     *launches = 1;

@@ -679,13 +679,17 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
             float fa[2][CH][TM], fb[2][CH][TN];
             const float *pa = sa + ((lane >> 5) + kg * 16) * RSA + wm * WTM + (lane & 31);
             const float *pb = sb + ((lane >> 5) + kg * 16) * RSB + wn * WTN + (lane & 31);
+            // Issue order: with two accumulator sets the steps of the two chains alternate
+            // (chain A's step p, chain B's step p, ...), so consecutive MFMAs never depend on
+            // each other; each chain still sees its own steps in increasing k order.
+            auto stepof = [](int v) { return NACC == 2 ? (v & 1) * 4 + (v >> 1) : v; };
             auto fetch_chunk = [&](int c, int buf) {
 #pragma unroll
                 for (int u = 0; u < CH; u++) {
 #pragma unroll
-                    for (int j = 0; j < TM; j++) fa[buf][u][j] = pa[krow(c * CH + u) * RSA + j * 32];
+                    for (int j = 0; j < TM; j++) fa[buf][u][j] = pa[krow(stepof(c * CH + u)) * RSA + j * 32];
 #pragma unroll
-                    for (int i = 0; i < TN; i++) fb[buf][u][i] = pb[krow(c * CH + u) * RSB + i * 32];
+                    for (int i = 0; i < TN; i++) fb[buf][u][i] = pb[krow(stepof(c * CH + u)) * RSB + i * 32];
                 }
             };
             if constexpr (FRAG == 1) {
@@ -730,7 +734,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
                     for (int i = 0; i < TN; i++)
 #pragma unroll
                         for (int j = 0; j < TM; j++) {
-                            if (NACC == 2 && (c & 1)) // steps 4..7 of the slab: the group's second chain
+                            if (NACC == 2 && stepof(c * CH + u) >= 4) // steps 4..7 of the slab: the group's second chain
                                 acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[c & 1][u][i], fa[c & 1][u][j], acc2[i][j], 0, 0, 0);
                             else
                                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[c & 1][u][i], fa[c & 1][u][j], acc[i][j], 0, 0, 0);

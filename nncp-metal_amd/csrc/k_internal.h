@@ -101,6 +101,8 @@ struct FusedAttnBwdArgs {
     float b_r_scale, scale;
 };
 bool k_attn_fused_shape_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr);
+// the single-query (per-timestep) mode: heads of up to 128 keys only
+bool k_attn_fused_step_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr);
 int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk);
 // returns 0, -1 (path unavailable, nothing launched) or -2 (launch failed)
 int k_attn_fused_bwd(hipStream_t st, const FusedAttnBwdArgs &a, int dk, float *dw_r, float *db_r,

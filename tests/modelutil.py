@@ -25,9 +25,16 @@ def hip_host():
     GPU tests without a GPU - the same sources built for the host (tests/hipcpu)."""
     pkg = load_pkg()
     emu, emu_host = os.environ.get("NNCP_TEST_HIP_LIB"), os.environ.get("NNCP_TEST_HOST_HIP_LIB")
-    if emu and emu_host:
-        return pkg.host.Host(emu_host, emu)
-    return pkg.host.Host()
+    host = pkg.host.Host(emu_host, emu) if emu and emu_host else pkg.host.Host()
+    # The library's HIP runtime comes up now, before any test has a chance to let torch bring
+    # up the copy it bundles (its autograd engine counts the devices at its first backward
+    # pass): the runtime that initialises second in a process finds no device, and the
+    # library then ends the process ("no HIP device 0 (found 0)").
+    nc = host.ncl
+    ctx = nc.nc_context_init(1)
+    nc.nc_new_cuda_device(ctx, 0)
+    nc.nc_context_end(ctx)
+    return host
 
 
 def rmsprop(lr=3e-4):

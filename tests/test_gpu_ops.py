@@ -150,7 +150,12 @@ def test_gemm_bf16_from_rounded_copies(hip, ref, rng, m, n, k, ta, tb):
                                  dict(H=2, dk=64, dv=64, B=1, T=64, M=64, d_pos=64, attn_len=100),
                                  dict(H=2, dk=64, dv=64, B=2, T=48, M=80, d_pos=128, attn_len=128),
                                  dict(H=2, dk=64, dv=64, B=2, T=64, M=96, d_pos=160, attn_len=160),
-                                 dict(H=2, dk=64, dv=64, B=19, T=64, M=192, d_pos=256, attn_len=256)])
+                                 dict(H=2, dk=64, dv=64, B=19, T=64, M=192, d_pos=256, attn_len=256),
+                                 # more than 128 keys: the key-chunked single-kernel path (12, 16, 20 key tiles)
+                                 dict(H=2, dk=64, dv=64, B=3, T=64, M=256, d_pos=320, attn_len=320),
+                                 dict(H=1, dk=64, dv=64, B=2, T=40, M=160, d_pos=40, attn_len=90),
+                                 dict(H=2, dk=64, dv=64, B=2, T=64, M=140, d_pos=204, attn_len=204),
+                                 dict(H=2, dk=64, dv=64, B=2, T=17, M=283, d_pos=300, attn_len=150)])
 def test_relpos_attention_model_shapes(hip, ref, rng, cfg):
     H, dk, dv, B, T, M, d_pos = (cfg[k] for k in ("H", "dk", "dv", "B", "T", "M", "d_pos"))
     K = M + T
@@ -169,6 +174,10 @@ def test_relpos_attention_model_shapes(hip, ref, rng, cfg):
     assert relerr(res[0][0], res[1][0]) <= TOL
     for gh, gr in zip(res[0][1], res[1][1]):
         assert relerr(gh, gr) <= 5 * TOL
+    if dk == 64 and K % 4 == 0 and K <= 320:
+        # these shapes take one kernel each way (plus the sum of the per-stream partials)
+        lib = C.CDLL(hip.lib._name)
+        assert lib.nchip_relpos_attn_last_launches() <= 2
 
 
 def _adversarial_logits(rng, V, n):
