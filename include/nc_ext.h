@@ -49,6 +49,14 @@ NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv_mem,
                               NCTensor *w_r, NCTensor *b_r, int n_head,
                               int d_key, int attn_len, float b_r_scale);
 
+/* The two projections of one decoder timestep (nncp.c:801-812) in one launch: returns
+   w0 x + bias0 (m0, n) and writes w1 x (m1, n) into slice `index` of the last axis of dst
+   (m1, n, T), the key / value cache.  w0 (m0, k), w1 (m1, k), x (k, n); bias0 may be NULL.
+   Consumes w0, bias0, w1 and x, not dst.  The values are those of nc_linear(w0, x, bias0)
+   and nc_matmul(w1, x), bit for bit.  No gradient. */
+NCTensor *nc_linear_pair_into(NCTensor *w0, NCTensor *bias0, NCTensor *w1, NCTensor *x,
+                              NCTensor *dst, int index);
+
 /* One query position of nc_relpos_attention: q (H*dk, B) is the query of
    position t, kv_cache (H*dk+H*dv, B, T) holds the keys / values of positions
    0..t of the current segment (later columns finite, e.g. zero), kv_mem, w_r,

@@ -114,6 +114,19 @@ int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launch
    choice.  The environment variable NCHIP_GEMM_CFG sets the initial value. */
 void nchip_gemm_force_config(int cfg);
 
+/* Two width-invariant fp32 products that share their right operand, in one launch:
+   C0 (m0 x n) = A0 (m0 x k) B (k x n) + bias0 and C1 (m1 x n) = A1 (m1 x k) B + bias1, column
+   major, untransposed, bias pointers may be NULL (the per-timestep query and key/value
+   projections of the decoder, nncp.c:801-812, whose second result goes straight into its
+   cache slot).  The bits are those of two nchip_gemm calls with NCHIP_GEMM_WIDTH_INVARIANT.
+   Returns 0, 1 when the shapes are not the few-column kernel's (n <= 64, k and both m
+   multiples of 32, 16-byte aligned operands; nothing was launched), negative on error. */
+int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, int k,
+                                const float *A0, int64_t lda0, const float *A1, int64_t lda1,
+                                const float *B, int64_t ldb,
+                                float *C0, int64_t ldc0, float *C1, int64_t ldc1,
+                                const float *bias0, const float *bias1);
+
 /* Testing aid: width-invariant fp32 products (NCHIP_GEMM_WIDTH_INVARIANT) with at most 64
    columns, untransposed operands and beta = 0 run a register-streaming kernel that issues the
    tile kernel's MFMA sequence without its LDS pipeline (the decoder's per-timestep products);

@@ -63,6 +63,11 @@ struct GemmArgs {
     int dbg;
     const NchipGemmProblem *grp; // grouped launch: one problem per table row
     int n_grp;
+    // second product of a few-column pair launch (gemm_skinny_nn, blockIdx.z = 1): same B, N, K
+    const float *A_1, *bias_1;
+    float *C_1;
+    int64_t lda_1, ldc_1;
+    int M_1;
 };
 
 __device__ __forceinline__ float gelu_tanh(float x)
@@ -431,7 +436,11 @@ __global__ __launch_bounds__(256) void gemm_skinny_nn(GemmArgs g)
     __shared__ __attribute__((aligned(16))) float stage[4][8 * AST + 32 * BST];
     __shared__ float red[3][16 * 64];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (blockIdx.z == 1) { // the pair's second product: its own A, C, bias and row count
+        g.A = g.A_1; g.C = g.C_1; g.bias = g.bias_1; g.lda = g.lda_1; g.ldc = g.ldc_1; g.M = g.M_1;
+    }
     const int m0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
+    if (m0 >= g.M) return; // (uniform: the grid covers the taller of the two products)
     const int kh = lane >> 5;
     const int ak = lane >> 3, am = (lane & 7) * 4; // this lane's k row and first of four rows m of the A slab
     const int bn = lane >> 1, bk = (lane & 1) * 4; // this lane's column and first of four k of the B slab
@@ -1328,6 +1337,36 @@ extern "C" void nchip_gemm_force_config(int cfg)
 extern "C" void nchip_gemm_few_columns_kernel(int on)
 {
     g_skinny = on;
+}
+
+// Two width-invariant few-column products with one operand in common, in ONE launch:
+// C0 (m0 x n) = A0 B + bias0 and C1 (m1 x n) = A1 B + bias1 (bias pointers may be NULL),
+// the decoder's query and key/value projections of a timestep.  Same kernel and the same
+// bits as two nchip_gemm calls in width-invariant mode.  Returns 1 when the shapes are not
+// the few-column kernel's (nothing launched: the caller issues the two products itself).
+extern "C" int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, int k,
+                                           const float *A0, int64_t lda0, const float *A1, int64_t lda1,
+                                           const float *B, int64_t ldb,
+                                           float *C0, int64_t ldc0, float *C1, int64_t ldc1,
+                                           const float *bias0, const float *bias1)
+{
+    if (m0 <= 0 || m1 <= 0 || n <= 0 || !A0 || !A1 || !B || !C0 || !C1) return -1;
+    if (!g_skinny || g_prof_on || n > 64 || k < 32 || k % 32 || m0 % 32 || m1 % 32 || lda0 % 4 || lda1 % 4 || ldb % 4 ||
+        lda0 < m0 || lda1 < m1 || ldb < k || ldc0 < m0 || ldc1 < m1 ||
+        (((uintptr_t)A0 | (uintptr_t)A1 | (uintptr_t)B) & 15) != 0)
+        return 1;
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.A = A0; g.B = B; g.C = C0; g.bias = bias0; g.lda = lda0; g.ldb = ldb; g.ldc = ldc0;
+    g.M = m0; g.N = n; g.K = k; g.batch = 1; g.batch_in = 1; g.ksplit = 1; g.alpha = 1.0f;
+    g.A_1 = A1; g.C_1 = C1; g.bias_1 = bias1; g.lda_1 = lda1; g.ldc_1 = ldc1; g.M_1 = m1;
+    const int mt = (m0 > m1 ? m0 : m1) / 32;
+    hipLaunchKernelGGL(gemm_skinny_nn<16>, dim3(mt, (n + 31) / 32, 2), dim3(256), 0, (hipStream_t)stream, g);
+    if (hipGetLastError() != hipSuccess) {
+        fprintf(stderr, "nchip_gemm_pair_few_columns: launch failed\n");
+        return -2;
+    }
+    return 0;
 }
 
 // 0: bf16 products always round their operands inside the tile loader;

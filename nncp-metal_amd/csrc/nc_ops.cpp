@@ -732,6 +732,47 @@ extern "C" NCTensor *nc_linear_add(NCTensor *w, NCTensor *x, NCTensor *bias, int
     return linear_impl(w, x, bias, act, res);
 }
 
+// nc_ext.h: the two projections of one decoder timestep in one launch.  Returns w0 x + bias0
+// and writes w1 x into slice `index` of the last axis of dst.  No gradient.
+extern "C" NCTensor *nc_linear_pair_into(NCTensor *w0, NCTensor *bias0, NCTensor *w1, NCTensor *x,
+                                         NCTensor *dst, int index)
+{
+    w0 = nc_contig(w0); w1 = nc_contig(w1); x = nc_contig(x);
+    need_f32(w0, "nc_linear_pair_into"); need_f32(w1, "nc_linear_pair_into"); need_f32(x, "nc_linear_pair_into");
+    need_f32(dst, "nc_linear_pair_into");
+    if (bias0) { bias0 = nc_contig(bias0); need_f32(bias0, "nc_linear_pair_into"); }
+    NCContext *m = nc_ctx(w0);
+    if (w0->n_dims != 2 || w1->n_dims != 2 || x->n_dims != 2 || w0->dims[1] != x->dims[0] || w1->dims[1] != x->dims[0])
+        nc_fatal("nc_linear_pair_into: w0 (m0, k), w1 (m1, k) and x (k, n) expected");
+    const size_t m0 = w0->dims[0], m1 = w1->dims[0], k = x->dims[0], n = x->dims[1];
+    if (dst->n_dims != 3 || dst->dims[0] != m1 || dst->dims[1] != n || index < 0 || (size_t)index >= dst->dims[2] ||
+        !nc_is_contig(dst))
+        nc_fatal("nc_linear_pair_into: dst must be a contiguous (m1, n, T) tensor and 0 <= index < T");
+    if (bias0 && nc_numel(bias0) != m0) nc_fatal("nc_linear_pair_into: bias0 must have m0 elements");
+    size_t dims[2] = { m0, n };
+    NCTensor *y0 = new_f32(w0, 2, dims);
+    float *slot = nc_f32(dst) + (size_t)index * m1 * n;
+    int rc = 1;
+    if (m->matmul_invariant && !m->matmul_bf16)
+        rc = nchip_gemm_pair_few_columns(m->stream, (int)m0, (int)m1, (int)n, (int)k, nc_f32(w0), (int64_t)m0,
+                                         nc_f32(w1), (int64_t)m1, nc_f32(x), (int64_t)k, nc_f32(y0), (int64_t)m0,
+                                         slot, (int64_t)m1, bias0 ? nc_f32(bias0) : nullptr, nullptr);
+    if (rc < 0) nc_fatal("nc_linear_pair_into: kernel rejected the shapes");
+    if (rc == 0) {
+        m->launches++;
+    } else {
+        // other shapes and modes: the two products one after the other (the second one
+        // writes its columns straight into the slot: ldc = m1)
+        dev_gemm(m, false, false, m0, n, k, 1.0f, w0, x, 0.0f, y0, 1, bias0 ? nc_f32(bias0) : nullptr, 0, nullptr, nullptr, true);
+        NCTensor *view = nc_slice_alias(dst, 2, (size_t)index, (size_t)index + 1);
+        view = nc_reshape_2d(view, m1, n);
+        dev_gemm(m, false, false, m1, n, k, 1.0f, w1, x, 0.0f, view, 1, nullptr, 0, nullptr, nullptr, true);
+        nc_free_tensor(view);
+    }
+    nc_free_tensor(w0); nc_free_tensor(bias0); nc_free_tensor(w1); nc_free_tensor(x);
+    return y0;
+}
+
 // ---- embedding, softmax, loss, norms ----------------------------------------
 extern "C" NCTensor *nc_get_col(NCTensor *w, NCTensor *x) // libnc.h:374-375
 {

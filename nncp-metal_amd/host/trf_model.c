@@ -656,7 +656,7 @@ NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
     for (int l = 0; l < c->n_layer; l++) {
         Layer *tl = &s->layers[l];
         Layer *pr = &s->layers[c->tied_w_r ? 0 : l], *pb = &s->layers[c->tied_b_r ? 0 : l];
-        NCTensor *x1 = nc_dup_tensor(x), *ff_in, *q, *kv, *att;
+        NCTensor *x1 = nc_dup_tensor(x), *ff_in, *q, *att;
         if (c->ln_flags & NNCP_LN_PRE)
             x1 = layer_norm(s, x1, tl->ln_g1, tl->ln_b1);
         if (t == 0 && c->mem_len > 0) { /* K/V of the memory: once per segment */
@@ -664,11 +664,10 @@ NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
             m2 = nc_matmul(nc_dup_tensor(tl->w_kv), m2);
             s->step_kvm[l] = nc_reshape_3d(m2, HDk + HDv, B, c->mem_len);
         }
-        q = nc_linear(nc_dup_tensor(tl->w_q), nc_dup_tensor(x1), c->query_bias ? nc_dup_tensor(tl->b_q) : NULL, NC_ACT_NONE);
-        kv = nc_matmul(nc_dup_tensor(tl->w_kv), x1);
-        kv = nc_reshape_3d(kv, HDk + HDv, B, 1);
-        nc_tensor_copy_slice(s->step_kv[l], kv, 2, t, t + 1, 0);
-        nc_free_tensor(kv);
+        /* query and key / value of this position in one launch; the latter goes straight into
+           column t of the cache */
+        q = nc_linear_pair_into(nc_dup_tensor(tl->w_q), c->query_bias ? nc_dup_tensor(tl->b_q) : NULL,
+                                nc_dup_tensor(tl->w_kv), x1, s->step_kv[l], t);
         att = nc_relpos_attention_step(q, nc_dup_tensor(s->step_kv[l]),
                                        c->mem_len > 0 ? nc_dup_tensor(s->step_kvm[l]) : NULL,
                                        c->use_w_r ? nc_dup_tensor(pr->w_r) : NULL, nc_dup_tensor(pb->b_r),

@@ -152,6 +152,24 @@ NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv_mem,
 
 /* one query position: the whole-segment routine on a query tensor that holds
    the query in column t, then that column of the result (see nc_ext.h) */
+/* nc_ext.h: the decoder's two projections of a timestep, stated with the plain ops: the first
+   result is nc_matmul + bias, the second goes into slice `index` of dst. */
+NCTensor *nc_linear_pair_into(NCTensor *w0, NCTensor *bias0, NCTensor *w1, NCTensor *x,
+                              NCTensor *dst, int index)
+{
+    NCTensor *y0, *y1;
+    if (dst->n_dims != 3 || index < 0 || (size_t)index >= dst->dims[2])
+        nc_fatal("nc_linear_pair_into: dst must be (m1, n, T) and 0 <= index < T");
+    y0 = nc_matmul(w0, nc_dup_tensor(x));
+    if (bias0)
+        y0 = nc_add(y0, bias0);
+    y1 = nc_matmul(w1, x);
+    y1 = nc_reshape_3d(y1, y1->dims[0], y1->dims[1], 1);
+    nc_tensor_copy_slice(dst, y1, 2, index, index + 1, 0);
+    nc_free_tensor(y1);
+    return y0;
+}
+
 NCTensor *nc_relpos_attention_step(NCTensor *q, NCTensor *kv_cache, NCTensor *kv_mem,
                                    NCTensor *w_r, NCTensor *b_r, int n_head, int d_key,
                                    int attn_len, float b_r_scale, int t)

@@ -102,6 +102,37 @@ def test_few_column_products_are_the_wide_products_columns(hip, rng, m, k, n):
     assert relerr(few[0], ref64) <= TOL
 
 
+@pytest.mark.parametrize("m0,m1,k,n,T", [(512, 1024, 512, 32, 4), (64, 96, 64, 5, 3), (40, 24, 19, 3, 2)])
+def test_projection_pair_of_a_timestep(hip, ref, rng, m0, m1, k, n, T):
+    """nc_linear_pair_into: the query projection and the key / value projection of one decoder
+    timestep in one launch, the second written into its cache slot.  In width-invariant mode
+    the values are the bits of nc_linear and nc_matmul; in every mode they match the checker,
+    and the other slots of the cache are left alone."""
+    w0 = rng.standard_normal((k, m0)).astype(np.float32)
+    w1 = rng.standard_normal((k, m1)).astype(np.float32)
+    b0 = rng.standard_normal(m0).astype(np.float32)
+    x = rng.standard_normal((n, k)).astype(np.float32)
+    cache = rng.standard_normal((T, n, m1)).astype(np.float32)
+    outs = {}
+    for name, nc, inv in (("inv", hip, 1), ("plain", hip, 0), ("ref", ref, 0)):
+        if nc is hip:
+            nc.nc_set_matmul_width_invariant(nc.ctx, inv)
+        dst = nc.tensor(cache)
+        q = nc.nc_linear_pair_into(nc.tensor(w0), nc.tensor(b0), nc.tensor(w1), nc.tensor(x), dst, T - 1)
+        outs[name] = (nc.numpy(q, free=True), nc.numpy(dst, free=True))
+        if nc is hip and inv:
+            outs["two"] = (nc.numpy(nc.nc_linear(nc.tensor(w0), nc.tensor(x), nc.tensor(b0), 0), free=True),
+                           nc.numpy(nc.nc_matmul(nc.tensor(w1), nc.tensor(x)), free=True))
+        if nc is hip:
+            nc.nc_set_matmul_width_invariant(nc.ctx, 0)
+    assert np.array_equal(outs["inv"][0], outs["two"][0])
+    assert np.array_equal(outs["inv"][1][T - 1], outs["two"][1])
+    for name in ("inv", "plain"):
+        assert relerr(outs[name][0], outs["ref"][0]) <= TOL
+        assert relerr(outs[name][1][T - 1], outs["ref"][1][T - 1]) <= TOL
+        assert np.array_equal(outs[name][1][:T - 1], cache[:T - 1])
+
+
 def test_gemm_bf16_variant(hip, ref, rng):
     w = rng.standard_normal((256, 320)).astype(np.float32)
     x = rng.standard_normal((200, 256)).astype(np.float32)
