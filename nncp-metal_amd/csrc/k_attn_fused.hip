@@ -86,6 +86,21 @@ __device__ __forceinline__ void put_rows(float *dst, const floatx4_t (&v)[ROWS *
     }
 }
 
+// a slice [it0, it1) of put_rows' stores, for callers that spread a tile's stores over a loop
+template <int DK, int ROWS>
+__device__ __forceinline__ void put_rows_part(float *dst, const floatx4_t (&v)[ROWS * (DK / 4) / 256], int rows_valid,
+                                              int it0, int it1)
+{
+    constexpr int RS = DK + 4, C4 = DK / 4;
+#pragma unroll
+    for (int it = 0; it < ROWS * C4 / 256; it++) {
+        if (it < it0 || it >= it1) continue;
+        int idx = threadIdx.x + it * 256;
+        int row = idx / C4, c = (idx % C4) * 4;
+        *reinterpret_cast<floatx4_t *>(dst + row * RS + c) = row < rows_valid ? v[it] : floatx4_t{ 0, 0, 0, 0 };
+    }
+}
+
 // Optional per-phase shader-clock stamps of one workgroup (debug builds only).
 #ifdef NCHIP_ATTN_PHASE_CLOCKS
 __device__ long long *g_phase_clk = nullptr;
@@ -213,11 +228,18 @@ void relpos_attn_fwd_fused(FusedAttnFwdArgs a)
                 Rw[(2 * pp) * 16 + 4 * g + r] = acc0[r];
                 Rw[(2 * pp + 1) * 16 + 4 * g + r] = acc1[r];
             }
+            // K and V are parked in their own regions a slice per tile pair, under the MFMAs of
+            // the next pair (they arrive during this phase; the key slices come first, in load order)
+            constexpr int NV = KR * (DK / 4) / 256, PER = (2 * NV + NT / 2 - 1) / (NT / 2);
+#pragma unroll
+            for (int e = 0; e < PER; e++) {
+                const int u = pp * PER + e; // 0 .. 2 NV - 1: first the key stores, then the value stores
+                if (u < NV) put_rows_part<DK, KR>(Ks, vk, a.K, u, u + 1);
+                else if (u < 2 * NV) put_rows_part<DK, KR>(Vs, vv, a.K, u - NV, u - NV + 1);
+            }
         }
         wave_lds_sync();
     }
-    put_rows<DK, KR>(Ks, vk, a.K);
-    put_rows<DK, KR>(Vs, vv, a.K); // (its own region: parked here, while no store is in flight behind it)
     __syncthreads();
     PHASE_MARK(2);
 
