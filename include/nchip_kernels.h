@@ -114,6 +114,19 @@ int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launch
    choice.  The environment variable NCHIP_GEMM_CFG sets the initial value. */
 void nchip_gemm_force_config(int cfg);
 
+/* nchip_gemm_dact that also leaves partial row sums of C (the bias gradient of the layer whose
+   pre-activation gradient C is): `rowsum` holds nchip_gemm_rowsum_rows(n) rows of m floats;
+   *rows_written of them are written, row p = the sum over 16 consecutive columns of C (columns
+   past n count as zero), so their sum in row order is the row sum of C.  *rows_written is 0
+   when the kernel chosen for this product does not write them (split-K, bf16 operand copies):
+   the caller then sums C itself. */
+int nchip_gemm_rowsum_rows(int n);
+int nchip_gemm_dact_rowsum(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                           const float *A, int64_t lda, const float *B, int64_t ldb,
+                           float *C, int64_t ldc, const float *pre_act, int act,
+                           int precision, int ksplit, float *workspace,
+                           float *rowsum, int *rows_written);
+
 /* Two width-invariant fp32 products that share their right operand, in one launch:
    C0 (m0 x n) = A0 (m0 x k) B (k x n) + bias0 and C1 (m1 x n) = A1 (m1 x k) B + bias1, column
    major, untransposed, bias pointers may be NULL (the per-timestep query and key/value
@@ -219,6 +232,20 @@ int nchip_norm_bwd_rows(int d, int64_t n);
 int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float *rstd,
                    const float *w, float *dx, const float *dx_add, float *dw, float *db,
                    float *partial, int d, int64_t n, int avg);
+
+/* nchip_norm_bwd that also leaves partial row sums of the dx it writes (the bias gradient of
+   a linear layer whose output went straight into this norm): dx_partial holds
+   nchip_norm_bwd_rows(d, n) rows of d floats, their sum in row order is the sum of dx over
+   its n columns.  Only for the widths nchip_norm_bwd_has_dx_rowsum() names; NULL = plain
+   nchip_norm_bwd. */
+#ifdef __cplusplus
+bool nchip_norm_bwd_has_dx_rowsum(int d);
+#else
+_Bool nchip_norm_bwd_has_dx_rowsum(int d);
+#endif
+int nchip_norm_bwd_rowsum(void *stream, const float *g, const float *xhat, const float *rstd,
+                          const float *w, float *dx, const float *dx_add, float *dw, float *db,
+                          float *partial, int d, int64_t n, int avg, float *dx_partial);
 
 /* nchip_norm_bwd for callers that cannot allocate device memory (code under HIP graph
    capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the

@@ -63,6 +63,7 @@ struct GemmArgs {
     int dbg;
     const NchipGemmProblem *grp; // grouped launch: one problem per table row
     int n_grp;
+    float *rowsum; // activation-gradient epilogue only: partial row sums of the result, one row per (tile column, wavefront column, lane half)
     // second product of a few-column pair launch (gemm_skinny_nn, blockIdx.z = 1): same B, N, K
     const float *A_1, *bias_1;
     float *C_1;
@@ -347,7 +348,7 @@ struct TileLoaderBf16Src {
 __device__ __forceinline__ void epilogue_tile(const GemmArgs &g, const floatx16 &acc, int m, int nb,
                                               float NCHIP_GLOBAL *C, float NCHIP_GLOBAL *P,
                                               const float NCHIP_GLOBAL *Radd, const float NCHIP_GLOBAL *Dp,
-                                              bool full, bool plain)
+                                              bool full, bool plain, float NCHIP_GLOBAL *rowsum = nullptr)
 {
     if (!full && m >= g.M) return;
     float NCHIP_GLOBAL *Cp = C + (int64_t)nb * g.ldc + m; // element r lives at Cp + nofs(r)*ldc
@@ -405,6 +406,12 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs &g, const floatx16 
 #pragma unroll
         for (int r = 0; r < 16; r++)
             if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r];
+        if (rowsum) { // this lane's 16 columns of row m, in column order: one entry of a partial row
+            float sum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) sum += ok[r] ? v[r] : 0.0f;
+            rowsum[m] = sum;
+        }
         return;
     }
 #pragma unroll
@@ -949,7 +956,10 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     for (int i = 0; i < TN; i++)
 #pragma unroll
         for (int j = 0; j < TM; j++) {
-            epilogue_tile(g, acc[i][j], mm_base + j * 32, nn_base + i * 32, C, P, Radd, Dp, full, plain);
+            float NCHIP_GLOBAL *rs = nullptr;
+            if (g.rowsum) // partial row of this (tile column, wavefront column, accumulator column, lane half)
+                rs = as_global(g.rowsum) + (int64_t)((((tile_n * WN + wn) * TN + i) * 2) + (lane >> 5)) * g.M;
+            epilogue_tile(g, acc[i][j], mm_base + j * 32, nn_base + i * 32, C, P, Radd, Dp, full, plain, rs);
         }
 #ifdef NCHIP_GEMM_CLOCKS
     if (g_gemm_clk && blockIdx.y == 0 && t == 0) g_gemm_clk[6 + 3 * blockIdx.x] = wall_clock64(); // stores issued
@@ -1138,8 +1148,10 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
                       float beta, float *C, int64_t ldc, int64_t sc_out, int64_t sc_in,
                       int batch, int batch_in,
                       const float *bias, int act, float *pre, const float *addend, int precision,
-                      int ksplit, float *workspace, const float *dpre = nullptr, int dact = 0)
+                      int ksplit, float *workspace, const float *dpre = nullptr, int dact = 0,
+                      float *rowsum = nullptr, int *rowsum_rows = nullptr)
 {
+    if (rowsum_rows) *rowsum_rows = 0;
     if (m <= 0 || n <= 0 || batch <= 0)
         return 0;
     if (k < 0 || !A || !B || !C || lda < (ta ? k : m) || ldb < (tb ? n : k) || ldc < m || batch_in < 1) {
@@ -1161,6 +1173,7 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     GemmArgs g;
     g.A = A; g.B = B; g.C = C; g.bias = bias; g.add = addend; g.pre = pre; g.ws = workspace;
     g.dpre = dpre; g.dact = dact;
+    g.rowsum = nullptr;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.sa = sa_out; g.sb = sb_out; g.sc = sc_out;
     g.sa_in = sa_in; g.sb_in = sb_in; g.sc_in = sc_in; g.batch_in = batch_in;
     g.M = m; g.N = n; g.K = k; g.batch = batch; g.ksplit = ksplit;
@@ -1224,6 +1237,14 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
             g.K = kpad; g.kchunk = kpad;
             from_bf16 = true;
         }
+    }
+    // partial row sums of the result (activation-gradient epilogue): one row per 16 columns of
+    // the padded column range; only the plain tile classes write them
+    if (rowsum && rowsum_rows && dpre && ksplit == 1 && batch == 1 && !from_bf16 &&
+        (cfg == 7 || cfg == 4 || cfg == 10 || cfg == 30)) {
+        const int bn = cfg == 7 ? 128 : 64;
+        g.rowsum = rowsum;
+        *rowsum_rows = (n + bn - 1) / bn * bn / 16;
     }
     if (from_bf16) {
         // 64x64 per wavefront, 64-deep tiles: with enough tiles for two workgroups
@@ -1312,6 +1333,21 @@ extern "C" int nchip_gemm_dact(void *stream, int ta, int tb, int m, int n, int k
 {
     return gemm2_impl(stream, ta, tb, m, n, k, alpha, A, lda, 0, 0, B, ldb, 0, 0, 0.0f, C, ldc, 0, 0, 1, 1,
                       nullptr, 0, nullptr, nullptr, precision, ksplit, workspace, pre_act, act);
+}
+
+// nchip_gemm_dact that also leaves partial row sums of C: rowsum holds nchip_gemm_rowsum_rows(n)
+// rows of m floats, of which *rows_written are written (row p = the sum over 16 columns of C;
+// 0 when this product's kernel does not write them: the caller then sums C itself)
+extern "C" int nchip_gemm_rowsum_rows(int n) { return (n + 127) / 128 * 8; }
+
+extern "C" int nchip_gemm_dact_rowsum(void *stream, int ta, int tb, int m, int n, int k, float alpha,
+                                      const float *A, int64_t lda, const float *B, int64_t ldb,
+                                      float *C, int64_t ldc, const float *pre_act, int act,
+                                      int precision, int ksplit, float *workspace,
+                                      float *rowsum, int *rows_written)
+{
+    return gemm2_impl(stream, ta, tb, m, n, k, alpha, A, lda, 0, 0, B, ldb, 0, 0, 0.0f, C, ldc, 0, 0, 1, 1,
+                      nullptr, 0, nullptr, nullptr, precision, ksplit, workspace, pre_act, act, rowsum, rows_written);
 }
 
 extern "C" int nchip_gemm(void *stream, int ta, int tb, int m, int n, int k, float alpha,

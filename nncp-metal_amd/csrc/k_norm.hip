@@ -147,14 +147,15 @@ __global__ __launch_bounds__(TPB) void norm_bwd_wb_stage1(const float *g, const 
 template <int NV>
 __global__ __launch_bounds__(TPB) void norm_bwd_fused(const float *g, const float *xhat, const float *rstd,
                                                       const float *w, float *dx, const float *dx_add,
-                                                      float *partial, int64_t n, int avg, int cw)
+                                                      float *partial, int64_t n, int avg, int cw,
+                                                      float *dx_partial)
 {
     constexpr int D = NV * 64;
-    __shared__ float sh[WPB - 1][2][D];
+    __shared__ float sh[WPB - 1][3][D];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    float wr[NV], aw[NV], ab[NV];
+    float wr[NV], aw[NV], ab[NV], ax[NV]; // ax: row sums of the dx written (dx_partial)
 #pragma unroll
-    for (int v = 0; v < NV; v++) { wr[v] = w ? w[lane + 64 * v] : 1.0f; aw[v] = 0.0f; ab[v] = 0.0f; }
+    for (int v = 0; v < NV; v++) { wr[v] = w ? w[lane + 64 * v] : 1.0f; aw[v] = 0.0f; ab[v] = 0.0f; ax[v] = 0.0f; }
     const int64_t c0 = ((int64_t)blockIdx.x * WPB + wv) * cw;
     for (int k = 0; k < cw; k++) {
         const int64_t c = c0 + k;
@@ -178,25 +179,40 @@ __global__ __launch_bounds__(TPB) void norm_bwd_fused(const float *g, const floa
 #pragma unroll
             for (int v = 0; v < NV; v++) {
                 float val = r * (gv[v] * wr[v] - s1 - hv[v] * s2);
-                dx[c * D + lane + 64 * v] = dx_add ? dx_add[c * D + lane + 64 * v] + val : val;
+                val = dx_add ? dx_add[c * D + lane + 64 * v] + val : val;
+                dx[c * D + lane + 64 * v] = val;
+                ax[v] += val;
             }
         }
     }
-    if (!partial) return;
+    if (!partial && !dx_partial) return;
     if (wv > 0) {
 #pragma unroll
-        for (int v = 0; v < NV; v++) { sh[wv - 1][0][lane + 64 * v] = aw[v]; sh[wv - 1][1][lane + 64 * v] = ab[v]; }
+        for (int v = 0; v < NV; v++) {
+            sh[wv - 1][0][lane + 64 * v] = aw[v]; sh[wv - 1][1][lane + 64 * v] = ab[v]; sh[wv - 1][2][lane + 64 * v] = ax[v];
+        }
     }
     __syncthreads();
     if (wv == 0) {
-        float *pw = partial + (int64_t)blockIdx.x * 2 * D, *pb = pw + D;
+        if (partial) {
+            float *pw = partial + (int64_t)blockIdx.x * 2 * D, *pb = pw + D;
 #pragma unroll
-        for (int v = 0; v < NV; v++) {
-            float a = aw[v], b = ab[v];
+            for (int v = 0; v < NV; v++) {
+                float a = aw[v], b = ab[v];
 #pragma unroll
-            for (int u = 0; u < WPB - 1; u++) { a += sh[u][0][lane + 64 * v]; b += sh[u][1][lane + 64 * v]; }
-            pw[lane + 64 * v] = a;
-            pb[lane + 64 * v] = b;
+                for (int u = 0; u < WPB - 1; u++) { a += sh[u][0][lane + 64 * v]; b += sh[u][1][lane + 64 * v]; }
+                pw[lane + 64 * v] = a;
+                pb[lane + 64 * v] = b;
+            }
+        }
+        if (dx_partial) { // row blockIdx.x of the partial row sums of dx, wavefronts in order
+#pragma unroll
+            for (int v = 0; v < NV; v++) {
+                float a = ax[v];
+#pragma unroll
+                for (int u = 0; u < WPB - 1; u++) a += sh[u][2][lane + 64 * v];
+                dx_partial[(int64_t)blockIdx.x * D + lane + 64 * v] = a;
+            }
         }
     }
 }
@@ -474,11 +490,24 @@ int nchip_norm_bwd_rows(int d, int64_t n)
     return (int)(n / 16 > 32 ? 32 : (n / 16 < 1 ? 1 : n / 16));
 }
 
+bool nchip_norm_bwd_has_dx_rowsum(int d) { return d == 128 || d == 256 || d == 512 || d == 1024; }
+
 int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float *rstd, const float *w,
                    float *dx, const float *dx_add, float *dw, float *db, float *partial, int d, int64_t n,
                    int avg)
 {
+    return nchip_norm_bwd_rowsum(stream, g, xhat, rstd, w, dx, dx_add, dw, db, partial, d, n, avg, nullptr);
+}
+
+int nchip_norm_bwd_rowsum(void *stream, const float *g, const float *xhat, const float *rstd, const float *w,
+                          float *dx, const float *dx_add, float *dw, float *db, float *partial, int d, int64_t n,
+                          int avg, float *dx_partial)
+{
     if (n <= 0 || d <= 0) return 0;
+    if (dx_partial && (!dx || !nchip_norm_bwd_has_dx_rowsum(d))) {
+        fprintf(stderr, "nchip_norm_bwd_rowsum: row sums of dx need dx and d in {128, 256, 512, 1024}\n");
+        return -1;
+    }
     hipStream_t st = (hipStream_t)stream;
     const bool wb = dw || db;
     if (wb && !partial) { fprintf(stderr, "nchip_norm_bwd: partial buffer missing\n"); return -1; }
@@ -487,7 +516,7 @@ int nchip_norm_bwd(void *stream, const float *g, const float *xhat, const float 
         const int cw = norm_bwd_cw(n);
         const int rows = nchip_norm_bwd_rows(d, n);
         float *pp = partial;
-#define NORM_BWD(NV) hipLaunchKernelGGL(norm_bwd_fused<NV>, dim3(rows), dim3(TPB), 0, st, g, xhat, rstd, w, dx, dx_add, pp, n, avg, cw)
+#define NORM_BWD(NV) hipLaunchKernelGGL(norm_bwd_fused<NV>, dim3(rows), dim3(TPB), 0, st, g, xhat, rstd, w, dx, dx_add, pp, n, avg, cw, dx_partial)
         if (d == 128) NORM_BWD(2); else if (d == 256) NORM_BWD(4); else if (d == 512) NORM_BWD(8); else NORM_BWD(16);
 #undef NORM_BWD
         if (wb)

@@ -156,6 +156,12 @@ struct NCNode {
     int pending = 0;
     int consumers = 0; // edges into this node in the current backward walk
     int mark = 0;
+    // Partial row sums of the gradient this node is about to receive, left by the kernel that
+    // produced that gradient (rows x n floats from the scratch pool): the node's backward step
+    // takes its bias gradient from them instead of summing the gradient again.
+    float *grad_rowsum = nullptr;
+    size_t grad_rowsum_cap = 0;
+    int grad_rowsum_rows = 0;
 };
 
 // nc_core.cpp

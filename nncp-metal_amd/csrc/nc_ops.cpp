@@ -665,11 +665,23 @@ static void matmul_bw(NCNode *nd, NCTensor *g, NCTensor **ga, int ia, int ib)
             int ks = nchip_gemm_pick_ksplit((int)s.k, (int)s.n, (int)s.m, 1);
             size_t cap = 0;
             float *ws = ks > 1 ? nc_tmp_f32(m, (size_t)ks * s.k * s.n, &cap) : nullptr;
-            if (nchip_gemm_dact(m->stream, !ta, 0, (int)s.k, (int)s.n, (int)s.m, alpha,
-                                nc_f32(a), (int64_t)(!ta ? s.m : s.k), nc_f32(g), (int64_t)s.m,
-                                nc_f32(db), (int64_t)s.k, nc_f32(px->saved[2]), px->ia[3],
-                                m->matmul_bf16, ks, ws))
+            // px's bias gradient is the row sum of this product: its partial sums come out of
+            // the same epilogue when px's bias can wait for the batched sum at the end
+            float *rs = nullptr;
+            size_t rs_cap = 0;
+            int rs_rows = 0;
+            if (px->n_args > 2 && px->parents.size() > 2 && px->parents[2] && nc_can_defer_sum(m, px->parents[2]) && ks == 1)
+                rs = nc_tmp_f32(m, (size_t)nchip_gemm_rowsum_rows((int)s.n) * s.k, &rs_cap);
+            if (nchip_gemm_dact_rowsum(m->stream, !ta, 0, (int)s.k, (int)s.n, (int)s.m, alpha,
+                                       nc_f32(a), (int64_t)(!ta ? s.m : s.k), nc_f32(g), (int64_t)s.m,
+                                       nc_f32(db), (int64_t)s.k, nc_f32(px->saved[2]), px->ia[3],
+                                       m->matmul_bf16, ks, ws, rs, &rs_rows))
                 nc_fatal("gemm failed (activation-gradient epilogue)");
+            if (rs && rs_rows > 0) {
+                px->grad_rowsum = rs; px->grad_rowsum_cap = rs_cap; px->grad_rowsum_rows = rs_rows;
+            } else if (rs) {
+                nc_tmp_free(m, rs, rs_cap);
+            }
             if (ws) nc_tmp_free(m, ws, cap);
             m->launches += ks > 1 ? 2 : 1;
             px->ia[5] = 1; // the gradient delivered to px is already d(pre-activation)
@@ -1398,11 +1410,21 @@ void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
             gz = t;
         }
         matmul_bw(nd, gz, ga, 0, 1);
-        if (nd->parents[2]) {
+        if (nd->parents[2] && nd->grad_rowsum && (already || nd->ia[3] == NC_ACT_NONE)) {
+            // the kernel that produced gz left its partial row sums: they join the batched sum
+            size_t nb = nd->saved[0]->dims[0];
+            NCTensor *dbias = nc_alloc(g->dev, NC_TYPE_F32, 1, &nb, false);
+            defer_sum(m, nd->grad_rowsum, dbias, nd->grad_rowsum_rows, (int64_t)nb, (int)nb, nd->parents[2]);
+            DeferredTmp dt = { nd->grad_rowsum, nd->grad_rowsum_cap };
+            m->deferred_tmp.push_back(dt);
+            nd->grad_rowsum = nullptr;
+            ga[2] = dbias;
+        } else if (nd->parents[2]) {
             Shape bs;
             bs.nd = 1; bs.d[0] = nd->saved[0]->dims[0];
             ga[2] = dev_unbroadcast(nc_dup_tensor(gz), bs, nd->parents[2]);
         }
+        if (nd->grad_rowsum) { nc_tmp_free(m, nd->grad_rowsum, nd->grad_rowsum_cap); nd->grad_rowsum = nullptr; }
         nc_free_tensor(gz);
         break;
     }
@@ -1448,10 +1470,22 @@ void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
         // dw / db that go straight to once-used parameters: their sums over the
         // partial rows join the batched sum at the end of nc_backward
         const bool late = dw && db && nc_can_defer_sum(m, nd->parents[1]) && nc_can_defer_sum(m, nd->parents[2]);
-        if (nchip_norm_bwd(st, nc_f32(g), nc_f32(xhat), nc_f32(rstd), w ? nc_f32(w) : nullptr,
-                           dx ? nc_f32(dx) : nullptr, prev, (dw && !late) ? nc_f32(dw) : nullptr,
-                           (db && !late) ? nc_f32(db) : nullptr, partial, d, cols, nd->ia[0]))
+        // the input came straight out of a linear layer with a bias (and feeds nothing else):
+        // that bias gradient is the row sum of dx, whose partial sums this kernel can leave
+        NCNode *pl = nd->parents[0];
+        float *dxp = nullptr;
+        size_t dxp_cap = 0;
+        if (dx && pl && pl->op == OP_LINEAR && pl->ia[3] == NC_ACT_NONE && pl->consumers == 1 && !pl->grad_rowsum &&
+            pl->parents.size() > 2 && pl->parents[2] && nc_can_defer_sum(m, pl->parents[2]) &&
+            nchip_norm_bwd_has_dx_rowsum(d) && pl->saved[0] && (int)pl->saved[0]->dims[0] == d)
+            dxp = nc_tmp_f32(m, (size_t)nchip_norm_bwd_rows(d, cols) * d, &dxp_cap);
+        if (nchip_norm_bwd_rowsum(st, nc_f32(g), nc_f32(xhat), nc_f32(rstd), w ? nc_f32(w) : nullptr,
+                                  dx ? nc_f32(dx) : nullptr, prev, (dw && !late) ? nc_f32(dw) : nullptr,
+                                  (db && !late) ? nc_f32(db) : nullptr, partial, d, cols, nd->ia[0], dxp))
             nc_fatal("layer norm backward failed");
+        if (dxp) {
+            pl->grad_rowsum = dxp; pl->grad_rowsum_cap = dxp_cap; pl->grad_rowsum_rows = nchip_norm_bwd_rows(d, cols);
+        }
         if (late) {
             const int rows = nchip_norm_bwd_rows(d, cols);
             defer_sum(m, partial, dw, rows, 2 * (int64_t)d, d, nd->parents[1]);
