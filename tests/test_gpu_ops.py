@@ -398,3 +398,62 @@ def test_bias_gradient_model_shapes(hip, ref, rng, f, n):
     exact = weight.astype(np.float64).sum(axis=0)
     assert relerr(gh[1], exact) <= TOL
     assert relerr(gh[1], gr[1]) <= 5 * TOL
+
+
+def _dev(nc, arr):
+    t = nc.tensor(np.ascontiguousarray(arr, dtype=np.float32))
+    return t, C.c_void_p(nc.lib.nc_tensor_get_ptr(t, None))
+
+
+@pytest.mark.parametrize("d,n", [(512, 2048), (128, 80), (1024, 333), (256, 5)])
+def test_norm_backward_leaves_the_row_sums_of_dx(hip, rng, d, n):
+    """nchip_norm_bwd_rowsum: the partial rows it leaves sum, in row order, to the sum of the dx
+    it wrote over the columns (what the bias gradient of the layer before the norm is), and dx
+    itself is the bits of the plain call."""
+    lib = C.CDLL(hip.lib._name)
+    st = C.c_void_p(hip.nc_context_stream(hip.ctx))
+    g = rng.standard_normal((n, d)); xhat = rng.standard_normal((n, d)); rstd = 0.5 + rng.random(n)
+    w = 1.0 + 0.1 * rng.standard_normal(d); add = rng.standard_normal((n, d))
+    rows = lib.nchip_norm_bwd_rows(C.c_int(d), C.c_int64(n))
+    t = {k: _dev(hip, v) for k, v in dict(g=g, xhat=xhat, rstd=rstd, w=w, add=add, dx_a=np.zeros((n, d)), dx_b=np.ones((n, d)),
+                                          part=np.full((rows, d), 7.0)).items()}
+    P = {k: v[1] for k, v in t.items()}
+    assert lib.nchip_norm_bwd(st, P["g"], P["xhat"], P["rstd"], P["w"], P["dx_a"], P["add"], None, None, None,
+                              C.c_int(d), C.c_int64(n), C.c_int(1)) == 0
+    assert lib.nchip_norm_bwd_rowsum(st, P["g"], P["xhat"], P["rstd"], P["w"], P["dx_b"], P["add"], None, None, None,
+                                     C.c_int(d), C.c_int64(n), C.c_int(1), P["part"]) == 0
+    dx_a, dx_b, part = (hip.numpy(t[k][0]) for k in ("dx_a", "dx_b", "part"))
+    hip.free(*[v[0] for v in t.values()])
+    assert np.array_equal(dx_a.view(np.uint32), dx_b.view(np.uint32))
+    want = dx_b.astype(np.float64).sum(axis=0)
+    assert relerr(part.astype(np.float64).sum(axis=0), want) <= 1e-6
+
+
+@pytest.mark.parametrize("m,n,k", [(2048, 1024, 64), (512, 2048, 128), (300, 70, 96), (128, 4100, 64)])
+def test_activation_gradient_product_leaves_its_row_sums(hip, rng, m, n, k):
+    """nchip_gemm_dact_rowsum: C = (A^T B) .* gelu'(pre) as nchip_gemm_dact computes it, plus
+    partial row sums of C whose total is the sum of C over its columns."""
+    lib = C.CDLL(hip.lib._name)
+    st = C.c_void_p(hip.nc_context_stream(hip.ctx))
+    A = rng.standard_normal((m, k)) * 0.1      # stored (k rows, m columns): op(A) = A^T is m x k
+    Bm = rng.standard_normal((n, k)) * 0.1     # (k, n)
+    pre = rng.standard_normal((n, m))
+    rows_cap = lib.nchip_gemm_rowsum_rows(C.c_int(n))
+    t = {key: _dev(hip, v) for key, v in dict(A=A, B=Bm, pre=pre, Ca=np.zeros((n, m)), Cb=np.ones((n, m)),
+                                              rs=np.full((rows_cap, m), 3.0)).items()}
+    P = {key: v[1] for key, v in t.items()}
+    NC_ACT_GELU = 1
+    i64, f32, ci = C.c_int64, C.c_float, C.c_int
+    assert lib.nchip_gemm_dact(st, ci(1), ci(0), ci(m), ci(n), ci(k), f32(1.0), P["A"], i64(k), P["B"], i64(k),
+                               P["Ca"], i64(m), P["pre"], ci(NC_ACT_GELU), ci(0), ci(1), None) == 0
+    written = C.c_int(-1)
+    assert lib.nchip_gemm_dact_rowsum(st, ci(1), ci(0), ci(m), ci(n), ci(k), f32(1.0), P["A"], i64(k), P["B"], i64(k),
+                                      P["Cb"], i64(m), P["pre"], ci(NC_ACT_GELU), ci(0), ci(1), None,
+                                      P["rs"], C.byref(written)) == 0
+    Ca, Cb, rs = (hip.numpy(t[key][0]) for key in ("Ca", "Cb", "rs"))
+    hip.free(*[v[0] for v in t.values()])
+    assert np.array_equal(Ca.view(np.uint32), Cb.view(np.uint32))
+    assert 0 < written.value <= rows_cap
+    want = Cb.astype(np.float64).sum(axis=0)
+    got = rs[:written.value].astype(np.float64).sum(axis=0)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(Cb).sum(axis=0).max()
