@@ -1,20 +1,24 @@
-// GEMM for gfx950 (MI355X): column-major C = act(alpha*op(A)*op(B) + beta*C + bias).
+// GEMM for gfx950 (MI355X): column-major C = act(alpha*op(A)*op(B) + beta*C + bias) [+ addend].
 //
-// One workgroup of 256 threads (4 wavefronts of 64 lanes, arranged 2x2) owns a
-// BM x BN tile of C.  A and B tiles of depth BK = 16 are staged through LDS
-// (double buffered, k-major rows so a wavefront reads 32 consecutive floats),
-// and every wavefront accumulates its (BM/2) x (BN/2) part with
-// v_mfma_f32_32x32x2_f32.  The MFMA is issued as D[n][m] = sum_k B[k][n]*A[k][m]
-// so that the 32 lanes of a half-wavefront hold 32 consecutive m of one column:
-// the epilogue stores are 128-byte coalesced in column-major C.
+// A workgroup of WM x WN wavefronts (times KW k groups) owns a BM x BN tile of C.  A and B
+// tiles of depth BK are staged through LDS (double buffered, PF register sets of tiles in
+// flight from global memory, k-major rows so a wavefront reads 32 consecutive floats), and
+// every wavefront accumulates its part with v_mfma_f32_32x32x2_f32.  The MFMA is issued as
+// D[n][m] = sum_k B[k][n]*A[k][m] so that the 32 lanes of a half-wavefront hold 32
+// consecutive m of one column: the epilogue stores are 128-byte coalesced in column-major C.
 //
-// Each C element is one sequential chain of MFMA accumulations over
-// k = 0, 2, 4, ... ; the chain does not depend on the tile shape, on m/n or on
-// the number of columns, so a column computed alone equals the same column
-// computed inside a larger matrix (needed for bit-exact decode).
+// Tile classes (chosen from the shape only): 128x128x32 with 8 wavefronts, 128x64x32 with 8
+// wavefronts, 64x64x32 with two k groups of 4 wavefronts (KW = 2: the groups split every
+// 32-deep slab, C = chain0 + chain1).  Inside a class a C element is a fixed sequence of MFMA
+// accumulations that does not depend on m, n or the number of columns.  The width-invariant
+// class (NCHIP_GEMM_WIDTH_INVARIANT: 64x64x32, KW = 2, two accumulator sets per group = four
+// chains per element, no split-K) is used by encoder and decoder alike when a column computed
+// alone must equal the same column computed inside a larger matrix (bit-exact decode);
+// gemm_skinny_nn issues the same sequence for products of a few columns.
 //
-// precision 1 rounds both operands to bf16 (nearest-even) while they are
-// written to LDS and feeds v_mfma_f32_32x32x16_bf16 (fp32 accumulate).
+// precision 1 rounds both operands to bf16 (nearest-even) while they are written to LDS and
+// feeds v_mfma_f32_32x32x16_bf16 (fp32 accumulate); large products go through bf16 copies of
+// the operands instead (cast_bf16_kernel + the BF16 = 2 tile kernels).
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 #include <stdint.h>
@@ -618,7 +622,8 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
 
     // PF register sets: while tile it is computed, tiles it+1 .. it+PF are landing
     // or in flight, so a load has PF compute phases to arrive.  Two sets are
-    // enough on MI355X: four or six measured no faster on any model shape.
+    // enough for the wide classes; the 64x64 class, whose tiles are consumed in
+    // half the time, keeps four.
     using LoaderA = std::conditional_t<BF16 == 2, TileLoaderBf16Src<BM, BK, TA ? 0 : 1, NT>,
                     std::conditional_t<BF16 == 1, TileLoaderBf16<BM, BK, TA ? 0 : 1, NT>, TileLoader<BM, BK, TA ? 0 : 1, NT>>>;
     using LoaderB = std::conditional_t<BF16 == 2, TileLoaderBf16Src<BN, BK, TB ? 1 : 0, NT>,
