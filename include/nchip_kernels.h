@@ -140,12 +140,14 @@ int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, int k,
                                 float *C0, int64_t ldc0, float *C1, int64_t ldc1,
                                 const float *bias0, const float *bias1);
 
-/* Testing aid: width-invariant fp32 products (NCHIP_GEMM_WIDTH_INVARIANT) with at most 64
-   columns, untransposed operands and beta = 0 run a register-streaming kernel that issues the
-   tile kernel's MFMA sequence without its LDS pipeline (the decoder's per-timestep products);
-   0 sends them through the tile kernel again, 1 (default) restores the choice.  The results
-   are the same bits either way. */
-void nchip_gemm_few_columns_kernel(int on);
+/* Testing aid: which kernel takes width-invariant fp32 products (NCHIP_GEMM_WIDTH_INVARIANT)
+   with at most 64 columns, untransposed operands and beta = 0 (the decoder's per-timestep
+   products).  2 (default): the vector-ALU kernel - an fp32 MFMA accumulates its k values one
+   after the other with fused multiply-adds, so the four chains of an element are formed by
+   plain fma instructions, one chain per thread, 8 x 8 outputs per workgroup; 1: the
+   few-column MFMA kernel (one 32-row tile per workgroup, its four wavefronts the four chains);
+   0: the tile kernel.  The results are the same bits in all three. */
+void nchip_gemm_few_columns_kernel(int kernel);
 
 /* Tuning aid: tiles are ordered, inside each XCD's run, in bands of `gm` tile
    rows (1 = plain column-major tile order; a negative value restores the
@@ -190,6 +192,12 @@ int nchip_relpos_attn_fwd_step(void *stream, const float *q, int64_t ldq,
                                const float *w_r, const float *b_r, float *out, int64_t ldo,
                                int H, int dk, int dv, int B, int T, int M, int d_pos,
                                int attn_len, float b_r_scale, int t);
+
+/* Testing aid for the call above: 1 (default) runs the one-query kernel on the vector ALUs
+   (fused multiply-add chains in the order the MFMAs of the whole-segment kernel accumulate),
+   0 runs the whole-segment kernel with every query row the one query.  Same bits.  No
+   counterpart in the reference. */
+void nchip_relpos_attn_step_kernel(int scalar);
 
 /* Kernel launches issued by the calling thread's last successful
    nchip_relpos_attn_fwd (1 when the head fits the single-kernel path). */

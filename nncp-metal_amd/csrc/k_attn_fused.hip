@@ -1167,6 +1167,136 @@ void relpos_attn_bwd_tiled(FusedAttnBwdArgs a)
     }
 }
 
+// ---- one query per (stream, head): the decoder's timestep ---------------------------------
+// The single query of a timestep through the arithmetic of relpos_attn_fwd_fused, on the
+// vector ALUs.  An fp32 MFMA accumulates its k values one after the other with fused
+// multiply-adds in increasing k, so every number of that kernel's column q_only can be
+// formed by plain code in the same order: the score of key j is a chain of DK fmas over the
+// features plus the position term (its own chain over w_r row d_pos-1-delta, clamped) plus the
+// scaled bias; the sum of the exponentials is taken the way the four lanes of a column hold
+// it (lane g: keys 16 jt + 4g + r in increasing order, then (s0 + s1) + (s2 + s3)); output
+// feature d is one chain over the keys in the order the PV MFMAs meet them (tile jt, step r,
+// k slot g: key 16 jt + 4g + r).  Masked keys contribute exact zeros there and are skipped.
+// A workgroup of 128 threads is one (stream, head): thread j owns key j (only keys inside
+// the attention window are fetched), then thread d owns output feature d.
+// a product that is rounded on its own (the whole-segment kernel keeps the scaled bias in
+// LDS, so no multiply-add can swallow it)
+__device__ __forceinline__ float rounded_product(float x, float y)
+{
+#pragma clang fp contract(off)
+    return x * y;
+}
+
+template <int DK>
+__global__ __launch_bounds__(128) void relpos_attn_step_scalar(FusedAttnFwdArgs a)
+{
+    constexpr int RS = DK + 4, NS = DK / 4;
+    __shared__ __attribute__((aligned(16))) float Vs[128 * RS];
+    __shared__ __attribute__((aligned(16))) float qs[DK];
+    __shared__ __attribute__((aligned(16))) float es[128];
+    __shared__ float red[4];
+    const int j = threadIdx.x;
+    const int b = blockIdx.x % a.B, h = blockIdx.x / a.B;
+    const int i = a.q_only;
+    const int delta = i + a.M - j;
+    const bool valid = j < a.K && (unsigned)delta < (unsigned)a.attn_len;
+    const bool has_w = a.w_r != nullptr;
+    floatx4_t kr[NS], vr[NS], wr[NS];
+    float bias_t = 0.0f;
+    if (valid) {
+        const float *row = (j < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * j)
+                                    : a.kv + a.ldkv * (b + (int64_t)a.B * (j - a.M))) + (int64_t)h * DK;
+        const floatx4_t NCHIP_GLOBAL *kp = reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(as_global(row));
+        const floatx4_t NCHIP_GLOBAL *vp = reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(as_global(row + (int64_t)a.H * DK));
+#pragma unroll
+        for (int s = 0; s < NS; s++) kr[s] = kp[s];
+        if (has_w) {
+            int pi = a.d_pos - 1 - delta;
+            pi = pi < 0 ? 0 : pi; // (delta >= 0: never above d_pos - 1)
+            const floatx4_t NCHIP_GLOBAL *wp = reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(
+                as_global(a.w_r + ((int64_t)h * a.d_pos + pi) * DK));
+#pragma unroll
+            for (int s = 0; s < NS; s++) wr[s] = wp[s];
+        }
+#pragma unroll
+        for (int s = 0; s < NS; s++) vr[s] = vp[s];
+        if (a.b_r) bias_t = as_global(a.b_r)[(int64_t)h * a.K + (a.K - 1 - delta)];
+    }
+    if (j < NS) {
+        floatx4_t q4 = *reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(as_global(a.q + (int64_t)h * DK + a.ldq * b) + 4 * j);
+#pragma unroll
+        for (int r = 0; r < 4; r++) qs[4 * j + r] = q4[r] * a.scale; // 1/sqrt(dk) folded in
+    }
+    __syncthreads();
+    float v = -INFINITY;
+    if (valid) {
+        float sc = 0.0f, rl = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const floatx4_t q4 = *reinterpret_cast<const floatx4_t *>(qs + 4 * s);
+#pragma unroll
+            for (int r = 0; r < 4; r++) sc = __builtin_fmaf(kr[s][r], q4[r], sc);
+            if (has_w) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) rl = __builtin_fmaf(wr[s][r], q4[r], rl);
+            }
+        }
+        v = sc + rl + rounded_product(bias_t, a.b_r_scale * a.scale);
+#pragma unroll
+        for (int s = 0; s < NS; s++) *reinterpret_cast<floatx4_t *>(Vs + j * RS + 4 * s) = vr[s];
+    } else { // a masked key's probability is an exact zero: its value row must only be finite
+#pragma unroll
+        for (int s = 0; s < NS; s++) *reinterpret_cast<floatx4_t *>(Vs + j * RS + 4 * s) = floatx4_t{ 0, 0, 0, 0 };
+    }
+    // maximum over the keys (exact in any order)
+    float mx = v;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if ((j & 63) == 0) red[j >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(red[0], red[1]);
+    if (mx == -INFINITY) mx = 0.0f;
+    const float e = __expf(v - mx); // exp(-inf) = 0 for masked keys
+    es[j] = e;
+    __syncthreads();
+    if (j < 4) { // the partial sum lane group g of the column holds in the whole-segment kernel
+        floatx4_t e4[8];
+#pragma unroll
+        for (int jt = 0; jt < 8; jt++) e4[jt] = *reinterpret_cast<const floatx4_t *>(es + jt * 16 + 4 * j);
+        float sum = 0.0f;
+#pragma unroll
+        for (int jt = 0; jt < 8; jt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) sum += e4[jt][r];
+        red[j] = sum;
+    }
+    __syncthreads();
+    const float sum = (red[0] + red[1]) + (red[2] + red[3]);
+    const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+    es[j] = e * inv; // (every thread read its own e above; the sums are done)
+    __syncthreads();
+    if (j < DK) {
+        const int j_hi = i + a.M, j_lo = j_hi - a.attn_len + 1; // keys inside the window (uniform)
+        float acc = 0.0f;
+        for (int jt = 0; jt < 8; jt++) {
+            if (jt * 16 > j_hi || jt * 16 + 15 < j_lo) continue; // a tile of masked keys: sixteen exact no-ops
+            floatx4_t p4[4];
+            float vv[16];
+#pragma unroll
+            for (int g = 0; g < 4; g++) p4[g] = *reinterpret_cast<const floatx4_t *>(es + jt * 16 + 4 * g);
+#pragma unroll
+            for (int u = 0; u < 16; u++) vv[u] = Vs[(jt * 16 + u) * RS + j];
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) acc = __builtin_fmaf(vv[4 * g + r], p4[g][r], acc);
+        }
+        as_global(a.out)[(int64_t)h * DK + j + a.ldo * b] = acc;
+    }
+}
+
+int g_attn_step_scalar = 1; // 0: single-query calls go through the whole-segment kernel (testing aid)
+
 template <typename KernelT>
 bool allow_lds(KernelT kern, size_t bytes)
 {
@@ -1259,8 +1389,20 @@ bool k_attn_fused_shape_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr)
     return dk == 64 && dv == 64 && T <= FA_TMAX && tiled_ntt(K, has_wr ? d_pos : 1) != 0;
 }
 
+// testing aid: 0 sends single-query calls through the whole-segment kernel again (every row
+// of its query tile the one query), 1 (default) through the vector-ALU kernel: same bits
+extern "C" void nchip_relpos_attn_step_kernel(int scalar)
+{
+    g_attn_step_scalar = scalar;
+}
+
 int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk)
 {
+    if (a.q_only >= 0 && g_attn_step_scalar && a.K <= 128 && a.d_pos <= 128 && !a.probs) {
+        if (dk == 64) hipLaunchKernelGGL(relpos_attn_step_scalar<64>, dim3(a.B * a.H), dim3(128), 0, st, a);
+        else hipLaunchKernelGGL(relpos_attn_step_scalar<32>, dim3(a.B * a.H), dim3(128), 0, st, a);
+        return hipGetLastError() == hipSuccess ? 0 : -1;
+    }
     if (const int ntt = (a.K > 128 || a.d_pos > 128) ? tiled_ntt(a.K, a.d_pos) : 0) {
         if (dk != 64 || a.q_only >= 0 || !a.probs || !probs_vec(a)) return -1;
         return ntt == 12 ? launch_fwd_tiled<64, 12>(st, a) : ntt == 16 ? launch_fwd_tiled<64, 16>(st, a)

@@ -528,6 +528,120 @@ __global__ __launch_bounds__(256) void gemm_skinny_nn(GemmArgs g)
     epilogue_tile(g, acc, m0 + (lane & 31), n0 + kh * 4, as_global(g.C), P, Radd, Dp, full, plain);
 }
 
+// The same few-column product on the vector ALUs.  An fp32 MFMA accumulates its k values
+// one after the other with fused multiply-adds, in increasing k (checked bit for bit against
+// v_mfma_f32_32x32x2_f32 chains, denormal products included), so an output element of the
+// width-invariant class is four chains of K/4 dependent v_fma_f32 - chain c takes k%32 in
+// [8c, 8c+8) - summed as (c0 + c1) + (c2 + c3).  A thread is one chain of one element: a
+// workgroup of 256 threads owns an 8 x 8 tile of C (4 chains each), so a 512 x 32 product
+// spreads over 256 workgroups instead of 16 and a chain costs K/4 FMAs (0.3 microseconds at
+// K = 512) instead of K/8 MFMAs of 64 cycles.  Its 8 rows of A and 8 columns of B pass
+// through LDS in chunks of 256 k ([row][k] with k contiguous, two buffers, one barrier per
+// chunk); the loads of up to PF chunks are in flight from the start (K = 2048 whole), since
+// one memory round trip is longer than all the arithmetic.  Bias and addend are fetched
+// before the k loop.  alpha = 1, beta = 0, no activation gradient; M a multiple of 8.
+constexpr int FC_KC = 256, FC_RS = FC_KC + 4;
+template <int PF>
+__global__ __launch_bounds__(256) void gemm_fewcol_fma(GemmArgs g)
+{
+    __shared__ __attribute__((aligned(16))) float tile[2][16 * FC_RS]; // rows 0-7: A rows, 8-15: B columns
+    const int t = threadIdx.x;
+    if (blockIdx.z == 1) { // the pair's second product: its own A, C, bias and row count
+        g.A = g.A_1; g.C = g.C_1; g.bias = g.bias_1; g.lda = g.lda_1; g.ldc = g.ldc_1; g.M = g.M_1;
+    }
+    const int m0 = blockIdx.x * 8, n0 = blockIdx.y * 8;
+    if (m0 >= g.M) return; // (uniform: the grid covers the taller of the two products)
+    const int ch = t & 3, ei = (t >> 2) & 7, ej = t >> 5; // chain, row and column of this thread's element
+    const int nslab = g.K / 32, nch = (g.K + FC_KC - 1) / FC_KC;
+    // A chunk: 256 k x 8 rows = 512 16-byte pieces (k = piece / 2, four rows each);
+    // B chunk: 8 columns x 256 k = 512 pieces (column = piece / 64, four k each)
+    const int ak[2] = { t >> 1, (t + 256) >> 1 }, ah = (t & 1) * 4;
+    const int bj[2] = { t >> 6, (t + 256) >> 6 }, bk = (t & 63) * 4;
+    const float NCHIP_GLOBAL *Ab = as_global(g.A) + m0 + ah;
+    const float NCHIP_GLOBAL *Bb[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int col = n0 + bj[u] < g.N ? n0 + bj[u] : g.N - 1;
+        Bb[u] = as_global(g.B) + (int64_t)col * g.ldb;
+    }
+    floatx4 ra[PF][2], rb[PF][2];
+    auto load = [&](floatx4 (&a)[2], floatx4 (&b)[2], int q) { // past the end: clamped, never used
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            int ka = q * FC_KC + ak[u], kb = q * FC_KC + bk;
+            ka = ka < g.K ? ka : g.K - 1;
+            kb = kb < g.K ? kb : g.K - 4;
+            a[u] = *reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(Ab + (int64_t)ka * g.lda);
+            b[u] = *reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(Bb[u] + kb);
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < PF; j++) {
+        load(ra[j], rb[j], j);
+        __builtin_amdgcn_sched_barrier(0); // oldest chunk first
+    }
+    const int row = m0 + ei, col = n0 + ej;
+    const bool ok = col < g.N;
+    float NCHIP_GLOBAL *P = g.pre ? as_global(g.pre) : nullptr;
+    const float NCHIP_GLOBAL *Radd = g.add ? as_global(g.add) : nullptr;
+    const bool plain = !g.bias && !P && !Radd && g.act == NCHIP_ACT_NONE;
+    const float bv = g.bias ? as_global(g.bias)[row] : 0.0f;
+    const float extra = (Radd && ok) ? Radd[(int64_t)col * g.ldc + row] : 0.0f;
+    auto park = [&](const floatx4 (&a)[2], const floatx4 (&b)[2], float *dst) { // registers -> [row][k]
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) dst[(ah + r) * FC_RS + ak[u]] = a[u][r];
+            *reinterpret_cast<floatx4 *>(dst + (8 + bj[u]) * FC_RS + bk) = b[u];
+        }
+    };
+    float acc = 0.0f;
+    for (int q0 = 0; q0 < nch; q0 += PF) {
+#pragma unroll
+        for (int j = 0; j < PF; j++) {
+            const int q = q0 + j;
+            if (q < nch) { // uniform
+                float *buf = tile[q & 1];
+                park(ra[j], rb[j], buf);
+                load(ra[j], rb[j], q + PF);
+                __syncthreads();
+                const float *wr = buf + ei * FC_RS + 8 * ch, *xr = buf + (8 + ej) * FC_RS + 8 * ch;
+                const int ns = nslab - 8 * q < 8 ? nslab - 8 * q : 8;
+                auto slab = [&](int s) {
+                    const floatx4 w0 = *reinterpret_cast<const floatx4 *>(wr + 32 * s);
+                    const floatx4 w1 = *reinterpret_cast<const floatx4 *>(wr + 32 * s + 4);
+                    const floatx4 x0 = *reinterpret_cast<const floatx4 *>(xr + 32 * s);
+                    const floatx4 x1 = *reinterpret_cast<const floatx4 *>(xr + 32 * s + 4);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc = __builtin_fmaf(x0[r], w0[r], acc);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc = __builtin_fmaf(x1[r], w1[r], acc);
+                };
+                if (ns == 8) { // a whole chunk, unrolled: the LDS reads run ahead of the chain
+#pragma unroll
+                    for (int s = 0; s < 8; s++) slab(s);
+                } else {
+                    for (int s = 0; s < ns; s++) slab(s);
+                }
+            }
+        }
+    }
+    // (c0 + c1) + (c2 + c3): the four chains of an element sit in four neighbouring lanes
+    float v = acc + __shfl_xor(acc, 1, 64);
+    v = v + __shfl_xor(v, 2, 64);
+    if (ch != 0 || !ok) return;
+    float NCHIP_GLOBAL *Cp = as_global(g.C) + (int64_t)col * g.ldc + row;
+    if (plain) {
+        *Cp = g.alpha * v;
+        return;
+    }
+    v = g.alpha * v + bv;
+    if (P) P[(int64_t)col * g.ldc + row] = v;
+    if (g.act == NCHIP_ACT_GELU) v = gelu_tanh(v);
+    else if (g.act == NCHIP_ACT_RELU) v = v > 0.0f ? v : 0.0f;
+    *Cp = v + extra;
+}
+
 // KW = 2 doubles the wavefronts of a workgroup without shrinking its tile: the
 // two groups of WM x WN wavefronts share the LDS tiles and split every 32-deep
 // k slab, group 0 taking k%32 < 16 and group 1 the rest; group 1 hands its
@@ -1033,7 +1147,16 @@ struct ProfRec {
 };
 bool g_prof_on = false;
 int g_force_cfg = getenv("NCHIP_GEMM_CFG") ? atoi(getenv("NCHIP_GEMM_CFG")) : 0;
-int g_skinny = 1; // width-invariant products with <= 64 columns take the register-streaming kernel
+int g_skinny = 2; // width-invariant products with <= 64 columns: 2 = the vector-ALU kernel, 1 = the MFMA few-column kernel, 0 = tiles
+
+// chunks of 256 k in flight: as many as the product has, up to 8
+static void launch_fewcol_fma(const GemmArgs &g, dim3 grid, hipStream_t st)
+{
+    const int nch = (g.K + FC_KC - 1) / FC_KC;
+    if (nch <= 2) hipLaunchKernelGGL(gemm_fewcol_fma<2>, grid, dim3(256), 0, st, g);
+    else if (nch <= 4) hipLaunchKernelGGL(gemm_fewcol_fma<4>, grid, dim3(256), 0, st, g);
+    else hipLaunchKernelGGL(gemm_fewcol_fma<8>, grid, dim3(256), 0, st, g);
+}
 int g_force_gm = -1;
 std::vector<ProfRec> g_prof;
 
@@ -1200,7 +1323,10 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     if (invariant && g_skinny && !ta && !tb && batch == 1 && precision == 0 && n <= 64 && k >= 32 && k % 32 == 0 &&
         m % 32 == 0 && lda % 4 == 0 && ldb % 4 == 0 && (((uintptr_t)A | (uintptr_t)B) & 15) == 0 && beta == 0.0f && !g_prof_on) {
         // a few token columns: the same arithmetic without the tile pipeline
-        hipLaunchKernelGGL(gemm_skinny_nn<16>, dim3(m / 32, (n + 31) / 32), dim3(256), 0, st, g);
+        if (g_skinny == 2 && alpha == 1.0f && !dpre)
+            launch_fewcol_fma(g, dim3(m / 8, (n + 7) / 8), st);
+        else
+            hipLaunchKernelGGL(gemm_skinny_nn<16>, dim3(m / 32, (n + 31) / 32), dim3(256), 0, st, g);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) {
             fprintf(stderr, "nchip_gemm: launch failed: %s\n", hipGetErrorString(e));
@@ -1374,7 +1500,8 @@ extern "C" void nchip_gemm_force_config(int cfg)
 }
 
 // testing aid: 0 sends width-invariant products of a few columns through the tile
-// kernel again (same bits, by construction: the tests compare the two)
+// kernel again, 1 through the MFMA few-column kernel, 2 (default) through the vector-ALU
+// kernel (same bits, by construction: the tests compare the three)
 extern "C" void nchip_gemm_few_columns_kernel(int on)
 {
     g_skinny = on;
@@ -1401,8 +1528,11 @@ extern "C" int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, 
     g.A = A0; g.B = B; g.C = C0; g.bias = bias0; g.lda = lda0; g.ldb = ldb; g.ldc = ldc0;
     g.M = m0; g.N = n; g.K = k; g.batch = 1; g.batch_in = 1; g.ksplit = 1; g.alpha = 1.0f;
     g.A_1 = A1; g.C_1 = C1; g.bias_1 = bias1; g.lda_1 = lda1; g.ldc_1 = ldc1; g.M_1 = m1;
-    const int mt = (m0 > m1 ? m0 : m1) / 32;
-    hipLaunchKernelGGL(gemm_skinny_nn<16>, dim3(mt, (n + 31) / 32, 2), dim3(256), 0, (hipStream_t)stream, g);
+    const int mmax = m0 > m1 ? m0 : m1;
+    if (g_skinny == 2)
+        launch_fewcol_fma(g, dim3(mmax / 8, (n + 7) / 8, 2), (hipStream_t)stream);
+    else
+        hipLaunchKernelGGL(gemm_skinny_nn<16>, dim3(mmax / 32, (n + 31) / 32, 2), dim3(256), 0, (hipStream_t)stream, g);
     if (hipGetLastError() != hipSuccess) {
         fprintf(stderr, "nchip_gemm_pair_few_columns: launch failed\n");
         return -2;

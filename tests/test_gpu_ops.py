@@ -67,12 +67,14 @@ def test_gemm_columns_do_not_depend_on_batch_width(hip, rng):
 
 
 @pytest.mark.parametrize("m,k,n", [(512, 512, 32), (2048, 512, 32), (512, 2048, 32), (256, 512, 32), (100, 70, 7),
-                                   (64, 33, 33), (130, 1, 64), (1024, 96, 40)])
+                                   (64, 33, 33), (130, 1, 64), (1024, 96, 40), (512, 1024, 32), (96, 4096, 16),
+                                   (64, 288, 9), (32, 32, 1), (32, 2304, 64)])
 def test_few_column_products_are_the_wide_products_columns(hip, rng, m, k, n):
     """Width-invariant mode: a product with a few token columns (the decoder's per-timestep
-    shape, which takes the register-streaming kernel) equals, bit for bit, the same product
-    through the tile kernel and the matching columns of a wide product, with every epilogue
-    option the forward pass uses (bias, GELU, residual addend)."""
+    shape, which takes the vector-ALU kernel: chains of fused multiply-adds in the order an
+    fp32 MFMA accumulates) equals, bit for bit, the same product through the MFMA few-column
+    kernel, through the tile kernel, and the matching columns of a wide product, with every
+    epilogue option the forward pass uses (bias, GELU, residual addend)."""
     lib = C.CDLL(hip.lib._name)
     w = rng.standard_normal((k, m)).astype(np.float32)
     wide = rng.standard_normal((200 + n, k)).astype(np.float32)
@@ -90,14 +92,17 @@ def test_few_column_products_are_the_wide_products_columns(hip, rng, m, k, n):
     try:
         whole = products(wide, res)
         few = products(wide[150:150 + n], res[150:150 + n])
+        lib.nchip_gemm_few_columns_kernel(1)
+        few_mfma = products(wide[150:150 + n], res[150:150 + n])
         lib.nchip_gemm_few_columns_kernel(0)
         few_tiles = products(wide[150:150 + n], res[150:150 + n])
     finally:
-        lib.nchip_gemm_few_columns_kernel(1)
+        lib.nchip_gemm_few_columns_kernel(2)
         hip.nc_set_matmul_width_invariant(hip.ctx, 0)
-    for a, b, c in zip(whole, few, few_tiles):
+    for a, b, c, d in zip(whole, few, few_tiles, few_mfma):
         assert np.array_equal(a[150:150 + n], b)
         assert np.array_equal(b, c)
+        assert np.array_equal(b, d)
     ref64 = wide[150:150 + n].astype(np.float64) @ w.astype(np.float64)
     assert relerr(few[0], ref64) <= TOL
 
@@ -403,6 +408,53 @@ def test_bias_gradient_model_shapes(hip, ref, rng, f, n):
 def _dev(nc, arr):
     t = nc.tensor(np.ascontiguousarray(arr, dtype=np.float32))
     return t, C.c_void_p(nc.lib.nc_tensor_get_ptr(t, None))
+
+
+@pytest.mark.parametrize("H,dk,B,T,M,d_pos,attn_len,has_w,t", [
+    (8, 64, 32, 64, 64, 128, 128, 1, 63), (8, 64, 32, 64, 64, 128, 128, 1, 0), (8, 64, 4, 64, 64, 128, 100, 1, 17),
+    (2, 32, 3, 9, 7, 13, 11, 1, 5), (2, 32, 3, 9, 7, 13, 16, 1, 8), (3, 64, 2, 20, 0, 20, 20, 1, 19),
+    (2, 64, 5, 33, 40, 1, 50, 0, 32), (4, 32, 2, 64, 64, 128, 3, 1, 40)])
+def test_one_query_attention_kernels_agree(hip, rng, H, dk, B, T, M, d_pos, attn_len, has_w, t):
+    """nchip_relpos_attn_fwd_step: the vector-ALU kernel (fused multiply-add chains in the order
+    an fp32 MFMA accumulates) writes the bits of the whole-segment kernel run with every query
+    row the one query, and both are the attention of query t in float64 up to rounding."""
+    lib = C.CDLL(hip.lib._name)
+    st = C.c_void_p(hip.nc_context_stream(hip.ctx))
+    K, D = M + T, H * dk
+    q = rng.standard_normal((B, D)); kv = rng.standard_normal((T, B, 2 * D)); kvm = rng.standard_normal((max(M, 1), B, 2 * D))
+    w_r = rng.standard_normal((H, d_pos, dk)); b_r = rng.standard_normal((H, K))
+    b_r_scale = float(np.sqrt(dk * D))
+    tens = {k: _dev(hip, v) for k, v in dict(q=q, kv=kv, kvm=kvm, w_r=w_r, b_r=b_r, o0=np.zeros((B, D)), o1=np.ones((B, D))).items()}
+    P = {k: v[1] for k, v in tens.items()}
+    i64, ci = C.c_int64, C.c_int
+    try:
+        for mode, out in ((0, "o0"), (1, "o1")):
+            lib.nchip_relpos_attn_step_kernel(mode)
+            assert lib.nchip_relpos_attn_fwd_step(st, P["q"], i64(D), P["kv"], P["kvm"] if M else None, i64(2 * D),
+                                                  P["w_r"] if has_w else None, P["b_r"], P[out], i64(D), ci(H), ci(dk), ci(dk),
+                                                  ci(B), ci(T), ci(M), ci(d_pos), ci(attn_len), C.c_float(b_r_scale), ci(t)) == 0
+    finally:
+        lib.nchip_relpos_attn_step_kernel(1)
+    o0, o1 = hip.numpy(tens["o0"][0]), hip.numpy(tens["o1"][0])
+    hip.free(*[v[0] for v in tens.values()])
+    assert np.array_equal(o0.view(np.uint32), o1.view(np.uint32))
+    f = lambda a: np.asarray(a, np.float32).astype(np.float64)
+    keys = np.concatenate([f(kvm)[:M], f(kv)], axis=0)              # (K, B, 2D), memory first
+    want = np.zeros((B, D))
+    for h in range(H):
+        for b in range(B):
+            qv = f(q)[b, h * dk:(h + 1) * dk]
+            js = [j for j in range(K) if 0 <= t + M - j < attn_len]
+            sc = []
+            for j in js:
+                delta = t + M - j
+                s_ = keys[j, b, h * dk:(h + 1) * dk] @ qv + b_r_scale * f(b_r)[h, K - 1 - delta]
+                if has_w:
+                    s_ += f(w_r)[h, max(d_pos - 1 - delta, 0)] @ qv
+                sc.append(s_ / np.sqrt(dk))
+            pr = np.exp(np.array(sc) - max(sc)); pr /= pr.sum()
+            want[b, h * dk:(h + 1) * dk] = sum(p_ * keys[j, b, D + h * dk:D + (h + 1) * dk] for p_, j in zip(pr, js))
+    assert relerr(o1, want) <= TOL
 
 
 @pytest.mark.parametrize("d,n", [(512, 2048), (128, 80), (1024, 333), (256, 5)])
