@@ -57,6 +57,19 @@ NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv_mem,
 NCTensor *nc_linear_pair_into(NCTensor *w0, NCTensor *bias0, NCTensor *w1, NCTensor *x,
                               NCTensor *dst, int index);
 
+/* The layer norm (avg_flag 1) or RMS norm (0) of x (k, n) with gain g and bias b (both or
+   neither), followed by y0 = act0(w0 norm(x) + bias0) and, when w1 and dst are given,
+   w1 norm(x) written into slice `index` of the last axis of dst (m1, n, T) - one launch in
+   width-invariant fp32 mode for k = 128, 256 or 512 and at most 64 columns (the decoder's
+   timestep: the norm that ends one block rides on the first product of the next,
+   nncp.c:896-987), the separate steps otherwise.  *pnormed, when pnormed is not NULL,
+   receives norm(x) as a new tensor.  The values are those of nc_fused_layer_norm followed by
+   nc_linear / nc_linear_pair_into, bit for bit.  Consumes x, g, b, w0, bias0 and w1, not
+   dst.  With a pair act0 must be NC_ACT_NONE.  No gradient. */
+NCTensor *nc_norm_linear_pair_into(NCTensor *x, NCTensor *g, NCTensor *b, float eps, BOOL avg_flag,
+                                   NCTensor *w0, NCTensor *bias0, int act0,
+                                   NCTensor *w1, NCTensor *dst, int index, NCTensor **pnormed);
+
 /* One query position of nc_relpos_attention: q (H*dk, B) is the query of
    position t, kv_cache (H*dk+H*dv, B, T) holds the keys / values of positions
    0..t of the current segment (later columns finite, e.g. zero), kv_mem, w_r,

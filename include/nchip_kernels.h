@@ -140,13 +140,29 @@ int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, int k,
                                 float *C0, int64_t ldc0, float *C1, int64_t ldc1,
                                 const float *bias0, const float *bias1);
 
+/* One or two width-invariant few-column products of the layer norm (avg = 1) or RMS norm
+   (avg = 0) of B's columns, in one launch: C0 (m0 x n) = act0(A0 norm(B) + bias0) and, when
+   m1 > 0, C1 (m1 x n) = A1 norm(B) + bias1.  B holds k = 128, 256 or 512 raw features per
+   column; ln_w / ln_b are gain and bias (both or neither); the normalised columns are also
+   written to ln_out (leading dimension ld_ln) when it is not NULL.  The decoder's timestep:
+   the norm that ends one block (nncp.c:896-987, layer_norm of nncp.c:279-288) rides on the
+   first product of the next.  The bits are those of nchip_norm_fwd followed by the products
+   with NCHIP_GEMM_WIDTH_INVARIANT.  Returns 0, 1 when the shapes are not this kernel's
+   (nothing was launched), negative on error. */
+int nchip_norm_gemm_few_columns(void *stream, const float *ln_w, const float *ln_b, float eps, int avg,
+                                float *ln_out, int64_t ld_ln, int m0, int m1, int n, int k,
+                                const float *A0, int64_t lda0, const float *A1, int64_t lda1,
+                                const float *B, int64_t ldb, float *C0, int64_t ldc0,
+                                float *C1, int64_t ldc1, const float *bias0, const float *bias1, int act0);
+
 /* Testing aid: which kernel takes width-invariant fp32 products (NCHIP_GEMM_WIDTH_INVARIANT)
    with at most 64 columns, untransposed operands and beta = 0 (the decoder's per-timestep
-   products).  2 (default): the vector-ALU kernel - an fp32 MFMA accumulates its k values one
-   after the other with fused multiply-adds, so the four chains of an element are formed by
-   plain fma instructions, one chain per thread, 8 x 8 outputs per workgroup; 1: the
-   few-column MFMA kernel (one 32-row tile per workgroup, its four wavefronts the four chains);
-   0: the tile kernel.  The results are the same bits in all three. */
+   products).  3 (default): 16 x 16 tiles with v_mfma_f32_16x16x4_f32, the four wavefronts of a
+   workgroup the four chains of the width-invariant class; 2: the vector-ALU kernel - an fp32
+   MFMA accumulates its k values one after the other with fused multiply-adds, so the chains
+   are formed by plain fma instructions, one chain per thread, 8 x 8 outputs per workgroup;
+   1: 32-row tiles with v_mfma_f32_32x32x2_f32; 0: the tile kernel.  The results are the same
+   bits in all four. */
 void nchip_gemm_few_columns_kernel(int kernel);
 
 /* Tuning aid: tiles are ordered, inside each XCD's run, in bands of `gm` tile

@@ -29,6 +29,7 @@
 #include <vector>
 #include "../../include/nchip_kernels.h"
 #include "k_addrspace.h"
+#include "k_norm_inline.h"
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -73,6 +74,14 @@ struct GemmArgs {
     float *C_1;
     int64_t lda_1, ldc_1;
     int M_1;
+    // few-column kernel that normalises B on the way in (gemm_fewcol_mfma with NV > 0): gain and
+    // bias (both or neither), the normalised columns written to ln_out (leading dimension
+    // ld_ln) by the first row tile when it is not NULL
+    const float *ln_w, *ln_b;
+    float *ln_out;
+    int64_t ld_ln;
+    float ln_eps;
+    int ln_avg;
 };
 
 __device__ __forceinline__ float gelu_tanh(float x)
@@ -642,6 +651,178 @@ __global__ __launch_bounds__(256) void gemm_fewcol_fma(GemmArgs g)
     *Cp = v + extra;
 }
 
+// The few-column product with v_mfma_f32_16x16x4_f32.  That instruction accumulates its
+// four k in increasing order like the 32x32x2 one its two, at a quarter of the chain latency
+// per k (a 16x16 tile: 8 passes per 4 k instead of 16 passes per 2 k), so chain c of a slab
+// is two of them (k%32 = 8c..8c+3, 8c+4..8c+7) and the result is again the bits of the tile
+// kernel.  A workgroup is a 16 x 16 tile of C and its four wavefronts are the four chains
+// (combined as (c0 + c1) + (c2 + c3) through LDS at the end); a wavefront fetches only the
+// 8 k per slab of its own chain - 16 rows of A and 16 columns of B, in chunks of 256 k, up
+// to PF chunks in flight - into a private corner of LDS and reads its fragments from there,
+// so the k loop has no workgroup barrier.  Against the vector-ALU kernel: a quarter of the
+// workgroups, but 1 KB of LDS reads per slab and wavefront for 256 outputs instead of 4 KB
+// for 16, which is what bounds that kernel on the taller products.  alpha = 1, beta = 0.
+//
+// NV > 0: B holds K = 64 NV raw features per column and the product is taken with their
+// layer norm (or RMS norm) - the arithmetic of norm_fwd_reg, wavefront c normalising columns
+// 4c..4c+3 of the tile before the k loop, the result kept whole in LDS (every workgroup
+// repeats it for its 16 columns, which costs less than a launch of its own); the first row
+// tile also writes the normalised columns out for the later consumers of that tensor.
+template <int PF, int NV = 0>
+__global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
+{
+    constexpr int BST = 68, WSZ = 64 * 16 + (NV ? 0 : 16 * BST); // per wavefront: A [64 k][16 rows], B [16 columns][64 k]
+    constexpr int XS = 64 * NV + 4;
+    __shared__ __attribute__((aligned(16))) float stage[4][WSZ];
+    __shared__ float red[3][4 * 64];
+    __shared__ float xn[NV ? 16 * XS : 1]; // normalised B: [16 columns][K]
+    const int lane = threadIdx.x & 63, c = threadIdx.x >> 6; // wavefront = chain
+    if (blockIdx.z == 1) { // the pair's second product: its own A, C, bias and row count
+        g.A = g.A_1; g.C = g.C_1; g.bias = g.bias_1; g.lda = g.lda_1; g.ldc = g.ldc_1; g.M = g.M_1;
+    }
+    const int m0 = blockIdx.x * 16, n0 = blockIdx.y * 16;
+    if (m0 >= g.M) return; // (uniform: the grid covers the taller of the two products)
+    const int il = lane & 15, gq = lane >> 4;
+    const int nslab = g.K / 32, nch = (g.K + 255) / 256;
+    float *As = stage[c], *Bs = As + 64 * 16;
+    // this lane's four 16-byte pieces of A (k_local = piece / 4, four rows) and of B
+    // (column = piece / 16, slab = (piece % 16) / 2, half a chain's 8 k)
+    const float NCHIP_GLOBAL *Ab = as_global(g.A) + m0 + (lane & 3) * 4;
+    const float NCHIP_GLOBAL *Bb[4];
+    int a_k[4], b_k[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int pa = lane + 64 * u, kl = pa >> 2;
+        a_k[u] = 32 * (kl >> 3) + 8 * c + (kl & 7);
+        const int pb = lane + 64 * u, colb = pb >> 4, kq = pb & 15;
+        const int col = n0 + colb < g.N ? n0 + colb : g.N - 1;
+        Bb[u] = as_global(g.B) + (int64_t)col * g.ldb;
+        b_k[u] = 32 * (kq >> 1) + 8 * c + 4 * (kq & 1);
+    }
+    floatx4 ra[PF][4], rb[NV ? 1 : PF][4];
+    auto load = [&](floatx4 (&a)[4], floatx4 (&b)[4], int q) { // past the end: clamped, never used
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            int ka = q * 256 + a_k[u], kb = q * 256 + b_k[u];
+            ka = ka < g.K ? ka : g.K - 1;
+            kb = kb < g.K ? kb : g.K - 4;
+            a[u] = *reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(Ab + (int64_t)ka * g.lda);
+            if (NV == 0) b[u] = *reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(Bb[u] + kb);
+        }
+    };
+    // the raw columns first: they are needed first
+    float xv[NV ? 4 : 1][NV ? NV : 1], lw[NV ? NV : 1], lb[NV ? NV : 1];
+    if (NV > 0) {
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) {
+            const int colb = 4 * c + cc, gcol = n0 + colb < g.N ? n0 + colb : g.N - 1;
+            const float NCHIP_GLOBAL *xc = as_global(g.B) + (int64_t)gcol * g.ldb + lane;
+#pragma unroll
+            for (int v = 0; v < NV; v++) xv[cc][v] = xc[64 * v];
+        }
+        if (g.ln_w) {
+#pragma unroll
+            for (int v = 0; v < NV; v++) { lw[v] = as_global(g.ln_w)[lane + 64 * v]; lb[v] = as_global(g.ln_b)[lane + 64 * v]; }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int j = 0; j < PF; j++) {
+        load(ra[j], rb[NV ? 0 : j], j);
+        __builtin_amdgcn_sched_barrier(0); // oldest chunk first
+    }
+    if (NV > 0) {
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) {
+            const int colb = 4 * c + cc;
+            float hh[NV ? NV : 1], yy[NV ? NV : 1];
+            norm_column_reg<(NV ? NV : 1)>(xv[cc], lw, lb, g.ln_w != nullptr, g.ln_eps, g.ln_avg, hh, yy);
+#pragma unroll
+            for (int v = 0; v < NV; v++) xn[colb * XS + lane + 64 * v] = yy[v];
+            if (g.ln_out && blockIdx.x == 0 && blockIdx.z == 0 && n0 + colb < g.N) {
+                float NCHIP_GLOBAL *yo = as_global(g.ln_out) + (int64_t)(n0 + colb) * g.ld_ln + lane;
+#pragma unroll
+                for (int v = 0; v < NV; v++) yo[64 * v] = yy[v];
+            }
+        }
+        __syncthreads();
+    }
+    // epilogue operands, fetched before the k loop (wavefront 0 finishes the tile)
+    const int col = n0 + il;
+    const bool ok = col < g.N;
+    float NCHIP_GLOBAL *P = g.pre ? as_global(g.pre) : nullptr;
+    const float NCHIP_GLOBAL *Radd = g.add ? as_global(g.add) : nullptr;
+    const bool plain = !g.bias && !P && !Radd && g.act == NCHIP_ACT_NONE;
+    float bv[4], extra[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int row = m0 + 4 * gq + r;
+        bv[r] = (c == 0 && g.bias) ? as_global(g.bias)[row] : 0.0f;
+        extra[r] = (c == 0 && Radd && ok) ? Radd[(int64_t)col * g.ldc + row] : 0.0f;
+    }
+    floatx4 acc = { 0, 0, 0, 0 };
+    for (int q0 = 0; q0 < nch; q0 += PF) {
+#pragma unroll
+        for (int j = 0; j < PF; j++) {
+            const int q = q0 + j;
+            if (q < nch) { // uniform
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int pa = lane + 64 * u;
+                    *reinterpret_cast<floatx4 *>(As + (pa >> 2) * 16 + (pa & 3) * 4) = ra[j][u];
+                    if (NV == 0) *reinterpret_cast<floatx4 *>(Bs + (pa >> 4) * BST + (pa & 15) * 4) = rb[j][u];
+                }
+                load(ra[j], rb[NV ? 0 : j], q + PF);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                float fa[16], fb[16];
+#pragma unroll
+                for (int e = 0; e < 16; e++) { // MFMA e of the chunk: slab e / 2, k_local = 4 e + gq
+                    fa[e] = As[(4 * e + gq) * 16 + il];
+                    int kx = 256 * q + 32 * (e >> 1) + 8 * c + 4 * (e & 1) + gq;
+                    kx = kx < g.K ? kx : g.K - 1; // (past a short last chunk: read, never used)
+                    fb[e] = NV ? xn[il * XS + kx] : Bs[il * BST + 4 * e + gq];
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier(); // the fragments are in registers: the corner may be rewritten
+                const int ne = (nslab - 8 * q < 8 ? nslab - 8 * q : 8) * 2;
+                if (ne == 16) {
+#pragma unroll
+                    for (int e = 0; e < 16; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[e], fb[e], acc, 0, 0, 0);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                        if (e < ne) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[e], fb[e], acc, 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (c > 0) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[c - 1][r * 64 + lane] = acc[r];
+    }
+    __syncthreads();
+    if (c > 0 || !ok) return;
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc[r] = (acc[r] + red[0][r * 64 + lane]) + (red[1][r * 64 + lane] + red[2][r * 64 + lane]);
+    // lane (il, gq) holds rows m0 + 4 gq + r of column n0 + il
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int row = m0 + 4 * gq + r;
+        float NCHIP_GLOBAL *Cp = as_global(g.C) + (int64_t)col * g.ldc + row;
+        if (plain) {
+            *Cp = g.alpha * acc[r];
+            continue;
+        }
+        float v = g.alpha * acc[r] + bv[r];
+        if (P) P[(int64_t)col * g.ldc + row] = v;
+        if (g.act == NCHIP_ACT_GELU) v = gelu_tanh(v);
+        else if (g.act == NCHIP_ACT_RELU) v = v > 0.0f ? v : 0.0f;
+        *Cp = v + extra[r];
+    }
+}
+
 // KW = 2 doubles the wavefronts of a workgroup without shrinking its tile: the
 // two groups of WM x WN wavefronts share the LDS tiles and split every 32-deep
 // k slab, group 0 taking k%32 < 16 and group 1 the rest; group 1 hands its
@@ -1147,7 +1328,7 @@ struct ProfRec {
 };
 bool g_prof_on = false;
 int g_force_cfg = getenv("NCHIP_GEMM_CFG") ? atoi(getenv("NCHIP_GEMM_CFG")) : 0;
-int g_skinny = 2; // width-invariant products with <= 64 columns: 2 = the vector-ALU kernel, 1 = the MFMA few-column kernel, 0 = tiles
+int g_skinny = 3; // width-invariant products with <= 64 columns: 3 = the 16x16x4 MFMA kernel, 2 = the vector-ALU kernel, 1 = the 32x32x2 MFMA kernel, 0 = tiles
 
 // chunks of 256 k in flight: as many as the product has, up to 8
 static void launch_fewcol_fma(const GemmArgs &g, dim3 grid, hipStream_t st)
@@ -1156,6 +1337,14 @@ static void launch_fewcol_fma(const GemmArgs &g, dim3 grid, hipStream_t st)
     if (nch <= 2) hipLaunchKernelGGL(gemm_fewcol_fma<2>, grid, dim3(256), 0, st, g);
     else if (nch <= 4) hipLaunchKernelGGL(gemm_fewcol_fma<4>, grid, dim3(256), 0, st, g);
     else hipLaunchKernelGGL(gemm_fewcol_fma<8>, grid, dim3(256), 0, st, g);
+}
+
+// (grid in 16 x 16 tiles)
+static void launch_fewcol_mfma(const GemmArgs &g, dim3 grid, hipStream_t st)
+{
+    const int nch = (g.K + 255) / 256;
+    if (nch <= 2) hipLaunchKernelGGL(gemm_fewcol_mfma<2>, grid, dim3(256), 0, st, g);
+    else hipLaunchKernelGGL(gemm_fewcol_mfma<4>, grid, dim3(256), 0, st, g);
 }
 int g_force_gm = -1;
 std::vector<ProfRec> g_prof;
@@ -1299,6 +1488,7 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
         return -1;
     }
     GemmArgs g;
+    memset(&g, 0, sizeof(g));
     g.A = A; g.B = B; g.C = C; g.bias = bias; g.add = addend; g.pre = pre; g.ws = workspace;
     g.dpre = dpre; g.dact = dact;
     g.rowsum = nullptr;
@@ -1323,7 +1513,10 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     if (invariant && g_skinny && !ta && !tb && batch == 1 && precision == 0 && n <= 64 && k >= 32 && k % 32 == 0 &&
         m % 32 == 0 && lda % 4 == 0 && ldb % 4 == 0 && (((uintptr_t)A | (uintptr_t)B) & 15) == 0 && beta == 0.0f && !g_prof_on) {
         // a few token columns: the same arithmetic without the tile pipeline
-        if (g_skinny == 2 && alpha == 1.0f && !dpre)
+        // (a long reduction keeps the vector-ALU kernel: four times the workgroups to stream its operands)
+        if (g_skinny == 3 && alpha == 1.0f && !dpre && k <= 1024)
+            launch_fewcol_mfma(g, dim3(m / 16, (n + 15) / 16), st);
+        else if (g_skinny >= 2 && alpha == 1.0f && !dpre)
             launch_fewcol_fma(g, dim3(m / 8, (n + 7) / 8), st);
         else
             hipLaunchKernelGGL(gemm_skinny_nn<16>, dim3(m / 32, (n + 31) / 32), dim3(256), 0, st, g);
@@ -1500,8 +1693,9 @@ extern "C" void nchip_gemm_force_config(int cfg)
 }
 
 // testing aid: 0 sends width-invariant products of a few columns through the tile
-// kernel again, 1 through the MFMA few-column kernel, 2 (default) through the vector-ALU
-// kernel (same bits, by construction: the tests compare the three)
+// kernel again, 1 through the 32x32x2 MFMA few-column kernel, 2 through the vector-ALU
+// kernel, 3 (default) through the 16x16x4 MFMA kernel (same bits, by construction: the
+// tests compare the four)
 extern "C" void nchip_gemm_few_columns_kernel(int on)
 {
     g_skinny = on;
@@ -1529,12 +1723,53 @@ extern "C" int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, 
     g.M = m0; g.N = n; g.K = k; g.batch = 1; g.batch_in = 1; g.ksplit = 1; g.alpha = 1.0f;
     g.A_1 = A1; g.C_1 = C1; g.bias_1 = bias1; g.lda_1 = lda1; g.ldc_1 = ldc1; g.M_1 = m1;
     const int mmax = m0 > m1 ? m0 : m1;
-    if (g_skinny == 2)
+    if (g_skinny == 3)
+        launch_fewcol_mfma(g, dim3(mmax / 16, (n + 15) / 16, 2), (hipStream_t)stream);
+    else if (g_skinny == 2)
         launch_fewcol_fma(g, dim3(mmax / 8, (n + 7) / 8, 2), (hipStream_t)stream);
     else
         hipLaunchKernelGGL(gemm_skinny_nn<16>, dim3(mmax / 32, (n + 31) / 32, 2), dim3(256), 0, (hipStream_t)stream, g);
     if (hipGetLastError() != hipSuccess) {
         fprintf(stderr, "nchip_gemm_pair_few_columns: launch failed\n");
+        return -2;
+    }
+    return 0;
+}
+
+// One or two width-invariant few-column products of the layer norm (avg = 1) or RMS norm
+// (avg = 0) of B's columns, in ONE launch: C0 (m0 x n) = act0(A0 norm(B) + bias0) and, when
+// m1 > 0, C1 (m1 x n) = A1 norm(B) + bias1.  B holds k = 128, 256 or 512 raw features per
+// column; ln_w / ln_b are the gain and bias (both or neither); the normalised columns are
+// also written to ln_out (leading dimension ld_ln) when it is not NULL.  The bits are those
+// of nchip_norm_fwd followed by the products in width-invariant mode.  Returns 1 when the
+// shapes are not this kernel's (nothing launched: the caller issues the steps itself).
+extern "C" int nchip_norm_gemm_few_columns(void *stream, const float *ln_w, const float *ln_b, float eps, int avg,
+                                           float *ln_out, int64_t ld_ln, int m0, int m1, int n, int k,
+                                           const float *A0, int64_t lda0, const float *A1, int64_t lda1,
+                                           const float *B, int64_t ldb, float *C0, int64_t ldc0,
+                                           float *C1, int64_t ldc1, const float *bias0, const float *bias1, int act0)
+{
+    if (m0 <= 0 || m1 < 0 || n <= 0 || !A0 || !B || !C0 || (m1 > 0 && (!A1 || !C1)) || (ln_w == nullptr) != (ln_b == nullptr))
+        return -1;
+    if (g_skinny != 3 || g_prof_on || n > 64 || (k != 128 && k != 256 && k != 512) || m0 % 32 || m1 % 32 || lda0 % 4 ||
+        (m1 > 0 && lda1 % 4) || lda0 < m0 || (m1 > 0 && lda1 < m1) || ldb < k || ldc0 < m0 || (m1 > 0 && ldc1 < m1) ||
+        (ln_out && ld_ln < k) || (((uintptr_t)A0 | (uintptr_t)A1) & 15) != 0 ||
+        (act0 != NCHIP_ACT_NONE && act0 != NCHIP_ACT_GELU && act0 != NCHIP_ACT_RELU))
+        return 1;
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.A = A0; g.B = B; g.C = C0; g.bias = bias0; g.lda = lda0; g.ldb = ldb; g.ldc = ldc0; g.act = act0;
+    g.M = m0; g.N = n; g.K = k; g.batch = 1; g.batch_in = 1; g.ksplit = 1; g.alpha = 1.0f;
+    g.A_1 = A1; g.C_1 = C1; g.bias_1 = bias1; g.lda_1 = lda1; g.ldc_1 = ldc1; g.M_1 = m1;
+    g.ln_w = ln_w; g.ln_b = ln_b; g.ln_out = ln_out; g.ld_ln = ld_ln; g.ln_eps = eps; g.ln_avg = avg;
+    const int mmax = m0 > m1 ? m0 : m1;
+    const dim3 grid(mmax / 16, (n + 15) / 16, m1 > 0 ? 2 : 1);
+    hipStream_t st = (hipStream_t)stream;
+    if (k == 128) hipLaunchKernelGGL((gemm_fewcol_mfma<2, 2>), grid, dim3(256), 0, st, g);
+    else if (k == 256) hipLaunchKernelGGL((gemm_fewcol_mfma<2, 4>), grid, dim3(256), 0, st, g);
+    else hipLaunchKernelGGL((gemm_fewcol_mfma<2, 8>), grid, dim3(256), 0, st, g);
+    if (hipGetLastError() != hipSuccess) {
+        fprintf(stderr, "nchip_norm_gemm_few_columns: launch failed\n");
         return -2;
     }
     return 0;

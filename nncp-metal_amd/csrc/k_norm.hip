@@ -9,6 +9,7 @@
 #include <stdlib.h>
 #include <mutex>
 #include "../../include/nchip_kernels.h"
+#include "k_norm_inline.h"
 
 // Scratch of nchip_norm_bwd_static: the partial dw / db rows of the norm backward, held by the
 // library itself so that the call allocates nothing.  In host code this name is only a
@@ -80,20 +81,13 @@ __global__ __launch_bounds__(TPB) void norm_fwd_reg(const float *x, const float 
 #pragma unroll
         for (int v = 0; v < NV; v++) { wv[v] = w[lane + 64 * v]; bv[v] = b[lane + 64 * v]; }
     }
-    float s = 0.0f;
-#pragma unroll
-    for (int v = 0; v < NV; v++) s += xv[v];
-    const float mean = avg ? wave_sum(s) / (float)D : 0.0f;
-    float q = 0.0f;
-#pragma unroll
-    for (int v = 0; v < NV; v++) { float t = xv[v] - mean; q += t * t; }
-    const float r = 1.0f / sqrtf(wave_sum(q) / (float)D + eps);
+    float h[NV], yv[NV];
+    const float r = norm_column_reg<NV>(xv, wv, bv, w != nullptr, eps, avg, h, yv);
     if (lane == 0) rstd[c] = r;
 #pragma unroll
     for (int v = 0; v < NV; v++) {
-        const float h = (xv[v] - mean) * r;
-        if (xhat) xhat[c * D + lane + 64 * v] = h;
-        y[c * D + lane + 64 * v] = w ? h * wv[v] + bv[v] : h;
+        if (xhat) xhat[c * D + lane + 64 * v] = h[v];
+        y[c * D + lane + 64 * v] = yv[v];
     }
 }
 

@@ -889,6 +889,64 @@ extern "C" NCTensor *nc_fused_layer_norm(NCTensor *x, NCTensor *w, NCTensor *b, 
     return norm_op(x, w, b, eps, avg_flag != 0);
 }
 
+// nc_ext.h: one or two products of the normalised x in one launch, the decoder's way of not
+// paying a launch for the layer norm between two blocks.  y0 = act0(w0 norm(x) + bias0);
+// with w1, w1 norm(x) goes into slice `index` of dst; *pnormed (when asked for) is norm(x).
+// Same bits as nc_fused_layer_norm + nc_linear / nc_linear_pair_into.  No gradient.
+extern "C" NCTensor *nc_norm_linear_pair_into(NCTensor *x, NCTensor *g, NCTensor *b, float eps, BOOL avg_flag,
+                                              NCTensor *w0, NCTensor *bias0, int act0,
+                                              NCTensor *w1, NCTensor *dst, int index, NCTensor **pnormed)
+{
+    const char *me = "nc_norm_linear_pair_into";
+    if ((g == nullptr) != (b == nullptr)) nc_fatal("%s: g and b go together", me);
+    if ((w1 == nullptr) != (dst == nullptr)) nc_fatal("%s: w1 and dst go together", me);
+    x = nc_contig(x); w0 = nc_contig(w0);
+    need_f32(x, me); need_f32(w0, me);
+    NCContext *m = nc_ctx(w0);
+    int rc = 1;
+    NCTensor *y0 = nullptr, *normed = nullptr;
+    if (x->n_dims == 2 && w0->n_dims == 2 && w0->dims[1] == x->dims[0] && m->matmul_invariant && !m->matmul_bf16 &&
+        (!g || (g->type == NC_TYPE_F32 && b->type == NC_TYPE_F32 && nc_is_contig(g) && nc_is_contig(b) &&
+                nc_numel(g) == x->dims[0] && nc_numel(b) == x->dims[0])) &&
+        (!bias0 || (bias0->type == NC_TYPE_F32 && nc_is_contig(bias0) && nc_numel(bias0) == w0->dims[0])) &&
+        (!w1 || (w1->type == NC_TYPE_F32 && nc_is_contig(w1) && w1->n_dims == 2 && w1->dims[1] == x->dims[0] &&
+                 dst->type == NC_TYPE_F32 && nc_is_contig(dst) && dst->n_dims == 3 && dst->dims[0] == w1->dims[0] &&
+                 dst->dims[1] == x->dims[1] && index >= 0 && (size_t)index < dst->dims[2])) &&
+        (act0 == NC_ACT_NONE || act0 == NC_ACT_GELU || act0 == NC_ACT_RELU)) {
+        const size_t k = x->dims[0], n = x->dims[1], m0 = w0->dims[0], m1 = w1 ? w1->dims[0] : 0;
+        size_t d0[2] = { m0, n }, dn[2] = { k, n };
+        y0 = new_f32(w0, 2, d0);
+        if (pnormed) normed = new_f32(w0, 2, dn);
+        rc = nchip_norm_gemm_few_columns(m->stream, g ? nc_f32(g) : nullptr, b ? nc_f32(b) : nullptr, eps, avg_flag != 0,
+                                         normed ? nc_f32(normed) : nullptr, (int64_t)k, (int)m0, (int)m1, (int)n, (int)k,
+                                         nc_f32(w0), (int64_t)m0, w1 ? nc_f32(w1) : nullptr, (int64_t)m1, nc_f32(x), (int64_t)k,
+                                         nc_f32(y0), (int64_t)m0, w1 ? nc_f32(dst) + (size_t)index * m1 * n : nullptr, (int64_t)m1,
+                                         bias0 ? nc_f32(bias0) : nullptr, nullptr,
+                                         act0 == NC_ACT_GELU ? NCHIP_ACT_GELU : act0 == NC_ACT_RELU ? NCHIP_ACT_RELU : NCHIP_ACT_NONE);
+        if (rc < 0) nc_fatal("%s: kernel rejected the shapes", me);
+        if (rc != 0) {
+            nc_free_tensor(y0); nc_free_tensor(normed);
+            y0 = normed = nullptr;
+        }
+    }
+    if (rc == 0) {
+        m->launches++;
+        nc_free_tensor(x); nc_free_tensor(g); nc_free_tensor(b);
+        nc_free_tensor(w0); nc_free_tensor(bias0); nc_free_tensor(w1);
+    } else { // other shapes and modes: the steps one after the other
+        normed = g ? nc_fused_layer_norm(x, g, b, eps, avg_flag) : nc_fused_layer_norm(x, nullptr, nullptr, eps, avg_flag);
+        if (w1) {
+            if (act0 != NC_ACT_NONE) nc_fatal("%s: no activation on the first product of a pair", me);
+            y0 = nc_linear_pair_into(w0, bias0, w1, nc_dup_tensor(normed), dst, index);
+        } else {
+            y0 = nc_linear(w0, nc_dup_tensor(normed), bias0, act0);
+        }
+        if (!pnormed) { nc_free_tensor(normed); normed = nullptr; }
+    }
+    if (pnormed) *pnormed = normed;
+    return y0;
+}
+
 // ---- fused attention (nc_ext.h) ---------------------------------------------
 struct AttnDims {
     int H, dk, dv, B, T, M, K, d_pos;

@@ -653,12 +653,24 @@ NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
     t0 = nc_reshape_1d(t0, (size_t)B);
     x = nc_get_col(nc_dup_tensor(s->embed), t0);
     x = nc_mul(x, scalar(s, s->embed_mult));
+    /* Post-norm blocks with a plain activation (nncp's default structure, nncp.c:2489-2513):
+       a norm is followed by a product, so it rides on that product's launch
+       (nc_norm_linear_pair_into) - the norm after the attention on the first feed-forward
+       product, the norm that ends a block on the projections of the next block or on the
+       output product.  `pend` is the block whose closing norm x still waits for. */
+    const int ride = (c->ln_flags & (NNCP_LN_PRE | NNCP_LN_POST | NNCP_LN_FINAL | NNCP_LN_COEF)) == NNCP_LN_POST &&
+                     (c->ff_act == NNCP_FF_GELU || c->ff_act == NNCP_FF_RELU);
+    const int is_ln = !(c->ln_flags & NNCP_LN_RMSNORM);
+    Layer *pend = NULL;
     for (int l = 0; l < c->n_layer; l++) {
         Layer *tl = &s->layers[l];
         Layer *pr = &s->layers[c->tied_w_r ? 0 : l], *pb = &s->layers[c->tied_b_r ? 0 : l];
-        NCTensor *x1 = nc_dup_tensor(x), *ff_in, *q, *att;
-        if (c->ln_flags & NNCP_LN_PRE)
-            x1 = layer_norm(s, x1, tl->ln_g1, tl->ln_b1);
+        NCTensor *x1 = NULL, *ff_in, *q, *att;
+        if (!pend) {
+            x1 = nc_dup_tensor(x);
+            if (c->ln_flags & NNCP_LN_PRE)
+                x1 = layer_norm(s, x1, tl->ln_g1, tl->ln_b1);
+        }
         if (t == 0 && c->mem_len > 0) { /* K/V of the memory: once per segment */
             NCTensor *m2 = nc_reshape_2d(nc_dup_tensor(s->mem_h[l]), c->d_model, (size_t)c->mem_len * B);
             m2 = nc_matmul(nc_dup_tensor(tl->w_kv), m2);
@@ -666,14 +678,35 @@ NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
         }
         /* query and key / value of this position in one launch; the latter goes straight into
            column t of the cache */
-        q = nc_linear_pair_into(nc_dup_tensor(tl->w_q), c->query_bias ? nc_dup_tensor(tl->b_q) : NULL,
-                                nc_dup_tensor(tl->w_kv), x1, s->step_kv[l], t);
+        if (pend) {
+            NCTensor *xn;
+            q = nc_norm_linear_pair_into(x, nc_dup_tensor(pend->ln_g2), nc_dup_tensor(pend->ln_b2), 1e-5f, is_ln,
+                                         nc_dup_tensor(tl->w_q), c->query_bias ? nc_dup_tensor(tl->b_q) : NULL, NC_ACT_NONE,
+                                         nc_dup_tensor(tl->w_kv), s->step_kv[l], t, &xn);
+            x = xn;
+            pend = NULL;
+        } else {
+            q = nc_linear_pair_into(nc_dup_tensor(tl->w_q), c->query_bias ? nc_dup_tensor(tl->b_q) : NULL,
+                                    nc_dup_tensor(tl->w_kv), x1, s->step_kv[l], t);
+        }
         att = nc_relpos_attention_step(q, nc_dup_tensor(s->step_kv[l]),
                                        c->mem_len > 0 ? nc_dup_tensor(s->step_kvm[l]) : NULL,
                                        c->use_w_r ? nc_dup_tensor(pr->w_r) : NULL, nc_dup_tensor(pb->b_r),
                                        H, c->d_key, c->attn_len[l], sqrtf((float)(c->d_key * c->d_model)), t);
         if (!tl->w_o)
             die("the fused path needs d_value != d_model (an output projection)");
+        if (ride) {
+            NCTensor *h;
+            int act = c->ff_act == NNCP_FF_GELU ? NC_ACT_GELU : NC_ACT_RELU;
+            t0 = nc_matmul_add(nc_dup_tensor(tl->w_o), att, x, 0, 0, 1.0f);
+            h = nc_norm_linear_pair_into(t0, nc_dup_tensor(tl->ln_g1), nc_dup_tensor(tl->ln_b1), 1e-5f, is_ln,
+                                         nc_dup_tensor(tl->ff1), tl->ff_bias1 ? nc_dup_tensor(tl->ff_bias1) : NULL, act,
+                                         NULL, NULL, 0, &ff_in);
+            x = nc_linear_add(nc_dup_tensor(tl->ff2), h, tl->ff_bias2 ? nc_dup_tensor(tl->ff_bias2) : NULL,
+                              NC_ACT_NONE, ff_in);
+            pend = tl;
+            continue;
+        }
         int fold = !(c->ln_flags & NNCP_LN_COEF);
         int fold_ff = fold && (c->ff_act == NNCP_FF_GELU || c->ff_act == NNCP_FF_RELU);
         if (fold) {
@@ -702,7 +735,12 @@ NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
     }
     if (c->ln_flags & NNCP_LN_FINAL)
         x = layer_norm(s, x, s->ln_g, s->ln_b);
-    t0 = nc_linear(nc_dup_tensor(s->embed_out), x, s->out_bias ? nc_dup_tensor(s->out_bias) : NULL, NC_ACT_NONE);
+    if (pend)
+        t0 = nc_norm_linear_pair_into(x, nc_dup_tensor(pend->ln_g2), nc_dup_tensor(pend->ln_b2), 1e-5f, is_ln,
+                                      nc_dup_tensor(s->embed_out), s->out_bias ? nc_dup_tensor(s->out_bias) : NULL,
+                                      NC_ACT_NONE, NULL, NULL, 0, NULL);
+    else
+        t0 = nc_linear(nc_dup_tensor(s->embed_out), x, s->out_bias ? nc_dup_tensor(s->out_bias) : NULL, NC_ACT_NONE);
     t0 = nc_reshape_3d(t0, c->n_symbols, B, 1);
     nc_free_tensor(s->logits);
     s->logits = nc_dup_tensor(t0);

@@ -170,6 +170,30 @@ NCTensor *nc_linear_pair_into(NCTensor *w0, NCTensor *bias0, NCTensor *w1, NCTen
     return y0;
 }
 
+/* nc_ext.h: the norm that ends one block together with the first product(s) of the next,
+   stated with the plain ops */
+NCTensor *nc_norm_linear_pair_into(NCTensor *x, NCTensor *g, NCTensor *b, float eps, BOOL avg_flag,
+                                   NCTensor *w0, NCTensor *bias0, int act0,
+                                   NCTensor *w1, NCTensor *dst, int index, NCTensor **pnormed)
+{
+    NCTensor *normed, *y0;
+    if ((w1 == NULL) != (dst == NULL))
+        nc_fatal("nc_norm_linear_pair_into: w1 and dst go together");
+    normed = nc_fused_layer_norm(x, g, b, eps, avg_flag);
+    if (w1) {
+        if (act0 != NC_ACT_NONE)
+            nc_fatal("nc_norm_linear_pair_into: no activation on the first product of a pair");
+        y0 = nc_linear_pair_into(w0, bias0, w1, nc_dup_tensor(normed), dst, index);
+    } else {
+        y0 = nc_linear(w0, nc_dup_tensor(normed), bias0, act0);
+    }
+    if (pnormed)
+        *pnormed = normed;
+    else
+        nc_free_tensor(normed);
+    return y0;
+}
+
 NCTensor *nc_relpos_attention_step(NCTensor *q, NCTensor *kv_cache, NCTensor *kv_mem,
                                    NCTensor *w_r, NCTensor *b_r, int n_head, int d_key,
                                    int attn_len, float b_r_scale, int t)

@@ -97,4 +97,42 @@ for case in range(n_cases):
         assert np.abs(gp - np.swapaxes(pre, 1, 2)).max() / (np.abs(pre).max() + 1e-9) < 2e-5
     for p in (dA, dB, dC, dbias, dpre, dadd, ws):
         if p: lib.hipFree(p)
+# the few-column kernels of the width-invariant class (16x16x4 MFMA, vector ALU, 32x32x2 MFMA)
+# against the tile kernel, bit for bit, at exact-size operands
+lib.nchip_gemm_force_config(0)
+for case in range(max(4, n_cases // 8)):
+    m = 32 * int(rng.integers(1, 9)); n = int(rng.integers(1, 65)); k = 32 * int(rng.choice([1, 2, 3, 8, 9, 16, 24, 40, 72]))
+    lda, ldb, ldc = m + 4 * int(rng.integers(3)), k + 4 * int(rng.integers(3)), m + int(rng.choice([0, 1, 4]))
+    A = rng.standard_normal((k, lda)).astype(np.float32); Bm = rng.standard_normal((n, ldb)).astype(np.float32)
+    bias = rng.standard_normal(m).astype(np.float32); add = rng.standard_normal((n, ldc)).astype(np.float32)
+    use_bias, act, use_pre, use_add = int(rng.integers(2)), int(rng.integers(3)), int(rng.integers(2)), int(rng.integers(2))
+    dA, dB = dev(A), dev(Bm)
+    dbias = dev(bias) if use_bias else None
+    dadd = dev(add) if use_add else None
+    outs = []
+    for kernel in (0, 1, 2, 3):
+        lib.nchip_gemm_few_columns_kernel(kernel)
+        dC = dev(np.full((n, ldc), 9.0, np.float32)); dpre = dev(np.zeros((n, ldc), np.float32)) if use_pre else None
+        if use_add:
+            rc = lib.nchip_gemm_add(None, 0, 0, m, n, k, 1.0, dA, lda, 0, dB, ldb, 0, dC, ldc, 0, 1, dbias, act, dpre, dadd, 0x100, 1, None)
+        else:
+            rc = lib.nchip_gemm2(None, 0, 0, m, n, k, 1.0, dA, lda, 0, 0, dB, ldb, 0, 0, 0.0, dC, ldc, 0, 0, 1, 1, dbias, act, dpre, 0x100, 1, None)
+        assert rc == 0, rc
+        outs.append((back(dC, n * ldc), back(dpre, n * ldc) if use_pre else None))
+        for q in (dC, dpre):
+            if q: lib.hipFree(q)
+    lib.nchip_gemm_few_columns_kernel(3)
+    for o, pz in outs[1:]:
+        assert np.array_equal(o.view(np.uint32), outs[0][0].view(np.uint32)), ("few-column kernels differ", m, n, k, act, use_bias, use_add)
+        if use_pre: assert np.array_equal(pz.view(np.uint32), outs[0][1].view(np.uint32))
+    v = Bm[:, :k].astype(np.float64) @ A[:, :m].astype(np.float64)
+    if use_bias: v = v + bias[None, :]
+    if act == 1: v = 0.5 * v * (1 + np.tanh(0.7978845608 * (v + 0.044715 * v ** 3)))
+    elif act == 2: v = np.maximum(v, 0)
+    if use_add: v = v + add[:, :m]
+    got = outs[0][0].reshape(n, ldc)
+    assert np.abs(got[:, :m] - v).max() / (np.abs(v).max() + 1e-9) < 2e-5
+    if ldc > m: assert np.all(got[:, m:] == 9.0), "padding rows of C written"
+    for q in (dA, dB, dbias, dadd):
+        if q: lib.hipFree(q)
 print("ok: %d cases in %.1fs" % (n_cases, time.time() - t0))

@@ -71,10 +71,11 @@ def test_gemm_columns_do_not_depend_on_batch_width(hip, rng):
                                    (64, 288, 9), (32, 32, 1), (32, 2304, 64)])
 def test_few_column_products_are_the_wide_products_columns(hip, rng, m, k, n):
     """Width-invariant mode: a product with a few token columns (the decoder's per-timestep
-    shape, which takes the vector-ALU kernel: chains of fused multiply-adds in the order an
-    fp32 MFMA accumulates) equals, bit for bit, the same product through the MFMA few-column
-    kernel, through the tile kernel, and the matching columns of a wide product, with every
-    epilogue option the forward pass uses (bias, GELU, residual addend)."""
+    shape, which takes the 16x16x4 MFMA few-column kernel) equals, bit for bit, the same
+    product through the vector-ALU kernel (chains of fused multiply-adds in the order an fp32
+    MFMA accumulates), through the 32x32x2 MFMA few-column kernel, through the tile kernel, and
+    the matching columns of a wide product, with every epilogue option the forward pass uses
+    (bias, GELU, residual addend)."""
     lib = C.CDLL(hip.lib._name)
     w = rng.standard_normal((k, m)).astype(np.float32)
     wide = rng.standard_normal((200 + n, k)).astype(np.float32)
@@ -92,17 +93,17 @@ def test_few_column_products_are_the_wide_products_columns(hip, rng, m, k, n):
     try:
         whole = products(wide, res)
         few = products(wide[150:150 + n], res[150:150 + n])
-        lib.nchip_gemm_few_columns_kernel(1)
-        few_mfma = products(wide[150:150 + n], res[150:150 + n])
-        lib.nchip_gemm_few_columns_kernel(0)
-        few_tiles = products(wide[150:150 + n], res[150:150 + n])
+        others = []
+        for kernel in (2, 1, 0):
+            lib.nchip_gemm_few_columns_kernel(kernel)
+            others.append(products(wide[150:150 + n], res[150:150 + n]))
     finally:
-        lib.nchip_gemm_few_columns_kernel(2)
+        lib.nchip_gemm_few_columns_kernel(3)
         hip.nc_set_matmul_width_invariant(hip.ctx, 0)
-    for a, b, c, d in zip(whole, few, few_tiles, few_mfma):
+    for i, (a, b) in enumerate(zip(whole, few)):
         assert np.array_equal(a[150:150 + n], b)
-        assert np.array_equal(b, c)
-        assert np.array_equal(b, d)
+        for other in others:
+            assert np.array_equal(b, other[i])
     ref64 = wide[150:150 + n].astype(np.float64) @ w.astype(np.float64)
     assert relerr(few[0], ref64) <= TOL
 
@@ -408,6 +409,49 @@ def test_bias_gradient_model_shapes(hip, ref, rng, f, n):
 def _dev(nc, arr):
     t = nc.tensor(np.ascontiguousarray(arr, dtype=np.float32))
     return t, C.c_void_p(nc.lib.nc_tensor_get_ptr(t, None))
+
+
+@pytest.mark.parametrize("k,m0,m1,n,avg,act", [(512, 512, 1024, 32, 1, 0), (512, 2048, 0, 32, 1, 1), (512, 256, 0, 32, 1, 0),
+                                               (256, 64, 96, 5, 0, 0), (128, 96, 0, 64, 0, 2), (512, 64, 0, 17, 1, 1),
+                                               (192, 64, 32, 4, 1, 0)])
+def test_norm_riding_on_a_product(hip, ref, rng, k, m0, m1, n, avg, act):
+    """nc_norm_linear_pair_into: in width-invariant mode the one-launch kernel (k = 128, 256, 512)
+    gives the bits of nc_fused_layer_norm followed by nc_linear / nc_linear_pair_into - the
+    normalised tensor, the product(s) and the cache slot - and in every mode the values match
+    the checker's separate steps."""
+    T = 3
+    x = rng.standard_normal((n, k)).astype(np.float32) * 2 + 0.3
+    g = (1 + 0.2 * rng.standard_normal(k)).astype(np.float32); b = (0.1 * rng.standard_normal(k)).astype(np.float32)
+    w0 = rng.standard_normal((k, m0)).astype(np.float32); b0 = rng.standard_normal(m0).astype(np.float32)
+    w1 = rng.standard_normal((k, max(m1, 1))).astype(np.float32)
+    cache = rng.standard_normal((T, n, max(m1, 1))).astype(np.float32)
+    outs = {}
+    for name, nc, inv in (("inv", hip, 1), ("plain", hip, 0), ("ref", ref, 0)):
+        if nc is hip:
+            nc.nc_set_matmul_width_invariant(nc.ctx, inv)
+        dst = nc.tensor(cache)
+        pn = C.c_void_p()
+        y0 = nc.nc_norm_linear_pair_into(nc.tensor(x), nc.tensor(g), nc.tensor(b), 1e-5, avg, nc.tensor(w0), nc.tensor(b0), act,
+                                         nc.tensor(w1) if m1 else None, dst if m1 else None, T - 1, C.byref(pn))
+        outs[name] = (nc.numpy(y0, free=True), nc.numpy(pn, free=True), nc.numpy(dst, free=True))
+        if nc is hip and inv:
+            xn = nc.nc_fused_layer_norm(nc.tensor(x), nc.tensor(g), nc.tensor(b), 1e-5, avg)
+            xn_np = nc.numpy(xn)
+            y = nc.nc_linear(nc.tensor(w0), nc.nc_dup_tensor(xn), nc.tensor(b0), act)
+            y1 = nc.nc_matmul(nc.tensor(w1), xn) if m1 else None
+            outs["steps"] = (nc.numpy(y, free=True), xn_np, nc.numpy(y1, free=True) if m1 else None)
+            if not m1:
+                nc.nc_free_tensor(xn)
+        if nc is hip:
+            nc.nc_set_matmul_width_invariant(nc.ctx, 0)
+    assert np.array_equal(outs["inv"][1].view(np.uint32), outs["steps"][1].view(np.uint32))
+    assert np.array_equal(outs["inv"][0].view(np.uint32), outs["steps"][0].view(np.uint32))
+    if m1:
+        assert np.array_equal(outs["inv"][2][T - 1].view(np.uint32), outs["steps"][2].view(np.uint32))
+        assert np.array_equal(outs["inv"][2][:T - 1], cache[:T - 1])
+    for name in ("inv", "plain"):
+        for i in range(3 if m1 else 2):
+            assert relerr(outs[name][i], outs["ref"][i]) <= TOL, (name, i)
 
 
 @pytest.mark.parametrize("H,dk,B,T,M,d_pos,attn_len,has_w,t", [
