@@ -204,6 +204,10 @@ NCTensor *nncp_model_last_logits(NNCPModel *s);
 void trf_step_begin(NNCPModel *s);
 NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input);
 void trf_step_end(NNCPModel *s);
+/* until the next trf_step_begin / trf_step_end: trf_eval_step returns the logits (V, B, 1)
+   instead of the probabilities - for a caller that builds integer CDFs from them and has no
+   use for the softmax launch */
+void trf_step_logits_only(NNCPModel *s, int on);
 
 /* ---- block loop (process_block, nncp.c:2968-3147) ------------------------------ */
 #define NNCP_MODE_SEQ_EVAL 0   /* one trf_eval per timestep: decodable, as nncp c/d */

@@ -32,6 +32,8 @@ struct NNCPModel {
     NCTensor *ln_g, *ln_b, *embed, *embed_out, *out_bias;
     NCTensor **mem_h, **train_h, **outputs;
     NCTensor **step_kv, **step_kvm; /* per-timestep decoding: K/V of the segment so far, K/V of the memory */
+    NCTensor *step_embed_mult; /* the embedding scale as a device scalar, kept for the timesteps of a segment */
+    int step_logits_only;      /* trf_eval_step returns the logits: the caller builds integer CDFs from them */
     NCTensor *logits;
     NCSGDOptState *opt;
     int seq_eval;

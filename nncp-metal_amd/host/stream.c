@@ -165,6 +165,7 @@ static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int ful
     if (mode == NNCP_MODE_SEGMENT && c->step_decode) {
         /* decoder, one token column per timestep against the K/V caches */
         trf_step_begin(s);
+        trf_step_logits_only(s, c->coder == NNCP_CODER_CDF16); /* the CDFs come from the logits: no softmax launch */
         for (int t = 0; t < n_t; t++) {
             for (int b = 0; b < B; b++)
                 nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));

@@ -619,6 +619,8 @@ void trf_step_end(NNCPModel *s)
         nc_free_tensor(s->step_kv[l]); s->step_kv[l] = NULL;
         nc_free_tensor(s->step_kvm[l]); s->step_kvm[l] = NULL;
     }
+    nc_free_tensor(s->step_embed_mult); s->step_embed_mult = NULL;
+    s->step_logits_only = 0;
 }
 
 void trf_step_begin(NNCPModel *s)
@@ -637,6 +639,12 @@ void trf_step_begin(NNCPModel *s)
     for (int l = 0; l < c->n_layer; l++) /* zero: columns not yet reached are masked but must be finite */
         s->step_kv[l] = nc_new_tensor_3d(s->dev, NC_TYPE_F32, (size_t)c->n_head * (c->d_key + c->d_value),
                                          c->batch_size, c->seg_len);
+    s->step_embed_mult = scalar(s, s->embed_mult);
+}
+
+void trf_step_logits_only(NNCPModel *s, int on)
+{
+    s->step_logits_only = on;
 }
 
 NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
@@ -652,7 +660,7 @@ NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
     t0 = nc_tensor_to_device(t0, s->dev);
     t0 = nc_reshape_1d(t0, (size_t)B);
     x = nc_get_col(nc_dup_tensor(s->embed), t0);
-    x = nc_mul(x, scalar(s, s->embed_mult));
+    x = nc_mul(x, nc_dup_tensor(s->step_embed_mult));
     /* Post-norm blocks with a plain activation (nncp's default structure, nncp.c:2489-2513):
        a norm is followed by a product, so it rides on that product's launch
        (nc_norm_linear_pair_into) - the norm after the attention on the first feed-forward
@@ -744,6 +752,8 @@ NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
     t0 = nc_reshape_3d(t0, c->n_symbols, B, 1);
     nc_free_tensor(s->logits);
     s->logits = nc_dup_tensor(t0);
+    if (s->step_logits_only)
+        return t0;
     return nc_soft_max(t0);
 }
 
