@@ -70,6 +70,18 @@ NCTensor *nc_norm_linear_pair_into(NCTensor *x, NCTensor *g, NCTensor *b, float 
                                    NCTensor *w0, NCTensor *bias0, int act0,
                                    NCTensor *w1, NCTensor *dst, int index, NCTensor **pnormed);
 
+/* Keeps a k-major copy of the weight matrix w (m, k) until nc_forget_k_major_weights: forward
+   products with at most 64 columns in width-invariant fp32 mode whose left operand is w
+   (nc_matmul, nc_matmul_add, nc_linear, nc_linear_add, nc_linear_pair_into,
+   nc_norm_linear_pair_into) read the copy instead - the same arithmetic and the same bits;
+   such a product is bound by the cache lines it brings in, one per k for a matrix stored with
+   rows contiguous, a quarter of that for the copy.  The matrix is found by its address: w
+   must neither be written nor freed while the copy is kept (the decoder keeps copies of its
+   weights for the timesteps of a segment, between two training steps).  Does not consume w.
+   No counterpart in the reference. */
+void nc_keep_k_major_weight(NCTensor *w);
+void nc_forget_k_major_weights(NCContext *m);
+
 /* One query position of nc_relpos_attention: q (H*dk, B) is the query of
    position t, kv_cache (H*dk+H*dv, B, T) holds the keys / values of positions
    0..t of the current segment (later columns finite, e.g. zero), kv_mem, w_r,

@@ -132,13 +132,15 @@ int nchip_gemm_dact_rowsum(void *stream, int ta, int tb, int m, int n, int k, fl
    major, untransposed, bias pointers may be NULL (the per-timestep query and key/value
    projections of the decoder, nncp.c:801-812, whose second result goes straight into its
    cache slot).  The bits are those of two nchip_gemm calls with NCHIP_GEMM_WIDTH_INVARIANT.
+   a_k_major != 0: A0 and A1 are stored with k contiguous (element (i, kk) at A[kk + i * lda]: the
+   transposed copy of a weight matrix), which a quarter of the cache lines serves; same bits.
    Returns 0, 1 when the shapes are not the few-column kernel's (n <= 64, k and both m
    multiples of 32, 16-byte aligned operands; nothing was launched), negative on error. */
 int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, int k,
                                 const float *A0, int64_t lda0, const float *A1, int64_t lda1,
                                 const float *B, int64_t ldb,
                                 float *C0, int64_t ldc0, float *C1, int64_t ldc1,
-                                const float *bias0, const float *bias1);
+                                const float *bias0, const float *bias1, int a_k_major);
 
 /* One or two width-invariant few-column products of the layer norm (avg = 1) or RMS norm
    (avg = 0) of B's columns, in one launch: C0 (m0 x n) = act0(A0 norm(B) + bias0) and, when
@@ -147,13 +149,14 @@ int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, int k,
    written to ln_out (leading dimension ld_ln) when it is not NULL.  The decoder's timestep:
    the norm that ends one block (nncp.c:896-987, layer_norm of nncp.c:279-288) rides on the
    first product of the next.  The bits are those of nchip_norm_fwd followed by the products
-   with NCHIP_GEMM_WIDTH_INVARIANT.  Returns 0, 1 when the shapes are not this kernel's
-   (nothing was launched), negative on error. */
+   with NCHIP_GEMM_WIDTH_INVARIANT.  a_k_major as for nchip_gemm_pair_few_columns.  Returns 0, 1
+   when the shapes are not this kernel's (nothing was launched), negative on error. */
 int nchip_norm_gemm_few_columns(void *stream, const float *ln_w, const float *ln_b, float eps, int avg,
                                 float *ln_out, int64_t ld_ln, int m0, int m1, int n, int k,
                                 const float *A0, int64_t lda0, const float *A1, int64_t lda1,
                                 const float *B, int64_t ldb, float *C0, int64_t ldc0,
-                                float *C1, int64_t ldc1, const float *bias0, const float *bias1, int act0);
+                                float *C1, int64_t ldc1, const float *bias0, const float *bias1, int act0,
+                                int a_k_major);
 
 /* Testing aid: which kernel takes width-invariant fp32 products (NCHIP_GEMM_WIDTH_INVARIANT)
    with at most 64 columns, untransposed operands and beta = 0 (the decoder's per-timestep

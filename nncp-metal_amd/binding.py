@@ -115,6 +115,7 @@ _PROTOS = {
     "nc_linear": (_P, [_P, _P, _P, _I]),
     "nc_linear_add": (_P, [_P, _P, _P, _I, _P]),
     "nc_relpos_attention_step": (_P, [_P, _P, _P, _P, _P, _I, _I, _I, C.c_float, _I]),
+    "nc_keep_k_major_weight": (None, [_P]), "nc_forget_k_major_weights": (None, [_P]),
     "nc_norm_linear_pair_into": (_P, [_P, _P, _P, C.c_float, _I, _P, _P, _I, _P, _P, _I, C.POINTER(_P)]),
     "nc_linear_pair_into": (_P, [_P, _P, _P, _P, _P, _I]),
     "nc_set_matmul_width_invariant": (_I, [_P, _I]),

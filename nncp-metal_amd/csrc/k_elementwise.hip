@@ -338,9 +338,35 @@ __global__ void pad_bwd_kernel(const float *gy, float *gx, int64_t n_in, int64_t
     }
 }
 
+// dst (k-major copy) [i][kk] = src (m x k, rows contiguous) [kk][i]: 32 x 32 tiles through LDS,
+// reads and writes both coalesced
+__global__ __launch_bounds__(256) void transpose_f32_kernel(const float *src, float *dst, int m, int k)
+{
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 32 x 8
+    const int i0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int kk = k0 + ty + 8 * r, i = i0 + tx;
+        if (kk < k && i < m) tile[ty + 8 * r][tx] = src[(int64_t)kk * m + i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int i = i0 + ty + 8 * r, kk = k0 + tx;
+        if (i < m && kk < k) dst[(int64_t)i * k + kk] = tile[tx][ty + 8 * r];
+    }
+}
+
 } // namespace
 
 extern "C" {
+
+void k_transpose_f32(hipStream_t st, const float *src, float *dst, int m, int k)
+{
+    if (m > 0 && k > 0)
+        hipLaunchKernelGGL(transpose_f32_kernel, dim3((m + 31) / 32, (k + 31) / 32), dim3(256), 0, st, src, dst, m, k);
+}
 
 void k_copy_nd(hipStream_t st, const void *src, void *dst, const NdDesc *d, int esize)
 {

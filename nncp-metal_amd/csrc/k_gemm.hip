@@ -549,6 +549,18 @@ __global__ __launch_bounds__(256) void gemm_skinny_nn(GemmArgs g)
 // chunk); the loads of up to PF chunks are in flight from the start (K = 2048 whole), since
 // one memory round trip is longer than all the arithmetic.  Bias and addend are fetched
 // before the k loop.  alpha = 1, beta = 0, no activation gradient; M a multiple of 8.
+// Row tile of workgroup x of a few-column kernel.  Consecutive workgroups go to the eight XCDs
+// in turn, each with an L2 of its own, and a 128-byte line of A (32 rows of one k) spans R
+// row tiles: the R tiles that share lines are given to workgroups of one XCD (x, x + 8, ...),
+// so that a line is fetched into one L2 and not into R of them.
+__device__ __forceinline__ int fewcol_row_tile(int x, int ntiles, int R)
+{
+    const int span = 8 * R, group = x / span;
+    if ((group + 1) * span > ntiles) return x; // a last, partial group keeps its order
+    const int in = x - group * span, xcd = in & 7, r = in >> 3;
+    return group * span + xcd * R + r;
+}
+
 constexpr int FC_KC = 256, FC_RS = FC_KC + 4;
 template <int PF>
 __global__ __launch_bounds__(256) void gemm_fewcol_fma(GemmArgs g)
@@ -558,7 +570,7 @@ __global__ __launch_bounds__(256) void gemm_fewcol_fma(GemmArgs g)
     if (blockIdx.z == 1) { // the pair's second product: its own A, C, bias and row count
         g.A = g.A_1; g.C = g.C_1; g.bias = g.bias_1; g.lda = g.lda_1; g.ldc = g.ldc_1; g.M = g.M_1;
     }
-    const int m0 = blockIdx.x * 8, n0 = blockIdx.y * 8;
+    const int m0 = fewcol_row_tile(blockIdx.x, gridDim.x, 4) * 8, n0 = blockIdx.y * 8;
     if (m0 >= g.M) return; // (uniform: the grid covers the taller of the two products)
     const int ch = t & 3, ei = (t >> 2) & 7, ej = t >> 5; // chain, row and column of this thread's element
     const int nslab = g.K / 32, nch = (g.K + FC_KC - 1) / FC_KC;
@@ -668,10 +680,25 @@ __global__ __launch_bounds__(256) void gemm_fewcol_fma(GemmArgs g)
 // 4c..4c+3 of the tile before the k loop, the result kept whole in LDS (every workgroup
 // repeats it for its 16 columns, which costs less than a launch of its own); the first row
 // tile also writes the normalised columns out for the later consumers of that tensor.
-template <int PF, int NV = 0>
+//
+// TR = 8: tiles of 8 x 8 outputs on the same instruction (rows and columns 8-15 of the MFMA
+// tile repeat 0-7 and are not stored): four times the workgroups for a long reduction.  What
+// bounds these kernels there is not the chain (0.85 microseconds per 1024 k) nor LDS but the
+// cache lines a workgroup must bring in - one 128-byte line of A per k whatever the tile
+// height up to 32 rows - at the miss parallelism of one CU: 2.2-2.5 microseconds per 1024 k,
+// with warm or cold weights, in every form tried (also with the LDS reads of the next chunk
+// placed between the MFMAs of the current one, and with all chunks in flight).
+//
+// AK = 1: A is stored with k contiguous (lda between rows: a k-major copy of a weight matrix).
+// The lines a workgroup brings in for A are then TR x K/32 instead of K, which is what the
+// kernel is bound by; the arithmetic is the same.
+template <int PF, int NV = 0, int TR = 16, int AK = 0>
 __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
 {
-    constexpr int BST = 68, WSZ = 64 * 16 + (NV ? 0 : 16 * BST); // per wavefront: A [64 k][16 rows], B [16 columns][64 k]
+    static_assert(TR == 16 || (TR == 8 && NV == 0), "8 x 8 tiles: plain products only");
+    constexpr int NU = TR / 4; // 16-byte pieces per lane, chunk and operand
+    constexpr int BST = 68, ASZ = AK ? TR * BST : 64 * TR; // per wavefront: A [64 k][TR rows] (AK: [TR rows][64 k]), B [TR columns][64 k]
+    constexpr int WSZ = ASZ + (NV ? 0 : TR * BST);
     constexpr int XS = 64 * NV + 4;
     __shared__ __attribute__((aligned(16))) float stage[4][WSZ];
     __shared__ float red[3][4 * 64];
@@ -680,33 +707,36 @@ __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
     if (blockIdx.z == 1) { // the pair's second product: its own A, C, bias and row count
         g.A = g.A_1; g.C = g.C_1; g.bias = g.bias_1; g.lda = g.lda_1; g.ldc = g.ldc_1; g.M = g.M_1;
     }
-    const int m0 = blockIdx.x * 16, n0 = blockIdx.y * 16;
+    const int m0 = fewcol_row_tile(blockIdx.x, gridDim.x, 32 / TR) * TR, n0 = blockIdx.y * TR;
     if (m0 >= g.M) return; // (uniform: the grid covers the taller of the two products)
-    const int il = lane & 15, gq = lane >> 4;
+    const int il = lane & 15, gq = lane >> 4, it = il & (TR - 1); // (it: this lane's row / column of the tile)
     const int nslab = g.K / 32, nch = (g.K + 255) / 256;
-    float *As = stage[c], *Bs = As + 64 * 16;
-    // this lane's four 16-byte pieces of A (k_local = piece / 4, four rows) and of B
+    float *As = stage[c], *Bs = As + ASZ;
+    // this lane's NU 16-byte pieces of A (k_local = piece / NU, four rows) and of B
     // (column = piece / 16, slab = (piece % 16) / 2, half a chain's 8 k)
-    const float NCHIP_GLOBAL *Ab = as_global(g.A) + m0 + (lane & 3) * 4;
-    const float NCHIP_GLOBAL *Bb[4];
-    int a_k[4], b_k[4];
+    const float NCHIP_GLOBAL *Ab = as_global(g.A) + m0 + (lane & (NU - 1)) * 4;
+    const float NCHIP_GLOBAL *Ar[NU]; // AK: the row of each piece (pieces laid out as those of B)
+    const float NCHIP_GLOBAL *Bb[NU];
+    int a_k[NU], b_k[NU];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-        const int pa = lane + 64 * u, kl = pa >> 2;
+    for (int u = 0; u < NU; u++) {
+        const int pa = lane + 64 * u, kl = pa / NU;
         a_k[u] = 32 * (kl >> 3) + 8 * c + (kl & 7);
         const int pb = lane + 64 * u, colb = pb >> 4, kq = pb & 15;
         const int col = n0 + colb < g.N ? n0 + colb : g.N - 1;
         Bb[u] = as_global(g.B) + (int64_t)col * g.ldb;
         b_k[u] = 32 * (kq >> 1) + 8 * c + 4 * (kq & 1);
+        Ar[u] = as_global(g.A) + (int64_t)(m0 + colb) * g.lda;
     }
-    floatx4 ra[PF][4], rb[NV ? 1 : PF][4];
-    auto load = [&](floatx4 (&a)[4], floatx4 (&b)[4], int q) { // past the end: clamped, never used
+    floatx4 ra[PF][NU], rb[NV ? 1 : PF][NU];
+    auto load = [&](floatx4 (&a)[NU], floatx4 (&b)[NU], int q) { // past the end: clamped, never used
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < NU; u++) {
             int ka = q * 256 + a_k[u], kb = q * 256 + b_k[u];
             ka = ka < g.K ? ka : g.K - 1;
             kb = kb < g.K ? kb : g.K - 4;
-            a[u] = *reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(Ab + (int64_t)ka * g.lda);
+            if (AK) a[u] = *reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(Ar[u] + kb);
+            else a[u] = *reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(Ab + (int64_t)ka * g.lda);
             if (NV == 0) b[u] = *reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(Bb[u] + kb);
         }
     };
@@ -731,25 +761,25 @@ __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
         load(ra[j], rb[NV ? 0 : j], j);
         __builtin_amdgcn_sched_barrier(0); // oldest chunk first
     }
-    if (NV > 0) {
+    if constexpr (NV > 0) {
+        float hh[4][NV], yy[4][NV], rr[4];
+        norm_columns_reg<NV, 4>(xv, lw, lb, g.ln_w != nullptr, g.ln_eps, g.ln_avg, hh, yy, rr);
 #pragma unroll
         for (int cc = 0; cc < 4; cc++) {
             const int colb = 4 * c + cc;
-            float hh[NV ? NV : 1], yy[NV ? NV : 1];
-            norm_column_reg<(NV ? NV : 1)>(xv[cc], lw, lb, g.ln_w != nullptr, g.ln_eps, g.ln_avg, hh, yy);
 #pragma unroll
-            for (int v = 0; v < NV; v++) xn[colb * XS + lane + 64 * v] = yy[v];
+            for (int v = 0; v < NV; v++) xn[colb * XS + lane + 64 * v] = yy[cc][v];
             if (g.ln_out && blockIdx.x == 0 && blockIdx.z == 0 && n0 + colb < g.N) {
                 float NCHIP_GLOBAL *yo = as_global(g.ln_out) + (int64_t)(n0 + colb) * g.ld_ln + lane;
 #pragma unroll
-                for (int v = 0; v < NV; v++) yo[64 * v] = yy[v];
+                for (int v = 0; v < NV; v++) yo[64 * v] = yy[cc][v];
             }
         }
         __syncthreads();
     }
     // epilogue operands, fetched before the k loop (wavefront 0 finishes the tile)
     const int col = n0 + il;
-    const bool ok = col < g.N;
+    const bool ok = col < g.N && il < TR && gq < TR / 4; // (8 x 8 tiles: the repeated rows and columns are not stored)
     float NCHIP_GLOBAL *P = g.pre ? as_global(g.pre) : nullptr;
     const float NCHIP_GLOBAL *Radd = g.add ? as_global(g.add) : nullptr;
     const bool plain = !g.bias && !P && !Radd && g.act == NCHIP_ACT_NONE;
@@ -757,7 +787,7 @@ __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         const int row = m0 + 4 * gq + r;
-        bv[r] = (c == 0 && g.bias) ? as_global(g.bias)[row] : 0.0f;
+        bv[r] = (c == 0 && g.bias && gq < TR / 4) ? as_global(g.bias)[row] : 0.0f;
         extra[r] = (c == 0 && Radd && ok) ? Radd[(int64_t)col * g.ldc + row] : 0.0f;
     }
     floatx4 acc = { 0, 0, 0, 0 };
@@ -767,9 +797,10 @@ __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
             const int q = q0 + j;
             if (q < nch) { // uniform
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
+                for (int u = 0; u < NU; u++) {
                     const int pa = lane + 64 * u;
-                    *reinterpret_cast<floatx4 *>(As + (pa >> 2) * 16 + (pa & 3) * 4) = ra[j][u];
+                    if (AK) *reinterpret_cast<floatx4 *>(As + (pa >> 4) * BST + (pa & 15) * 4) = ra[j][u];
+                    else *reinterpret_cast<floatx4 *>(As + (pa / NU) * TR + (pa & (NU - 1)) * 4) = ra[j][u];
                     if (NV == 0) *reinterpret_cast<floatx4 *>(Bs + (pa >> 4) * BST + (pa & 15) * 4) = rb[j][u];
                 }
                 load(ra[j], rb[NV ? 0 : j], q + PF);
@@ -779,10 +810,10 @@ __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
                 float fa[16], fb[16];
 #pragma unroll
                 for (int e = 0; e < 16; e++) { // MFMA e of the chunk: slab e / 2, k_local = 4 e + gq
-                    fa[e] = As[(4 * e + gq) * 16 + il];
+                    fa[e] = AK ? As[it * BST + 4 * e + gq] : As[(4 * e + gq) * TR + it];
                     int kx = 256 * q + 32 * (e >> 1) + 8 * c + 4 * (e & 1) + gq;
                     kx = kx < g.K ? kx : g.K - 1; // (past a short last chunk: read, never used)
-                    fb[e] = NV ? xn[il * XS + kx] : Bs[il * BST + 4 * e + gq];
+                    fb[e] = NV ? xn[il * XS + kx] : Bs[it * BST + 4 * e + gq];
                 }
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier(); // the fragments are in registers: the corner may be rewritten
@@ -1339,12 +1370,26 @@ static void launch_fewcol_fma(const GemmArgs &g, dim3 grid, hipStream_t st)
     else hipLaunchKernelGGL(gemm_fewcol_fma<8>, grid, dim3(256), 0, st, g);
 }
 
-// (grid in 16 x 16 tiles)
-static void launch_fewcol_mfma(const GemmArgs &g, dim3 grid, hipStream_t st)
+// 16 x 16 tiles; 8 x 8 tiles from K = 1280 on (up to 8 chunks in flight) and, with a k-major A,
+// whenever 16 x 16 tiles would leave most CUs without a workgroup (mmax: the taller product
+// of the launch, nz: 1 or 2 products, ak: A is k-major)
+static void launch_fewcol_mfma(const GemmArgs &g, int mmax, int nz, hipStream_t st, bool ak = false)
 {
     const int nch = (g.K + 255) / 256;
-    if (nch <= 2) hipLaunchKernelGGL(gemm_fewcol_mfma<2>, grid, dim3(256), 0, st, g);
-    else hipLaunchKernelGGL(gemm_fewcol_mfma<4>, grid, dim3(256), 0, st, g);
+    const dim3 grid16(mmax / 16, (g.N + 15) / 16, nz), grid8(mmax / 8, (g.N + 7) / 8, nz);
+    const bool small = nch > 4 || (ak && grid16.x * grid16.y * grid16.z < 192);
+    if (!ak) {
+        if (small) hipLaunchKernelGGL((gemm_fewcol_mfma<8, 0, 8>), grid8, dim3(256), 0, st, g);
+        else if (nch <= 2) hipLaunchKernelGGL(gemm_fewcol_mfma<2>, grid16, dim3(256), 0, st, g);
+        else hipLaunchKernelGGL(gemm_fewcol_mfma<4>, grid16, dim3(256), 0, st, g);
+    } else if (small) {
+        if (nch <= 2) hipLaunchKernelGGL((gemm_fewcol_mfma<2, 0, 8, 1>), grid8, dim3(256), 0, st, g);
+        else if (nch <= 4) hipLaunchKernelGGL((gemm_fewcol_mfma<4, 0, 8, 1>), grid8, dim3(256), 0, st, g);
+        else hipLaunchKernelGGL((gemm_fewcol_mfma<8, 0, 8, 1>), grid8, dim3(256), 0, st, g);
+    } else {
+        if (nch <= 2) hipLaunchKernelGGL((gemm_fewcol_mfma<2, 0, 16, 1>), grid16, dim3(256), 0, st, g);
+        else hipLaunchKernelGGL((gemm_fewcol_mfma<4, 0, 16, 1>), grid16, dim3(256), 0, st, g);
+    }
 }
 int g_force_gm = -1;
 std::vector<ProfRec> g_prof;
@@ -1510,12 +1555,23 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
         rec.flops = 2.0 * m * n * (double)k * batch;
     }
     ProfRec *pr = g_prof_on ? &rec : nullptr;
+    if (invariant && g_skinny == 3 && ta && !tb && batch == 1 && precision == 0 && n <= 64 && k >= 32 && k % 32 == 0 &&
+        m % 32 == 0 && lda % 4 == 0 && ldb % 4 == 0 && (((uintptr_t)A | (uintptr_t)B) & 15) == 0 && beta == 0.0f &&
+        alpha == 1.0f && !dpre && !g_prof_on) {
+        // a few token columns against a k-major A (a weight matrix's transposed copy): same chains
+        launch_fewcol_mfma(g, m, 1, st, true);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            fprintf(stderr, "nchip_gemm: launch failed: %s\n", hipGetErrorString(e));
+            return -2;
+        }
+        return 0;
+    }
     if (invariant && g_skinny && !ta && !tb && batch == 1 && precision == 0 && n <= 64 && k >= 32 && k % 32 == 0 &&
         m % 32 == 0 && lda % 4 == 0 && ldb % 4 == 0 && (((uintptr_t)A | (uintptr_t)B) & 15) == 0 && beta == 0.0f && !g_prof_on) {
         // a few token columns: the same arithmetic without the tile pipeline
-        // (a long reduction keeps the vector-ALU kernel: four times the workgroups to stream its operands)
-        if (g_skinny == 3 && alpha == 1.0f && !dpre && k <= 1024)
-            launch_fewcol_mfma(g, dim3(m / 16, (n + 15) / 16), st);
+        if (g_skinny == 3 && alpha == 1.0f && !dpre)
+            launch_fewcol_mfma(g, m, 1, st);
         else if (g_skinny >= 2 && alpha == 1.0f && !dpre)
             launch_fewcol_fma(g, dim3(m / 8, (n + 7) / 8), st);
         else
@@ -1710,11 +1766,12 @@ extern "C" int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, 
                                            const float *A0, int64_t lda0, const float *A1, int64_t lda1,
                                            const float *B, int64_t ldb,
                                            float *C0, int64_t ldc0, float *C1, int64_t ldc1,
-                                           const float *bias0, const float *bias1)
+                                           const float *bias0, const float *bias1, int a_k_major)
 {
     if (m0 <= 0 || m1 <= 0 || n <= 0 || !A0 || !A1 || !B || !C0 || !C1) return -1;
+    if (a_k_major && g_skinny != 3) return 1;
     if (!g_skinny || g_prof_on || n > 64 || k < 32 || k % 32 || m0 % 32 || m1 % 32 || lda0 % 4 || lda1 % 4 || ldb % 4 ||
-        lda0 < m0 || lda1 < m1 || ldb < k || ldc0 < m0 || ldc1 < m1 ||
+        lda0 < (a_k_major ? k : m0) || lda1 < (a_k_major ? k : m1) || ldb < k || ldc0 < m0 || ldc1 < m1 ||
         (((uintptr_t)A0 | (uintptr_t)A1 | (uintptr_t)B) & 15) != 0)
         return 1;
     GemmArgs g;
@@ -1724,7 +1781,7 @@ extern "C" int nchip_gemm_pair_few_columns(void *stream, int m0, int m1, int n, 
     g.A_1 = A1; g.C_1 = C1; g.bias_1 = bias1; g.lda_1 = lda1; g.ldc_1 = ldc1; g.M_1 = m1;
     const int mmax = m0 > m1 ? m0 : m1;
     if (g_skinny == 3)
-        launch_fewcol_mfma(g, dim3(mmax / 16, (n + 15) / 16, 2), (hipStream_t)stream);
+        launch_fewcol_mfma(g, mmax, 2, (hipStream_t)stream, a_k_major != 0);
     else if (g_skinny == 2)
         launch_fewcol_fma(g, dim3(mmax / 8, (n + 7) / 8, 2), (hipStream_t)stream);
     else
@@ -1747,12 +1804,13 @@ extern "C" int nchip_norm_gemm_few_columns(void *stream, const float *ln_w, cons
                                            float *ln_out, int64_t ld_ln, int m0, int m1, int n, int k,
                                            const float *A0, int64_t lda0, const float *A1, int64_t lda1,
                                            const float *B, int64_t ldb, float *C0, int64_t ldc0,
-                                           float *C1, int64_t ldc1, const float *bias0, const float *bias1, int act0)
+                                           float *C1, int64_t ldc1, const float *bias0, const float *bias1, int act0,
+                                           int a_k_major)
 {
     if (m0 <= 0 || m1 < 0 || n <= 0 || !A0 || !B || !C0 || (m1 > 0 && (!A1 || !C1)) || (ln_w == nullptr) != (ln_b == nullptr))
         return -1;
     if (g_skinny != 3 || g_prof_on || n > 64 || (k != 128 && k != 256 && k != 512) || m0 % 32 || m1 % 32 || lda0 % 4 ||
-        (m1 > 0 && lda1 % 4) || lda0 < m0 || (m1 > 0 && lda1 < m1) || ldb < k || ldc0 < m0 || (m1 > 0 && ldc1 < m1) ||
+        (m1 > 0 && lda1 % 4) || lda0 < (a_k_major ? k : m0) || (m1 > 0 && lda1 < (a_k_major ? k : m1)) || ldb < k || ldc0 < m0 || (m1 > 0 && ldc1 < m1) ||
         (ln_out && ld_ln < k) || (((uintptr_t)A0 | (uintptr_t)A1) & 15) != 0 ||
         (act0 != NCHIP_ACT_NONE && act0 != NCHIP_ACT_GELU && act0 != NCHIP_ACT_RELU))
         return 1;
@@ -1765,7 +1823,11 @@ extern "C" int nchip_norm_gemm_few_columns(void *stream, const float *ln_w, cons
     const int mmax = m0 > m1 ? m0 : m1;
     const dim3 grid(mmax / 16, (n + 15) / 16, m1 > 0 ? 2 : 1);
     hipStream_t st = (hipStream_t)stream;
-    if (k == 128) hipLaunchKernelGGL((gemm_fewcol_mfma<2, 2>), grid, dim3(256), 0, st, g);
+    if (a_k_major) {
+        if (k == 128) hipLaunchKernelGGL((gemm_fewcol_mfma<2, 2, 16, 1>), grid, dim3(256), 0, st, g);
+        else if (k == 256) hipLaunchKernelGGL((gemm_fewcol_mfma<2, 4, 16, 1>), grid, dim3(256), 0, st, g);
+        else hipLaunchKernelGGL((gemm_fewcol_mfma<2, 8, 16, 1>), grid, dim3(256), 0, st, g);
+    } else if (k == 128) hipLaunchKernelGGL((gemm_fewcol_mfma<2, 2>), grid, dim3(256), 0, st, g);
     else if (k == 256) hipLaunchKernelGGL((gemm_fewcol_mfma<2, 4>), grid, dim3(256), 0, st, g);
     else hipLaunchKernelGGL((gemm_fewcol_mfma<2, 8>), grid, dim3(256), 0, st, g);
     if (hipGetLastError() != hipSuccess) {

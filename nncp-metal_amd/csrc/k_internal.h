@@ -25,6 +25,8 @@ extern "C" {
 void k_copy_nd(hipStream_t st, const void *src, void *dst, const NdDesc *d, int esize);
 // i32/i8/u16 -> f32 style conversions are not needed on the device path
 void k_fill_f32(hipStream_t st, float *p, float v, int64_t n);
+// dst[i*k + kk] = src[kk*m + i]: the k-major copy of an m x k matrix stored with rows contiguous
+void k_transpose_f32(hipStream_t st, const float *src, float *dst, int m, int k);
 void k_fill_bytes(hipStream_t st, void *p, int v, int64_t nbytes);
 // y[i] = a[i] op b[i % nb]   (b's shape is a prefix of a's)
 void k_binary_prefix(hipStream_t st, int op, const float *a, const float *b, float *y,

@@ -125,6 +125,7 @@ static void staging_reclaim(NCContext *m);
 extern "C" void nc_context_end(NCContext *m)
 {
     if (!m) return;
+    nc_forget_k_major_weights(m);
     if (m->hip_ready) {
         (void)hipStreamSynchronize(m->stream);
         m->sync_count++;

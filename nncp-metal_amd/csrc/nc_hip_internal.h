@@ -78,6 +78,8 @@ struct DeferredShared {
 
 // a pinned table that was released while its upload may still be queued
 struct StagingRetired { void *p; size_t cap; uint64_t stamp; };
+// a weight matrix (m x k, rows contiguous) and its k-major copy (nc_keep_k_major_weight)
+struct KMajorCopy { const float *src; size_t m, k; NCTensor *copy; };
 
 struct NCContext {
     int nb_threads;
@@ -104,6 +106,7 @@ struct NCContext {
     // one flush later, and only once the stream has been waited for since its
     // upload was enqueued (nc_staging_retire)
     std::vector<StagingRetired> staging_retired; // released tables the stream may still read
+    std::vector<KMajorCopy> k_major;             // copies the few-column products read instead of their weights
     void *grp_staging;
     size_t grp_staging_cap;
     uint64_t grp_staging_stamp;
@@ -180,6 +183,9 @@ static inline float *nc_f32(const NCTensor *x) { return (float *)nc_data(x); }
 void need_dev(const NCTensor *x, const char *op);
 NCContext *nc_ctx(const NCTensor *x);
 static inline hipStream_t nc_stream(const NCTensor *x) { return x->dev->ctx->stream; }
+// the k-major copy kept for the m x k matrix at `a`, or NULL
+const float *nc_k_major_of(const NCContext *m, const float *a, size_t rows, size_t k);
+extern "C" void nc_forget_k_major_weights(NCContext *m);
 float *nc_tmp_f32(NCContext *m, size_t n, size_t *cap); // pool scratch; give back with nc_tmp_free
 void nc_tmp_free(NCContext *m, void *p, size_t cap);
 NCTensor *nc_reshape_view(NCTensor *x, int nd, const size_t *dims); // consumes, no graph

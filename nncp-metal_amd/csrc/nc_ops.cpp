@@ -537,6 +537,38 @@ static MMShape mm_shape(const NCTensor *a, const NCTensor *b, bool ta, bool tb)
 // C (contiguous m x n per batch) = alpha op(A) op(B) + beta C [+ bias, act]
 // `addend` (laid out like C, or NULL) is added after the activation; beta must be 0 with it
 // forward: a product of the forward pass (honours nc_set_matmul_width_invariant)
+// ---- k-major copies of weight matrices (nc_ext.h) -----------------------------------------
+// A product with a few columns is bound by the cache lines its workgroups bring in; for a
+// matrix stored with rows contiguous that is one line per k and workgroup, for a k-major
+// copy a quarter of it.  The decoder keeps such copies of its weights for the timesteps of
+// a segment; the products find them by the address of the matrix.
+const float *nc_k_major_of(const NCContext *m, const float *a, size_t rows, size_t k)
+{
+    for (const KMajorCopy &e : m->k_major)
+        if (e.src == a && e.m == rows && e.k == k) return nc_f32(e.copy);
+    return nullptr;
+}
+
+extern "C" void nc_keep_k_major_weight(NCTensor *w)
+{
+    need_f32(w, "nc_keep_k_major_weight");
+    if (w->n_dims != 2 || !nc_is_contig(w)) nc_fatal("nc_keep_k_major_weight: a contiguous (m, k) matrix expected");
+    NCContext *m = nc_ctx(w);
+    const size_t rows = w->dims[0], k = w->dims[1];
+    if (nc_k_major_of(m, nc_f32(w), rows, k)) return;
+    size_t dims[2] = { k, rows };
+    NCTensor *copy = new_f32(w, 2, dims);
+    k_transpose_f32(m->stream, nc_f32(w), nc_f32(copy), (int)rows, (int)k);
+    m->launches++;
+    m->k_major.push_back(KMajorCopy{ nc_f32(w), rows, k, copy });
+}
+
+extern "C" void nc_forget_k_major_weights(NCContext *m)
+{
+    for (KMajorCopy &e : m->k_major) nc_free_tensor(e.copy);
+    m->k_major.clear();
+}
+
 static void dev_gemm(NCContext *m, bool ta, bool tb, size_t M, size_t N, size_t K, float alpha,
                      const NCTensor *a, const NCTensor *b, float beta, NCTensor *c, size_t batch,
                      const float *bias, int act, float *pre, const float *addend = nullptr,
@@ -549,15 +581,24 @@ static void dev_gemm(NCContext *m, bool ta, bool tb, size_t M, size_t N, size_t 
     float *ws = nullptr;
     if (ks > 1) ws = nc_tmp_f32(m, batch * ks * M * N, &cap);
     int rc;
+    // a few columns against a weight matrix with a k-major copy: the same chains from the copy
+    const float *a_data = nc_f32(a);
+    if (invariant && !ta && !tb && batch == 1 && !m->matmul_bf16 && N <= 64 && M % 32 == 0 && K % 32 == 0 && K >= 32 &&
+        alpha == 1.0f && beta == 0.0f && !m->k_major.empty()) {
+        if (const float *km = nc_k_major_of(m, a_data, M, K)) {
+            a_data = km;
+            ta = true;
+        }
+    }
     if (addend)
         rc = nchip_gemm_add(m->stream, ta, tb, (int)M, (int)N, (int)K, alpha,
-                            nc_f32(a), (int64_t)(ta ? K : M), (int64_t)(M * K),
+                            a_data, (int64_t)(ta ? K : M), (int64_t)(M * K),
                             nc_f32(b), (int64_t)(tb ? N : K), (int64_t)(K * N),
                             nc_f32(c), (int64_t)M, (int64_t)(M * N), (int)batch,
                             bias, act, pre, addend, prec, ks, ws);
     else
         rc = nchip_gemm(m->stream, ta, tb, (int)M, (int)N, (int)K, alpha,
-                        nc_f32(a), (int64_t)(ta ? K : M), (int64_t)(M * K),
+                        a_data, (int64_t)(ta ? K : M), (int64_t)(M * K),
                         nc_f32(b), (int64_t)(tb ? N : K), (int64_t)(K * N),
                         beta, nc_f32(c), (int64_t)M, (int64_t)(M * N), (int)batch,
                         bias, act, pre, prec, ks, ws);
@@ -765,10 +806,13 @@ extern "C" NCTensor *nc_linear_pair_into(NCTensor *w0, NCTensor *bias0, NCTensor
     NCTensor *y0 = new_f32(w0, 2, dims);
     float *slot = nc_f32(dst) + (size_t)index * m1 * n;
     int rc = 1;
-    if (m->matmul_invariant && !m->matmul_bf16)
-        rc = nchip_gemm_pair_few_columns(m->stream, (int)m0, (int)m1, (int)n, (int)k, nc_f32(w0), (int64_t)m0,
-                                         nc_f32(w1), (int64_t)m1, nc_f32(x), (int64_t)k, nc_f32(y0), (int64_t)m0,
-                                         slot, (int64_t)m1, bias0 ? nc_f32(bias0) : nullptr, nullptr);
+    if (m->matmul_invariant && !m->matmul_bf16) {
+        const float *k0 = nc_k_major_of(m, nc_f32(w0), m0, k), *k1 = nc_k_major_of(m, nc_f32(w1), m1, k);
+        const bool km = k0 && k1;
+        rc = nchip_gemm_pair_few_columns(m->stream, (int)m0, (int)m1, (int)n, (int)k, km ? k0 : nc_f32(w0), (int64_t)(km ? k : m0),
+                                         km ? k1 : nc_f32(w1), (int64_t)(km ? k : m1), nc_f32(x), (int64_t)k, nc_f32(y0), (int64_t)m0,
+                                         slot, (int64_t)m1, bias0 ? nc_f32(bias0) : nullptr, nullptr, km);
+    }
     if (rc < 0) nc_fatal("nc_linear_pair_into: kernel rejected the shapes");
     if (rc == 0) {
         m->launches++;
@@ -917,12 +961,16 @@ extern "C" NCTensor *nc_norm_linear_pair_into(NCTensor *x, NCTensor *g, NCTensor
         size_t d0[2] = { m0, n }, dn[2] = { k, n };
         y0 = new_f32(w0, 2, d0);
         if (pnormed) normed = new_f32(w0, 2, dn);
+        const float *k0 = nc_k_major_of(m, nc_f32(w0), m0, k), *k1 = w1 ? nc_k_major_of(m, nc_f32(w1), m1, k) : nullptr;
+        const bool km = k0 && (!w1 || k1);
         rc = nchip_norm_gemm_few_columns(m->stream, g ? nc_f32(g) : nullptr, b ? nc_f32(b) : nullptr, eps, avg_flag != 0,
                                          normed ? nc_f32(normed) : nullptr, (int64_t)k, (int)m0, (int)m1, (int)n, (int)k,
-                                         nc_f32(w0), (int64_t)m0, w1 ? nc_f32(w1) : nullptr, (int64_t)m1, nc_f32(x), (int64_t)k,
+                                         km ? k0 : nc_f32(w0), (int64_t)(km ? k : m0), w1 ? (km ? k1 : nc_f32(w1)) : nullptr,
+                                         (int64_t)(km ? k : m1), nc_f32(x), (int64_t)k,
                                          nc_f32(y0), (int64_t)m0, w1 ? nc_f32(dst) + (size_t)index * m1 * n : nullptr, (int64_t)m1,
                                          bias0 ? nc_f32(bias0) : nullptr, nullptr,
-                                         act0 == NC_ACT_GELU ? NCHIP_ACT_GELU : act0 == NC_ACT_RELU ? NCHIP_ACT_RELU : NCHIP_ACT_NONE);
+                                         act0 == NC_ACT_GELU ? NCHIP_ACT_GELU : act0 == NC_ACT_RELU ? NCHIP_ACT_RELU : NCHIP_ACT_NONE,
+                                         km);
         if (rc < 0) nc_fatal("%s: kernel rejected the shapes", me);
         if (rc != 0) {
             nc_free_tensor(y0); nc_free_tensor(normed);

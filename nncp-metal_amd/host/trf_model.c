@@ -621,6 +621,7 @@ void trf_step_end(NNCPModel *s)
     }
     nc_free_tensor(s->step_embed_mult); s->step_embed_mult = NULL;
     s->step_logits_only = 0;
+    nc_forget_k_major_weights(s->ctx);
 }
 
 void trf_step_begin(NNCPModel *s)
@@ -640,6 +641,17 @@ void trf_step_begin(NNCPModel *s)
         s->step_kv[l] = nc_new_tensor_3d(s->dev, NC_TYPE_F32, (size_t)c->n_head * (c->d_key + c->d_value),
                                          c->batch_size, c->seg_len);
     s->step_embed_mult = scalar(s, s->embed_mult);
+    /* the weights do not change until the training step that follows the last timestep: the
+       products of a timestep (a few token columns each) read k-major copies of them */
+    for (int l = 0; l < c->n_layer; l++) {
+        Layer *tl = &s->layers[l];
+        nc_keep_k_major_weight(tl->w_q);
+        nc_keep_k_major_weight(tl->w_kv);
+        if (tl->w_o) nc_keep_k_major_weight(tl->w_o);
+        nc_keep_k_major_weight(tl->ff1);
+        nc_keep_k_major_weight(tl->ff2);
+    }
+    nc_keep_k_major_weight(s->embed_out);
 }
 
 void trf_step_logits_only(NNCPModel *s, int on)

@@ -170,6 +170,17 @@ NCTensor *nc_linear_pair_into(NCTensor *w0, NCTensor *bias0, NCTensor *w1, NCTen
     return y0;
 }
 
+/* nc_ext.h: a layout hint for the GPU library's few-column products; nothing to do here */
+void nc_keep_k_major_weight(NCTensor *w)
+{
+    (void)w;
+}
+
+void nc_forget_k_major_weights(NCContext *m)
+{
+    (void)m;
+}
+
 /* nc_ext.h: the norm that ends one block together with the first product(s) of the next,
    stated with the plain ops */
 NCTensor *nc_norm_linear_pair_into(NCTensor *x, NCTensor *g, NCTensor *b, float eps, BOOL avg_flag,

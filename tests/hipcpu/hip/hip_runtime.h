@@ -147,6 +147,7 @@ static void hipcpu_launch_impl(F kernel, dim3 grid, dim3 block, size_t shmem, A.
 #define __syncthreads() hipcpu_syncthreads()
 #define __builtin_amdgcn_wave_barrier() hipcpu_wave_barrier()
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
+#define __builtin_amdgcn_sched_group_barrier(mask, size, id) ((void)0)
 #define __builtin_amdgcn_fence(...) ((void)0)
 #define __builtin_amdgcn_s_setprio(x) ((void)0)
 static inline long long clock64(void) { return 0; }

@@ -411,6 +411,50 @@ def _dev(nc, arr):
     return t, C.c_void_p(nc.lib.nc_tensor_get_ptr(t, None))
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 512, 32), (2048, 512, 32), (512, 2048, 32), (256, 512, 5), (64, 96, 64),
+                                   (1024, 1024, 33), (32, 4096, 8), (96, 288, 16)])
+def test_k_major_weight_copies_change_no_bit(hip, rng, m, k, n):
+    """nc_keep_k_major_weight: the few-column products of the width-invariant class read a
+    k-major copy of their weight matrix (a quarter of the cache lines) and write the bits they
+    write from the matrix itself - plain, with bias and GELU, with a residual, as a pair into a
+    cache slot, and behind a norm."""
+    w = hip.tensor(rng.standard_normal((k, m)).astype(np.float32))
+    w1 = hip.tensor(rng.standard_normal((k, 2 * m)).astype(np.float32))
+    x = rng.standard_normal((n, k)).astype(np.float32)
+    bias = rng.standard_normal(m).astype(np.float32); res = rng.standard_normal((n, m)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32); b = (0.1 * rng.standard_normal(k)).astype(np.float32)
+    cache = rng.standard_normal((2, n, 2 * m)).astype(np.float32)
+    d, t = hip.dup, hip.tensor
+
+    def products():
+        outs = [hip.numpy(hip.nc_matmul(d(w), t(x)), free=True),
+                hip.numpy(hip.nc_linear(d(w), t(x), t(bias), 1), free=True),
+                hip.numpy(hip.nc_linear_add(d(w), t(x), t(bias), 0, t(res)), free=True),
+                hip.numpy(hip.nc_matmul_add(d(w), t(x), t(res), 0, 0, 1.0), free=True)]
+        dst = t(cache)
+        outs.append(hip.numpy(hip.nc_linear_pair_into(d(w), t(bias), d(w1), t(x), dst, 1), free=True))
+        outs.append(hip.numpy(dst, free=True))
+        dst = t(cache)
+        pn = C.c_void_p()
+        outs.append(hip.numpy(hip.nc_norm_linear_pair_into(t(x), t(g), t(b), 1e-5, 1, d(w), t(bias), 0, d(w1), dst, 0, C.byref(pn)), free=True))
+        outs.append(hip.numpy(dst, free=True)); outs.append(hip.numpy(pn, free=True))
+        return outs
+    hip.nc_set_matmul_width_invariant(hip.ctx, 1)
+    try:
+        plain = products()
+        hip.nc_keep_k_major_weight(w); hip.nc_keep_k_major_weight(w1)
+        kept = products()
+        hip.nc_forget_k_major_weights(hip.ctx)
+        again = products()
+    finally:
+        hip.nc_forget_k_major_weights(hip.ctx)
+        hip.nc_set_matmul_width_invariant(hip.ctx, 0)
+        hip.free(w, w1)
+    for a, b_, c in zip(plain, kept, again):
+        assert np.array_equal(a.view(np.uint32), b_.view(np.uint32))
+        assert np.array_equal(a.view(np.uint32), c.view(np.uint32))
+
+
 @pytest.mark.parametrize("k,m0,m1,n,avg,act", [(512, 512, 1024, 32, 1, 0), (512, 2048, 0, 32, 1, 1), (512, 256, 0, 32, 1, 0),
                                                (256, 64, 96, 5, 0, 0), (128, 96, 0, 64, 0, 2), (512, 64, 0, 17, 1, 1),
                                                (192, 64, 32, 4, 1, 0)])
