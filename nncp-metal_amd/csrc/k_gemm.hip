@@ -682,12 +682,12 @@ __global__ __launch_bounds__(256) void gemm_fewcol_fma(GemmArgs g)
 // tile also writes the normalised columns out for the later consumers of that tensor.
 //
 // TR = 8: tiles of 8 x 8 outputs on the same instruction (rows and columns 8-15 of the MFMA
-// tile repeat 0-7 and are not stored): four times the workgroups for a long reduction.  What
-// bounds these kernels there is not the chain (0.85 microseconds per 1024 k) nor LDS but the
-// cache lines a workgroup must bring in - one 128-byte line of A per k whatever the tile
-// height up to 32 rows - at the miss parallelism of one CU: 2.2-2.5 microseconds per 1024 k,
-// with warm or cold weights, in every form tried (also with the LDS reads of the next chunk
-// placed between the MFMAs of the current one, and with all chunks in flight).
+// tile repeat 0-7 and are not stored): four times the workgroups, for a long reduction and for
+// products that would otherwise leave most CUs idle.  What bounds these kernels is not the
+// chain (0.85 microseconds per 1024 k) but the 128-byte lines a workgroup must bring in, at
+// about 0.4 lines per nanosecond and CU, with warm or cold weights alike: a launch costs about
+// 2.6 microseconds plus 2.3 nanoseconds per line of its busiest workgroup.  With A stored
+// rows-contiguous that is one line of A per k whatever the tile height up to 32 rows.
 //
 // AK = 1: A is stored with k contiguous (lda between rows: a k-major copy of a weight matrix).
 // The lines a workgroup brings in for A are then TR x K/32 instead of K, which is what the

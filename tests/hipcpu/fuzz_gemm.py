@@ -122,6 +122,19 @@ for case in range(max(4, n_cases // 8)):
         for q in (dC, dpre):
             if q: lib.hipFree(q)
     lib.nchip_gemm_few_columns_kernel(3)
+    # the same product from a k-major copy of A (element (i, kk) at kk + i * ldat), exact size
+    ldat = k + 4 * int(rng.integers(3))
+    At = np.zeros((m, ldat), np.float32); At[:, :k] = A[:, :m].T
+    dAt = dev(At)
+    dC = dev(np.full((n, ldc), 9.0, np.float32)); dpre = dev(np.zeros((n, ldc), np.float32)) if use_pre else None
+    if use_add:
+        rc = lib.nchip_gemm_add(None, 1, 0, m, n, k, 1.0, dAt, ldat, 0, dB, ldb, 0, dC, ldc, 0, 1, dbias, act, dpre, dadd, 0x100, 1, None)
+    else:
+        rc = lib.nchip_gemm2(None, 1, 0, m, n, k, 1.0, dAt, ldat, 0, 0, dB, ldb, 0, 0, 0.0, dC, ldc, 0, 0, 1, 1, dbias, act, dpre, 0x100, 1, None)
+    assert rc == 0, rc
+    outs.append((back(dC, n * ldc), back(dpre, n * ldc) if use_pre else None))
+    for q in (dC, dpre, dAt):
+        if q: lib.hipFree(q)
     for o, pz in outs[1:]:
         assert np.array_equal(o.view(np.uint32), outs[0][0].view(np.uint32)), ("few-column kernels differ", m, n, k, act, use_bias, use_add)
         if use_pre: assert np.array_equal(pz.view(np.uint32), outs[0][1].view(np.uint32))
