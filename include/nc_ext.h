@@ -109,6 +109,18 @@ int nc_set_matmul_width_invariant(NCContext *m, int enable);
      cdf[i] = floor(Q_i * (65536 - V) / Q_V) + i.                          */
 NCTensor *nc_soft_max_cdf16(NCTensor *logits);
 
+/* nc_soft_max_cdf16 with the result on the host device, written there by the kernel itself
+   (pinned memory): for a few columns - a decoder timestep - this saves the launch and the
+   latency of a copy.  The contents are valid after the next nc_synchronize of the logits'
+   device.  Same values.  No counterpart in the reference. */
+NCTensor *nc_soft_max_cdf16_to_host(NCTensor *logits);
+
+/* nc_get_col (libnc.h:374-375) with the contiguous i32 indices x on the host device, read
+   by the kernel itself from pinned memory instead of being uploaded first (a decoder
+   timestep's tokens).  x must not change until the device has been synchronised.  Consumes
+   w and x.  No gradient.  No counterpart in the reference. */
+NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x);
+
 /* cdf (V, n) U16, targets (m, n) U16 -> (m, n) U16 symbols: the largest s
    with cdf[s, col] <= target (cumulative-frequency search of a decoder). */
 NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets);

@@ -1177,8 +1177,8 @@ void relpos_attn_bwd_tiled(FusedAttnBwdArgs a)
 // it (lane g: keys 16 jt + 4g + r in increasing order, then (s0 + s1) + (s2 + s3)); output
 // feature d is one chain over the keys in the order the PV MFMAs meet them (tile jt, step r,
 // k slot g: key 16 jt + 4g + r).  Masked keys contribute exact zeros there and are skipped.
-// A workgroup of 128 threads is one (stream, head): thread j owns key j (only keys inside
-// the attention window are fetched), then thread d owns output feature d.
+// A workgroup is one (stream, head): four neighbouring lanes own a key (only keys inside the
+// attention window are fetched), then thread d owns output feature d.
 // a product that is rounded on its own (the whole-segment kernel keeps the scaled bias in
 // LDS, so no multiply-add can swallow it)
 __device__ __forceinline__ float rounded_product(float x, float y)
@@ -1188,94 +1188,109 @@ __device__ __forceinline__ float rounded_product(float x, float y)
 }
 
 template <int DK>
-__global__ __launch_bounds__(128) void relpos_attn_step_scalar(FusedAttnFwdArgs a)
+__global__ __launch_bounds__(512) void relpos_attn_step_scalar(FusedAttnFwdArgs a)
 {
-    constexpr int RS = DK + 4, NS = DK / 4;
+    constexpr int RS = DK + 4, NS = DK / 4, QP = NS / 4; // QP: 16-byte pieces of a row per lane
     __shared__ __attribute__((aligned(16))) float Vs[128 * RS];
     __shared__ __attribute__((aligned(16))) float qs[DK];
     __shared__ __attribute__((aligned(16))) float es[128];
     __shared__ float red[4];
-    const int j = threadIdx.x;
+    // four neighbouring lanes share a key: each fetches a quarter of its rows (a wavefront's
+    // load then touches 16 rows instead of 64) and the chain over the features passes from
+    // quarter to quarter
+    const int t = threadIdx.x, j = t >> 2, sq = t & 3;
     const int b = blockIdx.x % a.B, h = blockIdx.x / a.B;
     const int i = a.q_only;
     const int delta = i + a.M - j;
     const bool valid = j < a.K && (unsigned)delta < (unsigned)a.attn_len;
     const bool has_w = a.w_r != nullptr;
-    floatx4_t kr[NS], vr[NS], wr[NS];
+    floatx4_t kr[QP], vr[QP], wr[QP];
     float bias_t = 0.0f;
     if (valid) {
         const float *row = (j < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * j)
-                                    : a.kv + a.ldkv * (b + (int64_t)a.B * (j - a.M))) + (int64_t)h * DK;
+                                    : a.kv + a.ldkv * (b + (int64_t)a.B * (j - a.M))) + (int64_t)h * DK + 4 * QP * sq;
         const floatx4_t NCHIP_GLOBAL *kp = reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(as_global(row));
         const floatx4_t NCHIP_GLOBAL *vp = reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(as_global(row + (int64_t)a.H * DK));
 #pragma unroll
-        for (int s = 0; s < NS; s++) kr[s] = kp[s];
+        for (int p = 0; p < QP; p++) kr[p] = kp[p];
         if (has_w) {
             int pi = a.d_pos - 1 - delta;
             pi = pi < 0 ? 0 : pi; // (delta >= 0: never above d_pos - 1)
             const floatx4_t NCHIP_GLOBAL *wp = reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(
-                as_global(a.w_r + ((int64_t)h * a.d_pos + pi) * DK));
+                as_global(a.w_r + ((int64_t)h * a.d_pos + pi) * DK + 4 * QP * sq));
 #pragma unroll
-            for (int s = 0; s < NS; s++) wr[s] = wp[s];
+            for (int p = 0; p < QP; p++) wr[p] = wp[p];
         }
 #pragma unroll
-        for (int s = 0; s < NS; s++) vr[s] = vp[s];
-        if (a.b_r) bias_t = as_global(a.b_r)[(int64_t)h * a.K + (a.K - 1 - delta)];
+        for (int p = 0; p < QP; p++) vr[p] = vp[p];
+        if (a.b_r && sq == 3) bias_t = as_global(a.b_r)[(int64_t)h * a.K + (a.K - 1 - delta)];
     }
-    if (j < NS) {
-        floatx4_t q4 = *reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(as_global(a.q + (int64_t)h * DK + a.ldq * b) + 4 * j);
+    if (t < NS) {
+        floatx4_t q4 = *reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(as_global(a.q + (int64_t)h * DK + a.ldq * b) + 4 * t);
 #pragma unroll
-        for (int r = 0; r < 4; r++) qs[4 * j + r] = q4[r] * a.scale; // 1/sqrt(dk) folded in
+        for (int r = 0; r < 4; r++) qs[4 * t + r] = q4[r] * a.scale; // 1/sqrt(dk) folded in
     }
     __syncthreads();
-    float v = -INFINITY;
-    if (valid) {
-        float sc = 0.0f, rl = 0.0f;
+    float sc = 0.0f, rl = 0.0f;
 #pragma unroll
-        for (int s = 0; s < NS; s++) {
-            const floatx4_t q4 = *reinterpret_cast<const floatx4_t *>(qs + 4 * s);
+    for (int r = 0; r < 4; r++) { // quarter r of the features, by the lane that holds it
+        if (sq == r && valid) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) sc = __builtin_fmaf(kr[s][r], q4[r], sc);
-            if (has_w) {
+            for (int p = 0; p < QP; p++) {
+                const floatx4_t q4 = *reinterpret_cast<const floatx4_t *>(qs + 4 * (r * QP + p));
 #pragma unroll
-                for (int r = 0; r < 4; r++) rl = __builtin_fmaf(wr[s][r], q4[r], rl);
+                for (int e = 0; e < 4; e++) sc = __builtin_fmaf(kr[p][e], q4[e], sc);
+                if (has_w) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) rl = __builtin_fmaf(wr[p][e], q4[e], rl);
+                }
             }
         }
-        v = sc + rl + rounded_product(bias_t, a.b_r_scale * a.scale);
+        if (r < 3) { // the chains so far go to the lane of the next quarter
+            const float sc_up = __shfl_up(sc, 1, 64), rl_up = __shfl_up(rl, 1, 64);
+            if (sq == r + 1) { sc = sc_up; rl = rl_up; }
+        }
+    }
+    if (valid) {
 #pragma unroll
-        for (int s = 0; s < NS; s++) *reinterpret_cast<floatx4_t *>(Vs + j * RS + 4 * s) = vr[s];
+        for (int p = 0; p < QP; p++) *reinterpret_cast<floatx4_t *>(Vs + j * RS + 4 * (QP * sq + p)) = vr[p];
+        if (sq == 3) es[j] = sc + rl + rounded_product(bias_t, a.b_r_scale * a.scale);
     } else { // a masked key's probability is an exact zero: its value row must only be finite
 #pragma unroll
-        for (int s = 0; s < NS; s++) *reinterpret_cast<floatx4_t *>(Vs + j * RS + 4 * s) = floatx4_t{ 0, 0, 0, 0 };
+        for (int p = 0; p < QP; p++) *reinterpret_cast<floatx4_t *>(Vs + j * RS + 4 * (QP * sq + p)) = floatx4_t{ 0, 0, 0, 0 };
+        if (sq == 3) es[j] = -INFINITY;
     }
+    __syncthreads();
+    // from here on thread k < 128 is key k (then output feature k)
+    const float v = t < 128 ? es[t] : -INFINITY;
     // maximum over the keys (exact in any order)
     float mx = v;
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-    if ((j & 63) == 0) red[j >> 6] = mx;
+    if ((t & 63) == 0 && t < 128) red[t >> 6] = mx;
     __syncthreads();
     mx = fmaxf(red[0], red[1]);
     if (mx == -INFINITY) mx = 0.0f;
     const float e = __expf(v - mx); // exp(-inf) = 0 for masked keys
-    es[j] = e;
+    if (t < 128) es[t] = e;
     __syncthreads();
-    if (j < 4) { // the partial sum lane group g of the column holds in the whole-segment kernel
+    if (t < 4) { // the partial sum lane group g of the column holds in the whole-segment kernel
         floatx4_t e4[8];
 #pragma unroll
-        for (int jt = 0; jt < 8; jt++) e4[jt] = *reinterpret_cast<const floatx4_t *>(es + jt * 16 + 4 * j);
+        for (int jt = 0; jt < 8; jt++) e4[jt] = *reinterpret_cast<const floatx4_t *>(es + jt * 16 + 4 * t);
         float sum = 0.0f;
 #pragma unroll
         for (int jt = 0; jt < 8; jt++)
 #pragma unroll
             for (int r = 0; r < 4; r++) sum += e4[jt][r];
-        red[j] = sum;
+        red[t] = sum;
     }
     __syncthreads();
     const float sum = (red[0] + red[1]) + (red[2] + red[3]);
     const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
-    es[j] = e * inv; // (every thread read its own e above; the sums are done)
+    if (t < 128) es[t] = e * inv; // (every thread read its own e above; the sums are done)
     __syncthreads();
-    if (j < DK) {
+    if (t < DK) {
         const int j_hi = i + a.M, j_lo = j_hi - a.attn_len + 1; // keys inside the window (uniform)
         float acc = 0.0f;
         for (int jt = 0; jt < 8; jt++) {
@@ -1285,13 +1300,13 @@ __global__ __launch_bounds__(128) void relpos_attn_step_scalar(FusedAttnFwdArgs 
 #pragma unroll
             for (int g = 0; g < 4; g++) p4[g] = *reinterpret_cast<const floatx4_t *>(es + jt * 16 + 4 * g);
 #pragma unroll
-            for (int u = 0; u < 16; u++) vv[u] = Vs[(jt * 16 + u) * RS + j];
+            for (int u = 0; u < 16; u++) vv[u] = Vs[(jt * 16 + u) * RS + t];
 #pragma unroll
             for (int r = 0; r < 4; r++)
 #pragma unroll
                 for (int g = 0; g < 4; g++) acc = __builtin_fmaf(vv[4 * g + r], p4[g][r], acc);
         }
-        as_global(a.out)[(int64_t)h * DK + j + a.ldo * b] = acc;
+        as_global(a.out)[(int64_t)h * DK + t + a.ldo * b] = acc;
     }
 }
 
@@ -1399,8 +1414,8 @@ extern "C" void nchip_relpos_attn_step_kernel(int scalar)
 int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk)
 {
     if (a.q_only >= 0 && g_attn_step_scalar && a.K <= 128 && a.d_pos <= 128 && !a.probs) {
-        if (dk == 64) hipLaunchKernelGGL(relpos_attn_step_scalar<64>, dim3(a.B * a.H), dim3(128), 0, st, a);
-        else hipLaunchKernelGGL(relpos_attn_step_scalar<32>, dim3(a.B * a.H), dim3(128), 0, st, a);
+        if (dk == 64) hipLaunchKernelGGL(relpos_attn_step_scalar<64>, dim3(a.B * a.H), dim3(512), 0, st, a);
+        else hipLaunchKernelGGL(relpos_attn_step_scalar<32>, dim3(a.B * a.H), dim3(512), 0, st, a);
         return hipGetLastError() == hipSuccess ? 0 : -1;
     }
     if (const int ntt = (a.K > 128 || a.d_pos > 128) ? tiled_ntt(a.K, a.d_pos) : 0) {

@@ -849,6 +849,25 @@ extern "C" NCTensor *nc_get_col(NCTensor *w, NCTensor *x) // libnc.h:374-375
     return y;
 }
 
+// nc_ext.h: nc_get_col with the indices read by the kernel straight from pinned host memory
+// (a decoder timestep's 32 tokens: an upload of their own costs a launch and its latency).
+// The index tensor must stay as it is until the stream has been waited for.  No gradient.
+extern "C" NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x)
+{
+    w = nc_contig(w);
+    need_f32(w, "nc_get_col_host_indices");
+    if (x->dev->is_hip || x->type != NC_TYPE_I32 || !nc_is_contig(x) || w->n_dims != 2)
+        nc_fatal("nc_get_col_host_indices: (D,V) f32 matrix on the GPU and contiguous i32 indices on the host expected");
+    size_t dims[2] = { w->dims[0], nc_numel(x) };
+    NCTensor *y = new_f32(w, 2, dims);
+    if (nchip_get_col(nc_stream(w), nc_f32(w), (const int32_t *)nc_data(x), nc_f32(y), (int)dims[0],
+                      (int)w->dims[1], (int64_t)dims[1]))
+        nc_fatal("nc_get_col_host_indices failed");
+    LAUNCHED(w);
+    nc_free_tensor(w); nc_free_tensor(x);
+    return y;
+}
+
 extern "C" NCTensor *nc_soft_max(NCTensor *x) // libnc.h:382
 {
     x = nc_contig(x);
@@ -1166,6 +1185,23 @@ extern "C" NCTensor *nc_soft_max_cdf16(NCTensor *logits)
                             (int64_t)(nc_numel(logits) / v)))
         nc_fatal("nc_soft_max_cdf16 failed");
     LAUNCHED(logits);
+    nc_free_tensor(logits);
+    return y;
+}
+
+// nc_ext.h: the same CDFs written by the kernel straight into pinned host memory (the rows
+// of a decoder timestep are 16 KB: a copy of their own costs a launch and its latency).  The
+// tensor is on the host device; its contents are there after the next nc_synchronize.
+extern "C" NCTensor *nc_soft_max_cdf16_to_host(NCTensor *logits)
+{
+    logits = nc_contig(logits);
+    need_f32(logits, "nc_soft_max_cdf16_to_host");
+    NCContext *m = nc_ctx(logits);
+    size_t v = logits->dims[0];
+    NCTensor *y = nc_alloc(&m->cpu, NC_TYPE_U16, logits->n_dims, logits->dims, false);
+    if (nchip_softmax_cdf16(m->stream, nc_f32(logits), (uint16_t *)nc_data(y), (int)v, (int64_t)(nc_numel(logits) / v)))
+        nc_fatal("nc_soft_max_cdf16_to_host failed");
+    m->launches++;
     nc_free_tensor(logits);
     return y;
 }

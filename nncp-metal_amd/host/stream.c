@@ -80,9 +80,18 @@ static HostDist fetch_dist(Coder *c, NCTensor *output)
     HostDist d;
     memset(&d, 0, sizeof(d));
     if (c->coder == NNCP_CODER_CDF16) {
-        NCTensor *cdf = nc_soft_max_cdf16(nc_dup_tensor(c->cls->last_logits(c->s)));
+        NCTensor *logits = c->cls->last_logits(c->s);
+        size_t dims[NC_N_DIMS_MAX], cols = 1;
+        int nd = nc_tensor_get_dims(logits, dims);
+        for (int i = 1; i < nd; i++) cols *= dims[i];
         nc_free_tensor(output);
-        d.host = nc_tensor_to_cpu_device(cdf);
+        if (cols <= 64) { /* a timestep's rows: the kernel writes them to the host itself */
+            NCDevice *dev = nc_get_tensor_device(logits);
+            d.host = nc_soft_max_cdf16_to_host(nc_dup_tensor(logits));
+            nc_synchronize(dev);
+        } else {
+            d.host = nc_tensor_to_cpu_device(nc_soft_max_cdf16(nc_dup_tensor(logits)));
+        }
         d.cdf = nc_tensor_get_ptr(d.host, &d.stride);
     } else {
         d.host = nc_tensor_to_cpu_device(output);

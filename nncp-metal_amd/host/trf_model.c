@@ -669,9 +669,11 @@ NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
     if (t < 0 || t >= c->seg_len)
         die("trf_eval_step: position outside the segment");
     t0 = nc_slice_alias(input, 1, t, t + 1);
-    t0 = nc_tensor_to_device(t0, s->dev);
     t0 = nc_reshape_1d(t0, (size_t)B);
-    x = nc_get_col(nc_dup_tensor(s->embed), t0);
+    if (s->dev != s->cpu && nc_get_tensor_device(input) == s->cpu)
+        x = nc_get_col_host_indices(nc_dup_tensor(s->embed), t0); /* the kernel reads the tokens where they are */
+    else
+        x = nc_get_col(nc_dup_tensor(s->embed), nc_tensor_to_device(t0, s->dev));
     x = nc_mul(x, nc_dup_tensor(s->step_embed_mult));
     /* Post-norm blocks with a plain activation (nncp's default structure, nncp.c:2489-2513):
        a norm is followed by a product, so it rides on that product's launch

@@ -170,6 +170,18 @@ NCTensor *nc_linear_pair_into(NCTensor *w0, NCTensor *bias0, NCTensor *w1, NCTen
     return y0;
 }
 
+/* nc_ext.h: forms of nc_soft_max_cdf16 / nc_get_col that spare the GPU library a copy; every
+   tensor of this library is on the host already */
+NCTensor *nc_soft_max_cdf16_to_host(NCTensor *logits)
+{
+    return nc_soft_max_cdf16(logits);
+}
+
+NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x)
+{
+    return nc_get_col(w, x);
+}
+
 /* nc_ext.h: a layout hint for the GPU library's few-column products; nothing to do here */
 void nc_keep_k_major_weight(NCTensor *w)
 {
