@@ -117,9 +117,10 @@ NCTensor *nc_soft_max_cdf16_to_host(NCTensor *logits);
 
 /* nc_get_col (libnc.h:374-375) with the contiguous i32 indices x on the host device, read
    by the kernel itself from pinned memory instead of being uploaded first (a decoder
-   timestep's tokens).  x must not change until the device has been synchronised.  Consumes
-   w and x.  No gradient.  No counterpart in the reference. */
-NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x);
+   timestep's tokens), times `scale` (nncp.c:625-630: the embedding multiplier; the values are
+   those of nc_mul(nc_get_col(w, x), scale)).  x must not change until the device has been
+   synchronised.  Consumes w and x.  No gradient.  No counterpart in the reference. */
+NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x, float scale);
 
 /* cdf (V, n) U16, targets (m, n) U16 -> (m, n) U16 symbols: the largest s
    with cdf[s, col] <= target (cumulative-frequency search of a decoder). */

@@ -311,6 +311,9 @@ int nchip_nll_bwd(void *stream, const float *p, const int32_t *idx, const float 
    backward (libnc.h:374-377; nncp.c:625): dw (d, v) overwritten; columns that
    share an index are summed in increasing c. */
 int nchip_get_col(void *stream, const float *w, const int32_t *idx, float *y, int d, int v, int64_t n);
+/* the same gather times a scale (nncp.c:625-630: the embedding and its multiplier in one
+   launch; one rounding per element, as the separate product has) */
+int nchip_get_col_scaled(void *stream, const float *w, const int32_t *idx, float *y, int d, int v, int64_t n, float scale);
 int nchip_add_col(void *stream, const float *g, const int32_t *idx, float *dw, int d, int v, int64_t n);
 
 /* fused optimiser step over one parameter (libnc.h:540-572 semantics as

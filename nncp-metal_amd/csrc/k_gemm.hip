@@ -701,7 +701,7 @@ __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
     constexpr int WSZ = ASZ + (NV ? 0 : TR * BST);
     constexpr int XS = 64 * NV + 4;
     __shared__ __attribute__((aligned(16))) float stage[4][WSZ];
-    __shared__ float red[3][4 * 64];
+    __shared__ float red[4][4 * 64];
     __shared__ float xn[NV ? 16 * XS : 1]; // normalised B: [16 columns][K]
     const int lane = threadIdx.x & 63, c = threadIdx.x >> 6; // wavefront = chain
     if (blockIdx.z == 1) { // the pair's second product: its own A, C, bias and row count
@@ -777,19 +777,16 @@ __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
         }
         __syncthreads();
     }
-    // epilogue operands, fetched before the k loop (wavefront 0 finishes the tile)
-    const int col = n0 + il;
+    // epilogue operands, fetched before the k loop: wavefront c finishes row 4 gq + c of the
+    // four rows a lane holds (the four chains of an element meet through LDS either way, and
+    // bias, activation and addend then take a quarter of the time on each wavefront)
+    const int col = n0 + il, row = m0 + 4 * gq + c;
     const bool ok = col < g.N && il < TR && gq < TR / 4; // (8 x 8 tiles: the repeated rows and columns are not stored)
     float NCHIP_GLOBAL *P = g.pre ? as_global(g.pre) : nullptr;
     const float NCHIP_GLOBAL *Radd = g.add ? as_global(g.add) : nullptr;
     const bool plain = !g.bias && !P && !Radd && g.act == NCHIP_ACT_NONE;
-    float bv[4], extra[4];
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int row = m0 + 4 * gq + r;
-        bv[r] = (c == 0 && g.bias && gq < TR / 4) ? as_global(g.bias)[row] : 0.0f;
-        extra[r] = (c == 0 && Radd && ok) ? Radd[(int64_t)col * g.ldc + row] : 0.0f;
-    }
+    const float bv = (g.bias && gq < TR / 4) ? as_global(g.bias)[row] : 0.0f;
+    const float extra = (Radd && ok) ? Radd[(int64_t)col * g.ldc + row] : 0.0f;
     floatx4 acc = { 0, 0, 0, 0 };
     for (int q0 = 0; q0 < nch; q0 += PF) {
 #pragma unroll
@@ -829,29 +826,22 @@ __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
             }
         }
     }
-    if (c > 0) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) red[c - 1][r * 64 + lane] = acc[r];
-    }
+    for (int r = 0; r < 4; r++) red[c][r * 64 + lane] = acc[r];
     __syncthreads();
-    if (c > 0 || !ok) return;
-#pragma unroll
-    for (int r = 0; r < 4; r++) acc[r] = (acc[r] + red[0][r * 64 + lane]) + (red[1][r * 64 + lane] + red[2][r * 64 + lane]);
-    // lane (il, gq) holds rows m0 + 4 gq + r of column n0 + il
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int row = m0 + 4 * gq + r;
-        float NCHIP_GLOBAL *Cp = as_global(g.C) + (int64_t)col * g.ldc + row;
-        if (plain) {
-            *Cp = g.alpha * acc[r];
-            continue;
-        }
-        float v = g.alpha * acc[r] + bv[r];
-        if (P) P[(int64_t)col * g.ldc + row] = v;
-        if (g.act == NCHIP_ACT_GELU) v = gelu_tanh(v);
-        else if (g.act == NCHIP_ACT_RELU) v = v > 0.0f ? v : 0.0f;
-        *Cp = v + extra[r];
+    if (!ok) return;
+    // lane (il, gq) of wavefront c finishes row m0 + 4 gq + c of column n0 + il: (c0 + c1) + (c2 + c3)
+    const float sum = (red[0][c * 64 + lane] + red[1][c * 64 + lane]) + (red[2][c * 64 + lane] + red[3][c * 64 + lane]);
+    float NCHIP_GLOBAL *Cp = as_global(g.C) + (int64_t)col * g.ldc + row;
+    if (plain) {
+        *Cp = g.alpha * sum;
+        return;
     }
+    float v = g.alpha * sum + bv;
+    if (P) P[(int64_t)col * g.ldc + row] = v;
+    if (g.act == NCHIP_ACT_GELU) v = gelu_tanh(v);
+    else if (g.act == NCHIP_ACT_RELU) v = v > 0.0f ? v : 0.0f;
+    *Cp = v + extra;
 }
 
 // KW = 2 doubles the wavefronts of a workgroup without shrinking its tile: the

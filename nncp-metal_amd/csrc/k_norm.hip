@@ -295,14 +295,15 @@ __global__ void nll_bwd_kernel(const float *p, const int32_t *idx, const float *
     }
 }
 
-__global__ void get_col_kernel(const float *w, const int32_t *idx, float *y, int d, int v, int64_t total, int *bad)
+__global__ void get_col_kernel(const float *w, const int32_t *idx, float *y, int d, int v, int64_t total, int *bad,
+                               float scale)
 {
     for (int64_t e = (int64_t)blockIdx.x * TPB + threadIdx.x; e < total; e += (int64_t)gridDim.x * TPB) {
         int64_t c = e / d;
         int i = (int)(e % d);
         const int s = idx[c];
         const bool ok = (unsigned)s < (unsigned)v;
-        y[e] = ok ? w[(int64_t)s * d + i] : 0.0f;
+        y[e] = ok ? w[(int64_t)s * d + i] * scale : 0.0f; // (scale 1: the value itself)
         if (!ok && i == 0) *bad = 1;
     }
 }
@@ -638,9 +639,14 @@ int nchip_nll_bwd(void *stream, const float *p, const int32_t *idx, const float 
 
 int nchip_get_col(void *stream, const float *w, const int32_t *idx, float *y, int d, int v, int64_t n)
 {
+    return nchip_get_col_scaled(stream, w, idx, y, d, v, n, 1.0f);
+}
+
+int nchip_get_col_scaled(void *stream, const float *w, const int32_t *idx, float *y, int d, int v, int64_t n, float scale)
+{
     if (n <= 0) return 0;
     hipLaunchKernelGGL(get_col_kernel, dim3(grid_for(n * d)), dim3(TPB), 0, (hipStream_t)stream, w, idx, y, d, v, n * d,
-                       index_flag());
+                       index_flag(), scale);
     return check("nchip_get_col");
 }
 

@@ -851,8 +851,9 @@ extern "C" NCTensor *nc_get_col(NCTensor *w, NCTensor *x) // libnc.h:374-375
 
 // nc_ext.h: nc_get_col with the indices read by the kernel straight from pinned host memory
 // (a decoder timestep's 32 tokens: an upload of their own costs a launch and its latency).
-// The index tensor must stay as it is until the stream has been waited for.  No gradient.
-extern "C" NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x)
+// The index tensor must stay as it is until the stream has been waited for.  The columns come
+// out multiplied by `scale` (the embedding multiplier: one launch less).  No gradient.
+extern "C" NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x, float scale)
 {
     w = nc_contig(w);
     need_f32(w, "nc_get_col_host_indices");
@@ -860,8 +861,8 @@ extern "C" NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x)
         nc_fatal("nc_get_col_host_indices: (D,V) f32 matrix on the GPU and contiguous i32 indices on the host expected");
     size_t dims[2] = { w->dims[0], nc_numel(x) };
     NCTensor *y = new_f32(w, 2, dims);
-    if (nchip_get_col(nc_stream(w), nc_f32(w), (const int32_t *)nc_data(x), nc_f32(y), (int)dims[0],
-                      (int)w->dims[1], (int64_t)dims[1]))
+    if (nchip_get_col_scaled(nc_stream(w), nc_f32(w), (const int32_t *)nc_data(x), nc_f32(y), (int)dims[0],
+                             (int)w->dims[1], (int64_t)dims[1], scale))
         nc_fatal("nc_get_col_host_indices failed");
     LAUNCHED(w);
     nc_free_tensor(w); nc_free_tensor(x);

@@ -670,11 +670,13 @@ NCTensor *trf_eval_step(NNCPModel *s, int t, const NCTensor *input)
         die("trf_eval_step: position outside the segment");
     t0 = nc_slice_alias(input, 1, t, t + 1);
     t0 = nc_reshape_1d(t0, (size_t)B);
-    if (s->dev != s->cpu && nc_get_tensor_device(input) == s->cpu)
-        x = nc_get_col_host_indices(nc_dup_tensor(s->embed), t0); /* the kernel reads the tokens where they are */
-    else
+    if (s->dev != s->cpu && nc_get_tensor_device(input) == s->cpu) {
+        /* the kernel reads the tokens where they are and applies the multiplier */
+        x = nc_get_col_host_indices(nc_dup_tensor(s->embed), t0, s->embed_mult);
+    } else {
         x = nc_get_col(nc_dup_tensor(s->embed), nc_tensor_to_device(t0, s->dev));
-    x = nc_mul(x, nc_dup_tensor(s->step_embed_mult));
+        x = nc_mul(x, nc_dup_tensor(s->step_embed_mult));
+    }
     /* Post-norm blocks with a plain activation (nncp's default structure, nncp.c:2489-2513):
        a norm is followed by a product, so it rides on that product's launch
        (nc_norm_linear_pair_into) - the norm after the attention on the first feed-forward

@@ -177,9 +177,10 @@ NCTensor *nc_soft_max_cdf16_to_host(NCTensor *logits)
     return nc_soft_max_cdf16(logits);
 }
 
-NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x)
+NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x, float scale)
 {
-    return nc_get_col(w, x);
+    NCTensor *y = nc_get_col(w, x);
+    return nc_mul(y, nc_new_f32(y->dev, scale));
 }
 
 /* nc_ext.h: a layout hint for the GPU library's few-column products; nothing to do here */

@@ -411,6 +411,27 @@ def _dev(nc, arr):
     return t, C.c_void_p(nc.lib.nc_tensor_get_ptr(t, None))
 
 
+def test_timestep_rows_without_copy_launches(hip, rng):
+    """nc_soft_max_cdf16_to_host and nc_get_col_host_indices: the CDF rows the kernel writes
+    into host memory are those of nc_soft_max_cdf16, and the gather that reads its indices from
+    host memory (times the embedding multiplier) is nc_mul(nc_get_col(...), scale), bit for bit."""
+    V, B, D = 256, 32, 512
+    logits = (3 * rng.standard_normal((B, V))).astype(np.float32)
+    want = hip.numpy(hip.nc_soft_max_cdf16(hip.tensor(logits)), free=True)
+    host = hip.nc_soft_max_cdf16_to_host(hip.tensor(logits))
+    hip.nc_synchronize(hip.dev)
+    got = hip.numpy(host, free=True)
+    assert got.dtype == np.uint16 and np.array_equal(got, want)
+    w = rng.standard_normal((V, D)).astype(np.float32)
+    idx = rng.integers(0, V, B).astype(np.int32)
+    scale = float(np.sqrt(D))
+    a = hip.nc_mul(hip.nc_get_col(hip.tensor(w), hip.tensor(idx)), hip.nc_new_f32(hip.dev, scale))
+    b = hip.nc_get_col_host_indices(hip.tensor(w), hip.tensor(idx, device=hip.cpu), scale)
+    a, b = hip.numpy(a, free=True), hip.numpy(b, free=True)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.array_equal(a, w[idx] * np.float32(scale))
+
+
 @pytest.mark.parametrize("m,k,n", [(512, 512, 32), (2048, 512, 32), (512, 2048, 32), (256, 512, 5), (64, 96, 64),
                                    (1024, 1024, 33), (32, 4096, 8), (96, 288, 16)])
 def test_k_major_weight_copies_change_no_bit(hip, rng, m, k, n):
