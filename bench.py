@@ -447,7 +447,7 @@ def main():
                                                    "reported under `variants` (comma separated, empty for none)")
     ap.add_argument("--cpu-steps", type=int, default=4, help="0 skips the CPU baseline")
     ap.add_argument("--cpu-single-steps", type=int, default=1, help="steps of the single-thread CPU baseline (0 skips it)")
-    ap.add_argument("--decode-segments", type=int, default=2, help="segments decoded for the `decode` object (0 skips it)")
+    ap.add_argument("--decode-segments", type=int, default=4, help="segments decoded for the `decode` object (0 skips it)")
     ap.add_argument("--profile-steps", type=int, default=2)
     ap.add_argument("--attention-iters", type=int, default=50, help="0 skips the isolated attention timing")
     ap.add_argument("--cdf-iters", type=int, default=50, help="0 skips the coder-side CDF timing")

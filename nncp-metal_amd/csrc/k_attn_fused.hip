@@ -674,8 +674,18 @@ __global__ __launch_bounds__(256) void attn_param_grad_reduce(const float *dwp, 
     if (e < n_w) { src = dwp + e; dst = dw + e; n = n_w; }
     else if (e < n_w + n_b) { src = dbp + (e - n_w); dst = db + (e - n_w); n = n_b; }
     else return;
+    // the partials are added in stream order; eight loads at a time are in flight (added one
+    // after the other as they are: a loop of dependent load-and-add pays a memory round trip per stream)
     float acc = 0.0f;
-    for (int b = 0; b < B; b++) acc += src[(int64_t)b * n];
+    int b = 0;
+    for (; b + 8 <= B; b += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = src[(int64_t)(b + u) * n];
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc += v[u];
+    }
+    for (; b < B; b++) acc += src[(int64_t)b * n];
     *dst = acc;
 }
 
