@@ -68,6 +68,7 @@ struct GemmArgs {
     int dbg;
     const NchipGemmProblem *grp; // grouped launch: one problem per table row
     int n_grp;
+    int grp_chunk; // grouped launch: consecutive tiles of the list handed to one XCD at a time
     float *rowsum; // activation-gradient epilogue only: partial row sums of the result, one row per (tile column, wavefront column, lane half)
     // second product of a few-column pair launch (gemm_skinny_nn, blockIdx.z = 1): same B, N, K
     const float *A_1, *bias_1;
@@ -888,7 +889,18 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     const float *A2 = nullptr, *B2 = nullptr;
     int k1 = 0x7fffffff;
     if (g.grp) {
-        // grouped launch: find the problem that owns this workgroup
+        // grouped launch: consecutive workgroup ids go to the XCDs in turn; hand each XCD
+        // GC consecutive tiles of the list at a time (neighbours in a tile column, which share
+        // a B panel in that XCD's L2) while the turn-taking keeps the XCDs' work balanced
+        {
+            const int GC = g.grp_chunk;
+            const int total = gridDim.x, span = NXCD * GC;
+            if (GC > 1 && (bid / span + 1) * span <= total) {
+                const int in = bid % span, x = in % NXCD, slot = in / NXCD;
+                bid = (bid / span) * span + x * GC + slot;
+            }
+        }
+        // find the problem that owns this workgroup
         int lo = 0, hi = g.n_grp; // grp[lo].tile_start <= bid < grp[hi].tile_start
         while (hi - lo > 1) {
             int mid = (lo + hi) >> 1;
@@ -1891,6 +1903,10 @@ extern "C" int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmP
     GemmArgs g;
     memset(&g, 0, sizeof(g));
     g.grp = dev_table; g.n_grp = n_problems;
+    // 16 tiles per turn: measured at C3 (1156 tiles), FETCH_SIZE of the launch 3.18 GB at 1 (plain
+    // round robin), 2.67 at 8, 2.13 at 16, duration 1574 / 1555 / 1563 us; from 32 on the runs
+    // are long enough for the XCDs to finish apart (1692 us)
+    { static const int gc = getenv("NCHIP_GRP_CHUNK") ? atoi(getenv("NCHIP_GRP_CHUNK")) : 16; g.grp_chunk = gc; }
     g.batch = 1; g.batch_in = 1; g.ksplit = 1;
     g.beta = 0.0f; g.act = 0;
     hipStream_t st = (hipStream_t)stream;
