@@ -31,7 +31,36 @@
 extern "C" {
 #endif
 
+/* Profiling hooks of the boundary (libnc.h:14-67).  The reference's prof_start / prof_end are
+   inline in its header and count cycles into prof_cycles[] only when built with -DPROFILE;
+   here they are always live: they forward to the library, which adds the elapsed nanoseconds
+   to prof_cycles[idx], counts the sample and - when the environment variable NC_PROFILE is set
+   - opens / closes a roctx range of the section's name ("EVAL", "GRAD", ...), so the sections of
+   nncp.c:606/1027, 1108/1191, 1227/1234, 2881/2917 show up in a rocprofv3 marker trace.
+   nc_prof_dump (libnc.h:67) prints the table to stderr when NC_PROFILE is set. */
+void nc_prof_begin(int idx);
+void nc_prof_finish(int idx, int n_ops);
+
 #ifndef LIBNC_H /* ---- types (skipped when the reference header is present) */
+
+typedef enum { /* libnc.h:16-25 */
+    PROF_EVAL,
+    PROF_GRAD,
+    PROF_SGD,
+    PROF_UPDATE,
+    PROF_WRITE_SYM,
+    PROF_PROBE,
+    PROF_TOTAL,
+    PROF_COUNT,
+} ProfEnum;
+
+extern int64_t prof_cycles[PROF_COUNT];  /* libnc.h:29-31; nanoseconds here */
+extern int64_t prof_samples[PROF_COUNT];
+extern int64_t prof_ops[PROF_COUNT];
+
+static inline void prof_start(int idx) { nc_prof_begin(idx); }                      /* libnc.h:33 */
+static inline void prof_end(int idx) { nc_prof_finish(idx, 0); }                    /* libnc.h:38 */
+static inline void prof_end_ops(int idx, int n_ops) { nc_prof_finish(idx, n_ops); } /* libnc.h:44 */
 
 #ifndef CUTILS_H
 typedef int BOOL;

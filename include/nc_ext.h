@@ -138,6 +138,19 @@ float nc_exp_det(float x);
    Returns the previous setting.  libnc_ref.so emulates the same rounding. */
 int nc_set_matmul_bf16(NCContext *m, int enable);
 
+/* bf16 operand copies.  With nc_set_matmul_bf16 on, a product whose shape allows it reads
+   both operands as bf16 from memory: every f32 device buffer can carry a bf16 copy of itself
+   (same elements, rounded to nearest even), written by the kernel that produces the f32
+   values where there is one (layer norms, the optimiser's weight update, product epilogues
+   that feed another product) and by one cast pass otherwise, and dropped whenever the buffer
+   is written in place.  nc_get_bf16_cast_count: how many copies were made by a cast of their
+   own so far (the ones a producing kernel could still take over).  nc_set_bf16_shadow_check:
+   testing aid, process-wide - when non-zero, every use of a copy first compares it with a
+   fresh rounding of the buffer and ends the process if they differ (a writer that failed to
+   drop the copy); returns the previous setting.  Both 0 / no effect in libnc_ref.so. */
+int64_t nc_get_bf16_cast_count(NCContext *m);
+int nc_set_bf16_shadow_check(int enable);
+
 /* When non-zero, nc_backward() postpones the weight-gradient GEMMs
    dW = dY X^T of plain linear layers (weight used once in the graph) and runs
    them all in one grouped launch just before it returns.  The gradient
@@ -146,6 +159,19 @@ int nc_set_matmul_bf16(NCContext *m, int enable);
    forward to sgd_opt_update_var (nncp.c:1078-1096).  Returns the previous
    setting.  No effect in libnc_ref.so. */
 int nc_set_deferred_weight_grad(NCContext *m, int enable);
+
+/* The optimiser's per-parameter state, for checkpoints and for tests that put two models
+   into the same state: `which` 0 = first moment (Adam with beta1 != 0), 1 = second moment
+   (Adam, RMSProp).  nc_sgd_opt_get_state returns a new 1-D f32 tensor on the host device
+   holding a copy (NULL when the parameter has no optimiser or the algorithm keeps no such
+   moment); nc_sgd_opt_set_state copies the values of v (f32, same element count, any device)
+   into it.  nc_sgd_opt_get_step / nc_sgd_opt_set_step: the count of updates applied, which
+   Adam's bias correction reads.  No counterpart in libnc.h (its optimiser state is opaque:
+   libnc.h:561-571). */
+NCTensor *nc_sgd_opt_get_state(NCParam *p, int which);
+void nc_sgd_opt_set_state(NCParam *p, int which, const NCTensor *v);
+int64_t nc_sgd_opt_get_step(NCSGDOptState *s);
+void nc_sgd_opt_set_step(NCSGDOptState *s, int64_t step);
 
 /* Number of kernel launches issued so far (0 in libnc_ref.so). */
 int64_t nc_get_launch_count(NCContext *m);

@@ -96,8 +96,48 @@ typedef struct {
     float alpha;
 } NchipGemmProblem;
 int nchip_gemm_grouped_tiles(int m, int n);
+/* precision 0: fp32; 1: fp32 operands rounded to bf16 in the tile loader; 2: the operand
+   pointers of the table address bf16 copies (2 bytes per element, same layout and leading
+   dimensions as the fp32 matrices they were rounded from), read with unguarded 16-byte
+   loads - every k and k2 a multiple of 64, every row-contiguous operand extent (m with
+   ta = 0, n with tb = 1) a multiple of 128, leading dimensions multiples of 8, bases 16-byte
+   aligned; the caller checks.  C is fp32 in all three. */
 int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmProblem *dev_table,
                        int n_problems, int total_tiles, int precision, double total_flops);
+
+/* One product C = act(alpha op(A) op(B) + bias) [+ addend] whose operands are read as bf16
+   from memory: A16 / B16 address the bf16 copies of the fp32 matrices (element for element,
+   same column-major layout and leading dimensions, no padding), accumulation in fp32 on
+   v_mfma_f32_32x32x16_bf16.  The values are those of nchip_gemm with precision 1 up to the
+   order of the k sum inside a tile class.  Unguarded 16-byte loads throughout: k a multiple
+   of 64, leading dimensions multiples of 8, bases 16-byte aligned, and an operand whose long
+   axis is contiguous (A with ta = 0, B with tb = 1) must fill whole tiles of the class the
+   shape selects (128 or 64 rows / columns).  Returns 1 when the shape does not fit (nothing
+   launched: the caller takes another route), 0 when launched, negative on error.
+     pre / addend / dpre+dact / rowsum+rows_written: as in nchip_gemm_add, nchip_gemm_dact and
+     nchip_gemm_dact_rowsum (all optional);
+     C16: when not NULL, the result once more, rounded to bf16 (nearest even), laid out like
+     C with the same ldc - the operand copy of a later product, so that C is never cast. */
+typedef struct {
+    int ta, tb, m, n, k;
+    float alpha;
+    const uint16_t *A16, *B16;
+    int64_t lda, ldb;
+    float *C;
+    int64_t ldc;
+    uint16_t *C16;
+    const float *bias;
+    int act;
+    float *pre;
+    const float *addend;
+    const float *dpre;
+    int dact;
+    float *rowsum;
+    int *rows_written;
+} NchipGemmBf16Args;
+int nchip_gemm_bf16_operands(void *stream, const NchipGemmBf16Args *a);
+/* tuning aid: 0 = tile class from the shape, 1 = 128x128, 2 = 128x64, 3 = 64x64 (all 64 deep) */
+void nchip_gemm_bf16_operands_class(int cls);
 
 /* Optional timing of every GEMM launch with HIP events on the launch stream.
    After nchip_gemm_profile_enable(1), each nchip_gemm* dispatch carries an
@@ -116,8 +156,11 @@ void nchip_gemm_force_config(int cfg);
 
 /* nchip_gemm_dact that also leaves partial row sums of C (the bias gradient of the layer whose
    pre-activation gradient C is): `rowsum` holds nchip_gemm_rowsum_rows(n) rows of m floats;
-   *rows_written of them are written, row p = the sum over 16 consecutive columns of C (columns
-   past n count as zero), so their sum in row order is the row sum of C.  *rows_written is 0
+   *rows_written of them are written.  Row p is the sum over 16 columns of C, the 16 that one lane
+   of the epilogue holds: of the 32-column block p / 2, the columns c with c mod 8 in
+   [4 (p mod 2), 4 (p mod 2) + 4) - four runs of 4 consecutive columns, 8 apart - added in
+   increasing column order (columns past n count as zero).  Rows 2j and 2j + 1 together cover
+   block j, so the sum of all rows in row order is the row sum of C.  *rows_written is 0
    when the kernel chosen for this product does not write them (split-K, bf16 operand copies):
    the caller then sums C itself. */
 int nchip_gemm_rowsum_rows(int n);
@@ -247,6 +290,11 @@ int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
 int nchip_norm_fwd(void *stream, const float *x, const float *w, const float *b,
                    float *y, float *xhat, float *rstd, int d, int64_t n,
                    float eps, int avg);
+/* nchip_norm_fwd that also leaves y rounded to bf16 (nearest even) in y16 (d, n), the operand
+   copy the bf16 products read; y16 NULL = nchip_norm_fwd.  No counterpart in the reference. */
+int nchip_norm_fwd_bf16copy(void *stream, const float *x, const float *w, const float *b,
+                            float *y, float *xhat, float *rstd, int d, int64_t n,
+                            float eps, int avg, uint16_t *y16);
 /* dx (d,n) = gradient of the input, plus dx_add (d,n) when that is not NULL;
    dw, db (d) overwritten (may be NULL when w is NULL).  partial needs
    nchip_norm_bwd_partial_rows(n) * 2 * d floats. */
@@ -274,12 +322,19 @@ int nchip_norm_bwd_rowsum(void *stream, const float *g, const float *xhat, const
                           const float *w, float *dx, const float *dx_add, float *dw, float *db,
                           float *partial, int d, int64_t n, int avg, float *dx_partial);
 
+/* nchip_norm_bwd_rowsum that also leaves dx rounded to bf16 in dx16 (d, n); NULL = none. */
+int nchip_norm_bwd_bf16copy(void *stream, const float *g, const float *xhat, const float *rstd,
+                            const float *w, float *dx, const float *dx_add, float *dw, float *db,
+                            float *partial, int d, int64_t n, int avg, float *dx_partial, uint16_t *dx16);
+
 /* nchip_norm_bwd for callers that cannot allocate device memory (code under HIP graph
    capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
    reference.  Same arguments without `partial`: the partial dw / db rows go to a buffer the
    library itself holds in device memory, nchip_norm_bwd_static_capacity() floats (8 MiB)
-   per GPU for the life of the process, and the call allocates nothing.  (d, n) must satisfy
-   nchip_norm_bwd_rows(d, n) * 2 * d <= that capacity - true for every n when d is 128, 256,
+   per GPU for the life of the process, and the call allocates nothing.  The rows it holds
+   are the nchip_norm_bwd_rows(d, n) rows the kernels actually write (never more than the
+   nchip_norm_bwd_partial_rows(n) that size a caller's buffer for nchip_norm_bwd): (d, n) must
+   satisfy nchip_norm_bwd_rows(d, n) * 2 * d <= that capacity - true for every n when d is 128, 256,
    512 or 1024, and for d <= 32768 otherwise - else the call returns -3 with a message and
    launches nothing.  The stream must belong to the current device.  All calls on one GPU
    share the buffer: calls that may overlap there (different streams, different threads)
@@ -327,17 +382,23 @@ int nchip_opt_update(void *stream, int algo, float *w, float *m, float *v, const
    pure bandwidth: 16 B per parameter for RMSProp).  dev_table[n_tensors] and
    dev_chunk_prefix[n_tensors + 1] live in device memory; tensor i owns the
    workgroups chunk_prefix[i] .. chunk_prefix[i+1]-1, each covering `chunk`
-   consecutive elements.  m may be NULL (beta1 == 0), v may be NULL (SGD). */
+   consecutive elements.  m may be NULL (beta1 == 0), v may be NULL (SGD).  w16, when not
+   NULL, receives the updated w rounded to bf16 (nearest even), element for element: the
+   operand copy the bf16 products read, so that no weight is cast again after its update. */
 typedef struct {
     float *w, *m, *v;
     const float *g;
     int64_t n;
     float lr;
     int pad_;
+    uint16_t *w16;
 } NchipOptTensor;
 int nchip_opt_update_multi(void *stream, int algo, const NchipOptTensor *dev_table,
                            const int *dev_chunk_prefix, int n_tensors, int total_chunks, int chunk,
                            float beta1, float beta2, float eps, float clip, float c1, float c2);
+
+/* dst[i] = src[i] rounded to bf16 (nearest even), i < n: one streaming pass. */
+int nchip_cast_bf16(void *stream, const float *src, uint16_t *dst, int64_t n);
 
 /* logits (v, n) f32 -> cdf (v, n) u16 as specified in nc_ext.h
    (nc_soft_max_cdf16); bit-identical to the CPU checker. */

@@ -146,6 +146,15 @@ NCTensor **nncp_model_param(NNCPModel *s, const char *name);
 int nncp_model_param_count(NNCPModel *s);
 const char *nncp_model_param_name(NNCPModel *s, int index);
 int64_t nncp_model_train_step(NNCPModel *s);
+/* What a training step carries over to the next besides the parameters, for checkpoints and
+   for tests that put two models into the same state: the optimiser's moment `which` of the
+   named parameter (nc_sgd_opt_get_state / nc_sgd_opt_set_state of nc_ext.h; get returns an
+   owned host tensor or NULL, set copies v in) and the memory of layer l, the (d_model, B,
+   mem_len) tensor mem_h[l] of nncp.c:1205-1221 (borrowed; Transformer models only, NULL for
+   an LSTM or without memory). */
+NCTensor *nncp_model_opt_state(NNCPModel *s, const char *name, int which);
+void nncp_model_set_opt_state(NNCPModel *s, const char *name, int which, const NCTensor *v);
+NCTensor *nncp_model_memory(NNCPModel *s, int l);
 /* every registered parameter to / from a parameter file (nc_save_coefs / nc_load_coefs,
    libnc.h:530, 536; the file named by --load_coefs, nncp.c:3761).  Loading needs a model of
    the same configuration: names, shapes and types must match. */

@@ -29,6 +29,7 @@
 #include <vector>
 #include "../../include/nchip_kernels.h"
 #include "k_addrspace.h"
+#include "k_bf16.h"
 #include "k_norm_inline.h"
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -57,6 +58,7 @@ struct GemmArgs {
     int dact;
     float *pre;
     float *ws;
+    uint16_t *c16; // the result once more, rounded to bf16, laid out like C (may be NULL)
     int64_t lda, ldb, ldc, sa, sb, sc;   // outer batch strides
     int64_t sa_in, sb_in, sc_in;         // inner batch strides
     int batch_in;                        // batch index z -> (z / batch_in, z % batch_in)
@@ -195,15 +197,7 @@ struct TileLoader {
 // fetched as 2 columns x 2 rows (k, k+1) and stored as one 8-byte LDS write;
 // k-contiguous operands give two words per float4.  Rounding is to nearest
 // even (v_cvt_pk_bf16_f32).
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float floatx2_t __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
-{
-    floatx2_t f = { lo, hi };
-    bf16x2_t h = __builtin_convertvector(f, bf16x2_t);
-    return __builtin_bit_cast(uint32_t, h);
-}
+// (pack_bf16: k_bf16.h)
 
 template <int BT, int BK, int MAJOR, int NT>
 struct TileLoaderBf16 {
@@ -362,10 +356,12 @@ struct TileLoaderBf16Src {
 __device__ __forceinline__ void epilogue_tile(const GemmArgs &g, const floatx16 &acc, int m, int nb,
                                               float NCHIP_GLOBAL *C, float NCHIP_GLOBAL *P,
                                               const float NCHIP_GLOBAL *Radd, const float NCHIP_GLOBAL *Dp,
-                                              bool full, bool plain, float NCHIP_GLOBAL *rowsum = nullptr)
+                                              bool full, bool plain, float NCHIP_GLOBAL *rowsum = nullptr,
+                                              uint16_t NCHIP_GLOBAL *H = nullptr)
 {
     if (!full && m >= g.M) return;
     float NCHIP_GLOBAL *Cp = C + (int64_t)nb * g.ldc + m; // element r lives at Cp + nofs(r)*ldc
+    uint16_t NCHIP_GLOBAL *Hp = H ? H + (int64_t)nb * g.ldc + m : nullptr; // bf16 copy of the same elements
     auto nofs = [](int r) { return (r >> 2) * 8 + (r & 3); };
     if (plain && full) {
 #pragma unroll
@@ -420,6 +416,11 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs &g, const floatx16 
 #pragma unroll
         for (int r = 0; r < 16; r++)
             if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r];
+        if (Hp) {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                if (ok[r]) Hp[(int64_t)nofs(r) * g.ldc] = f32_to_bf16_rne(v[r]);
+        }
         if (rowsum) { // this lane's 16 columns of row m, in column order: one entry of a partial row
             float sum = 0.0f;
 #pragma unroll
@@ -429,8 +430,15 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs &g, const floatx16 
         return;
     }
 #pragma unroll
+    for (int r = 0; r < 16; r++) v[r] += extra[r];
+#pragma unroll
     for (int r = 0; r < 16; r++)
-        if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r] + extra[r];
+        if (ok[r]) Cp[(int64_t)nofs(r) * g.ldc] = v[r];
+    if (Hp) {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            if (ok[r]) Hp[(int64_t)nofs(r) * g.ldc] = f32_to_bf16_rne(v[r]);
+    }
 }
 
 // Product with a few token columns for the width-invariant class: C (M x N, 32 columns per
@@ -1284,7 +1292,8 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
     const float NCHIP_GLOBAL *Radd = g.add ? as_global(g.add + coff) : nullptr;
     const bool full = (m0 + BM <= g.M) && (n0 + BN <= g.N); // uniform
     const float NCHIP_GLOBAL *Dp = g.dpre ? as_global(g.dpre + coff) : nullptr;
-    const bool plain = !g.bias && !P && !Radd && !Dp && g.beta == 0.0f && g.act == NCHIP_ACT_NONE;
+    uint16_t NCHIP_GLOBAL *H16 = g.c16 ? as_global(g.c16 + coff) : nullptr;
+    const bool plain = !g.bias && !P && !Radd && !Dp && !H16 && g.beta == 0.0f && g.act == NCHIP_ACT_NONE;
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
@@ -1292,7 +1301,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
             float NCHIP_GLOBAL *rs = nullptr;
             if (g.rowsum) // partial row of this (tile column, wavefront column, accumulator column, lane half)
                 rs = as_global(g.rowsum) + (int64_t)((((tile_n * WN + wn) * TN + i) * 2) + (lane >> 5)) * g.M;
-            epilogue_tile(g, acc[i][j], mm_base + j * 32, nn_base + i * 32, C, P, Radd, Dp, full, plain, rs);
+            epilogue_tile(g, acc[i][j], mm_base + j * 32, nn_base + i * 32, C, P, Radd, Dp, full, plain, rs, H16);
         }
 #ifdef NCHIP_GEMM_CLOCKS
     if (g_gemm_clk && blockIdx.y == 0 && t == 0) g_gemm_clk[6 + 3 * blockIdx.x] = wall_clock64(); // stores issued
@@ -1353,6 +1362,21 @@ __global__ __launch_bounds__(256) void cast_bf16_kernel(const float *src, uint16
     }
 }
 
+// dst[i] = bf16(src[i]) for i < n, 8 elements per thread and step (two 16-byte loads, one
+// 16-byte store); both pointers 16-byte aligned
+__global__ __launch_bounds__(256) void cast_bf16_flat_kernel(const float *src, uint16_t *dst, int64_t n)
+{
+    const int64_t units = n / 8, stride = (int64_t)gridDim.x * 256;
+    const floatx4 NCHIP_GLOBAL *s4 = reinterpret_cast<const floatx4 NCHIP_GLOBAL *>(as_global(src));
+    u32x4 NCHIP_GLOBAL *d4 = reinterpret_cast<u32x4 NCHIP_GLOBAL *>(as_global(dst));
+    for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += stride) {
+        const floatx4 a = s4[2 * u], b = s4[2 * u + 1];
+        d4[u] = u32x4{ pack_bf16(a[0], a[1]), pack_bf16(a[2], a[3]), pack_bf16(b[0], b[1]), pack_bf16(b[2], b[3]) };
+    }
+    if (blockIdx.x == 0) // the last n % 8 elements
+        for (int64_t i = units * 8 + threadIdx.x; i < n; i += 256) as_global(dst)[i] = f32_to_bf16_rne(as_global(src)[i]);
+}
+
 // ---- optional per-launch timing (HIP events on the launch stream) ----------
 struct ProfRec {
     hipEvent_t start, stop;
@@ -1395,6 +1419,8 @@ static void launch_fewcol_mfma(const GemmArgs &g, int mmax, int nz, hipStream_t 
 }
 int g_force_gm = -1;
 std::vector<ProfRec> g_prof;
+int g_bf16ops_cls = getenv("NCHIP_GEMM_BF16OPS_CLASS") ? atoi(getenv("NCHIP_GEMM_BF16OPS_CLASS")) : 0;
+
 
 // With `rec` the kernel's own start / stop timestamps are bound to the record's
 // events (hipExtLaunchKernelGGL), so the measured time is the dispatch alone,
@@ -1852,6 +1878,86 @@ extern "C" void nchip_gemm_force_band(int gm)
     g_force_gm = gm;
 }
 
+extern "C" int nchip_cast_bf16(void *stream, const float *src, uint16_t *dst, int64_t n)
+{
+    if (n <= 0) return 0;
+    if (!src || !dst || (((uintptr_t)src | (uintptr_t)dst) & 15) != 0) {
+        fprintf(stderr, "nchip_cast_bf16: 16-byte aligned buffers expected\n");
+        return -1;
+    }
+    int64_t nb = (n / 8 + 255) / 256;
+    if (nb < 1) nb = 1;
+    if (nb > 4096) nb = 4096;
+    hipLaunchKernelGGL(cast_bf16_flat_kernel, dim3((unsigned)nb), dim3(256), 0, (hipStream_t)stream, src, dst, n);
+    if (hipGetLastError() != hipSuccess) { fprintf(stderr, "nchip_cast_bf16: launch failed\n"); return -2; }
+    return 0;
+}
+
+// Product whose operands are already bf16 in memory (the rounded copies of the fp32 matrices,
+// element for element in the same column-major layout: no padding).  Unguarded 16-byte loads
+// throughout, so the shapes must fit: k a multiple of 64; an operand whose long axis is
+// contiguous (A with ta = 0, B with tb = 1) must fill whole tiles (m resp. n a multiple of
+// 128: every tile class divides it); leading dimensions multiples of 8 elements; 16-byte
+// aligned bases.  Returns 1 when they do not (nothing launched: the caller takes another
+// route).  Epilogue options as in the fp32-operand calls; c16, when given, receives the
+// result rounded to bf16 next to C.
+extern "C" int nchip_gemm_bf16_operands(void *stream, const NchipGemmBf16Args *a)
+{
+    if (a->rows_written) *a->rows_written = 0;
+    const int m = a->m, n = a->n, k = a->k, ta = a->ta != 0, tb = a->tb != 0;
+    if (m <= 0 || n <= 0) return 0;
+    if (!a->A16 || !a->B16 || !a->C || k <= 0 || a->lda < (ta ? k : m) || a->ldb < (tb ? n : k) || a->ldc < m) {
+        fprintf(stderr, "nchip_gemm_bf16_operands: bad arguments (m=%d n=%d k=%d)\n", m, n, k);
+        return -1;
+    }
+    if (k % 64 || a->lda % 8 || a->ldb % 8 || (((uintptr_t)a->A16 | (uintptr_t)a->B16) & 15) != 0)
+        return 1;
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.A = reinterpret_cast<const float *>(a->A16); g.B = reinterpret_cast<const float *>(a->B16);
+    g.C = a->C; g.c16 = a->C16; g.bias = a->bias; g.add = a->addend; g.pre = a->pre;
+    g.dpre = a->dpre; g.dact = a->dact;
+    g.lda = a->lda; g.ldb = a->ldb; g.ldc = a->ldc;
+    g.batch_in = 1; g.M = m; g.N = n; g.K = k; g.batch = 1; g.ksplit = 1; g.kchunk = k;
+    g.alpha = a->alpha; g.beta = 0.0f; g.act = a->act;
+    hipStream_t st = (hipStream_t)stream;
+    // tile class from the tile counts: the largest tile that still gives every CU a workgroup
+    const int64_t t128 = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
+    const int64_t t128x64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64);
+    int cls = g_bf16ops_cls;
+    if (!cls) cls = t128 >= 224 ? 1 : (t128x64 >= 224 && m >= 128 ? 2 : 3);
+    {
+        const int bm = cls == 3 ? 64 : 128, bn = cls == 1 ? 128 : 64;
+        if ((!ta && m % bm) || (tb && n % bn)) return 1; // row-contiguous operands need whole tiles
+    }
+    if (a->rowsum && a->rows_written && a->dpre) {
+        const int bn = cls == 1 ? 128 : 64;
+        g.rowsum = a->rowsum;
+        *a->rows_written = (n + bn - 1) / bn * bn / 16;
+    }
+    ProfRec rec;
+    if (g_prof_on) {
+        (void)hipEventCreate(&rec.start);
+        (void)hipEventCreate(&rec.stop);
+        rec.flops = 2.0 * m * n * (double)k;
+        rec.variant = 32 + cls * 4 + ta * 2 + tb; // the bf16-operand classes
+    }
+    ProfRec *pr = g_prof_on ? &rec : nullptr;
+    if (cls == 1) launch_tile<128, 128, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+    else if (cls == 2) launch_tile<128, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+    else launch_tile<64, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+    if (g_prof_on) g_prof.push_back(rec);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        fprintf(stderr, "nchip_gemm_bf16_operands: launch failed: %s\n", hipGetErrorString(e));
+        return -2;
+    }
+    return 0;
+}
+
+// tuning aid: 0 = choose the bf16-operand tile class from the shape, 1 = 128x128, 2 = 128x64, 3 = 64x64
+extern "C" void nchip_gemm_bf16_operands_class(int cls) { g_bf16ops_cls = cls; }
+
 // ---- profiling entry points ---------------------------------------------------
 extern "C" void nchip_gemm_profile_enable(int on)
 {
@@ -1861,13 +1967,14 @@ extern "C" void nchip_gemm_profile_enable(int on)
 extern "C" int nchip_gemm_profile_read(int max_variants, char (*names)[48], int64_t *launches,
                                        double *flops, double *seconds)
 {
-    double fl[32] = { 0 }, sec[32] = { 0 };
-    int64_t cnt[32] = { 0 };
+    constexpr int NVAR = 64;
+    double fl[NVAR] = { 0 }, sec[NVAR] = { 0 };
+    int64_t cnt[NVAR] = { 0 };
     for (ProfRec &r : g_prof) {
         float ms = 0.0f;
         (void)hipEventSynchronize(r.stop);
         (void)hipEventElapsedTime(&ms, r.start, r.stop);
-        if (r.variant >= 0 && r.variant < 32) {
+        if (r.variant >= 0 && r.variant < NVAR) {
             fl[r.variant] += r.flops;
             sec[r.variant] += ms * 1e-3;
             cnt[r.variant]++;
@@ -1878,12 +1985,18 @@ extern "C" int nchip_gemm_profile_read(int max_variants, char (*names)[48], int6
     g_prof.clear();
     static const char *tiles_f32[4] = { "64,64,16,2,2", "128,64,32,4,2", "128,128,32,4,2", "64,64,32,2,2" };
     static const char *tiles_bf16[4] = { "64,64,32,2,2", "128,64,32,4,2", "128,128,32,4,2", "64,64,32,2,2" };
+    static const char *tiles_ops[4] = { "128,128,64,2,2", "128,128,64,2,2", "128,64,64,2,2", "64,64,64,2,2" }; // 0: the grouped launch
     int n = 0;
-    for (int v = 0; v < 32 && n < max_variants; v++) {
+    for (int v = 0; v < NVAR && n < max_variants; v++) {
         if (!cnt[v]) continue;
-        const bool two_groups = v / 8 == 3 || ((v & 1) && v / 8 == 0);
-        snprintf(names[n], 48, "gemm_kernel<%s,%d,%d,%d%s>", (v & 1) ? tiles_bf16[v / 8] : tiles_f32[v / 8],
-                 (v >> 2) & 1, (v >> 1) & 1, v & 1, two_groups ? ",2" : "");
+        if (v >= 32) { // operands read as bf16: gemm_kernel<tile, ta, tb, 2>
+            snprintf(names[n], 48, "gemm_kernel<%s,%d,%d,2%s>", tiles_ops[(v - 32) / 4], (v >> 1) & 1, v & 1,
+                     v < 36 ? ",grouped" : "");
+        } else {
+            const bool two_groups = v / 8 == 3 || ((v & 1) && v / 8 == 0);
+            snprintf(names[n], 48, "gemm_kernel<%s,%d,%d,%d%s>", (v & 1) ? tiles_bf16[v / 8] : tiles_f32[v / 8],
+                     (v >> 2) & 1, (v >> 1) & 1, v & 1, two_groups ? ",2" : "");
+        }
         launches[n] = cnt[v]; flops[n] = fl[v]; seconds[n] = sec[v];
         n++;
     }
@@ -1910,35 +2023,38 @@ extern "C" int nchip_gemm_grouped(void *stream, int ta, int tb, const NchipGemmP
     g.batch = 1; g.batch_in = 1; g.ksplit = 1;
     g.beta = 0.0f; g.act = 0;
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid(total_tiles, 1), block(512);
+    dim3 grid(total_tiles, 1), block(precision == 2 ? 256 : 512);
     ProfRec rec;
     if (g_prof_on) {
         (void)hipEventCreate(&rec.start);
         (void)hipEventCreate(&rec.stop);
-        rec.variant = 2 * 8 + (ta ? 4 : 0) + (tb ? 2 : 0) + (precision == 1 ? 1 : 0);
+        rec.variant = precision == 2 ? 32 + (ta ? 2 : 0) + (tb ? 1 : 0)
+                                     : 2 * 8 + (ta ? 4 : 0) + (tb ? 2 : 0) + (precision == 1 ? 1 : 0);
         rec.flops = total_flops;
     }
-#define GRP2(TA, TB, BF, SAV)                                                                                  \
+#define GRP_LAUNCH(KERNEL, BK_, TA, TB, BF)                                                                \
     do {                                                                                                   \
-        constexpr size_t dyn = lds_dynamic_bytes<128, 128, 32, TA, TB, BF>();                              \
+        constexpr size_t dyn = lds_dynamic_bytes<128, 128, BK_, TA, TB, BF>();                             \
         if (dyn) {                                                                                         \
-            static const bool ok = hipFuncSetAttribute(                                                    \
-                reinterpret_cast<const void *>(gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV, 1, (BF == 0)>),               \
+            static const bool ok = hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL),             \
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) == hipSuccess;                       \
             if (!ok) { fprintf(stderr, "nchip_gemm_grouped: cannot reserve %zu bytes of LDS\n", dyn); return -2; } \
         }                                                                                                  \
-        if (g_prof_on) hipExtLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV, 1, (BF == 0)>), grid, block, dyn, st, \
-                                             rec.start, rec.stop, 0, g);                                   \
-        else hipLaunchKernelGGL((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, SAV, 1, (BF == 0)>), grid, block, dyn, st, g);    \
+        if (g_prof_on) hipExtLaunchKernelGGL(KERNEL, grid, block, dyn, st, rec.start, rec.stop, 0, g);     \
+        else hipLaunchKernelGGL(KERNEL, grid, block, dyn, st, g);                                          \
     } while (0)
-#define GRP(TA, TB, BF) GRP2(TA, TB, BF, (BF == 2))
-    if (precision == 1) {
+#define GRP(TA, TB, BF) GRP_LAUNCH((gemm_kernel<128, 128, 32, 4, 2, TA, TB, BF, 1, 2, 0, 1, (BF == 0)>), 32, TA, TB, BF)
+#define GRP16(TA, TB) GRP_LAUNCH((gemm_kernel<128, 128, 64, 2, 2, TA, TB, 2, 1>), 64, TA, TB, 2)
+    if (precision == 2) {
+        if (!ta && !tb) GRP16(0, 0); else if (ta && !tb) GRP16(1, 0); else if (!ta && tb) GRP16(0, 1); else GRP16(1, 1);
+    } else if (precision == 1) {
         if (!ta && !tb) GRP(0, 0, 1); else if (ta && !tb) GRP(1, 0, 1); else if (!ta && tb) GRP(0, 1, 1); else GRP(1, 1, 1);
     } else {
         if (!ta && !tb) GRP(0, 0, 0); else if (ta && !tb) GRP(1, 0, 0); else if (!ta && tb) GRP(0, 1, 0); else GRP(1, 1, 0);
     }
 #undef GRP
-#undef GRP2
+#undef GRP16
+#undef GRP_LAUNCH
     if (g_prof_on) g_prof.push_back(rec);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

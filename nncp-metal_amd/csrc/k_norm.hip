@@ -10,6 +10,7 @@
 #include <mutex>
 #include "../../include/nchip_kernels.h"
 #include "k_norm_inline.h"
+#include "k_bf16.h"
 
 // Scratch of nchip_norm_bwd_static: the partial dw / db rows of the norm backward, held by the
 // library itself so that the call allocates nothing.  In host code this name is only a
@@ -41,7 +42,7 @@ __device__ __forceinline__ float wave_max(float v)
 
 __global__ __launch_bounds__(TPB) void norm_fwd_kernel(const float *x, const float *w, const float *b,
                                                        float *y, float *xhat, float *rstd,
-                                                       int d, int64_t n, float eps, int avg)
+                                                       int d, int64_t n, float eps, int avg, uint16_t *y16)
 {
     int lane = threadIdx.x & 63;
     int64_t c = (int64_t)blockIdx.x * WPB + (threadIdx.x >> 6);
@@ -57,7 +58,9 @@ __global__ __launch_bounds__(TPB) void norm_fwd_kernel(const float *x, const flo
     for (int i = lane; i < d; i += 64) {
         float h = (xc[i] - mean) * r;
         if (xhat) xhat[c * d + i] = h;
-        y[c * d + i] = w ? h * w[i] + b[i] : h;
+        const float out = w ? h * w[i] + b[i] : h;
+        y[c * d + i] = out;
+        if (y16) y16[c * d + i] = f32_to_bf16_rne(out);
     }
 }
 
@@ -67,7 +70,7 @@ __global__ __launch_bounds__(TPB) void norm_fwd_kernel(const float *x, const flo
 template <int NV>
 __global__ __launch_bounds__(TPB) void norm_fwd_reg(const float *x, const float *w, const float *b,
                                                     float *y, float *xhat, float *rstd,
-                                                    int64_t n, float eps, int avg)
+                                                    int64_t n, float eps, int avg, uint16_t *y16)
 {
     constexpr int D = 64 * NV;
     const int lane = threadIdx.x & 63;
@@ -89,12 +92,17 @@ __global__ __launch_bounds__(TPB) void norm_fwd_reg(const float *x, const float 
         if (xhat) xhat[c * D + lane + 64 * v] = h[v];
         y[c * D + lane + 64 * v] = yv[v];
     }
+    if (y16) { // the operand copy of the products that read y
+#pragma unroll
+        for (int v = 0; v < NV; v++) y16[c * D + lane + 64 * v] = f32_to_bf16_rne(yv[v]);
+    }
 }
 
 // dx = rstd * (gh - mean(gh) - xhat * mean(gh * xhat)),  gh = g * w
 __global__ __launch_bounds__(TPB) void norm_bwd_dx_kernel(const float *g, const float *xhat,
                                                           const float *rstd, const float *w,
-                                                          float *dx, const float *dx_add, int d, int64_t n, int avg)
+                                                          float *dx, const float *dx_add, int d, int64_t n, int avg,
+                                                          uint16_t *dx16)
 {
     int lane = threadIdx.x & 63;
     int64_t c = (int64_t)blockIdx.x * WPB + (threadIdx.x >> 6);
@@ -112,7 +120,9 @@ __global__ __launch_bounds__(TPB) void norm_bwd_dx_kernel(const float *g, const 
     for (int i = lane; i < d; i += 64) {
         float gh = w ? gc[i] * w[i] : gc[i];
         float v = r * (gh - s1 - hc[i] * s2);
-        dx[c * d + i] = dx_add ? dx_add[c * d + i] + v : v;
+        v = dx_add ? dx_add[c * d + i] + v : v;
+        dx[c * d + i] = v;
+        if (dx16) dx16[c * d + i] = f32_to_bf16_rne(v);
     }
 }
 
@@ -142,7 +152,7 @@ template <int NV>
 __global__ __launch_bounds__(TPB) void norm_bwd_fused(const float *g, const float *xhat, const float *rstd,
                                                       const float *w, float *dx, const float *dx_add,
                                                       float *partial, int64_t n, int avg, int cw,
-                                                      float *dx_partial)
+                                                      float *dx_partial, uint16_t *dx16)
 {
     constexpr int D = NV * 64;
     __shared__ float sh[WPB - 1][3][D];
@@ -175,6 +185,7 @@ __global__ __launch_bounds__(TPB) void norm_bwd_fused(const float *g, const floa
                 float val = r * (gv[v] * wr[v] - s1 - hv[v] * s2);
                 val = dx_add ? dx_add[c * D + lane + 64 * v] + val : val;
                 dx[c * D + lane + 64 * v] = val;
+                if (dx16) dx16[c * D + lane + 64 * v] = f32_to_bf16_rne(val);
                 ax[v] += val;
             }
         }
@@ -420,6 +431,7 @@ __global__ __launch_bounds__(TPB) void opt_update_multi_kernel(const NchipOptTen
         opt_step(algo, w, t.m ? t.m + i : nullptr, v, t.g[i], t.lr, b1, b2, eps, clip, c1, c2);
         t.w[i] = w;
         if (t.v) t.v[i] = v;
+        if (t.w16) t.w16[i] = f32_to_bf16_rne(w);
     }
 }
 
@@ -446,16 +458,22 @@ extern "C" {
 int nchip_norm_fwd(void *stream, const float *x, const float *w, const float *b, float *y,
                    float *xhat, float *rstd, int d, int64_t n, float eps, int avg)
 {
+    return nchip_norm_fwd_bf16copy(stream, x, w, b, y, xhat, rstd, d, n, eps, avg, nullptr);
+}
+
+int nchip_norm_fwd_bf16copy(void *stream, const float *x, const float *w, const float *b, float *y,
+                            float *xhat, float *rstd, int d, int64_t n, float eps, int avg, uint16_t *y16)
+{
     if (n <= 0 || d <= 0) return 0;
     if ((w == nullptr) != (b == nullptr)) { fprintf(stderr, "nchip_norm_fwd: w and b go together\n"); return -1; }
     const dim3 grid((unsigned)((n + WPB - 1) / WPB));
-#define NORM_FWD(NV) hipLaunchKernelGGL(norm_fwd_reg<NV>, grid, dim3(TPB), 0, (hipStream_t)stream, x, w, b, y, xhat, rstd, n, eps, avg)
+#define NORM_FWD(NV) hipLaunchKernelGGL(norm_fwd_reg<NV>, grid, dim3(TPB), 0, (hipStream_t)stream, x, w, b, y, xhat, rstd, n, eps, avg, y16)
     if (d == 128) NORM_FWD(2);
     else if (d == 256) NORM_FWD(4);
     else if (d == 512) NORM_FWD(8);
     else if (d == 1024) NORM_FWD(16);
     else
-        hipLaunchKernelGGL(norm_fwd_kernel, grid, dim3(TPB), 0, (hipStream_t)stream, x, w, b, y, xhat, rstd, d, n, eps, avg);
+        hipLaunchKernelGGL(norm_fwd_kernel, grid, dim3(TPB), 0, (hipStream_t)stream, x, w, b, y, xhat, rstd, d, n, eps, avg, y16);
 #undef NORM_FWD
     return check("nchip_norm_fwd");
 }
@@ -498,7 +516,15 @@ int nchip_norm_bwd_rowsum(void *stream, const float *g, const float *xhat, const
                           float *dx, const float *dx_add, float *dw, float *db, float *partial, int d, int64_t n,
                           int avg, float *dx_partial)
 {
+    return nchip_norm_bwd_bf16copy(stream, g, xhat, rstd, w, dx, dx_add, dw, db, partial, d, n, avg, dx_partial, nullptr);
+}
+
+int nchip_norm_bwd_bf16copy(void *stream, const float *g, const float *xhat, const float *rstd, const float *w,
+                            float *dx, const float *dx_add, float *dw, float *db, float *partial, int d, int64_t n,
+                            int avg, float *dx_partial, uint16_t *dx16)
+{
     if (n <= 0 || d <= 0) return 0;
+    if (dx16 && !dx) { fprintf(stderr, "nchip_norm_bwd_bf16copy: a copy of dx needs dx\n"); return -1; }
     if (dx_partial && (!dx || !nchip_norm_bwd_has_dx_rowsum(d))) {
         fprintf(stderr, "nchip_norm_bwd_rowsum: row sums of dx need dx and d in {128, 256, 512, 1024}\n");
         return -1;
@@ -511,7 +537,7 @@ int nchip_norm_bwd_rowsum(void *stream, const float *g, const float *xhat, const
         const int cw = norm_bwd_cw(n);
         const int rows = nchip_norm_bwd_rows(d, n);
         float *pp = partial;
-#define NORM_BWD(NV) hipLaunchKernelGGL(norm_bwd_fused<NV>, dim3(rows), dim3(TPB), 0, st, g, xhat, rstd, w, dx, dx_add, pp, n, avg, cw, dx_partial)
+#define NORM_BWD(NV) hipLaunchKernelGGL(norm_bwd_fused<NV>, dim3(rows), dim3(TPB), 0, st, g, xhat, rstd, w, dx, dx_add, pp, n, avg, cw, dx_partial, dx16)
         if (d == 128) NORM_BWD(2); else if (d == 256) NORM_BWD(4); else if (d == 512) NORM_BWD(8); else NORM_BWD(16);
 #undef NORM_BWD
         if (wb)
@@ -521,7 +547,7 @@ int nchip_norm_bwd_rowsum(void *stream, const float *g, const float *xhat, const
     }
     if (dx)
         hipLaunchKernelGGL(norm_bwd_dx_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, st,
-                           g, xhat, rstd, w, dx, dx_add, d, n, avg);
+                           g, xhat, rstd, w, dx, dx_add, d, n, avg, dx16);
     if (partial) {
         int rows = nchip_norm_bwd_rows(d, n);
         hipLaunchKernelGGL(norm_bwd_wb_stage1, dim3((d + TPB - 1) / TPB, rows), dim3(TPB), 0, st,

@@ -6,6 +6,8 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <dlfcn.h>
+#include <time.h>
 #include "nc_hip_internal.h"
 
 [[noreturn]] void nc_fatal(const char *fmt, ...)
@@ -104,6 +106,7 @@ extern "C" NCContext *nc_context_init(int nb_threads)
     m->matmul_bf16 = 0;
     m->matmul_invariant = 0;
     m->launches = 0;
+    m->shadow_casts = 0;
     m->node_seq = 0;
     m->epoch = 0;
     m->defer_wgrad = false;
@@ -201,13 +204,81 @@ void nc_staging_retire(NCContext *m, void *p, size_t cap, uint64_t stamp)
     else staging_reclaim(m);
 }
 
+void nc_mark_in_flight(NCTensor *x)
+{
+    x->buf->in_flight = x->buf->dev->ctx->sync_count + 1;
+}
+
 extern "C" void nc_synchronize(NCDevice *d)
 {
     if (d->ctx->hip_ready)
         nc_stream_wait(d->ctx);
 }
 
-extern "C" void nc_prof_dump(void) {}
+// ---- profiling hooks (libnc.h:14-67) -----------------------------------------------------
+// Section timers of the host code above the ABI: wall-clock nanoseconds per section (the
+// kernels of a section run asynchronously, so a section's time is the time the host spent
+// in it, waits included), plus - with NC_PROFILE set - a roctx range per section for
+// rocprofv3's marker trace.  The roctx library is looked up at run time and only then.
+extern "C" {
+int64_t prof_cycles[PROF_COUNT], prof_samples[PROF_COUNT], prof_ops[PROF_COUNT];
+}
+static const char *const PROF_NAMES[PROF_COUNT] = { "EVAL", "GRAD", "SGD", "UPDATE", "WRITE_SYM", "PROBE", "TOTAL" };
+static bool prof_enabled() { static const bool on = getenv("NC_PROFILE") && *getenv("NC_PROFILE"); return on; }
+typedef int (*RoctxPush)(const char *);
+typedef int (*RoctxPop)(void);
+static RoctxPush roctx_push;
+static RoctxPop roctx_pop;
+static void roctx_lookup()
+{
+    static bool done = false;
+    if (done) return;
+    done = true;
+    for (const char *name : { "libroctx64.so.4", "libroctx64.so", "librocprofiler-sdk-roctx.so.1" }) {
+        if (void *h = dlopen(name, RTLD_NOW | RTLD_LOCAL)) {
+            roctx_push = (RoctxPush)dlsym(h, "roctxRangePushA");
+            roctx_pop = (RoctxPop)dlsym(h, "roctxRangePop");
+            if (roctx_push && roctx_pop) return;
+            roctx_push = nullptr; roctx_pop = nullptr;
+        }
+    }
+}
+static int64_t prof_now()
+{
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (int64_t)ts.tv_sec * 1000000000 + ts.tv_nsec;
+}
+
+extern "C" void nc_prof_begin(int idx)
+{
+    if (idx < 0 || idx >= PROF_COUNT) return;
+    if (prof_enabled()) {
+        roctx_lookup();
+        if (roctx_push) roctx_push(PROF_NAMES[idx]);
+    }
+    prof_cycles[idx] -= prof_now();
+}
+
+extern "C" void nc_prof_finish(int idx, int n_ops)
+{
+    if (idx < 0 || idx >= PROF_COUNT) return;
+    prof_cycles[idx] += prof_now();
+    prof_samples[idx]++;
+    prof_ops[idx] += n_ops;
+    if (prof_enabled() && roctx_pop) roctx_pop();
+}
+
+extern "C" void nc_prof_dump(void) // libnc.h:67
+{
+    if (!prof_enabled()) return;
+    fprintf(stderr, "%-10s %10s %14s %12s %12s\n", "section", "samples", "total ms", "us/sample", "ops");
+    for (int i = 0; i < PROF_COUNT; i++) {
+        if (!prof_samples[i]) continue;
+        fprintf(stderr, "%-10s %10lld %14.3f %12.2f %12lld\n", PROF_NAMES[i], (long long)prof_samples[i],
+                prof_cycles[i] * 1e-6, prof_cycles[i] * 1e-3 / prof_samples[i], (long long)prof_ops[i]);
+    }
+}
 
 extern "C" int nc_set_matmul_width_invariant(NCContext *m, int enable) // nc_ext.h
 {
@@ -302,6 +373,7 @@ NCTensor *nc_alloc(NCDevice *d, NCTypeEnum t, int nd, const size_t *dims, bool z
     x->buf->ref = 1;
     x->buf->dev = d;
     size_t bytes = n * nc_type_size(t);
+    x->buf->elems = n;
     x->buf->ptr = pool_of(d).get(bytes ? bytes : 4, &x->buf->cap);
     if (zero && bytes) {
         if (d->is_hip) { k_fill_bytes(d->ctx->stream, x->buf->ptr, 0, (int64_t)bytes); d->ctx->launches++; }
@@ -332,6 +404,72 @@ NCTensor *nc_reshape_view(NCTensor *x, int nd, const size_t *dims)
     if (s != nc_numel(x)) nc_fatal("reshape: element count mismatch (%zu vs %zu)", s, nc_numel(x));
     nc_free_tensor(x);
     return y;
+}
+
+// ---- bf16 shadows --------------------------------------------------------------------------
+static bool shadow_capable(const NCTensor *x)
+{
+    return x->dev->is_hip && x->type == NC_TYPE_F32 && nc_is_contig(x) && x->off % 8 == 0 && x->buf->elems > 0;
+}
+
+static void shadow_alloc(NCContext *m, NCTensorBuffer *b)
+{
+    if (!b->sh) {
+        b->sh = (uint16_t *)m->dev_pool.get(b->elems * sizeof(uint16_t) + 64, &b->sh_cap);
+        b->sh_valid = false;
+    }
+}
+
+static int g_shadow_check = getenv("NCHIP_SHADOW_CHECK") ? atoi(getenv("NCHIP_SHADOW_CHECK")) : 0;
+static int shadow_check_mode() { return g_shadow_check; }
+
+extern "C" int nc_set_bf16_shadow_check(int enable) // nc_ext.h
+{
+    int old = g_shadow_check;
+    g_shadow_check = enable != 0;
+    return old;
+}
+
+extern "C" int64_t nc_get_bf16_cast_count(NCContext *m) { return m->shadow_casts; } // nc_ext.h
+
+const uint16_t *nc_shadow_of(NCContext *m, const NCTensor *x)
+{
+    if (!shadow_capable(x)) return nullptr;
+    NCTensorBuffer *b = x->buf;
+    if (b->sh_valid && shadow_check_mode()) {
+        // debugging aid: a shadow that claims to be valid must equal a fresh cast
+        size_t cap;
+        uint16_t *tmp = (uint16_t *)m->dev_pool.get(b->elems * sizeof(uint16_t) + 64, &cap);
+        if (nchip_cast_bf16(m->stream, (const float *)b->ptr, tmp, (int64_t)b->elems)) nc_fatal("bf16 cast failed");
+        std::vector<uint16_t> h0(b->elems), h1(b->elems);
+        hip_check(hipMemcpyAsync(h0.data(), tmp, b->elems * 2, hipMemcpyDeviceToHost, m->stream), "shadow check copy");
+        hip_check(hipMemcpyAsync(h1.data(), b->sh, b->elems * 2, hipMemcpyDeviceToHost, m->stream), "shadow check copy");
+        nc_stream_wait(m);
+        m->dev_pool.put(tmp, cap);
+        if (memcmp(h0.data(), h1.data(), b->elems * 2) != 0)
+            nc_fatal("bf16 shadow of a buffer of %zu elements is stale (a writer did not invalidate it)", b->elems);
+    }
+    if (!b->sh_valid) {
+        shadow_alloc(m, b);
+        if (nchip_cast_bf16(m->stream, (const float *)b->ptr, b->sh, (int64_t)b->elems)) nc_fatal("bf16 cast failed");
+        m->launches++;
+        m->shadow_casts++;
+        b->sh_valid = true;
+    }
+    return b->sh + x->off;
+}
+
+uint16_t *nc_shadow_for_write(NCContext *m, NCTensor *x)
+{
+    if (!shadow_capable(x) || x->off != 0 || nc_numel(x) != x->buf->elems) return nullptr;
+    shadow_alloc(m, x->buf);
+    x->buf->sh_valid = true;
+    return x->buf->sh;
+}
+
+void nc_shadow_invalidate(NCTensor *x)
+{
+    if (x && x->buf) x->buf->sh_valid = false;
 }
 
 float *nc_tmp_f32(NCContext *m, size_t n, size_t *cap)
@@ -373,7 +511,12 @@ extern "C" void nc_free_tensor(NCTensor *x) // libnc.h:174; NULL accepted (nncp.
     if (!x || --x->ref > 0) return;
     nc_free_node(x->node);
     if (--x->buf->ref == 0) {
-        pool_of(x->buf->dev).put(x->buf->ptr, x->buf->cap);
+        NCContext *m = x->buf->dev->ctx;
+        if (x->buf->sh) m->dev_pool.put(x->buf->sh, x->buf->sh_cap); // stream ordered, like the buffer itself
+        if (x->buf->in_flight && !x->buf->dev->is_hip && x->buf->in_flight > m->sync_count)
+            nc_staging_retire(m, x->buf->ptr, x->buf->cap, x->buf->in_flight - 1); // a queued kernel may still use it
+        else
+            pool_of(x->buf->dev).put(x->buf->ptr, x->buf->cap);
         free(x->buf);
     }
     free(x);
@@ -394,6 +537,7 @@ extern "C" int nc_tensor_get_dims(const NCTensor *x, size_t *dims)
 extern "C" void *nc_tensor_get_ptr(const NCTensor *x, size_t *pstride)
 {
     if (pstride) *pstride = x->n_dims >= 2 ? x->strides[1] : (x->n_dims ? x->dims[0] : 1);
+    x->buf->sh_valid = false; // the address leaves the library: whoever holds it may write
     return nc_data(x);
 }
 
@@ -426,6 +570,7 @@ void nc_copy_any(NCTensor *dst, const NCTensor *src)
     if (dst->dev != src->dev)
         nc_fatal("copy: tensors live on different devices");
     if (nc_numel(dst) == 0) return;
+    nc_shadow_invalidate(dst);
     if (!dst->dev->is_hip) { host_copy_strided(dst, src); return; }
     NCContext *m = dst->dev->ctx;
     if (nc_is_contig(dst) && nc_is_contig(src)) {
@@ -488,6 +633,7 @@ extern "C" void nc_tensor_set_zero(NCTensor *y) // libnc.h:192
 {
     size_t bytes = nc_numel(y) * nc_type_size(y->type);
     if (!bytes) return;
+    nc_shadow_invalidate(y);
     if (nc_is_contig(y)) {
         if (y->dev->is_hip) { k_fill_bytes(nc_stream(y), nc_data(y), 0, (int64_t)bytes); nc_ctx(y)->launches++; }
         else memset(nc_data(y), 0, bytes);
@@ -501,6 +647,7 @@ extern "C" void nc_tensor_set_zero(NCTensor *y) // libnc.h:192
 extern "C" void nc_tensor_set_f32(NCTensor *y, float val) // libnc.h:194
 {
     if (!nc_is_contig(y) || y->type != NC_TYPE_F32) nc_fatal("set_f32: contiguous f32 tensor expected");
+    nc_shadow_invalidate(y);
     if (y->dev->is_hip) { k_fill_f32(nc_stream(y), nc_f32(y), val, (int64_t)nc_numel(y)); nc_ctx(y)->launches++; }
     else for (size_t i = 0; i < nc_numel(y); i++) nc_f32(y)[i] = val;
 }
@@ -620,6 +767,7 @@ static void upload_f32(NCTensor *y, const float *host)
 extern "C" void nc_tensor_set_rnd_unif(NCTensor *y, float avg, float range, NCRNDState *rs)
 {
     if (!nc_is_contig(y) || y->type != NC_TYPE_F32) nc_fatal("set_rnd_unif: contiguous f32 tensor expected");
+    nc_shadow_invalidate(y);
     size_t n = nc_numel(y);
     float *tmp = (float *)nc_malloc(n * sizeof(float));
     for (size_t i = 0; i < n; i++) {
@@ -633,6 +781,7 @@ extern "C" void nc_tensor_set_rnd_unif(NCTensor *y, float avg, float range, NCRN
 extern "C" void nc_tensor_set_dropout(NCTensor *y, float prob, NCRNDState *rs) // libnc.h:201
 {
     if (!nc_is_contig(y) || y->type != NC_TYPE_F32) nc_fatal("set_dropout: contiguous f32 tensor expected");
+    nc_shadow_invalidate(y);
     size_t n = nc_numel(y);
     float *tmp = (float *)nc_malloc(n * sizeof(float)), keep = 1.0f / (1.0f - prob);
     for (size_t i = 0; i < n; i++) {
@@ -754,6 +903,29 @@ extern "C" void nc_sgd_opt_set_all(NCParamList *pl, NCSGDOptState *s)
 
 extern "C" void nc_sgd_opt_set_lr(NCSGDOptState *s, float lr) { s->p.lr = lr; }
 
+// nc_ext.h: the moments of one parameter, out as a host copy and in from any f32 tensor
+extern "C" NCTensor *nc_sgd_opt_get_state(NCParam *p, int which)
+{
+    SGDOptVarState *vs = p->sgd_opt;
+    NCTensor *t = !vs ? nullptr : which == 0 ? vs->m : which == 1 ? vs->v : nullptr;
+    return t ? nc_tensor_to_cpu_device(nc_dup_tensor(t)) : nullptr;
+}
+
+extern "C" void nc_sgd_opt_set_state(NCParam *p, int which, const NCTensor *v)
+{
+    SGDOptVarState *vs = p->sgd_opt;
+    NCTensor *t = !vs ? nullptr : which == 0 ? vs->m : which == 1 ? vs->v : nullptr;
+    if (!t) nc_fatal("nc_sgd_opt_set_state: '%s' keeps no moment %d", p->name, which);
+    if (v->type != NC_TYPE_F32 || nc_numel(v) != vs->n) nc_fatal("nc_sgd_opt_set_state: %zu f32 values expected for '%s'", vs->n, p->name);
+    size_t n1 = vs->n;
+    NCTensor *src = nc_reshape_view(nc_tensor_to_device(nc_dup_tensor(v), t->dev), 1, &n1);
+    nc_tensor_copy(t, src);
+    nc_free_tensor(src);
+}
+
+extern "C" int64_t nc_sgd_opt_get_step(NCSGDOptState *s) { return s->step; }
+extern "C" void nc_sgd_opt_set_step(NCSGDOptState *s, int64_t step) { s->step = step; }
+
 // libnc.h:563: the NCParamUpdateFunc nncp.c forwards to (nncp.c:1095); yg is
 // consumed.  Only accumulates; nc_sgd_opt_update applies.
 extern "C" void sgd_opt_update_var(void *opaque, NCTensor *yg, NCTensor *get_col_index)
@@ -805,6 +977,10 @@ extern "C" void nc_sgd_opt_update(NCSGDOptState *s)
         t.n = (int64_t)vs->n;
         t.lr = p->lr * vs->param->lr_mult;
         t.pad_ = 0;
+        // matrices are operands of the bf16 products: their shadow is written with the update
+        // (vectors - biases, gains - are not, and a shadow they may have is stale from here on)
+        t.w16 = (s->ctx->matmul_bf16 && w->n_dims >= 2) ? nc_shadow_for_write(s->ctx, w) : nullptr;
+        if (!t.w16) nc_shadow_invalidate(w);
         tab.push_back(t);
         prefix.push_back(prefix.back() + (int)((vs->n + chunk - 1) / chunk));
     }

@@ -90,6 +90,7 @@ struct NCContext {
     int matmul_bf16;
     int matmul_invariant; // forward products use the width-invariant GEMM class
     int64_t launches;
+    int64_t shadow_casts; // bf16 shadows made by a cast of their own (not by the producing kernel)
     int64_t node_seq;
     int epoch;
     bool defer_wgrad;
@@ -121,6 +122,19 @@ struct NCTensorBuffer {
     NCDevice *dev;
     void *ptr;
     size_t cap;
+    // host buffers that a queued kernel reads or writes in place (nc_mark_in_flight): the
+    // wait count when that kernel was enqueued, plus one (0 = never handed to a kernel)
+    uint64_t in_flight;
+    // bf16 shadow of a device f32 buffer (bf16-operand products only): the same elements in
+    // the same order, rounded to nearest even.  Written either by the kernel that produces
+    // the f32 values (norms, product epilogues, the optimiser) or by one cast the first time
+    // a product asks for it; every later product reads 2 bytes per element instead of 4.
+    // sh_valid says that sh holds the rounding of what the buffer holds NOW: whatever writes
+    // into an existing buffer clears it (nc_shadow_invalidate).
+    uint16_t *sh;
+    size_t sh_cap;
+    bool sh_valid;
+    size_t elems; // elements the buffer was allocated for
 };
 
 struct NCTensor {
@@ -197,6 +211,20 @@ void nc_stream_wait(NCContext *m);
 // caller that enqueues step after step without reading anything back), waits
 // first, so the buffer is never rewritten under a copy that has yet to run.
 void nc_staging_retire(NCContext *m, void *p, size_t cap, uint64_t stamp);
+// A kernel that was just enqueued reads or writes the pinned memory of host tensor x in
+// place: when the last reference goes, the buffer returns to the pool only after the stream
+// has been waited for (nc_free_tensor retires it like a pinned table).
+void nc_mark_in_flight(NCTensor *x);
+
+// bf16 shadows (nc_core.cpp).  nc_shadow_of: the shadow of contiguous f32 device tensor x,
+// made by one cast of the whole buffer if it is not valid yet; NULL when x cannot have one
+// (not f32, not on the device, not contiguous, offset not a multiple of 8 elements).
+// nc_shadow_for_write: the place where a kernel that is about to write ALL of x's buffer may
+// leave the shadow (marks it valid); NULL when x does not cover its buffer.
+// nc_shadow_invalidate: x's buffer is about to be written in place.
+const uint16_t *nc_shadow_of(NCContext *m, const NCTensor *x);
+uint16_t *nc_shadow_for_write(NCContext *m, NCTensor *x);
+void nc_shadow_invalidate(NCTensor *x);
 
 // nc_autodiff.cpp
 NCNode *nc_new_node(NCContext *m, int op, int n_args, NCTensor **args);

@@ -569,12 +569,53 @@ extern "C" void nc_forget_k_major_weights(NCContext *m)
     m->k_major.clear();
 }
 
+// The product through the operands' bf16 shadows (bf16 mode, plain unbatched products whose
+// shape the unguarded loaders take): no operand is converted inside the product, and none is
+// cast more than once however many products read it.  want_c16: also leave the result's own
+// shadow (it is the operand of a later product).  Returns false when this route does not
+// apply (nothing launched).
+struct Bf16Extra { const float *dpre = nullptr; int dact = 0; float *rowsum = nullptr; int *rows_written = nullptr; };
+static bool dev_gemm_bf16_operands(NCContext *m, bool ta, bool tb, size_t M, size_t N, size_t K, float alpha,
+                                   const NCTensor *a, const NCTensor *b, NCTensor *c, const float *bias, int act,
+                                   float *pre, const float *addend, bool want_c16, const Bf16Extra *ex = nullptr)
+{
+    static const bool off = getenv("NCHIP_BF16_SHADOWS") && atoi(getenv("NCHIP_BF16_SHADOWS")) == 0;
+    if (off || !m->matmul_bf16 || K % 64 || K < 64 || M < 64 || N < 16) return false;
+    const size_t lda = ta ? K : M, ldb = tb ? N : K;
+    if (lda % 8 || ldb % 8 || (!ta && M % 64) || (tb && N % 64)) return false;
+    const uint16_t *a16 = nc_shadow_of(m, a), *b16 = a16 ? nc_shadow_of(m, b) : nullptr;
+    if (!a16 || !b16) return false;
+    NchipGemmBf16Args g;
+    memset(&g, 0, sizeof(g));
+    g.ta = ta; g.tb = tb; g.m = (int)M; g.n = (int)N; g.k = (int)K; g.alpha = alpha;
+    g.A16 = a16; g.lda = (int64_t)lda; g.B16 = b16; g.ldb = (int64_t)ldb;
+    g.C = nc_f32(c); g.ldc = (int64_t)M;
+    g.bias = bias; g.act = act; g.pre = pre; g.addend = addend;
+    if (ex) { g.dpre = ex->dpre; g.dact = ex->dact; g.rowsum = ex->rowsum; g.rows_written = ex->rows_written; }
+    // (the result's shadow is claimed only once the launch is certain: a refused shape leaves it alone)
+    const bool had = c->buf->sh_valid;
+    g.C16 = want_c16 ? nc_shadow_for_write(m, c) : nullptr;
+    int rc = nchip_gemm_bf16_operands(m->stream, &g);
+    if (rc < 0) nc_fatal("gemm failed (bf16 operands, m=%zu n=%zu k=%zu)", M, N, K);
+    if (rc > 0) {
+        if (g.C16) c->buf->sh_valid = had;
+        return false;
+    }
+    if (!g.C16) nc_shadow_invalidate(c);
+    m->launches++;
+    return true;
+}
+
 static void dev_gemm(NCContext *m, bool ta, bool tb, size_t M, size_t N, size_t K, float alpha,
                      const NCTensor *a, const NCTensor *b, float beta, NCTensor *c, size_t batch,
                      const float *bias, int act, float *pre, const float *addend = nullptr,
-                     bool forward = false)
+                     bool forward = false, bool want_c16 = false)
 {
     const bool invariant = forward && m->matmul_invariant;
+    if (m->matmul_bf16 && !invariant && batch == 1 && beta == 0.0f &&
+        dev_gemm_bf16_operands(m, ta, tb, M, N, K, alpha, a, b, c, bias, act, pre, addend, want_c16))
+        return;
+    nc_shadow_invalidate(c);
     const int prec = m->matmul_bf16 | (invariant ? NCHIP_GEMM_WIDTH_INVARIANT : 0);
     int ks = invariant ? 1 : nchip_gemm_pick_ksplit((int)M, (int)N, (int)K, (int)batch);
     size_t cap = 0;
@@ -713,7 +754,18 @@ static void matmul_bw(NCNode *nd, NCTensor *g, NCTensor **ga, int ia, int ib)
             int rs_rows = 0;
             if (px->n_args > 2 && px->parents.size() > 2 && px->parents[2] && nc_can_defer_sum(m, px->parents[2]) && ks == 1)
                 rs = nc_tmp_f32(m, (size_t)nchip_gemm_rowsum_rows((int)s.n) * s.k, &rs_cap);
-            if (nchip_gemm_dact_rowsum(m->stream, !ta, 0, (int)s.k, (int)s.n, (int)s.m, alpha,
+            bool done = false;
+            if (m->matmul_bf16 && ks == 1) {
+                // operands from their bf16 shadows; the result (the gradient of the pre-activation) is
+                // the operand of the next two products, so its shadow comes out of this epilogue too
+                Bf16Extra ex;
+                ex.dpre = nc_f32(px->saved[2]); ex.dact = px->ia[3]; ex.rowsum = rs; ex.rows_written = &rs_rows;
+                done = dev_gemm_bf16_operands(m, !ta, false, s.k, s.n, s.m, alpha, a, g, db, nullptr, 0, nullptr, nullptr,
+                                              true, &ex);
+                if (done) m->launches--; // (counted below)
+            }
+            if (!done &&
+                nchip_gemm_dact_rowsum(m->stream, !ta, 0, (int)s.k, (int)s.n, (int)s.m, alpha,
                                        nc_f32(a), (int64_t)(!ta ? s.m : s.k), nc_f32(g), (int64_t)s.m,
                                        nc_f32(db), (int64_t)s.k, nc_f32(px->saved[2]), px->ia[3],
                                        m->matmul_bf16, ks, ws, rs, &rs_rows))
@@ -757,8 +809,10 @@ static NCTensor *linear_impl(NCTensor *w, NCTensor *x, NCTensor *bias, int act, 
     }
     bool graph = w->node || x->node || (bias && bias->node) || (res && res->node);
     NCTensor *pre = (act != NC_ACT_NONE && graph) ? nc_alloc_like(y) : nullptr;
+    // (an activated result feeds the next linear layer: in bf16 mode its operand copy is
+    // written by this product's epilogue)
     dev_gemm(m, false, false, s.m, s.n, s.k, 1.0f, w, x, 0.0f, y, 1, bias ? nc_f32(bias) : nullptr, act,
-             pre ? nc_f32(pre) : nullptr, res ? nc_f32(res) : nullptr, true);
+             pre ? nc_f32(pre) : nullptr, res ? nc_f32(res) : nullptr, true, act != NC_ACT_NONE);
     NCTensor *args[4] = { w, x, bias, res };
     NCNode *n = nc_new_node(m, OP_LINEAR, 4, args);
     if (graph) {
@@ -805,6 +859,7 @@ extern "C" NCTensor *nc_linear_pair_into(NCTensor *w0, NCTensor *bias0, NCTensor
     size_t dims[2] = { m0, n };
     NCTensor *y0 = new_f32(w0, 2, dims);
     float *slot = nc_f32(dst) + (size_t)index * m1 * n;
+    nc_shadow_invalidate(dst);
     int rc = 1;
     if (m->matmul_invariant && !m->matmul_bf16) {
         const float *k0 = nc_k_major_of(m, nc_f32(w0), m0, k), *k1 = nc_k_major_of(m, nc_f32(w1), m1, k);
@@ -865,6 +920,7 @@ extern "C" NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x, float sca
                              (int)w->dims[1], (int64_t)dims[1], scale))
         nc_fatal("nc_get_col_host_indices failed");
     LAUNCHED(w);
+    nc_mark_in_flight(x); // the kernel has yet to read the indices: their buffer outlives this reference
     nc_free_tensor(w); nc_free_tensor(x);
     return y;
 }
@@ -926,8 +982,11 @@ static NCTensor *norm_op(NCTensor *x, NCTensor *w, NCTensor *b, float eps, int a
     NCTensor *y = nc_alloc_like(x);
     NCTensor *xhat = w ? nc_alloc_like(x) : nc_dup_tensor(y);
     NCTensor *rstd = nc_alloc(x->dev, NC_TYPE_F32, 1, &cols, false);
-    if (nchip_norm_fwd(nc_stream(x), nc_f32(x), w ? nc_f32(w) : nullptr, b ? nc_f32(b) : nullptr, nc_f32(y),
-                       nc_f32(xhat), nc_f32(rstd), (int)d, (int64_t)cols, eps, avg))
+    // bf16 products: the normalised columns are the operand of the products that follow, so
+    // their bf16 copy is written here and never cast
+    uint16_t *y16 = nc_ctx(x)->matmul_bf16 ? nc_shadow_for_write(nc_ctx(x), y) : nullptr;
+    if (nchip_norm_fwd_bf16copy(nc_stream(x), nc_f32(x), w ? nc_f32(w) : nullptr, b ? nc_f32(b) : nullptr, nc_f32(y),
+                                nc_f32(xhat), nc_f32(rstd), (int)d, (int64_t)cols, eps, avg, y16))
         nc_fatal("layer norm failed");
     LAUNCHED(x);
     NCTensor *args[3] = { x, w, b };
@@ -964,6 +1023,9 @@ extern "C" NCTensor *nc_norm_linear_pair_into(NCTensor *x, NCTensor *g, NCTensor
     const char *me = "nc_norm_linear_pair_into";
     if ((g == nullptr) != (b == nullptr)) nc_fatal("%s: g and b go together", me);
     if ((w1 == nullptr) != (dst == nullptr)) nc_fatal("%s: w1 and dst go together", me);
+    if (dst) nc_shadow_invalidate(dst);
+    // (checked before a path is chosen: the pair kernel would apply act0 to the cache column too)
+    if (w1 && act0 != NC_ACT_NONE) nc_fatal("%s: no activation on the first product of a pair", me);
     x = nc_contig(x); w0 = nc_contig(w0);
     need_f32(x, me); need_f32(w0, me);
     NCContext *m = nc_ctx(w0);
@@ -1004,7 +1066,6 @@ extern "C" NCTensor *nc_norm_linear_pair_into(NCTensor *x, NCTensor *g, NCTensor
     } else { // other shapes and modes: the steps one after the other
         normed = g ? nc_fused_layer_norm(x, g, b, eps, avg_flag) : nc_fused_layer_norm(x, nullptr, nullptr, eps, avg_flag);
         if (w1) {
-            if (act0 != NC_ACT_NONE) nc_fatal("%s: no activation on the first product of a pair", me);
             y0 = nc_linear_pair_into(w0, bias0, w1, nc_dup_tensor(normed), dst, index);
         } else {
             y0 = nc_linear(w0, nc_dup_tensor(normed), bias0, act0);
@@ -1203,6 +1264,7 @@ extern "C" NCTensor *nc_soft_max_cdf16_to_host(NCTensor *logits)
     if (nchip_softmax_cdf16(m->stream, nc_f32(logits), (uint16_t *)nc_data(y), (int)v, (int64_t)(nc_numel(logits) / v)))
         nc_fatal("nc_soft_max_cdf16_to_host failed");
     m->launches++;
+    nc_mark_in_flight(y); // freed before the next wait, the buffer must not serve another tensor yet
     nc_free_tensor(logits);
     return y;
 }
@@ -1266,10 +1328,35 @@ static void flush_deferred_gemms(NCContext *m)
     std::stable_sort(m->deferred.begin(), m->deferred.end(), [](const DeferredGemm &x, const DeferredGemm &y) {
         return x.k + (x.a2 ? x.k2 : 0) > y.k + (y.a2 ? y.k2 : 0);
     });
+    // bf16 mode: when every problem fits the unguarded loaders, the operands are read from
+    // their bf16 shadows (which the forward and input-gradient products of the same tensors
+    // have left behind, or one cast each makes now)
+    bool from_shadows = m->matmul_bf16 != 0 && !(getenv("NCHIP_BF16_SHADOWS") && atoi(getenv("NCHIP_BF16_SHADOWS")) == 0);
+    for (const DeferredGemm &d : m->deferred)
+        if (d.m % 128 || d.n % 128 || d.k % 64 || (d.a2 && d.k2 % 64) || d.k < 64) from_shadows = false;
+    std::vector<const uint16_t *> sh;
+    if (from_shadows) {
+        for (const DeferredGemm &d : m->deferred) {
+            const NCTensor *ops[4] = { d.a, d.b, d.a2, d.b2 };
+            for (const NCTensor *t : ops) {
+                const uint16_t *q = t ? nc_shadow_of(m, t) : nullptr;
+                if (t && !q) from_shadows = false;
+                sh.push_back(q);
+            }
+        }
+    }
+    size_t di = 0;
     for (DeferredGemm &d : m->deferred) {
         NchipGemmProblem p;
-        p.A = nc_f32(d.a); p.B = nc_f32(d.b); p.C = nc_f32(d.c);
-        p.A2 = d.a2 ? nc_f32(d.a2) : nullptr; p.B2 = d.b2 ? nc_f32(d.b2) : nullptr;
+        if (from_shadows) {
+            p.A = (const float *)sh[4 * di]; p.B = (const float *)sh[4 * di + 1]; p.C = nc_f32(d.c);
+            p.A2 = (const float *)sh[4 * di + 2]; p.B2 = (const float *)sh[4 * di + 3];
+        } else {
+            p.A = nc_f32(d.a); p.B = nc_f32(d.b); p.C = nc_f32(d.c);
+            p.A2 = d.a2 ? nc_f32(d.a2) : nullptr; p.B2 = d.b2 ? nc_f32(d.b2) : nullptr;
+        }
+        di++;
+        nc_shadow_invalidate(d.c);
         p.m = d.m; p.n = d.n; p.k = d.k; p.k2 = d.a2 ? d.k2 : 0;
         flops += 2.0 * d.m * d.n * (double)(d.k + p.k2);
         p.lda = d.m; p.ldb = d.n; p.ldc = d.m;
@@ -1282,7 +1369,8 @@ static void flush_deferred_gemms(NCContext *m)
     void *dev = m->dev_pool.get(bytes, &dcap);
     memcpy(host, tab.data(), bytes);
     hip_check(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync gemm table");
-    if (nchip_gemm_grouped(m->stream, 0, 1, (const NchipGemmProblem *)dev, (int)tab.size(), tiles, m->matmul_bf16, flops))
+    if (nchip_gemm_grouped(m->stream, 0, 1, (const NchipGemmProblem *)dev, (int)tab.size(), tiles,
+                           from_shadows ? 2 : m->matmul_bf16, flops))
         nc_fatal("grouped weight-gradient GEMM failed");
     m->launches++;
     // pinned staging is recycled one flush later, after a wait for the stream
@@ -1622,9 +1710,11 @@ void nc_node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
             pl->parents.size() > 2 && pl->parents[2] && nc_can_defer_sum(m, pl->parents[2]) &&
             nchip_norm_bwd_has_dx_rowsum(d) && pl->saved[0] && (int)pl->saved[0]->dims[0] == d)
             dxp = nc_tmp_f32(m, (size_t)nchip_norm_bwd_rows(d, cols) * d, &dxp_cap);
-        if (nchip_norm_bwd_rowsum(st, nc_f32(g), nc_f32(xhat), nc_f32(rstd), w ? nc_f32(w) : nullptr,
-                                  dx ? nc_f32(dx) : nullptr, prev, (dw && !late) ? nc_f32(dw) : nullptr,
-                                  (db && !late) ? nc_f32(db) : nullptr, partial, d, cols, nd->ia[0], dxp))
+        // (bf16 products: dx is the operand of the products behind the layer that fed this norm)
+        uint16_t *dx16 = (dx && m->matmul_bf16) ? nc_shadow_for_write(m, dx) : nullptr;
+        if (nchip_norm_bwd_bf16copy(st, nc_f32(g), nc_f32(xhat), nc_f32(rstd), w ? nc_f32(w) : nullptr,
+                                    dx ? nc_f32(dx) : nullptr, prev, (dw && !late) ? nc_f32(dw) : nullptr,
+                                    (db && !late) ? nc_f32(db) : nullptr, partial, d, cols, nd->ia[0], dxp, dx16))
             nc_fatal("layer norm backward failed");
         if (dxp) {
             pl->grad_rowsum = dxp; pl->grad_rowsum_cap = dxp_cap; pl->grad_rowsum_rows = nchip_norm_bwd_rows(d, cols);

@@ -74,16 +74,33 @@ extern "C" NCTensor *nc_load_param(NCContext *m, FILE *f, char *name, size_t nam
 {
     uint32_t nl, type, nd;
     if (!get_u32(f, &nl)) return nullptr;
-    if (nl + 1 > name_size) nc_fatal("parameter file: a name of %u bytes does not fit the caller's buffer", nl);
+    // (compared as size_t: nl + 1 wraps to 0 for a name length of 0xffffffff)
+    if (name_size == 0 || (size_t)nl >= name_size)
+        nc_fatal("parameter file: a name of %u bytes does not fit the caller's buffer", nl);
     if (nl && fread(name, nl, 1, f) != 1) nc_fatal("parameter file: truncated record");
     name[nl] = 0;
-    if (!get_u32(f, &type) || !get_u32(f, &nd) || nd > NC_N_DIMS_MAX) nc_fatal("parameter file: bad record '%s'", name);
+    if (!get_u32(f, &type) || !get_u32(f, &nd)) nc_fatal("parameter file: truncated record '%s'", name);
+    // (no dimensions: a scalar parameter, one element)
+    if (nd > NC_N_DIMS_MAX || type >= (uint32_t)NC_TYPE_COUNT)
+        nc_fatal("parameter file: bad record '%s' (type %u, %u dimensions)", name, type, nd);
     size_t dims[NC_N_DIMS_MAX];
+    // what the file still holds bounds the record: checked before anything is allocated
+    const long here = ftell(f);
+    if (here < 0 || fseek(f, 0, SEEK_END) != 0) nc_fatal("parameter file: not seekable");
+    const long end = ftell(f);
+    if (end < here || fseek(f, here, SEEK_SET) != 0) nc_fatal("parameter file: not seekable");
+    const uint64_t left = (uint64_t)(end - here), esz = nc_type_size((NCTypeEnum)type);
+    if (left < 8ull * nd) nc_fatal("parameter file: truncated record '%s'", name);
+    uint64_t budget = (left - 8ull * nd) / esz, count = 1; // elements the rest of the file can hold
     for (uint32_t i = 0; i < nd; i++) {
         uint64_t d;
         if (!get_u64(f, &d)) nc_fatal("parameter file: truncated record '%s'", name);
+        if (d == 0 || d > budget / count)
+            nc_fatal("parameter file: record '%s' claims more elements than the file holds", name);
+        count *= d;
         dims[i] = (size_t)d;
     }
+    if (budget < count) nc_fatal("parameter file: truncated record '%s'", name);
     NCTensor *h = nc_new_tensor(nc_new_cpu_device(m), (NCTypeEnum)type, (int)nd, dims);
     size_t bytes = nc_numel(h) * nc_type_size(h->type);
     if (bytes && fread(nc_data(h), bytes, 1, f) != 1) nc_fatal("parameter file: truncated record '%s'", name);

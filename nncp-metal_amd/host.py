@@ -137,6 +137,11 @@ class Host:
         L.nncp_model_param.restype = C.POINTER(_P)
         L.nncp_model_param.argtypes = [_P, C.c_char_p]
         L.nncp_model_param_count.argtypes = [_P]
+        L.nncp_model_opt_state.restype = _P
+        L.nncp_model_opt_state.argtypes = [_P, C.c_char_p, C.c_int]
+        L.nncp_model_set_opt_state.argtypes = [_P, C.c_char_p, C.c_int, _P]
+        L.nncp_model_memory.restype = _P
+        L.nncp_model_memory.argtypes = [_P, C.c_int]
         L.nncp_model_param_name.restype = C.c_char_p
         L.nncp_model_param_name.argtypes = [_P, C.c_int]
         for n in ("nncp_model_save_coefs", "nncp_model_load_coefs"):
@@ -312,6 +317,38 @@ class Model:
 
     def params(self):
         return {n: self.get_param(n) for n in self.param_names()}
+
+    def state(self):
+        """Everything one training step hands to the next: parameters, the optimiser's second
+        moments and the per-layer memories, as numpy arrays (a checkpoint)."""
+        names = self.param_names()
+        v = {}
+        for n in names:
+            t = self.L.nncp_model_opt_state(self.ptr, n.encode(), 1)
+            if t:
+                v[n] = self._to_numpy(t)
+                self.nc.nc_free_tensor(t)
+        mem = []
+        for l in range(self.cfg.n_layer):
+            t = self.L.nncp_model_memory(self.ptr, l)
+            if t:
+                mem.append(self._to_numpy(t))
+        return dict(w={n: self.get_param(n) for n in names}, v=v, mem=mem)
+
+    def load_state(self, st):
+        """Puts the model into a state taken from another model of the same configuration,
+        on either library (see state())."""
+        for n, a in st["w"].items():
+            self.set_param(n, a)
+        for n, a in st["v"].items():
+            h = self._host_tensor(np.ascontiguousarray(a, dtype=np.float32).ravel())
+            self.L.nncp_model_set_opt_state(self.ptr, n.encode(), 1, h)
+            self.nc.nc_free_tensor(h)
+        for l, a in enumerate(st["mem"]):
+            dst = self.L.nncp_model_memory(self.ptr, l)
+            src = self.nc.nc_tensor_to_device(self._host_tensor(np.ascontiguousarray(a, dtype=np.float32)), self.dev)
+            self.nc.nc_tensor_copy(dst, src)
+            self.nc.nc_free_tensor(src)
 
     def save_coefs(self, path):
         """Every parameter to a parameter file (nc_save_coefs, libnc.h:530)."""

@@ -518,6 +518,7 @@ int nncp_encode_file(const char *in_name, const char *out_name, const NNCPConfig
         add_stats(retrain_st, &bs);
     }
     nncp_put_bit_flush(&pb);
+    nc_prof_dump(); /* nncp.c:3505 */
     nncp_model_free(s);
     free(block);
     free(arith_buf);
@@ -602,6 +603,7 @@ int nncp_decode_file(const char *in_name, const char *out_name, int use_device, 
         nncp_retrain_block(s, block, len, &fp.lr, &bs);
         add_stats(retrain_st, &bs);
     }
+    nc_prof_dump(); /* nncp.c:3676 */
     nncp_model_free(s);
     free(block);
     free(data);

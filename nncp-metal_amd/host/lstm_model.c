@@ -168,6 +168,7 @@ NCTensor *lstm_eval(NNCPModel *s, int output_index, const NCTensor *input) /* nn
     if (output_index < 0) { ls->seq_eval = 0; t0i = 0; t1i = T; }
     else { ls->seq_eval = 1; t0i = output_index; t1i = output_index + 1; }
     const int n = t1i - t0i;
+    prof_start(PROF_EVAL); /* nncp.c:1881 */
     NCTensor **layer_out = nc_mallocz(sizeof(NCTensor *) * T * L);
     NCTensor **pre = nc_mallocz(sizeof(NCTensor *) * T);
     NCTensor **tmp = nc_mallocz(sizeof(NCTensor *) * (T > L ? T : L));
@@ -266,6 +267,7 @@ NCTensor *lstm_eval(NNCPModel *s, int output_index, const NCTensor *input) /* nn
     nc_free(layer_out);
     nc_free(pre);
     nc_free(tmp);
+    prof_end(PROF_EVAL); /* nncp.c:2056 */
     return output;
 }
 
@@ -286,6 +288,7 @@ float lstm_eval_gradient(NNCPModel *s, const NCTensor *expected_output) /* nncp.
     struct LstmState *ls = s->lstm;
     NCTensor *output, *loss;
     float ret;
+    prof_start(PROF_GRAD); /* nncp.c:2079 */
     if (ls->seq_eval) {
         NCNode *node;
         output = nc_concat(ls->outputs, c->seg_len, 2);
@@ -307,12 +310,15 @@ float lstm_eval_gradient(NNCPModel *s, const NCTensor *expected_output) /* nncp.
     nc_free_tensor(loss);
     nc_free_tensor(ls->logits);
     ls->logits = NULL;
+    prof_end(PROF_GRAD); /* nncp.c:2131 */
     return ret;
 }
 
 void lstm_update(NNCPModel *s) /* nncp.c:2136-2142 */
 {
+    prof_start(PROF_UPDATE); /* nncp.c:2139 */
     nc_sgd_opt_update(s->opt);
+    prof_end(PROF_UPDATE); /* nncp.c:2141 */
     s->train_step++; /* counted by process_block in the reference (nncp.c:3056) */
 }
 

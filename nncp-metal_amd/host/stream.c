@@ -104,6 +104,7 @@ static HostDist fetch_dist(Coder *c, NCTensor *output)
 static int code_symbol(Coder *c, const HostDist *d, size_t col, int stream, int pos)
 {
     int sym;
+    prof_start(PROF_WRITE_SYM); /* nncp.c:3007, 3039 */
     if (!c->is_decode) {
         sym = get_symb(&c->view, stream, pos);
         if (d->cdf) nncp_write_sym_cdf(c->pb, d->cdf + col * d->stride, c->n_symbols, sym);
@@ -113,6 +114,7 @@ static int code_symbol(Coder *c, const HostDist *d, size_t col, int stream, int 
         else sym = nncp_read_sym(c->gb, d->prob + col * d->stride, c->n_symbols);
         put_symb(&c->view, stream, pos, sym);
     }
+    prof_end(PROF_WRITE_SYM); /* nncp.c:3018, 3041 */
     return sym;
 }
 
@@ -272,6 +274,7 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
     const int overlap = mode == NNCP_MODE_SEGMENT && !is_decode; /* code while the training kernels run */
     while (idx + T <= c.view.stride) { /* nncp.c:2993 */
         HostDist pending = { 0 };
+        prof_start(PROF_TOTAL); /* nncp.c:2994 */
         if (overlap)
             pending = encode_segment_eval(&c, idx, T, T, 1, input, expected);
         else
@@ -290,6 +293,7 @@ void nncp_process_block(NNCPModel *s, NNCPPutBit *pb, NNCPGetBit *gb, uint16_t *
         c.st->n_steps++;
         c.st->n_symbols += (int64_t)T * B;
         idx += T;
+        prof_end_ops(PROF_TOTAL, T * B); /* nncp.c:3056 */
     }
     int len2 = c.view.stride - idx, len1 = len2 + (c.view.rem != 0); /* nncp.c:3076-3077 */
     if (len1 > 0) {

@@ -216,6 +216,31 @@ const char *nncp_model_param_name(NNCPModel *s, int index)
     return NULL;
 }
 
+static NCParam *find_param_entry(NNCPModel *s, const char *name)
+{
+    NCParam *p = nc_find_param(&s->params, name);
+    if (!p)
+        die("no parameter of that name");
+    return p;
+}
+
+NCTensor *nncp_model_opt_state(NNCPModel *s, const char *name, int which)
+{
+    return nc_sgd_opt_get_state(find_param_entry(s, name), which);
+}
+
+void nncp_model_set_opt_state(NNCPModel *s, const char *name, int which, const NCTensor *v)
+{
+    nc_sgd_opt_set_state(find_param_entry(s, name), which, v);
+}
+
+NCTensor *nncp_model_memory(NNCPModel *s, int l)
+{
+    if (s->cfg.model_type == NNCP_MODEL_LSTM || s->cfg.mem_len <= 0 || l < 0 || l >= s->cfg.n_layer)
+        return NULL;
+    return s->mem_h[l];
+}
+
 /* parameter files: what --load_coefs names (nncp.c:3149, 3761; its use at nncp.c:3439-3442 and
    3604-3607 is compiled out in the reference, the calls are libnc.h:530, 536) */
 void nncp_model_save_coefs(NNCPModel *s, const char *filename) { nc_save_coefs(&s->params, filename); }
@@ -524,6 +549,7 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
     int seg_len, B = c->batch_size;
     NCTensor *t0, *x, *output;
 
+    prof_start(PROF_EVAL); /* nncp.c:606 */
     /* dropout masks sit between steps that the fused entry points merge, so a
        retrain pass goes through the op-by-op sequence */
     s->fused_now = c->fused && !s->dropout_enabled;
@@ -600,6 +626,7 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
     s->outputs[output_index < 0 ? 0 : output_index] = nc_dup_tensor(output);
     if (!fused && (output_index < 0 || output_index == c->seg_len - 1))
         free_position_tensors(s);
+    prof_end(PROF_EVAL); /* nncp.c:1027 */
     return output;
 }
 
@@ -826,6 +853,7 @@ float trf_eval_gradient(NNCPModel *s, const NCTensor *expected_output1) /* nncp.
     NCTensor *expected = nc_tensor_to_device(nc_dup_tensor(expected_output1), s->dev);
     NCTensor *output, *loss;
     float ret;
+    prof_start(PROF_GRAD); /* nncp.c:1108 */
     if (s->seq_eval) {
         NCNode **tab = nc_malloc(sizeof(NCNode *) * (c->n_layer * 2 + 1));
         int count = 0;
@@ -853,6 +881,7 @@ float trf_eval_gradient(NNCPModel *s, const NCTensor *expected_output1) /* nncp.
     nc_free_tensor(loss);
     nc_free_tensor(s->logits);
     s->logits = NULL;
+    prof_end(PROF_GRAD); /* nncp.c:1191 */
     return ret;
 }
 
@@ -865,6 +894,7 @@ void trf_reset(NNCPModel *s) /* nncp.c:1195-1203 */
 void trf_update(NNCPModel *s) /* nncp.c:1224-1235 with mem_update nncp.c:1205-1221 */
 {
     int M = s->cfg.mem_len, T = s->cfg.seg_len;
+    prof_start(PROF_UPDATE); /* nncp.c:1227 */
     nc_sgd_opt_update(s->opt);
     for (int l = 0; l < s->cfg.n_layer && M > 0; l++) {
         if (M > T) {
@@ -881,6 +911,7 @@ void trf_update(NNCPModel *s) /* nncp.c:1224-1235 with mem_update nncp.c:1205-12
         }
     }
     s->train_step++;
+    prof_end(PROF_UPDATE); /* nncp.c:1234 */
 }
 
 void trf_set_lr(NNCPModel *s, float lr) { nc_sgd_opt_set_lr(s->opt, lr); }

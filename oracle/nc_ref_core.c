@@ -17,6 +17,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include <omp.h>
+#include <time.h>
 #include "nc_ref_internal.h"
 
 void nc_fatal(const char *fmt, ...)
@@ -78,12 +79,44 @@ NCDevice *nc_new_cpu_device(NCContext *m) { return m->cpu; }
 NCDevice *nc_new_cuda_device(NCContext *m, int device_index) { (void)device_index; return m->cpu; }
 NCDevice *nc_new_device(NCContext *m, const char *name) { (void)name; return m->cpu; }
 void nc_synchronize(NCDevice *d) { (void)d; }
-void nc_prof_dump(void) {}
+/* libnc.h:14-67: the section timers (nanoseconds of wall clock); no marker ranges here */
+int64_t prof_cycles[PROF_COUNT], prof_samples[PROF_COUNT], prof_ops[PROF_COUNT];
+static int64_t prof_clock(void)
+{
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (int64_t)ts.tv_sec * 1000000000 + ts.tv_nsec;
+}
+void nc_prof_begin(int idx)
+{
+    if (idx >= 0 && idx < PROF_COUNT)
+        prof_cycles[idx] -= prof_clock();
+}
+void nc_prof_finish(int idx, int n_ops)
+{
+    if (idx < 0 || idx >= PROF_COUNT)
+        return;
+    prof_cycles[idx] += prof_clock();
+    prof_samples[idx]++;
+    prof_ops[idx] += n_ops;
+}
+void nc_prof_dump(void)
+{
+    static const char *const names[PROF_COUNT] = { "EVAL", "GRAD", "SGD", "UPDATE", "WRITE_SYM", "PROBE", "TOTAL" };
+    const char *on = getenv("NC_PROFILE");
+    if (!on || !*on)
+        return;
+    for (int i = 0; i < PROF_COUNT; i++)
+        if (prof_samples[i])
+            fprintf(stderr, "%-10s %10lld samples %14.3f ms\n", names[i], (long long)prof_samples[i], prof_cycles[i] * 1e-6);
+}
 int nc_set_matmul_bf16(NCContext *m, int enable);
 int64_t nc_get_launch_count(NCContext *m) { (void)m; return 0; }
 void *nc_context_stream(NCContext *m) { (void)m; return NULL; }
 int nc_set_deferred_weight_grad(NCContext *m, int enable) { (void)m; (void)enable; return 0; }
 int nc_set_matmul_width_invariant(NCContext *m, int enable) { (void)m; (void)enable; return 0; }
+int64_t nc_get_bf16_cast_count(NCContext *m) { (void)m; return 0; }
+int nc_set_bf16_shadow_check(int enable) { (void)enable; return 0; }
 
 size_t nc_type_size(NCTypeEnum t)
 {
@@ -558,6 +591,46 @@ void nc_sgd_opt_set_all(NCParamList *pl, NCSGDOptState *s)
 }
 
 void nc_sgd_opt_set_lr(NCSGDOptState *s, float lr) { s->p.lr = lr; }
+
+/* nc_ext.h: a parameter's moments as tensors (the checker keeps both for every algorithm;
+   the ones an algorithm never touches read as NULL, as in the product) */
+static float *moment_of(NCParam *p, int which)
+{
+    struct SGDOptVarState *vs = p->sgd_opt;
+    if (!vs)
+        return NULL;
+    int algo = (int)vs->opt->p.algo;
+    if (which == 0)
+        return algo == SGD_OPT_ADAM && vs->opt->p.u.adam.beta1 != 0.0f ? vs->m : NULL;
+    if (which == 1)
+        return algo != SGD_OPT_BASIC ? vs->v : NULL;
+    return NULL;
+}
+
+NCTensor *nc_sgd_opt_get_state(NCParam *p, int which)
+{
+    float *src = moment_of(p, which);
+    if (!src)
+        return NULL;
+    NCTensor *t = nc_new_tensor_1d(nc_new_cpu_device((*p->pval)->dev->ctx), NC_TYPE_F32, p->sgd_opt->n);
+    memcpy(nc_f32(t), src, p->sgd_opt->n * sizeof(float));
+    return t;
+}
+
+void nc_sgd_opt_set_state(NCParam *p, int which, const NCTensor *v)
+{
+    float *dst = moment_of(p, which);
+    if (!dst)
+        nc_fatal("nc_sgd_opt_set_state: '%s' keeps no moment %d", p->name, which);
+    if (v->type != NC_TYPE_F32 || nc_numel(v) != p->sgd_opt->n)
+        nc_fatal("nc_sgd_opt_set_state: %zu f32 values expected for '%s'", p->sgd_opt->n, p->name);
+    NCTensor *c = nc_contig(nc_dup_tensor(v));
+    memcpy(dst, nc_f32(c), p->sgd_opt->n * sizeof(float));
+    nc_free_tensor(c);
+}
+
+int64_t nc_sgd_opt_get_step(NCSGDOptState *s) { return s->step; }
+void nc_sgd_opt_set_step(NCSGDOptState *s, int64_t step) { s->step = step; }
 
 /* libnc.h:563: the NCParamUpdateFunc nncp.c forwards to (nncp.c:1095);
    opaque is the NCParam, yg is consumed. */

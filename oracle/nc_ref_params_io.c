@@ -71,26 +71,49 @@ void nc_save_param(FILE *f, const NCTensor *v1, const char *name)
     nc_free_tensor(h);
 }
 
+/* bytes between the read position and the end of the file */
+static uint64_t bytes_left(FILE *f)
+{
+    long pos = ftell(f), end;
+    if (pos < 0 || fseek(f, 0, SEEK_END))
+        nc_fatal("parameter file: not seekable");
+    end = ftell(f);
+    if (end < pos || fseek(f, pos, SEEK_SET))
+        nc_fatal("parameter file: not seekable");
+    return (uint64_t)(end - pos);
+}
+
 NCTensor *nc_load_param(NCContext *m, FILE *f, char *name, size_t name_size)
 {
     uint32_t nl, type, nd;
     size_t dims[NC_N_DIMS_MAX], n = 1, stride;
+    uint64_t room;
     if (fread(&nl, 4, 1, f) != 1)
         return NULL;
-    if (nl + 1 > name_size)
+    if ((size_t)nl >= name_size) /* in size_t: a 32-bit nl + 1 wraps for 0xffffffff */
         nc_fatal("parameter file: a name of %u bytes does not fit the caller's buffer", nl);
     if (nl && fread(name, nl, 1, f) != 1)
         nc_fatal("parameter file: truncated record");
     name[nl] = 0;
-    if (fread(&type, 4, 1, f) != 1 || fread(&nd, 4, 1, f) != 1 || nd > NC_N_DIMS_MAX)
-        nc_fatal("parameter file: bad record '%s'", name);
+    if (fread(&type, 4, 1, f) != 1 || fread(&nd, 4, 1, f) != 1)
+        nc_fatal("parameter file: truncated record '%s'", name);
+    if (nd > NC_N_DIMS_MAX || type >= NC_TYPE_COUNT) /* nd = 0: a scalar */
+        nc_fatal("parameter file: bad record '%s' (type %u, %u dimensions)", name, type, nd);
+    room = bytes_left(f);
+    if (room < (uint64_t)nd * 8)
+        nc_fatal("parameter file: truncated record '%s'", name);
+    room = (room - (uint64_t)nd * 8) / nc_type_size((NCTypeEnum)type);
     for (uint32_t i = 0; i < nd; i++) {
         uint64_t d;
         if (fread(&d, 8, 1, f) != 1)
             nc_fatal("parameter file: truncated record '%s'", name);
+        if (d == 0 || d > room / n)
+            nc_fatal("parameter file: record '%s' claims more elements than the file holds", name);
         dims[i] = (size_t)d;
         n *= dims[i];
     }
+    if (room < n)
+        nc_fatal("parameter file: truncated record '%s'", name);
     NCTensor *h = nc_new_tensor(nc_new_cpu_device(m), (NCTypeEnum)type, (int)nd, dims);
     size_t bytes = n * nc_type_size((NCTypeEnum)type);
     if (bytes && fread(nc_tensor_get_ptr(h, &stride), bytes, 1, f) != 1)

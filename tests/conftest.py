@@ -45,6 +45,30 @@ def pkg():
     return load_pkg()
 
 
+@pytest.fixture(scope="session", autouse=True)
+def library_runtime_first(request):
+    """Whenever a GPU test is selected, the product library's HIP runtime is brought up before
+    the first test runs.  torch bundles a HIP runtime of its own (its autograd engine counts the
+    devices at its first backward pass); of two runtimes in one process the one that
+    initialises second finds no device, and the library then ends the process
+    ("no HIP device 0 (found 0)").  Done here, no test can let torch's copy come up first,
+    whatever it does before it asks for the library."""
+    if any(item.get_closest_marker("gpu") is not None for item in request.session.items):
+        lib = hip_lib_path(load_pkg())
+        if not os.path.exists(lib):
+            pytest.fail("%s is missing: build it first (there is no fallback path)" % lib)
+        import ctypes
+        nc = ctypes.CDLL(lib, mode=ctypes.RTLD_LOCAL)
+        nc.nc_context_init.restype = ctypes.c_void_p
+        nc.nc_new_cuda_device.restype = ctypes.c_void_p
+        nc.nc_new_cuda_device.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        nc.nc_context_end.argtypes = [ctypes.c_void_p]
+        ctx = nc.nc_context_init(1)
+        nc.nc_new_cuda_device(ctx, 0)
+        nc.nc_context_end(ctx)
+    yield
+
+
 @pytest.fixture()
 def ref(pkg):
     if not os.path.exists(REF_LIB):

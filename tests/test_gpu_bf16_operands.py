@@ -1,0 +1,249 @@
+"""Products whose operands are read as bf16 from memory (nchip_gemm_bf16_operands, the grouped
+launch with precision 2, nchip_cast_bf16) and the shadow copies that feed them at the tensor
+level.  The yardstick is numpy: both operands rounded to bf16 (nearest even, the rounding
+tests/test_oracle_ops.py pins against torch), products and sums in float64 - the kernels
+accumulate the same rounded values in fp32, so they must agree to fp32 summation error (1e-5
+of the largest magnitude); bf16 copies of results must be the nearest-even rounding of the
+fp32 results, bit for bit."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from conftest import hip_lib_path
+
+pytestmark = pytest.mark.gpu
+
+
+def bf16_round(x):
+    """float32 -> the float32 value of its nearest-even bf16 rounding, and the 16 bits"""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint32)
+    return (r << 16).view(np.float32).reshape(np.shape(x)), r.astype(np.uint16).reshape(np.shape(x))
+
+
+def relerr(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return float(np.abs(a - b).max() / (np.abs(b).max() + 1e-30))
+
+
+class Args(C.Structure):
+    _fields_ = [("ta", C.c_int), ("tb", C.c_int), ("m", C.c_int), ("n", C.c_int), ("k", C.c_int),
+                ("alpha", C.c_float), ("A16", C.c_void_p), ("B16", C.c_void_p), ("lda", C.c_int64),
+                ("ldb", C.c_int64), ("C", C.c_void_p), ("ldc", C.c_int64), ("C16", C.c_void_p),
+                ("bias", C.c_void_p), ("act", C.c_int), ("pre", C.c_void_p), ("addend", C.c_void_p),
+                ("dpre", C.c_void_p), ("dact", C.c_int), ("rowsum", C.c_void_p), ("rows_written", C.POINTER(C.c_int))]
+
+
+class Problem(C.Structure):
+    _fields_ = [("A", C.c_void_p), ("B", C.c_void_p), ("C", C.c_void_p), ("A2", C.c_void_p), ("B2", C.c_void_p),
+                ("m", C.c_int), ("n", C.c_int), ("k", C.c_int), ("k2", C.c_int),
+                ("lda", C.c_int), ("ldb", C.c_int), ("ldc", C.c_int), ("tile_start", C.c_int), ("alpha", C.c_float)]
+
+
+@pytest.fixture()
+def raw(hip, pkg):
+    lib = C.CDLL(hip_lib_path(pkg))
+    lib.nchip_cast_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]
+    lib.nchip_gemm_bf16_operands.argtypes = [C.c_void_p, C.POINTER(Args)]
+    lib.nchip_gemm_grouped.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_double]
+    st = C.c_void_p(hip.nc_context_stream(hip.ctx))
+    ptr = lambda t: C.c_void_p(hip.lib.nc_tensor_get_ptr(t, None))
+    return lib, st, ptr
+
+
+def gelu(x):
+    return 0.5 * x * (1.0 + np.tanh(0.7978845608 * (x + 0.044715 * x ** 3)))
+
+
+def gelu_grad(x):
+    c0, c1 = 0.7978845608, 0.044715
+    t = np.tanh(c0 * (x + c1 * x ** 3))
+    return 0.5 * (1 + t) + 0.5 * x * (1 - t * t) * c0 * (1 + 3 * c1 * x * x)
+
+
+@pytest.mark.parametrize("n", [8, 4096, 1000003, 13])
+def test_cast_is_round_to_nearest_even(hip, raw, rng, n):
+    lib, st, ptr = raw
+    x = (rng.standard_normal(n) * np.exp(rng.uniform(-30, 30, n))).astype(np.float32)
+    x[: min(n, 6)] = np.array([0.0, -0.0, 1.00390625, 1.01171875, np.float32(2.0 ** -130), 3.0e38], np.float32)[: min(n, 6)]
+    src, dst = hip.tensor(x), hip.tensor(np.zeros(n, np.uint16))
+    assert lib.nchip_cast_bf16(st, ptr(src), ptr(dst), n) == 0
+    got = hip.numpy(dst)
+    hip.free(src, dst)
+    assert np.array_equal(got, bf16_round(x)[1])
+
+
+# (m, n, k): every tile class (forced below) must divide what it needs whole
+SHAPES = [(128, 128, 64), (256, 192, 128), (512, 2048, 512), (384, 100, 192), (128, 77, 64), (1024, 256, 320)]
+
+
+@pytest.mark.parametrize("cls", [0, 1, 2, 3])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_product_from_bf16_operands(hip, raw, rng, m, n, k, ta, tb, cls):
+    lib, st, ptr = raw
+    if tb and n % 128:
+        pytest.skip("a column-contiguous B must fill whole tiles")
+    a = rng.standard_normal((m, k) if ta else (k, m)).astype(np.float32)      # numpy order: (columns, rows)
+    b = rng.standard_normal((k, n) if tb else (n, k)).astype(np.float32)
+    bias = rng.standard_normal(m).astype(np.float32)
+    add = rng.standard_normal((n, m)).astype(np.float32)
+    A = bf16_round(a)[0].astype(np.float64)
+    B = bf16_round(b)[0].astype(np.float64)
+    Am = A if not ta else A.T                  # (k, m) numpy = column-major (m, k)
+    Bm = B if not tb else B.T                  # (n, k)
+    pre = 0.75 * (Bm @ Am) + bias              # (n, m): column-major (m, n)
+    want = gelu(pre) + add
+    t = {k_: hip.tensor(v) for k_, v in dict(a=a, b=b, bias=bias, add=add).items()}
+    t.update(a16=hip.tensor(np.zeros(a.shape, np.uint16)), b16=hip.tensor(np.zeros(b.shape, np.uint16)),
+             c=hip.tensor(np.full((n, m), 7.0, np.float32)), pre=hip.tensor(np.full((n, m), 7.0, np.float32)),
+             c16=hip.tensor(np.full((n, m), 7, np.uint16)))
+    assert lib.nchip_cast_bf16(st, ptr(t["a"]), ptr(t["a16"]), a.size) == 0
+    assert lib.nchip_cast_bf16(st, ptr(t["b"]), ptr(t["b16"]), b.size) == 0
+    lib.nchip_gemm_bf16_operands_class(cls)
+    g = Args(ta=ta, tb=tb, m=m, n=n, k=k, alpha=0.75, A16=ptr(t["a16"]), B16=ptr(t["b16"]),
+             lda=k if ta else m, ldb=n if tb else k, C=ptr(t["c"]), ldc=m, C16=ptr(t["c16"]),
+             bias=ptr(t["bias"]), act=1, pre=ptr(t["pre"]), addend=ptr(t["add"]))
+    rc = lib.nchip_gemm_bf16_operands(st, C.byref(g))
+    lib.nchip_gemm_bf16_operands_class(0)
+    assert rc == 0
+    c, p, c16 = hip.numpy(t["c"]), hip.numpy(t["pre"]), hip.numpy(t["c16"])
+    hip.free(*t.values())
+    assert relerr(p, pre) <= 1e-5
+    assert relerr(c, want) <= 1e-5
+    assert np.array_equal(c16, bf16_round(c)[1])        # the copy is the rounding of what C holds
+
+
+def test_activation_gradient_epilogue_and_row_sums(hip, raw, rng):
+    lib, st, ptr = raw
+    m, n, k = 256, 384, 128                      # dX (m, n) = W^T (m, k) dY (k, n), times gelu'(pre)
+    w = rng.standard_normal((m, k)).astype(np.float32)        # column-major (k, m): ta = 1
+    dy = rng.standard_normal((n, k)).astype(np.float32)
+    pre = rng.standard_normal((n, m)).astype(np.float32)
+    want = (bf16_round(dy)[0].astype(np.float64) @ bf16_round(w)[0].astype(np.float64).T) * gelu_grad(pre.astype(np.float64))
+    lib.nchip_gemm_rowsum_rows.restype = C.c_int
+    rows = lib.nchip_gemm_rowsum_rows(n)
+    t = dict(w=hip.tensor(w), dy=hip.tensor(dy), pre=hip.tensor(pre), w16=hip.tensor(np.zeros(w.shape, np.uint16)),
+             dy16=hip.tensor(np.zeros(dy.shape, np.uint16)), c=hip.tensor(np.zeros((n, m), np.float32)),
+             c16=hip.tensor(np.zeros((n, m), np.uint16)), rs=hip.tensor(np.full((rows, m), 9.0, np.float32)))
+    lib.nchip_cast_bf16(st, ptr(t["w"]), ptr(t["w16"]), w.size)
+    lib.nchip_cast_bf16(st, ptr(t["dy"]), ptr(t["dy16"]), dy.size)
+    written = C.c_int(0)
+    g = Args(ta=1, tb=0, m=m, n=n, k=k, alpha=1.0, A16=ptr(t["w16"]), B16=ptr(t["dy16"]), lda=k, ldb=k,
+             C=ptr(t["c"]), ldc=m, C16=ptr(t["c16"]), dpre=ptr(t["pre"]), dact=1, rowsum=ptr(t["rs"]),
+             rows_written=C.pointer(written))
+    assert lib.nchip_gemm_bf16_operands(st, C.byref(g)) == 0
+    c, c16, rs = hip.numpy(t["c"]), hip.numpy(t["c16"]), hip.numpy(t["rs"])
+    hip.free(*t.values())
+    assert relerr(c, want) <= 1e-5
+    assert np.array_equal(c16, bf16_round(c)[1])
+    assert 0 < written.value <= rows
+    assert relerr(rs[: written.value].sum(axis=0), c.astype(np.float64).sum(axis=0)) <= 1e-5
+
+
+def test_grouped_launch_from_bf16_operands(hip, raw, rng):
+    """dW = alpha (dY X^T + dY2 X2^T) for three problems of different sizes in one launch."""
+    lib, st, ptr = raw
+    probs = [(256, 128, 192, 64), (128, 384, 64, 0), (512, 256, 128, 128)]   # (m, n, k, k2)
+    keep, table, wants, outs, tiles, flops = [], [], [], [], 0, 0.0
+    for m, n, k, k2 in probs:
+        ops = [rng.standard_normal((kk, dim)).astype(np.float32) for kk, dim in ((k, m), (k, n), (k2, m), (k2, n)) if kk]
+        dev = [hip.tensor(o) for o in ops]
+        d16 = [hip.tensor(np.zeros(o.shape, np.uint16)) for o in ops]
+        for s_, d_, o in zip(dev, d16, ops):
+            assert lib.nchip_cast_bf16(st, ptr(s_), ptr(d_), o.size) == 0
+        r = [bf16_round(o)[0].astype(np.float64) for o in ops]
+        want = r[1].T @ r[0] + (r[3].T @ r[2] if k2 else 0.0)                 # (n, m) numpy = column-major (m, n)
+        out = hip.tensor(np.full((n, m), 5.0, np.float32))
+        table.append(Problem(A=ptr(d16[0]), B=ptr(d16[1]), C=ptr(out), A2=ptr(d16[2]) if k2 else None,
+                             B2=ptr(d16[3]) if k2 else None, m=m, n=n, k=k, k2=k2, lda=m, ldb=n, ldc=m,
+                             tile_start=tiles, alpha=0.5))
+        tiles += (m // 128) * (n // 128)
+        flops += 2.0 * m * n * (k + k2)
+        wants.append(0.5 * want)
+        outs.append(out)
+        keep += dev + d16
+    raw_table = np.frombuffer(b"".join(bytes(p) for p in table), dtype=np.uint8)
+    dev_table = hip.tensor(raw_table)
+    assert lib.nchip_gemm_grouped(st, 0, 1, ptr(dev_table), len(table), tiles, 2, flops) == 0
+    for out, want in zip(outs, wants):
+        assert relerr(hip.numpy(out), want) <= 1e-5
+    hip.free(dev_table, *outs, *keep)
+
+
+def test_tensor_products_in_bf16_mode_use_and_keep_shadows(hip, ref, rng):
+    """nc_linear / nc_matmul with bf16 products on: forward, the activation-gradient product,
+    the input gradients and the weight gradients of a two-layer perceptron agree with
+    the checker's emulation of the same rounding (2e-2 is the variant's bar; these agree to
+    fp32 summation error), on shapes that take the shadow route and on shapes that do not;
+    an operand rewritten in place between two products is read again, not remembered."""
+    for d, f, n in ((128, 256, 192), (128, 256, 50), (96, 200, 64)):
+        w1 = (rng.standard_normal((d, f)) * 0.1).astype(np.float32)       # numpy (d, f) = column-major (f, d)
+        w2 = (rng.standard_normal((f, d)) * 0.1).astype(np.float32)
+        b1 = rng.standard_normal(f).astype(np.float32)
+        x = rng.standard_normal((n, d)).astype(np.float32)
+        res = []
+        for nc in (hip, ref):
+            nc.nc_set_matmul_bf16(nc.ctx, 1)
+            (h1, p1), (h2, p2), (hb, pb) = nc.param(w1, "w1"), nc.param(w2, "w2"), nc.param(b1, "b1")
+            hx, px = nc.param(x, "x")
+            y = nc.nc_linear(nc.dup(h1.value), nc.dup(hx.value), nc.dup(hb.value), 1)
+            y = nc.nc_matmul(nc.dup(h2.value), y)
+            out = nc.numpy(y)
+            loss = nc.nc_sum(nc.nc_mul(y, nc.tensor(np.linspace(-1, 1, out.size, dtype=np.float32).reshape(out.shape))))
+            grads = nc.backward(loss)
+            nc.free(loss)
+            res.append((out, [grads[p] for p in (p1, p2, pb, px)]))
+            # the same product again after x was rewritten in place: must see the new values
+            x2 = x[::-1].copy()
+            src = nc.tensor(x2)
+            nc.nc_tensor_copy(hx.value, src)
+            nc.free(src)
+            y2 = nc.nc_matmul(nc.dup(h1.value), nc.dup(hx.value))
+            res[-1] = res[-1] + (nc.numpy(y2, free=True),)
+            nc.nc_set_matmul_bf16(nc.ctx, 0)
+        (o_h, g_h, y2_h), (o_r, g_r, y2_r) = res
+        # one product: fp32 summation error.  A chain of two: an activation that sits near a
+        # rounding boundary may round to the other bf16 neighbour on the two sides (2^-9 of
+        # that element), which is what the looser bars of the chained results allow for.
+        assert relerr(y2_h, y2_r) <= 2e-5, (d, f, n)
+        assert relerr(o_h, o_r) <= 5e-4, (d, f, n)
+        for a, b in zip(g_h, g_r):
+            assert relerr(a, b) <= 2e-3, (d, f, n)
+
+
+def test_training_steps_through_shadows_match_the_checkers_emulation():
+    """Three RMSProp steps of a two-layer model whose every product takes the bf16-operand
+    route (d_model 128, 128 tokens per segment: forward, input-gradient, activation-gradient
+    and the grouped weight-gradient launch), with the shadow checker on: every copy a product
+    reads is compared with a fresh rounding of its buffer first (a stale copy ends the
+    process).  Probabilities, loss and parameters against the checker emulating the same
+    operand rounding, at the variant's bar; memories shift between the steps (mem_len >
+    seg_len), so copies of rewritten buffers must be dropped."""
+    import modelutil as M
+    hp = M.load_pkg().host
+    cfg = dict(n_layer=2, d_model=128, n_head=2, d_inner=256, d_pos=48, mem_len=32, seg_len=16,
+               batch_size=8, n_symbols=64, seed=11)
+    syms = M.markov1(cfg["batch_size"] * cfg["seg_len"] * 3, cfg["n_symbols"], seed=12)
+    batches = M.segment_batches(syms, cfg["batch_size"], cfg["seg_len"], 3)
+    res = []
+    for host, dev in ((M.hip_host(), 1), (M.ref_host(), 0)):
+        m = hp.Model(host, hp.make_config(**dict(cfg, use_device=dev, fused=1, nb_threads=4, sgd_opt=M.rmsprop(3e-4))))
+        m.nc.nc_set_matmul_bf16(m.ctx, 1)
+        old = m.nc.nc_set_bf16_shadow_check(1)
+        steps = [m.train_step(tok, tgt, 3e-4) for tok, tgt in batches]
+        casts = m.nc.nc_get_bf16_cast_count(m.ctx)
+        w = m.params()
+        m.nc.nc_set_bf16_shadow_check(old)
+        m.nc.nc_set_matmul_bf16(m.ctx, 0)
+        m.close()
+        res.append((steps, w, casts))
+    (s_h, w_h, casts), (s_r, w_r, _) = res
+    assert casts > 0                                  # the route was taken (embedding output, attention output, ...)
+    for (p_h, l_h), (p_r, l_r) in zip(s_h, s_r):
+        assert M.relerr(p_h, p_r) <= 2e-2
+        assert abs(l_h - l_r) <= 2e-2 * abs(l_r)
+    for k in w_r:
+        if w_r[k].ndim >= 2 and not k.startswith("b_r"):
+            assert M.rel_l2(w_h[k], w_r[k]) <= 2e-2, k

@@ -88,6 +88,15 @@ def test_host_tensor_compute_is_refused(emulated):
     assert r.returncode != 0 and "GPU only" in r.stderr
 
 
+def test_malformed_parameter_files_end_with_a_message(emulated, tmp_path):
+    """The product's own reader of parameter files (csrc/nc_params_io.cpp) against the malformed
+    records of tests/test_host_model.py: each ends in nc_fatal's message, none in a fault."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import test_host_model as T
+    T.check_malformed_files_end_cleanly(
+        tmp_path, "pkg.host.Host(%r, %r)" % (EMU_HOST, EMU_LIB), 1, env=emulated)
+
+
 def test_token_outside_the_table_reads_nothing_and_ends_the_process_at_the_next_wait(emulated):
     """nc_get_col with an index >= the number of columns (and a negative one): the kernel reads
     nothing out of range (the guard pages of this build would end the process with SIGSEGV), the
