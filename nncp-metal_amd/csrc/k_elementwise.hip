@@ -5,6 +5,7 @@
 // axis 0; reductions use fixed-order two-stage sums (no atomics) so results
 // are run-to-run identical.
 #include "k_internal.h"
+#include "k_act.h"
 
 namespace {
 
@@ -89,18 +90,8 @@ __global__ void masked_fill_kernel(const float *x, const int8_t *mask, float *y,
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-__device__ __forceinline__ float gelu_f(float x)
-{
-    const float c0 = 0.7978845608f, c1 = 0.044715f;
-    return 0.5f * x * (1.0f + tanhf(c0 * (x + c1 * x * x * x)));
-}
-
-__device__ __forceinline__ float gelu_grad_f(float x)
-{
-    const float c0 = 0.7978845608f, c1 = 0.044715f;
-    float t = tanhf(c0 * (x + c1 * x * x * x));
-    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * c0 * (1.0f + 3.0f * c1 * x * x);
-}
+__device__ __forceinline__ float gelu_f(float x) { return nchip_gelu(x); }           // k_act.h
+__device__ __forceinline__ float gelu_grad_f(float x) { return nchip_gelu_grad(x); }
 
 __global__ void unary_fwd_kernel(int op, const float *x, float *y, int64_t n)
 {

@@ -30,6 +30,7 @@
 #include "../../include/nchip_kernels.h"
 #include "k_addrspace.h"
 #include "k_bf16.h"
+#include "k_act.h"
 #include "k_norm_inline.h"
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -87,19 +88,11 @@ struct GemmArgs {
     int ln_avg;
 };
 
-__device__ __forceinline__ float gelu_tanh(float x)
-{
-    const float c0 = 0.7978845608f, c1 = 0.044715f;
-    return 0.5f * x * (1.0f + tanhf(c0 * (x + c1 * x * x * x)));
-}
+__device__ __forceinline__ float gelu_tanh(float x) { return nchip_gelu(x); } // k_act.h
 
 __device__ __forceinline__ float act_grad(float x, int act)
 {
-    if (act == NCHIP_ACT_GELU) {
-        const float c0 = 0.7978845608f, c1 = 0.044715f;
-        float t = tanhf(c0 * (x + c1 * x * x * x));
-        return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * c0 * (1.0f + 3.0f * c1 * x * x);
-    }
+    if (act == NCHIP_ACT_GELU) return nchip_gelu_grad(x);
     if (act == NCHIP_ACT_RELU) return x > 0.0f ? 1.0f : 0.0f;
     return 1.0f;
 }
@@ -1172,18 +1165,35 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_kernel(GemmArgs g0)
             compute(sa, sa + LDS_A);
             __syncthreads();
         };
-#pragma unroll
-        for (int j = 0; j < PF; j++)
-            if (j < nk) fetch(j, std::false_type(), la[j], lb[j]);
-        if (nk > 0) park(0, la[0], lb[0]);
-        if (PF < nk) fetch(PF, std::false_type(), la[0], lb[0]);
-        __syncthreads();
         int it = 0;
-        if (a_full && b_full) // steady state: every tile fetched here is complete
+        if (a_full && b_full && 2 * PF < nk_full) {
+            // Steady state: every tile fetched here is complete.  The first PF + 1 tiles are
+            // fetched by the same straight-line sequence as inside the loop, with nothing
+            // conditional between them and the loop: the compiler then sees one and the same
+            // queue of outstanding loads on entry and on the back edge and waits for the
+            // oldest register set only (s_waitcnt vmcnt(n)).  With a conditional fetch in
+            // front of the loop it assumes the worst path and drains every load in flight at
+            // the top of each trip - which is what the prefetch is there to avoid.
+#pragma unroll
+            for (int j = 0; j < PF; j++) {
+                fetch(j, std::true_type(), la[j], lb[j]);
+                __builtin_amdgcn_sched_barrier(0); // oldest tile first, as on the back edge
+            }
+            park(0, la[0], lb[0]);
+            fetch(PF, std::true_type(), la[0], lb[0]);
+            __syncthreads();
             for (; it + 2 * PF < nk_full; it += PF) {
 #pragma unroll
                 for (int j = 0; j < PF; j++) body(it + j, std::true_type(), la[(j + 1) % PF], lb[(j + 1) % PF]);
             }
+        } else {
+#pragma unroll
+            for (int j = 0; j < PF; j++)
+                if (j < nk) fetch(j, std::false_type(), la[j], lb[j]);
+            if (nk > 0) park(0, la[0], lb[0]);
+            if (PF < nk) fetch(PF, std::false_type(), la[0], lb[0]);
+            __syncthreads();
+        }
         for (; it < nk; it += PF) {
 #pragma unroll
             for (int j = 0; j < PF; j++)
@@ -1943,9 +1953,20 @@ extern "C" int nchip_gemm_bf16_operands(void *stream, const NchipGemmBf16Args *a
         rec.variant = 32 + cls * 4 + ta * 2 + tb; // the bf16-operand classes
     }
     ProfRec *pr = g_prof_on ? &rec : nullptr;
-    if (cls == 1) launch_tile<128, 128, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
-    else if (cls == 2) launch_tile<128, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
-    else launch_tile<64, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+    static const int pf = getenv("NCHIP_BF16OPS_PF") ? atoi(getenv("NCHIP_BF16OPS_PF")) : 2;
+    if (pf == 4) {
+        if (cls == 1) launch_tile<128, 128, 64, 2, 2, 2, 1, 3>(st, ta, tb, g, pr);
+        else if (cls == 2) launch_tile<128, 64, 64, 2, 2, 2, 1, 4>(st, ta, tb, g, pr);
+        else launch_tile<64, 64, 64, 2, 2, 2, 1, 4>(st, ta, tb, g, pr);
+    } else if (pf == 3) {
+        if (cls == 1) launch_tile<128, 128, 64, 2, 2, 2, 1, 2>(st, ta, tb, g, pr);
+        else if (cls == 2) launch_tile<128, 64, 64, 2, 2, 2, 1, 3>(st, ta, tb, g, pr);
+        else launch_tile<64, 64, 64, 2, 2, 2, 1, 3>(st, ta, tb, g, pr);
+    } else {
+        if (cls == 1) launch_tile<128, 128, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+        else if (cls == 2) launch_tile<128, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+        else launch_tile<64, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+    }
     if (g_prof_on) g_prof.push_back(rec);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

@@ -455,6 +455,9 @@ const uint16_t *nc_shadow_of(NCContext *m, const NCTensor *x)
         m->launches++;
         m->shadow_casts++;
         b->sh_valid = true;
+        static const bool trace = getenv("NCHIP_SHADOW_TRACE") != nullptr;
+        if (trace) fprintf(stderr, "[cast] %zu elements, tensor dims %zu x %zu (rank %d)\n", b->elems,
+                           x->n_dims > 0 ? x->dims[0] : 1, x->n_dims > 1 ? x->dims[1] : 1, x->n_dims);
     }
     return b->sh + x->off;
 }
