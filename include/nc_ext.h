@@ -150,6 +150,12 @@ int nc_set_matmul_bf16(NCContext *m, int enable);
    drop the copy); returns the previous setting.  Both 0 / no effect in libnc_ref.so. */
 int64_t nc_get_bf16_cast_count(NCContext *m);
 int nc_set_bf16_shadow_check(int enable);
+/* While non-zero (and nc_set_matmul_bf16 is on), the forward products nc_matmul / nc_matmul_add /
+   nc_linear / nc_linear_add also leave the bf16 copy of their result: for results that go
+   straight into another consumer of bf16 operands (the query and key / value projections in
+   front of nc_relpos_attention), which then needs no cast of them.  Returns the previous
+   setting.  No effect on values; no effect in libnc_ref.so. */
+int nc_set_bf16_copy_of_results(NCContext *m, int enable);
 
 /* When non-zero, nc_backward() postpones the weight-gradient GEMMs
    dW = dY X^T of plain linear layers (weight used once in the graph) and runs

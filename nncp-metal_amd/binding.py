@@ -127,6 +127,7 @@ _PROTOS = {
     "nc_set_matmul_bf16": (_I, [_P, _I]),
     "nc_get_launch_count": (C.c_int64, [_P]),
     "nc_get_bf16_cast_count": (C.c_int64, [_P]), "nc_set_bf16_shadow_check": (_I, [_I]),
+    "nc_set_bf16_copy_of_results": (_I, [_P, _I]),
     "nc_context_stream": (_P, [_P]),
     "nc_set_deferred_weight_grad": (_I, [_P, _I]),
 }

@@ -11,7 +11,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 SOURCES = {
-    "k_gemm.hip": [], "k_elementwise.hip": [], "k_norm.hip": [], "k_attention.hip": [], "k_attn_fused.hip": [],
+    "k_gemm.hip": [], "k_elementwise.hip": [], "k_norm.hip": [], "k_attention.hip": [], "k_attn_fused.hip": [], "k_attn_bf16.hip": [],
     # bit-exact integer-CDF path: no contraction, no reassociation
     "k_cdf.hip": ["-ffp-contract=off"],
     "nc_core.cpp": ["-x", "hip"], "nc_autodiff.cpp": ["-x", "hip"], "nc_params_io.cpp": ["-x", "hip"],

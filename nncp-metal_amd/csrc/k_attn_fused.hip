@@ -689,6 +689,19 @@ __global__ __launch_bounds__(256) void attn_param_grad_reduce(const float *dwp, 
     *dst = acc;
 }
 
+} // namespace
+
+int k_attn_param_grad_reduce(hipStream_t st, const float *dwp, float *dw, int64_t n_w,
+                             const float *dbp, float *db, int64_t n_b, int B)
+{
+    if (n_w + n_b <= 0) return 0;
+    hipLaunchKernelGGL(attn_param_grad_reduce, dim3((unsigned)((n_w + n_b + 255) / 256)), dim3(256), 0, st,
+                       dwp, dw, n_w, dbp, db, n_b, B);
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
+namespace {
+
 // ---- more than 128 keys: the same arithmetic with the key / position axis in chunks ------
 // Up to 320 keys and relative positions (NTT 16-key tiles, a multiple of 4).  Q, the rel
 // strips and the bias row stay in LDS for the whole kernel; w_r, K and V pass through ONE

@@ -109,5 +109,33 @@ int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk);
 // returns 0, -1 (path unavailable, nothing launched) or -2 (launch failed)
 int k_attn_fused_bwd(hipStream_t st, const FusedAttnBwdArgs &a, int dk, float *dw_r, float *db_r,
                      int64_t n_w, int64_t n_b, int *launches, bool keep_partials);
+// dw_r (n_w) and db_r (n_b) = sums over the B per-stream partials, in stream order (either may be NULL / 0)
+int k_attn_param_grad_reduce(hipStream_t st, const float *dwp, float *dw, int64_t n_w,
+                             const float *dbp, float *db, int64_t n_b, int B);
+
+// k_attn_bf16.hip: the same attention on the bf16 matrix cores.  Operands are the bf16 copies
+// of the fp32 tensors of FusedAttnFwdArgs / FusedAttnBwdArgs (same layouts, leading
+// dimensions in elements); probs is (K, T, H, B) bf16; out16 / dq16 / dkv16 / dkvm16 (may be
+// NULL) receive bf16 copies of the fp32 results, laid out like them.
+struct Bf16AttnFwdArgs {
+    const uint16_t *q, *kv, *kvm, *w_r;
+    const float *b_r;
+    float *out;
+    uint16_t *out16, *probs;
+    int64_t ldq, ldkv, ldo;
+    int H, B, T, M, K, d_pos, attn_len;
+    float b_r_scale, scale;
+};
+struct Bf16AttnBwdArgs {
+    const uint16_t *q, *kv, *kvm, *w_r, *probs, *dout;
+    float *dq, *dkv, *dkvm, *dwp, *dbp; // dwp / dbp: per-stream partials in scratch
+    uint16_t *dq16, *dkv16, *dkvm16;
+    int64_t ldq, ldkv, ldo;
+    int H, B, T, M, K, d_pos, attn_len;
+    float b_r_scale, scale;
+};
+bool k_attn_bf16_shape_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr);
+int k_attn_bf16_fwd(hipStream_t st, const Bf16AttnFwdArgs &a); // 0 or -2 (launch failed)
+int k_attn_bf16_bwd(hipStream_t st, const Bf16AttnBwdArgs &a);
 
 #endif

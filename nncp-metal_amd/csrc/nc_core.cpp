@@ -105,6 +105,7 @@ extern "C" NCContext *nc_context_init(int nb_threads)
     m->host_pool.device = false;
     m->matmul_bf16 = 0;
     m->matmul_invariant = 0;
+    m->bf16_copy_results = 0;
     m->launches = 0;
     m->shadow_casts = 0;
     m->node_seq = 0;
@@ -284,6 +285,13 @@ extern "C" int nc_set_matmul_width_invariant(NCContext *m, int enable) // nc_ext
 {
     int old = m->matmul_invariant;
     m->matmul_invariant = enable != 0;
+    return old;
+}
+
+extern "C" int nc_set_bf16_copy_of_results(NCContext *m, int enable) // nc_ext.h
+{
+    int old = m->bf16_copy_results;
+    m->bf16_copy_results = enable != 0;
     return old;
 }
 

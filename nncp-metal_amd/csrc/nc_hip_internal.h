@@ -89,6 +89,7 @@ struct NCContext {
     Pool dev_pool, host_pool;
     int matmul_bf16;
     int matmul_invariant; // forward products use the width-invariant GEMM class
+    int bf16_copy_results; // bf16 mode: forward products also leave the bf16 copy of their result
     int64_t launches;
     int64_t shadow_casts; // bf16 shadows made by a cast of their own (not by the producing kernel)
     int64_t node_seq;

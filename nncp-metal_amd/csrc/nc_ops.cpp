@@ -612,6 +612,7 @@ static void dev_gemm(NCContext *m, bool ta, bool tb, size_t M, size_t N, size_t 
                      bool forward = false, bool want_c16 = false)
 {
     const bool invariant = forward && m->matmul_invariant;
+    if (forward && m->bf16_copy_results) want_c16 = true; // nc_set_bf16_copy_of_results
     if (m->matmul_bf16 && !invariant && batch == 1 && beta == 0.0f &&
         dev_gemm_bf16_operands(m, ta, tb, M, N, K, alpha, a, b, c, bias, act, pre, addend, want_c16))
         return;
@@ -779,7 +780,10 @@ static void matmul_bw(NCNode *nd, NCTensor *g, NCTensor **ga, int ia, int ib)
             m->launches += ks > 1 ? 2 : 1;
             px->ia[5] = 1; // the gradient delivered to px is already d(pre-activation)
         } else
-        if (!tb) dev_gemm(m, !ta, false, s.k, s.n, s.m, alpha, a, g, 0.0f, db, s.batch, nullptr, 0, nullptr, prev);
+        // (the gradient of an attention output is an operand of the bf16 attention backward:
+        // its bf16 copy comes out of this product's epilogue)
+        if (!tb) dev_gemm(m, !ta, false, s.k, s.n, s.m, alpha, a, g, 0.0f, db, s.batch, nullptr, 0, nullptr, prev, false,
+                          px->op == OP_ATTN);
         else     dev_gemm(m, true, ta, s.n, s.k, s.m, alpha, g, a, 0.0f, db, s.batch, nullptr, 0, nullptr, prev);
         ga[ib] = db;
     }
@@ -1122,10 +1126,34 @@ extern "C" NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv
     size_t od[3] = { (size_t)a.H * a.dv, (size_t)a.B, (size_t)a.T };
     size_t pd[4] = { (size_t)a.K, (size_t)a.T, (size_t)a.H, (size_t)a.B };
     NCTensor *y = new_f32(all[0], 3, od);
-    NCTensor *probs = new_f32(all[0], 4, pd);
+    // bf16 products: the attention runs on the bf16 matrix cores from the operands' bf16 copies
+    // (left behind by the products that made q / kv and by the optimiser for w_r) when the
+    // head shape is that kernel's; the probabilities are then kept as bf16
+    bool on_bf16 = false;
+    NCTensor *probs = nullptr;
+    static const bool bf16_attn_off = getenv("NCHIP_BF16_ATTENTION") && atoi(getenv("NCHIP_BF16_ATTENTION")) == 0;
+    if (m->matmul_bf16 && !bf16_attn_off && k_attn_bf16_shape_ok(a.dk, a.dv, a.T, a.K, a.d_pos, all[3] != nullptr) &&
+        all[0]->dims[0] % 8 == 0 && all[1]->dims[0] % 8 == 0) {
+        const uint16_t *q16 = nc_shadow_of(m, all[0]), *kv16 = nc_shadow_of(m, all[1]);
+        const uint16_t *kvm16 = all[2] ? nc_shadow_of(m, all[2]) : nullptr;
+        const uint16_t *w16 = all[3] ? nc_shadow_of(m, all[3]) : nullptr;
+        if (q16 && kv16 && (!all[2] || kvm16) && (!all[3] || w16)) {
+            probs = nc_alloc(all[0]->dev, NC_TYPE_U16, 4, pd, false);
+            Bf16AttnFwdArgs g;
+            g.q = q16; g.kv = kv16; g.kvm = kvm16; g.w_r = w16; g.b_r = all[4] ? nc_f32(all[4]) : nullptr;
+            g.out = nc_f32(y); g.out16 = nc_shadow_for_write(m, y); g.probs = (uint16_t *)nc_data(probs);
+            g.ldq = (int64_t)all[0]->dims[0]; g.ldkv = (int64_t)all[1]->dims[0]; g.ldo = (int64_t)od[0];
+            g.H = a.H; g.B = a.B; g.T = a.T; g.M = a.M; g.K = a.K; g.d_pos = a.d_pos; g.attn_len = attn_len;
+            g.b_r_scale = b_r_scale; g.scale = 1.0f / sqrtf((float)a.dk);
+            if (k_attn_bf16_fwd(m->stream, g)) nc_fatal("nc_relpos_attention: bf16 kernel launch failed");
+            m->launches++;
+            on_bf16 = true;
+        }
+    }
+    if (!probs) probs = new_f32(all[0], 4, pd);
     size_t cap = 0;
-    float *rel = all[3] ? nc_tmp_f32(m, (size_t)a.d_pos * a.T * a.H * a.B, &cap) : nullptr;
-    int rc = nchip_relpos_attn_fwd(m->stream, nc_f32(all[0]), (int64_t)all[0]->dims[0],
+    float *rel = (all[3] && !on_bf16) ? nc_tmp_f32(m, (size_t)a.d_pos * a.T * a.H * a.B, &cap) : nullptr;
+    int rc = on_bf16 ? 0 : nchip_relpos_attn_fwd(m->stream, nc_f32(all[0]), (int64_t)all[0]->dims[0],
                                    nc_f32(all[1]), all[2] ? nc_f32(all[2]) : nullptr, (int64_t)all[1]->dims[0],
                                    all[3] ? nc_f32(all[3]) : nullptr, all[4] ? nc_f32(all[4]) : nullptr,
                                    nc_f32(y), (int64_t)od[0], nc_f32(probs), rel,
@@ -1133,7 +1161,7 @@ extern "C" NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv
                                    0 /* attention stays fp32 in the bf16 variant */);
     if (rel) nc_tmp_free(m, rel, cap);
     if (rc) nc_fatal("nc_relpos_attention: kernel rejected the shapes");
-    m->launches += nchip_relpos_attn_last_launches();
+    if (!on_bf16) m->launches += nchip_relpos_attn_last_launches();
     NCNode *n = nc_new_node(m, OP_ATTN, 5, all);
     bool graph = false;
     for (int i = 0; i < 5; i++)
@@ -1204,7 +1232,34 @@ static void attn_bw(NCNode *nd, NCTensor *g, NCTensor **ga)
     const bool shared = (!dwr || nc_can_defer_shared_sum(m, nd->parents[3])) &&
                         (!dbr || nc_can_defer_shared_sum(m, nd->parents[4]));
     const int keep = (dwr || dbr) && (once || shared);
-    int rc = nchip_relpos_attn_bwd(m->stream, nc_f32(q), (int64_t)q->dims[0], nc_f32(kv),
+    int rc;
+    if (probs->type == NC_TYPE_U16) {
+        // the forward ran on the bf16 matrix cores: so does the backward, from the same copies
+        const uint16_t *q16 = nc_shadow_of(m, q), *kv16 = nc_shadow_of(m, kv), *kvm16 = kvm ? nc_shadow_of(m, kvm) : nullptr;
+        const uint16_t *w16 = w_r ? nc_shadow_of(m, w_r) : nullptr, *go16 = nc_shadow_of(m, gc);
+        if (!q16 || !kv16 || (kvm && !kvm16) || (w_r && !w16) || !go16)
+            nc_fatal("nc_relpos_attention backward: an operand has no bf16 copy");
+        const int64_t n_w = dwr ? (int64_t)nc_numel(dwr) : 0, n_b = dbr ? (int64_t)nc_numel(dbr) : 0;
+        Bf16AttnBwdArgs g;
+        g.q = q16; g.kv = kv16; g.kvm = kvm16; g.w_r = w16; g.probs = (const uint16_t *)nc_data(probs); g.dout = go16;
+        g.dq = nc_f32(dq); g.dkv = nc_f32(dkv); g.dkvm = dkvm ? nc_f32(dkvm) : nullptr;
+        g.dwp = dwr ? scratch : nullptr; g.dbp = dbr ? scratch + n_w * a.B : nullptr;
+        g.dq16 = nc_shadow_for_write(m, dq); g.dkv16 = nc_shadow_for_write(m, dkv);
+        g.dkvm16 = dkvm ? nc_shadow_for_write(m, dkvm) : nullptr;
+        g.ldq = (int64_t)q->dims[0]; g.ldkv = (int64_t)kv->dims[0]; g.ldo = (int64_t)gc->dims[0];
+        g.H = a.H; g.B = a.B; g.T = a.T; g.M = a.M; g.K = a.K; g.d_pos = a.d_pos; g.attn_len = nd->ia[2];
+        g.b_r_scale = nd->fa[0]; g.scale = 1.0f / sqrtf((float)a.dk);
+        if (k_attn_bf16_bwd(m->stream, g)) nc_fatal("nc_relpos_attention backward: bf16 kernel launch failed");
+        m->launches++;
+        rc = keep ? 1 : 0;
+        if (!keep && (dwr || dbr)) {
+            if (k_attn_param_grad_reduce(m->stream, scratch, dwr ? nc_f32(dwr) : nullptr, n_w, scratch + n_w * a.B,
+                                         dbr ? nc_f32(dbr) : nullptr, n_b, a.B))
+                nc_fatal("nc_relpos_attention backward: partial sums failed");
+            m->launches++;
+        }
+    } else
+    rc = nchip_relpos_attn_bwd(m->stream, nc_f32(q), (int64_t)q->dims[0], nc_f32(kv),
                                    kvm ? nc_f32(kvm) : nullptr, (int64_t)kv->dims[0],
                                    w_r ? nc_f32(w_r) : nullptr, nc_f32(probs), nc_f32(gc),
                                    (int64_t)gc->dims[0], nc_f32(dq), nc_f32(dkv),
@@ -1227,7 +1282,7 @@ static void attn_bw(NCNode *nd, NCTensor *g, NCTensor **ga)
     } else {
         nc_tmp_free(m, scratch, cap);
     }
-    m->launches += nchip_relpos_attn_last_launches();
+    if (probs->type != NC_TYPE_U16) m->launches += nchip_relpos_attn_last_launches();
     nc_free_tensor(gc);
     NCTensor *out[5] = { dq, dkv, dkvm, dwr, dbr };
     for (int i = 0; i < 5; i++) {

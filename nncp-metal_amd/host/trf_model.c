@@ -478,6 +478,9 @@ static NCTensor *attention_fused(NNCPModel *s, int l, NCTensor *x, NCTensor *res
     NCTensor *q, *kv, *kvm = NULL, *att;
     Layer *pr = &s->layers[c->tied_w_r ? 0 : l], *pb = &s->layers[c->tied_b_r ? 0 : l];
 
+    /* (bf16 products: the attention reads bf16 operands too, so these three products leave the
+       bf16 copies of their results) */
+    int copies = nc_set_bf16_copy_of_results(s->ctx, 1);
     q = nc_linear(nc_dup_tensor(tl->w_q), nc_dup_tensor(x), c->query_bias ? nc_dup_tensor(tl->b_q) : NULL, NC_ACT_NONE);
     kv = nc_matmul(nc_dup_tensor(tl->w_kv), x);
     if (c->mem_len > 0) {
@@ -485,6 +488,7 @@ static NCTensor *attention_fused(NNCPModel *s, int l, NCTensor *x, NCTensor *res
         kvm = nc_matmul(nc_dup_tensor(tl->w_kv), kvm);
         kvm = nc_reshape_3d(kvm, HDk + HDv, B, c->mem_len);
     }
+    nc_set_bf16_copy_of_results(s->ctx, copies);
     att = nc_relpos_attention(nc_reshape_3d(q, HDk, B, T), nc_reshape_3d(kv, HDk + HDv, B, T), kvm,
                               c->use_w_r ? nc_dup_tensor(pr->w_r) : NULL, nc_dup_tensor(pb->b_r),
                               H, c->d_key, c->attn_len[l], sqrtf((float)(c->d_key * c->d_model)));

@@ -117,6 +117,7 @@ int nc_set_deferred_weight_grad(NCContext *m, int enable) { (void)m; (void)enabl
 int nc_set_matmul_width_invariant(NCContext *m, int enable) { (void)m; (void)enable; return 0; }
 int64_t nc_get_bf16_cast_count(NCContext *m) { (void)m; return 0; }
 int nc_set_bf16_shadow_check(int enable) { (void)enable; return 0; }
+int nc_set_bf16_copy_of_results(NCContext *m, int enable) { (void)m; (void)enable; return 0; }
 
 size_t nc_type_size(NCTypeEnum t)
 {

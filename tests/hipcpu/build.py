@@ -14,7 +14,7 @@ CSRC = os.path.join(ROOT, "nncp-metal_amd", "csrc")
 BUILD = os.path.join(HERE, "_build")
 OUT = os.path.join(HERE, "libnc_hipcpu.so")
 CXX = os.environ.get("HIPCPU_CXX", "/opt/rocm/llvm/bin/clang++")
-SOURCES = ["k_gemm.hip", "k_elementwise.hip", "k_norm.hip", "k_attention.hip", "k_attn_fused.hip", "k_cdf.hip",
+SOURCES = ["k_gemm.hip", "k_elementwise.hip", "k_norm.hip", "k_attention.hip", "k_attn_fused.hip", "k_attn_bf16.hip", "k_cdf.hip",
            "nc_core.cpp", "nc_autodiff.cpp", "nc_ops.cpp", "nc_params_io.cpp"]
 NO_CONTRACT = {"k_cdf.hip", "nc_ops.cpp"}
 FLAGS = ["-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-fno-strict-aliasing", "-Wno-unknown-attributes",

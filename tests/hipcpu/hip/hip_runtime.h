@@ -265,6 +265,32 @@ static inline hipcpu_f16v hipcpu_mfma_32x32x16_bf16(V a, V b, hipcpu_f16v c, int
     hipcpu_wave_barrier();
     return c;
 }
+/* v_mfma_f32_16x16x32_bf16: lane l holds 8 consecutive k = (l/16)*8 .. +7 of row / column
+   l%16; D as for 16x16x4 */
+template <typename V>
+static inline hipcpu_f4v hipcpu_mfma_16x16x32_bf16(V a, V b, hipcpu_f4v c, int, int, int)
+{
+    static_assert(sizeof(V) == 16, "8 bf16 values");
+    uint32_t w[8];
+    memcpy(w, &a, 16);
+    memcpy(w + 4, &b, 16);
+    const uint32_t *tab = hipcpu_wave_exchange(w, 8);
+    const int l = hipcpu_cur->lane, j = l & 15;
+    for (int r = 0; r < 4; r++) {
+        const int i = (l / 16) * 4 + r;
+        float acc = c[r];
+        for (int kg = 0; kg < 4; kg++) {
+            const uint16_t *pa = (const uint16_t *)(tab + (kg * 16 + i) * 16);
+            const uint16_t *pb = (const uint16_t *)(tab + (kg * 16 + j) * 16 + 4);
+            for (int e = 0; e < 8; e++)
+                acc = fmaf(hipcpu_bf16_to_f32(pa[e]), hipcpu_bf16_to_f32(pb[e]), acc);
+        }
+        c[r] = acc;
+    }
+    hipcpu_wave_barrier();
+    return c;
+}
+#define __builtin_amdgcn_mfma_f32_16x16x32_bf16 hipcpu_mfma_16x16x32_bf16
 #define __builtin_amdgcn_mfma_f32_32x32x2f32 hipcpu_mfma_32x32x2f32
 #define __builtin_amdgcn_mfma_f32_16x16x4f32 hipcpu_mfma_16x16x4f32
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16 hipcpu_mfma_32x32x16_bf16

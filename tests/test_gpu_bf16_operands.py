@@ -247,3 +247,57 @@ def test_training_steps_through_shadows_match_the_checkers_emulation():
     for k in w_r:
         if w_r[k].ndim >= 2 and not k.startswith("b_r"):
             assert M.rel_l2(w_h[k], w_r[k]) <= 2e-2, k
+
+
+ATTN_CFGS = [dict(H=2, B=2, T=64, M=64, d_pos=128, attn_len=128),      # the headline head shape
+             dict(H=1, B=3, T=48, M=80, d_pos=128, attn_len=100),
+             dict(H=2, B=2, T=40, M=24, d_pos=64, attn_len=64),        # key tiles partly empty
+             dict(H=2, B=1, T=64, M=64, d_pos=40, attn_len=128),       # far keys share position row 0
+             dict(H=1, B=2, T=64, M=192, d_pos=256, attn_len=256),     # 256 keys: the 16-tile instantiation
+             dict(H=2, B=2, T=17, M=143, d_pos=160, attn_len=90),
+             dict(H=2, B=2, T=64, M=64, d_pos=0, attn_len=128),        # no position vectors
+             dict(H=2, B=2, T=33, M=17, d_pos=29, attn_len=25)]        # K not a multiple of 8: the fp32 kernels
+
+
+@pytest.mark.parametrize("cfg", ATTN_CFGS)
+def test_attention_on_the_bf16_matrix_cores(hip, ref, rng, cfg):
+    """nc_relpos_attention with bf16 products on: q, kv, kv_mem and w_r are read as bf16, the
+    probabilities, dS, dRel and dO are rounded to bf16 where a product multiplies them, sums are
+    fp32.  Against the checker's fp32 attention on inputs that are already bf16 values (so the
+    operand rounding is exact on both sides): what is left is the rounding of the
+    intermediate factors, 2^-9 each - output and every gradient within 1e-2 of their
+    largest magnitude, an order inside the variant's 2e-2 bar and an order above what the
+    fp32 path holds (1e-5).  The launch count shows which kernels ran."""
+    H, B, T, M, d_pos = (cfg[k] for k in ("H", "B", "T", "M", "d_pos"))
+    dk = dv = 64
+    K = M + T
+    shapes = [(T, B, H * dk), (T, B, H * (dk + dv)), (M, B, H * (dk + dv)), (H, max(d_pos, 1), dk), (H, K)]
+    arrays = [bf16_round((rng.standard_normal(s) * 0.5).astype(np.float32))[0] for s in shapes]
+    weight = bf16_round(rng.standard_normal((T, B, H * dv)).astype(np.float32))[0]
+    res = []
+    for nc in (hip, ref):
+        nc.nc_set_matmul_bf16(nc.ctx, 1)
+        old = nc.nc_set_bf16_shadow_check(1)
+        hs = [nc.param(a, "p%d" % i) for i, a in enumerate(arrays)]
+        args = [nc.dup(h.value) for h, _ in hs]
+        if d_pos == 0:
+            nc.free(args[3])
+            args[3] = None
+        l0 = nc.nc_get_launch_count(nc.ctx)
+        y = nc.nc_relpos_attention(*args, H, dk, cfg["attn_len"], 2.5)
+        fwd_launches = nc.nc_get_launch_count(nc.ctx) - l0
+        out = nc.numpy(y)
+        loss = nc.nc_sum(nc.nc_mul(y, nc.tensor(weight)))
+        g = nc.backward(loss)
+        nc.free(loss)
+        res.append((out, [g.get(p) for _, p in hs], fwd_launches))
+        nc.nc_set_bf16_shadow_check(old)
+        nc.nc_set_matmul_bf16(nc.ctx, 0)
+    (o_h, g_h, launches), (o_r, g_r, _) = res
+    assert relerr(o_h, o_r) <= 1e-2
+    for i, (a, b) in enumerate(zip(g_h, g_r)):
+        if d_pos == 0 and i == 3:
+            continue
+        assert relerr(a, b) <= 1e-2, i
+    if K % 8 == 0:
+        assert launches <= 5            # 4 casts at most (parameters here have no producer) + the one kernel
