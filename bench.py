@@ -245,15 +245,52 @@ def attention_c2(pkg, iters=50):
         return ms.value * 1e3 / iters
 
     us_f, us_b, us = timed([fwd]), timed([bwd]), timed([fwd, bwd])
+
+    # the same head shape on the bf16 matrix cores (the bf16-operand variant's attention):
+    # operands are the bf16 copies of the tensors above, made once outside the timed region
+    # (in the step they come out of the producing products' epilogues)
+    def u16(shape):
+        return nc.tensor(np.zeros(shape, np.uint16))
+    for k in ("q", "kv", "kvm", "w_r", "dout"):
+        dev[k + "16"] = u16(host[k].shape)
+        assert lib.nchip_cast_bf16(None, P[k], C.c_void_p(nc.lib.nc_tensor_get_ptr(dev[k + "16"], None)),
+                                   i64(host[k].size)) == 0
+    for k in ("out", "dq", "dkv", "dkvm"):
+        dev[k + "16"] = u16(outs[k])
+    dev["probs16"] = u16(outs["probs"])
+    P = {k: C.c_void_p(nc.lib.nc_tensor_get_ptr(v, None)) for k, v in dev.items()}
+
+    def fwd16():
+        return lib.nchip_relpos_attn_fwd_bf16(None, P["q16"], ld, P["kv16"], P["kvm16"], ldkv, P["w_r16"], P["b_r"],
+                                              P["out"], P["out16"], ld, P["probs16"], i32(Hh), i32(dk), i32(dk),
+                                              i32(B), i32(T), i32(M), i32(d_pos), i32(K), f32(1.0))
+
+    def bwd16():
+        return lib.nchip_relpos_attn_bwd_bf16(None, P["q16"], ld, P["kv16"], P["kvm16"], ldkv, P["w_r16"],
+                                              P["probs16"], P["dout16"], ld, P["dq"], P["dq16"], P["dkv"], P["dkv16"],
+                                              P["dkvm"], P["dkvm16"], P["dw_r"], P["db_r"], i32(Hh), i32(dk), i32(dk),
+                                              i32(B), i32(T), i32(M), i32(d_pos), i32(K), f32(1.0), P["scratch"])
+
+    us16_f, us16_b, us16 = timed([fwd16]), timed([bwd16]), timed([fwd16, bwd16])
     for v in dev.values():
         nc.free(v)
     nc.close()
+    # algorithmic bytes.  fp32: fwd Q + K + V + position table + O, bwd Q, K, V, O, dO in and
+    # dQ, dK, dV out = 72 MiB.  bf16: the same tensors at 2 bytes where they are read, fp32 +
+    # bf16 where they are written (results keep their fp32 form for the rest of the step)
     nbytes, flops = 72 * 2 ** 20, 2.95e9
+    n_q, n_kv, n_w = q.size, kv.size + kvm.size, w_r.size
+    nbytes16 = (2 * (n_q + n_kv + n_w) + 6 * n_q) + (2 * (2 * n_q + n_kv + n_w) + 6 * (n_q + n_kv))
     return {"workload": "BASELINE configs[1]: B32 H8 d64 T64 K128 fwd+bwd fp32",
             "us_fwd": round(us_f, 2), "us_bwd": round(us_b, 2), "us_fwd_bwd": round(us, 2),
             "algorithmic_GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / 8000, 4),
             "dense_TFLOPs": round(flops / us / 1e6, 2), "mfma_fp32_frac": round(flops / us / 1e6 / 157.3, 4),
-            "binding_bound": "mfma (39 flop/B > fp32 ridge 20)"}
+            "binding_bound": "mfma (39 flop/B > fp32 ridge 20)",
+            "bf16": {"workload": "the same head shape, operands as bf16 copies, v_mfma_f32_16x16x32_bf16",
+                     "us_fwd": round(us16_f, 2), "us_bwd": round(us16_b, 2), "us_fwd_bwd": round(us16, 2),
+                     "algorithmic_bytes": nbytes16,
+                     "algorithmic_GBps": round(nbytes16 / us16 / 1e3, 1), "hbm_frac": round(nbytes16 / us16 / 1e3 / 8000, 4),
+                     "dense_TFLOPs": round(flops / us16 / 1e6, 2), "mfma_bf16_frac": round(flops / us16 / 1e6 / 2500, 4)}}
 
 
 def cdf_c5(pkg, iters=50):

@@ -284,6 +284,27 @@ int nchip_relpos_attn_bwd(void *stream, const float *q, int64_t ldq,
                           int attn_len, float b_r_scale, int precision, float *scratch,
                           int keep_partials);
 
+/* The same attention on the bf16 matrix cores (v_mfma_f32_16x16x32_bf16, fp32 accumulation,
+   fp32 scores and softmax): every operand is the bf16 copy (nearest even) of the fp32 tensor
+   of nchip_relpos_attn_fwd / _bwd, in the same layout with the same leading dimensions;
+   probs16 is (K, T, H, B) bf16, written by the forward with the very values it multiplied
+   with V and read by the backward; out16 / dq16 / dkv16 / dkvm16 (each may be NULL) receive
+   bf16 copies of the fp32 results.  d_head 64 (keys and values), T <= 64, K = M + T <= 256 and
+   a multiple of 8, d_pos <= K, leading dimensions multiples of 8: returns 1 (nothing
+   launched) for anything else, 0 when launched, negative on error.  The backward writes
+   per-stream dw_r / db_r partials to scratch (nchip_relpos_attn_bwd_scratch floats) and sums
+   them over the streams in stream order.  No counterpart in the reference. */
+int nchip_relpos_attn_fwd_bf16(void *stream, const uint16_t *q16, int64_t ldq, const uint16_t *kv16,
+                               const uint16_t *kvm16, int64_t ldkv, const uint16_t *w_r16, const float *b_r,
+                               float *out, uint16_t *out16, int64_t ldo, uint16_t *probs16, int H, int dk,
+                               int dv, int B, int T, int M, int d_pos, int attn_len, float b_r_scale);
+int nchip_relpos_attn_bwd_bf16(void *stream, const uint16_t *q16, int64_t ldq, const uint16_t *kv16,
+                               const uint16_t *kvm16, int64_t ldkv, const uint16_t *w_r16,
+                               const uint16_t *probs16, const uint16_t *dout16, int64_t ldo,
+                               float *dq, uint16_t *dq16, float *dkv, uint16_t *dkv16, float *dkvm,
+                               uint16_t *dkvm16, float *dw_r, float *db_r, int H, int dk, int dv, int B,
+                               int T, int M, int d_pos, int attn_len, float b_r_scale, float *scratch);
+
 /* LayerNorm / RMSNorm over axis 0 of (d, n) with optional affine
    (nncp.c:279-288; libnc.h:389-395).  xhat (d, n) and rstd (n) are saved for
    the backward.  w/b may be NULL (then y == xhat may alias). */

@@ -60,6 +60,14 @@ __device__ __forceinline__ int slot_of(int j)
     return (j & ~31) | ((j & 12) << 1) | ((j & 16) >> 2) | (j & 3);
 }
 
+// element offset of 16-byte chunk `chunk` in row `frow` of a transposed tile (rows TS apart):
+// the chunks of feature rows 8c .. 8c+7 are stored at chunk ^ c (see park_transposed)
+template <int TS>
+__device__ __forceinline__ int tr_off(int frow, int chunk)
+{
+    return frow * TS + ((chunk ^ ((frow >> 3) & 7)) << 3);
+}
+
 // the 8 bf16 values of a lane for the pair of tiles (2u, 2u + 1): element e = 4t + r
 __device__ __forceinline__ u32x4 pack8(const float (&lo)[4], const float (&hi)[4])
 {
@@ -105,12 +113,15 @@ struct RowTile {
         for (int it = 0; it < N; it++) {
             const int idx = threadIdx.x + it * 256, row = idx / C8, c = idx % C8;
             const int col = SLOTS ? slot_of(row) : row;
+            // feature rows 8c .. 8c+7 keep their 16-byte chunks at chunk ^ c (tr_off): the 8 lanes
+            // that hold one token then write 8 different banks instead of one
+            const int pcol = (((col >> 3) ^ (c & 7)) << 3) | (col & 7);
             const bool on = row < rows_valid;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const uint32_t w = on ? v[it][e] : 0u;
-                dst[(c * 8 + 2 * e) * TS + col] = (uint16_t)(w & 0xffffu);
-                dst[(c * 8 + 2 * e + 1) * TS + col] = (uint16_t)(w >> 16);
+                dst[(c * 8 + 2 * e) * TS + pcol] = (uint16_t)(w & 0xffffu);
+                dst[(c * 8 + 2 * e + 1) * TS + pcol] = (uint16_t)(w >> 16);
             }
         }
     }
@@ -273,7 +284,7 @@ __global__ __launch_bounds__(256) void relpos_attn_fwd_bf16(Bf16AttnFwdArgs a)
     for (int u = 0; u < NT / 2; u++)
 #pragma unroll
         for (int dt = 0; dt < ND; dt++)
-            acc[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Vt + (dt * 16 + il) * TS + 32 * u + 8 * g), pb[u], acc[dt]);
+            acc[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Vt + tr_off<TS>(dt * 16 + il, 4 * u + g)), pb[u], acc[dt]);
     if (i < a.T) {
         const int64_t o = (int64_t)h * DK + 4 * g + a.ldo * (b + (int64_t)a.B * i);
 #pragma unroll
@@ -427,8 +438,8 @@ __global__ __launch_bounds__(256) void relpos_attn_bwd_bf16(Bf16AttnBwdArgs a)
             const u32x4 rb = { rv[0] | (rv[1] << 16), rv[2] | (rv[3] << 16), rv[4] | (rv[5] << 16), rv[6] | (rv[7] << 16) };
 #pragma unroll
             for (int dt = 0; dt < ND; dt++) {
-                dqa[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Kt + (dt * 16 + il) * TS + 32 * u + 8 * g), sb, dqa[dt]);
-                dqa[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Wt + (dt * 16 + il) * TS + 32 * u + 8 * g), rb, dqa[dt]);
+                dqa[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Kt + tr_off<TS>(dt * 16 + il, 4 * u + g)), sb, dqa[dt]);
+                dqa[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Wt + tr_off<TS>(dt * 16 + il, 4 * u + g)), rb, dqa[dt]);
             }
         }
         if (i < a.T) {
@@ -471,8 +482,8 @@ __global__ __launch_bounds__(256) void relpos_attn_bwd_bf16(Bf16AttnBwdArgs a)
             av[dt] = floatx4_t{ 0, 0, 0, 0 };
 #pragma unroll
             for (int s = 0; s < NQS; s++) {
-                ak[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Qt + (dt * 16 + il) * QS + 32 * s + 8 * g), sb[s], ak[dt]);
-                av[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Ot + (dt * 16 + il) * QS + 32 * s + 8 * g), pb[s], av[dt]);
+                ak[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Qt + tr_off<QS>(dt * 16 + il, 4 * s + g)), sb[s], ak[dt]);
+                av[dt] = mfma_bf16(*reinterpret_cast<const u32x4 *>(Ot + tr_off<QS>(dt * 16 + il, 4 * s + g)), pb[s], av[dt]);
             }
         }
         const int j = jt * 16 + il;
@@ -509,7 +520,7 @@ __global__ __launch_bounds__(256) void relpos_attn_bwd_bf16(Bf16AttnBwdArgs a)
                 floatx4_t acc = { 0, 0, 0, 0 };
 #pragma unroll
                 for (int s = 0; s < NQS; s++)
-                    acc = mfma_bf16(*reinterpret_cast<const u32x4 *>(Qt + (dt * 16 + il) * QS + 32 * s + 8 * g), rb[s], acc);
+                    acc = mfma_bf16(*reinterpret_cast<const u32x4 *>(Qt + tr_off<QS>(dt * 16 + il, 4 * s + g)), rb[s], acc);
                 if (pp < a.d_pos) *reinterpret_cast<floatx4_t NCHIP_GLOBAL *>(dwz + (int64_t)pp * DK + dt * 16 + 4 * g) = acc;
             }
         }
@@ -576,4 +587,46 @@ int k_attn_bf16_bwd(hipStream_t st, const Bf16AttnBwdArgs &a)
     const int kmax = a.K > a.d_pos ? a.K : a.d_pos;
     if (kmax <= 128) return launch_bwd<64, 8>(st, a);
     return launch_bwd<64, 16>(st, a);
+}
+
+// ---- raw entry points (include/nchip_kernels.h) -------------------------------------------
+extern "C" int nchip_relpos_attn_fwd_bf16(void *stream, const uint16_t *q16, int64_t ldq, const uint16_t *kv16,
+                                          const uint16_t *kvm16, int64_t ldkv, const uint16_t *w_r16, const float *b_r,
+                                          float *out, uint16_t *out16, int64_t ldo, uint16_t *probs16, int H, int dk,
+                                          int dv, int B, int T, int M, int d_pos, int attn_len, float b_r_scale)
+{
+    if (!q16 || !kv16 || !out || !probs16 || H < 1 || B < 1 || (M > 0 && !kvm16)) return -1;
+    if (!k_attn_bf16_shape_ok(dk, dv, T, M + T, d_pos, w_r16 != nullptr) || ldq % 8 || ldkv % 8 || ldo % 4) return 1;
+    Bf16AttnFwdArgs g;
+    g.q = q16; g.kv = kv16; g.kvm = kvm16; g.w_r = w_r16; g.b_r = b_r; g.out = out; g.out16 = out16; g.probs = probs16;
+    g.ldq = ldq; g.ldkv = ldkv; g.ldo = ldo;
+    g.H = H; g.B = B; g.T = T; g.M = M; g.K = M + T; g.d_pos = w_r16 ? d_pos : 1; g.attn_len = attn_len;
+    g.b_r_scale = b_r_scale; g.scale = 1.0f / sqrtf((float)dk);
+    return k_attn_bf16_fwd((hipStream_t)stream, g);
+}
+
+extern "C" int nchip_relpos_attn_bwd_bf16(void *stream, const uint16_t *q16, int64_t ldq, const uint16_t *kv16,
+                                          const uint16_t *kvm16, int64_t ldkv, const uint16_t *w_r16,
+                                          const uint16_t *probs16, const uint16_t *dout16, int64_t ldo,
+                                          float *dq, uint16_t *dq16, float *dkv, uint16_t *dkv16, float *dkvm,
+                                          uint16_t *dkvm16, float *dw_r, float *db_r, int H, int dk, int dv, int B,
+                                          int T, int M, int d_pos, int attn_len, float b_r_scale, float *scratch)
+{
+    if (!q16 || !kv16 || !probs16 || !dout16 || !dq || !dkv || H < 1 || B < 1 || (M > 0 && (!kvm16 || !dkvm)) ||
+        ((dw_r || db_r) && !scratch) || (dw_r && !w_r16))
+        return -1;
+    if (!k_attn_bf16_shape_ok(dk, dv, T, M + T, d_pos, w_r16 != nullptr) || ldq % 8 || ldkv % 8 || ldo % 8) return 1;
+    const int K = M + T, dp = w_r16 ? d_pos : 1;
+    const int64_t n_w = dw_r ? (int64_t)dk * dp * H : 0, n_b = db_r ? (int64_t)K * H : 0;
+    Bf16AttnBwdArgs g;
+    g.q = q16; g.kv = kv16; g.kvm = kvm16; g.w_r = w_r16; g.probs = probs16; g.dout = dout16;
+    g.dq = dq; g.dkv = dkv; g.dkvm = dkvm; g.dwp = dw_r ? scratch : nullptr; g.dbp = db_r ? scratch + n_w * B : nullptr;
+    g.dq16 = dq16; g.dkv16 = dkv16; g.dkvm16 = dkvm16;
+    g.ldq = ldq; g.ldkv = ldkv; g.ldo = ldo;
+    g.H = H; g.B = B; g.T = T; g.M = M; g.K = K; g.d_pos = dp; g.attn_len = attn_len;
+    g.b_r_scale = b_r_scale; g.scale = 1.0f / sqrtf((float)dk);
+    int rc = k_attn_bf16_bwd((hipStream_t)stream, g);
+    if (rc == 0 && (dw_r || db_r))
+        rc = k_attn_param_grad_reduce((hipStream_t)stream, scratch, dw_r, n_w, scratch + n_w * B, db_r, n_b, B);
+    return rc;
 }

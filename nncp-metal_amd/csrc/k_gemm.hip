@@ -1935,7 +1935,7 @@ extern "C" int nchip_gemm_bf16_operands(void *stream, const NchipGemmBf16Args *a
     const int64_t t128 = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
     const int64_t t128x64 = (int64_t)((m + 127) / 128) * ((n + 63) / 64);
     int cls = g_bf16ops_cls;
-    if (!cls) cls = t128 >= 224 ? 1 : (t128x64 >= 224 && m >= 128 ? 2 : 3);
+    if (cls < 1 || cls > 3) cls = t128 >= 224 ? 1 : (t128x64 >= 224 && m >= 128 ? 2 : 3);
     {
         const int bm = cls == 3 ? 64 : 128, bn = cls == 1 ? 128 : 64;
         if ((!ta && m % bm) || (tb && n % bn)) return 1; // row-contiguous operands need whole tiles
@@ -1953,20 +1953,12 @@ extern "C" int nchip_gemm_bf16_operands(void *stream, const NchipGemmBf16Args *a
         rec.variant = 32 + cls * 4 + ta * 2 + tb; // the bf16-operand classes
     }
     ProfRec *pr = g_prof_on ? &rec : nullptr;
-    static const int pf = getenv("NCHIP_BF16OPS_PF") ? atoi(getenv("NCHIP_BF16OPS_PF")) : 2;
-    if (pf == 4) {
-        if (cls == 1) launch_tile<128, 128, 64, 2, 2, 2, 1, 3>(st, ta, tb, g, pr);
-        else if (cls == 2) launch_tile<128, 64, 64, 2, 2, 2, 1, 4>(st, ta, tb, g, pr);
-        else launch_tile<64, 64, 64, 2, 2, 2, 1, 4>(st, ta, tb, g, pr);
-    } else if (pf == 3) {
-        if (cls == 1) launch_tile<128, 128, 64, 2, 2, 2, 1, 2>(st, ta, tb, g, pr);
-        else if (cls == 2) launch_tile<128, 64, 64, 2, 2, 2, 1, 3>(st, ta, tb, g, pr);
-        else launch_tile<64, 64, 64, 2, 2, 2, 1, 3>(st, ta, tb, g, pr);
-    } else {
-        if (cls == 1) launch_tile<128, 128, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
-        else if (cls == 2) launch_tile<128, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
-        else launch_tile<64, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
-    }
+    // (measured on the C3 and C4 shapes: deeper prefetch - 3 or 4 register sets - changes nothing
+    // once the loop waits for its oldest set only; 256 x 128 tiles with 8 wavefronts run at the
+    // rate of the 128 x 128 class, 256 x 256 tiles spill)
+    if (cls == 1) launch_tile<128, 128, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+    else if (cls == 2) launch_tile<128, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
+    else launch_tile<64, 64, 64, 2, 2, 2, 1>(st, ta, tb, g, pr);
     if (g_prof_on) g_prof.push_back(rec);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

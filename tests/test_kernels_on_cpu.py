@@ -76,6 +76,17 @@ def test_results_do_not_depend_on_work_item_order(emulated):
     assert p.returncode == 0 and " passed" in out, out[-3000:]
 
 
+def test_bf16_operand_paths_pass_on_the_cpu_build(emulated):
+    """The products that read bf16 operand copies (every tile class and transposition, the
+    grouped launch, the copies the epilogues and norms write), the tensor-level shadow route
+    with its consistency checker on, and attention on the bf16 matrix cores forward and
+    backward - the unguarded 16-byte loads and the transposed LDS tiles of these kernels are
+    exactly what guard pages behind every buffer are for."""
+    p = _pytest(emulated, ["-n", "7", "tests/test_gpu_bf16_operands.py"])
+    out = p.communicate(timeout=1500)[0]
+    assert p.returncode == 0 and " passed" in out, out[-3000:]
+
+
 def test_host_tensor_compute_is_refused(emulated):
     """No CPU fallback in the product library: compute on a host tensor aborts with a
     message.  (Host-side logic, so it is exercised on the CPU build and not by aborting
