@@ -35,17 +35,27 @@ PEAK_TFLOPS = {"fp32": 157.3, "bf16": 2500.0}
 PROFILES = os.path.join(ROOT, "profiles")
 
 
-def measured_traffic(kernel, summary="c3_fp32_hbm_traffic_pmc.txt"):
-    """HBM-side bytes per launch (read + written) of a kernel instantiation, from the committed
-    rocprofv3 summary (FETCH_SIZE / WRITE_SIZE runs of this script, scaled by a device copy of
-    known size; a counter run cannot be taken from inside the timed run).  The summary's rows
-    are `<kernel name> <launches> <FETCH KiB> <WRITE KiB> <read MB> <write MB>`; names are
-    compared without blanks and by prefix, because the event records name a kernel by its
-    leading template arguments only.  None when the summary does not hold the kernel."""
+TRAFFIC_SUMMARY = {"fp32": "c3_fp32_hbm_traffic_pmc.txt", "bf16": "c3_bf16_hbm_traffic_pmc.txt"}
+
+
+def measured_traffic(kernel, variant):
+    """(HBM-side bytes per launch (read + written) of a kernel instantiation, where the figure
+    comes from) out of the committed rocprofv3 summary of the variant (FETCH_SIZE / WRITE_SIZE
+    runs of this script, scaled by a device copy of known size; a counter run cannot be taken
+    from inside the timed run, so the figure is the committed one and `traffic_source` says
+    so).  The summary's rows are `<kernel name> <launches> <FETCH KiB> <WRITE KiB> <read MB>
+    <write MB>`; names are compared without blanks.  The event records name a kernel by its
+    leading template arguments only, so a row matches when its name starts with the record's;
+    two rows that both do are two instantiations the record cannot tell apart, and then no
+    figure is given.  (None, None) when the summary does not hold the kernel."""
+    summary = TRAFFIC_SUMMARY[variant]
     path = os.path.join(PROFILES, summary)
     if not os.path.exists(path):
-        return None
-    want = kernel.replace(" ", "").rstrip(">")
+        return None, None
+    # (the grouped launch runs the same template as single launches: its record carries a
+    # ",grouped" mark that kernel names do not have)
+    want = kernel.replace(" ", "").replace(",grouped>", ">").rstrip(">")
+    found = []
     for line in open(path):
         parts = line.rsplit(None, 5)
         if len(parts) != 6:
@@ -55,9 +65,11 @@ def measured_traffic(kernel, summary="c3_fp32_hbm_traffic_pmc.txt"):
             read_mb, write_mb = float(parts[4]), float(parts[5])
         except ValueError:
             continue
-        if name.startswith(want):
-            return (read_mb + write_mb) * 1e6
-    return None
+        if name.startswith(want) and name[len(want):len(want) + 1] in (",", ">"):
+            found.append((read_mb + write_mb) * 1e6)
+    if len(found) != 1:
+        return None, None
+    return found[0], "profiles/%s (committed counter summary of this command; not re-measured in this run)" % summary
 
 
 def markov3_dirichlet(n, seed=2024, alpha=0.05, n_symbols=256):
@@ -416,59 +428,63 @@ def decode_c3(pkg, data, n_segments, variant):
             "round_trip_ok": bool(np.array_equal(out, syms))}
 
 
-def main_c4(args):
-    """BASELINE configs[3] (not the headline metric; `--workload c4`): 20 layers,
-    d_model 1024, 16 heads x 64, d_ff 4096, 64 + 192 keys, batch 64, V 16384,
-    one step = 4096 tokens.  Same library calls as the default workload."""
-    import __graft_entry__ as G
-    pkg = G._load_pkg()
+def measure_c4(pkg, variant, warmup, steps, profile_steps):
+    """BASELINE configs[3] (not the headline metric): 20 layers, d_model 1024, 16 heads x 64,
+    d_ff 4096, 64 + 192 keys, batch 64, V 16384; one step = 4096 tokens.  Same library calls
+    as the default workload.  Returns the fields of its line / of the `c4` object."""
     H = pkg.host
     B, T = C4["batch_size"], C4["seg_len"]
     per_step = B * T
-    total_steps = args.warmup + args.steps + args.profile_steps
-    data = bigram_zipf_dirichlet(total_steps * per_step)
+    data = bigram_zipf_dirichlet((warmup + steps + profile_steps) * per_step)
     opt = pkg.binding.SGDOptParams(algo=pkg.binding.SGD_OPT_RMSPROP, beta2=0.99, eps=1e-8, lr=3e-4)
     model = H.Model(H.Host(), H.make_config(**dict(C4, use_device=1, fused=1, sgd_opt=opt)))
     init_weights(model)
-    model.nc.nc_set_matmul_bf16(model.ctx, 1 if args.variant == "bf16" else 0)
+    model.nc.nc_set_matmul_bf16(model.ctx, 1 if variant == "bf16" else 0)
     mode = H.MODE_SEGMENT | H.CODER_CDF16
     pos = 0
-    if args.warmup:
-        say("C4 %s: %d warm-up steps" % (args.variant, args.warmup))
-        run_block(model, H, data[pos:pos + args.warmup * per_step], mode)
-        pos += args.warmup * per_step
-    say("C4 %s: %d timed steps" % (args.variant, args.steps))
+    if warmup:
+        say("C4 %s: %d warm-up steps" % (variant, warmup))
+        run_block(model, H, data[pos:pos + warmup * per_step], mode)
+        pos += warmup * per_step
+    say("C4 %s: %d timed steps" % (variant, steps))
     l0 = model.nc.nc_get_launch_count(model.ctx)
-    sec, nbytes, st = run_block(model, H, data[pos:pos + args.steps * per_step], mode)
+    sec, nbytes, st = run_block(model, H, data[pos:pos + steps * per_step], mode)
     launches = model.nc.nc_get_launch_count(model.ctx) - l0
-    pos += args.steps * per_step
+    pos += steps * per_step
     roof = None
-    if args.profile_steps:
-        say("C4 %s: %d steps with per-launch GEMM events" % (args.variant, args.profile_steps))
-        rows = gemm_profile(model, H, data[pos:pos + args.profile_steps * per_step], mode, pkg.binding.HIP_LIB)
+    if profile_steps:
+        say("C4 %s: %d steps with per-launch GEMM events" % (variant, profile_steps))
+        rows = gemm_profile(model, H, data[pos:pos + profile_steps * per_step], mode, pkg.binding.HIP_LIB)
         if rows:
             dom = max(rows, key=lambda r: r["seconds"])
-            peak = PEAK_TFLOPS[args.variant]
+            peak = PEAK_TFLOPS[variant]
             achieved = dom["flops"] / dom["seconds"] / 1e12
             tot_f, tot_s = sum(r["flops"] for r in rows), sum(r["seconds"] for r in rows)
             roof = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 3), "peak": peak,
                     "unit": "TFLOP/s", "frac": round(achieved / peak, 4), "traffic": None,
-                    "launches_per_step": dom["launches"] / args.profile_steps,
+                    "launches_per_step": dom["launches"] / profile_steps,
                     "avg_launch_us": round(dom["seconds"] / dom["launches"] * 1e6, 2),
                     "all_gemm_tflops": round(tot_f / tot_s / 1e12, 3),
-                    "all_gemm_ms_per_step": round(tot_s / args.profile_steps * 1e3, 3)}
+                    "all_gemm_ms_per_step": round(tot_s / profile_steps * 1e3, 3)}
     model.close()
-    print(json.dumps({
-        "metric": "tokens/sec compressed (train+code) 20L d1024 V16384", "value": round(args.steps * per_step / sec, 1),
-        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(sec / args.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32" if args.variant == "fp32" else "bf16-in/f32-acc", "data": "synthetic",
-        "config": {"workload": "BASELINE configs[3]: 20L d1024 16x64 ff4096 T64 M192 B64 V16384, RMSProp, seeded "
-                               "bigram Zipf(1.0) x Dirichlet(0.1) tokens, weights N(0,0.02)",
-                   "tokens_per_step": per_step, "coder": "gpu cdf16 + host range coder", "variant": args.variant},
-        "bits_per_token": round(nbytes * 8 / (args.steps * per_step), 4),
-        "kernel_launches_per_step": launches / args.steps, "roofline": roof,
-        "cpu_baseline": None}))
+    return {"metric": "tokens/sec compressed (train+code) 20L d1024 V16384",
+            "value": round(steps * per_step / sec, 1), "unit": "tokens/s", "steps": steps, "warmup": warmup,
+            "ms_per_step": round(sec / steps * 1e3, 3),
+            "dtype": "f32" if variant == "fp32" else "bf16-in/f32-acc",
+            "config": {"workload": "BASELINE configs[3]: 20L d1024 16x64 ff4096 T64 M192 B64 V16384, RMSProp, seeded "
+                                   "bigram Zipf(1.0) x Dirichlet(0.1) tokens, weights N(0,0.02)",
+                       "tokens_per_step": per_step, "coder": "gpu cdf16 + host range coder", "variant": variant},
+            "bits_per_token": round(nbytes * 8 / (steps * per_step), 4),
+            "kernel_launches_per_step": launches / steps, "roofline": roof}
+
+
+def main_c4(args):
+    """`--workload c4`: the configs[3] measurement as a line of its own."""
+    import __graft_entry__ as G
+    r = measure_c4(G._load_pkg(), args.variant, args.warmup, args.steps, args.profile_steps)
+    r.update({"n_gpus": 1, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+              "data": "synthetic", "cpu_baseline": None})
+    print(json.dumps(r))
 
 
 def main():
@@ -486,6 +502,12 @@ def main():
     ap.add_argument("--cpu-single-steps", type=int, default=1, help="steps of the single-thread CPU baseline (0 skips it)")
     ap.add_argument("--decode-segments", type=int, default=4, help="segments decoded for the `decode` object (0 skips it)")
     ap.add_argument("--profile-steps", type=int, default=2)
+    ap.add_argument("--c4-steps", type=int, default=3,
+                    help="timed steps of BASELINE configs[3] in its bf16-operand variant for the `c4` object of "
+                         "the default line (after 1 warm-up step, plus 1 step under GEMM events; 0 skips it)")
+    ap.add_argument("--decodable-steps", type=int, default=10,
+                    help="timed steps of the width-invariant encoder (the stream format the per-timestep "
+                         "decoder reads) for `encode_step_decodable` (0 skips it)")
     ap.add_argument("--attention-iters", type=int, default=50, help="0 skips the isolated attention timing")
     ap.add_argument("--cdf-iters", type=int, default=50, help="0 skips the coder-side CDF timing")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
@@ -506,7 +528,8 @@ def main():
     B, T = C3["batch_size"], C3["seg_len"]
     per_step = B * T
     total_steps = args.warmup + args.steps + args.profile_steps
-    data = markov3_dirichlet(max(total_steps, args.cpu_steps, args.decode_segments) * per_step)
+    data = markov3_dirichlet(max(total_steps, args.warmup + args.decodable_steps, args.cpu_steps,
+                                 args.decode_segments) * per_step)
     opt = pkg.binding.SGDOptParams(algo=pkg.binding.SGD_OPT_RMSPROP, beta2=0.99, eps=1e-8, lr=3e-4)
     mode = H.MODE_SEGMENT | H.CODER_CDF16
 
@@ -523,7 +546,7 @@ def main():
         hip.hipFree(src)
         hip.hipFree(dst)
 
-    def measure(variant):
+    def measure(variant, mode=mode, steps=args.steps, profile_steps=args.profile_steps):
         """warm-up, the timed steps and the per-launch GEMM timing of one arithmetic variant"""
         model = H.Model(H.Host(), H.make_config(**dict(C3, use_device=1, fused=1, sgd_opt=opt)))
         init_weights(model)
@@ -533,15 +556,15 @@ def main():
             say("C3 %s: %d warm-up steps" % (variant, args.warmup))
             run_block(model, H, data[pos:pos + args.warmup * per_step], mode)
             pos += args.warmup * per_step
-        say("C3 %s: %d timed steps" % (variant, args.steps))
+        say("C3 %s: %d timed steps" % (variant, steps))
         l0 = model.nc.nc_get_launch_count(model.ctx)
-        sec, nbytes, st = run_block(model, H, data[pos:pos + args.steps * per_step], mode)
+        sec, nbytes, st = run_block(model, H, data[pos:pos + steps * per_step], mode)
         launches = model.nc.nc_get_launch_count(model.ctx) - l0
-        pos += args.steps * per_step
+        pos += steps * per_step
         roof = None
-        if args.profile_steps:
-            say("C3 %s: %d steps with per-launch GEMM events" % (variant, args.profile_steps))
-            rows = gemm_profile(model, H, data[pos:pos + args.profile_steps * per_step], mode,
+        if profile_steps:
+            say("C3 %s: %d steps with per-launch GEMM events" % (variant, profile_steps))
+            rows = gemm_profile(model, H, data[pos:pos + profile_steps * per_step], mode,
                                 pkg.binding.HIP_LIB)
             if rows:
                 dom = max(rows, key=lambda r: r["seconds"])
@@ -549,19 +572,20 @@ def main():
                 peak = PEAK_TFLOPS[variant]
                 tot_f = sum(r["flops"] for r in rows)
                 tot_s = sum(r["seconds"] for r in rows)
+                traffic, traffic_source = measured_traffic(dom["kernel"], variant)
                 roof = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 3),
                         "peak": peak, "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
-                        "traffic": measured_traffic(dom["kernel"]) if variant == "fp32" else None,
-                        "launches_per_step": dom["launches"] / args.profile_steps,
+                        "traffic": traffic, "traffic_source": traffic_source,
+                        "launches_per_step": dom["launches"] / profile_steps,
                         "avg_launch_us": round(dom["seconds"] / dom["launches"] * 1e6, 2),
                         "flops_per_launch": dom["flops"] / dom["launches"],
                         "all_gemm_tflops": round(tot_f / tot_s / 1e12, 3),
-                        "all_gemm_ms_per_step": round(tot_s / args.profile_steps * 1e3, 3)}
+                        "all_gemm_ms_per_step": round(tot_s / profile_steps * 1e3, 3)}
         model.close()
-        return {"value": round(args.steps * per_step / sec, 1), "ms_per_step": round(sec / args.steps * 1e3, 3),
+        return {"value": round(steps * per_step / sec, 1), "ms_per_step": round(sec / steps * 1e3, 3),
                 "dtype": "f32" if variant == "fp32" else "bf16-in/f32-acc",
-                "bits_per_symbol": round(nbytes * 8 / (args.steps * per_step), 4),
-                "kernel_launches_per_step": launches / args.steps,
+                "bits_per_symbol": round(nbytes * 8 / (steps * per_step), 4),
+                "kernel_launches_per_step": launches / steps,
                 "host_seconds": {"eval_and_copy": round(st.t_eval, 4), "code": round(st.t_code, 4),
                                  "grad": round(st.t_grad, 4), "update": round(st.t_update, 4)},
                 "roofline": roof}
@@ -573,6 +597,18 @@ def main():
             r = measure(v)
             variants[v] = {k: r[k] for k in ("value", "ms_per_step", "dtype", "bits_per_symbol")}
             variants[v]["all_gemm_tflops"] = r["roofline"]["all_gemm_tflops"] if r["roofline"] else None
+            variants[v]["kernel_launches_per_step"] = r["kernel_launches_per_step"]
+            variants[v]["roofline"] = r["roofline"]
+
+    step_dec = None
+    if args.decodable_steps:
+        # the same workload coded in the stream format of the per-timestep decoder: forward
+        # products in their width-invariant form (what `decode` below reads back)
+        r = measure(args.variant, mode | H.MODE_STEP_DECODE, args.decodable_steps, 0)
+        step_dec = {"value": r["value"], "unit": "symbols/s", "ms_per_step": r["ms_per_step"],
+                    "steps": args.decodable_steps, "warmup": args.warmup, "variant": args.variant,
+                    "kernel_launches_per_step": r["kernel_launches_per_step"],
+                    "mode": "NNCP_MODE_SEGMENT | NNCP_MODE_STEP_DECODE | NNCP_CODER_CDF16"}
 
     attn = cdf = dec = None
     if args.attention_iters:
@@ -584,6 +620,9 @@ def main():
     if args.decode_segments:
         say("decoding %d segments with the per-timestep decoder" % args.decode_segments)
         dec = decode_c3(pkg, data, args.decode_segments, args.variant)
+    c4 = None
+    if args.c4_steps:
+        c4 = measure_c4(pkg, "bf16", 1, args.c4_steps, 1)
 
     cpu = None
     if args.cpu_steps:
@@ -610,11 +649,15 @@ def main():
         "config": {"workload": "BASELINE configs[2]: 12L d512 8x64 ff2048 T64 M64 B32 V256, RMSProp, "
                                "order-3 Markov Dirichlet(0.05) prefix, weights N(0,0.02)",
                    "symbols_per_step": per_step, "coder": "gpu cdf16 + host range coder",
-                   "variant": args.variant},
+                   "variant": args.variant,
+                   "encoder": "whole-segment encoder (NNCP_MODE_SEGMENT | NNCP_CODER_CDF16): its stream is read "
+                              "back by a decoder that replays the segment evaluation per timestep; the stream "
+                              "format of the per-timestep decoder is timed under encode_step_decodable"},
         "bits_per_symbol": head["bits_per_symbol"],
         "kernel_launches_per_step": head["kernel_launches_per_step"],
         "host_seconds": head["host_seconds"],
-        "roofline": head["roofline"], "variants": variants, "attention": attn, "cdf": cdf, "decode": dec,
+        "roofline": head["roofline"], "encode_step_decodable": step_dec, "variants": variants,
+        "c4": c4, "attention": attn, "cdf": cdf, "decode": dec,
         "cpu_baseline": cpu}))
 
 

@@ -267,6 +267,7 @@ static double load_elem(const NCTensor *x, size_t off)
     case NC_TYPE_I32: return ((const int32_t *)p)[x->off + off];
     case NC_TYPE_I8: return ((const int8_t *)p)[x->off + off];
     case NC_TYPE_U16: return ((const uint16_t *)p)[x->off + off];
+    case NC_TYPE_BF16: return nc_bf16_widen(((const uint16_t *)p)[x->off + off]);
     default: nc_fatal("load: unsupported type");
     }
 }
@@ -279,6 +280,7 @@ static void store_elem(NCTensor *x, size_t off, double v)
     case NC_TYPE_I32: ((int32_t *)p)[x->off + off] = (int32_t)v; break;
     case NC_TYPE_I8: ((int8_t *)p)[x->off + off] = (int8_t)v; break;
     case NC_TYPE_U16: ((uint16_t *)p)[x->off + off] = (uint16_t)v; break;
+    case NC_TYPE_BF16: ((uint16_t *)p)[x->off + off] = nc_bf16_bits((float)v); break;
     default: nc_fatal("store: unsupported type");
     }
 }
@@ -374,10 +376,10 @@ void nc_tensor_set_zero(NCTensor *y) /* libnc.h:192 */
 void nc_tensor_set_f32(NCTensor *y, float val) /* libnc.h:194 */
 {
     size_t n = nc_numel(y);
-    if (!nc_is_contig(y) || y->type != NC_TYPE_F32)
-        nc_fatal("set_f32: contiguous f32 tensor expected");
+    if (!nc_is_contig(y) || (y->type != NC_TYPE_F32 && y->type != NC_TYPE_BF16))
+        nc_fatal("set_f32: contiguous f32 or bf16 tensor expected");
     for (size_t i = 0; i < n; i++)
-        nc_f32(y)[i] = val;
+        store_elem(y, i, val);
 }
 
 /* libnc.h:206: host-side single element write with conversion to the item
@@ -446,11 +448,11 @@ void nc_rnd_end(NCRNDState *s) { nc_free(s); }
 void nc_tensor_set_rnd_unif(NCTensor *y, float avg, float range, NCRNDState *rs)
 {
     size_t n = nc_numel(y);
-    if (!nc_is_contig(y) || y->type != NC_TYPE_F32)
-        nc_fatal("set_rnd_unif: contiguous f32 tensor expected");
+    if (!nc_is_contig(y) || (y->type != NC_TYPE_F32 && y->type != NC_TYPE_BF16))
+        nc_fatal("set_rnd_unif: contiguous f32 or bf16 tensor expected");
     for (size_t i = 0; i < n; i++) {
         float u = (float)(xorwow(rs) >> 8) * (1.0f / 16777216.0f); /* [0,1) */
-        nc_f32(y)[i] = avg + range * (2.0f * u - 1.0f);
+        store_elem(y, i, avg + range * (2.0f * u - 1.0f)); /* (a bf16 tensor keeps the rounding) */
     }
 }
 
@@ -538,6 +540,7 @@ struct SGDOptVarState {
     NCSGDOptState *opt;
     NCParam *param;
     float *m, *v, *g;
+    float *master; /* bf16 parameters: the fp32 values the update works on */
     size_t n;
     int has_grad;
     struct SGDOptVarState *next;
@@ -571,7 +574,7 @@ void nc_sgd_opt_set_all(NCParamList *pl, NCSGDOptState *s)
             struct SGDOptVarState *vs = p->sgd_opt, **pp;
             for (pp = &vs->opt->vars; *pp; pp = &(*pp)->next)
                 if (*pp == vs) { *pp = vs->next; break; }
-            free(vs->m); free(vs->v); free(vs->g);
+            free(vs->m); free(vs->v); free(vs->g); free(vs->master);
             nc_free(vs);
             p->sgd_opt = NULL;
         }
@@ -583,6 +586,15 @@ void nc_sgd_opt_set_all(NCParamList *pl, NCSGDOptState *s)
             vs->m = nc_mallocz(vs->n * sizeof(float));
             vs->v = nc_mallocz(vs->n * sizeof(float));
             vs->g = nc_mallocz(vs->n * sizeof(float));
+            if ((*p->pval)->type == NC_TYPE_BF16) {
+                /* the update works on an fp32 master that starts as the parameter's value;
+                   the parameter itself holds the master's rounding */
+                NCTensor *c = nc_contig(nc_dup_tensor(*p->pval));
+                vs->master = nc_malloc(vs->n * sizeof(float));
+                for (size_t i = 0; i < vs->n; i++)
+                    vs->master[i] = (float)load_elem(c, i);
+                nc_free_tensor(c);
+            }
             for (pp = &s->vars; *pp; pp = &(*pp)->next)
                 ;
             *pp = vs;
@@ -605,6 +617,8 @@ static float *moment_of(NCParam *p, int which)
         return algo == SGD_OPT_ADAM && vs->opt->p.u.adam.beta1 != 0.0f ? vs->m : NULL;
     if (which == 1)
         return algo != SGD_OPT_BASIC ? vs->v : NULL;
+    if (which == 2)
+        return vs->master;
     return NULL;
 }
 
@@ -669,9 +683,10 @@ void nc_sgd_opt_update(NCSGDOptState *s)
         if (!vs->has_grad)
             continue;
         NCTensor *wt = *vs->param->pval;
-        float *w = nc_f32(wt), lr = p->lr * vs->param->lr_mult;
-        if (!nc_is_contig(wt) || wt->type != NC_TYPE_F32)
-            nc_fatal("optimiser: contiguous f32 parameter expected");
+        float lr = p->lr * vs->param->lr_mult;
+        if (!nc_is_contig(wt) || (wt->type != NC_TYPE_F32 && !vs->master))
+            nc_fatal("optimiser: contiguous f32 or bf16 parameter expected");
+        float *w = vs->master ? vs->master : nc_f32(wt);
         #pragma omp parallel for if (vs->n > 65536)
         for (size_t i = 0; i < vs->n; i++) {
             float g = vs->g[i];
@@ -698,6 +713,11 @@ void nc_sgd_opt_update(NCSGDOptState *s)
             default:
                 nc_fatal("unsupported optimiser %d", p->algo);
             }
+        }
+        if (vs->master) {
+            uint16_t *w16 = (uint16_t *)wt->buf->data + wt->off;
+            for (size_t i = 0; i < vs->n; i++)
+                w16[i] = nc_bf16_bits(vs->master[i]);
         }
         vs->has_grad = 0;
     }

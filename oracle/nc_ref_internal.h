@@ -88,6 +88,22 @@ NCTensor *nc_view(const NCTensor *x); /* new header sharing the buffer, no node 
 float *nc_f32(const NCTensor *x);     /* data pointer (offset applied) */
 void nc_copy_strided(NCTensor *dst, const NCTensor *src);
 
+/* bf16 <-> f32: nearest even on the way down (NaN stays a quiet NaN), exact on the way up */
+static inline uint16_t nc_bf16_bits(float f)
+{
+    union { float f; uint32_t u; } v = { f };
+    if ((v.u & 0x7fffffffu) > 0x7f800000u)
+        return (uint16_t)((v.u >> 16) | 0x40);
+    v.u += 0x7fff + ((v.u >> 16) & 1);
+    return (uint16_t)(v.u >> 16);
+}
+
+static inline float nc_bf16_widen(uint16_t b)
+{
+    union { uint32_t u; float f; } v = { (uint32_t)b << 16 };
+    return v.f;
+}
+
 /* nc_ref_ops.c */
 NCNode *nc_new_node(NCContext *m, NCOpEnum op, int n_args, NCTensor **args);
 void nc_attach(NCTensor *y, NCNode *n);

@@ -13,7 +13,7 @@ that are sums of cancelling terms is amplified (zero-initialised vectors consist
 else).  There a float64 evaluation of the same steps is the arbiter: the kernels must be
 within the bar of it, or no further from it than 3x the checker's own distance (the same
 order of rounding noise); randomly initialised matrices stay within the bar of the checker or
-of the float64 evaluation itself.  Compressed sizes: within 0.5 %."""
+of the float64 evaluation itself, or within 3x the checker's own distance from the latter.  Compressed sizes: within 0.5 %."""
 import os
 
 import numpy as np
@@ -114,9 +114,12 @@ def _check_steps(hosts, cfg, batches, ref, bf16, tol):
     w, r, x = weights[ref.last], ref.weights[ref.last], ref.exact_weights[ref.last]
     mats = _matrices(r)
     vecs = [k for k in r if k not in mats]
-    for k in mats:          # within the bar of the fp32 checker, or of the float64 evaluation itself
-        e, ex = M.rel_l2(w[k], r[k]), M.rel_l2(w[k], x[k])
-        assert min(e, ex) <= tol, (k, e, ex)
+    for k in mats:          # within the bar of the fp32 checker, or of the float64 evaluation itself,
+        # or within 3x the checker's own distance from it, as for the vectors (embedding rows of
+        # symbols seen a few times have gradients near eps / 0.1, where the first RMSProp updates
+        # lr g / (0.1 |g| + eps) pass the relative rounding noise of g on undamped)
+        e, ex, rx = M.rel_l2(w[k], r[k]), M.rel_l2(w[k], x[k]), M.rel_l2(r[k], x[k])
+        assert min(e, ex) <= tol or M.within_or_no_worse(ex, rx, tol), (k, e, ex, rx)
     assert M.rel_l2(_joint(w, list(r)), _joint(r, list(r))) <= tol
     yard_v = max(M.rel_l2(yard_w[k], x[k]) for k in vecs)
     for k in vecs:
@@ -195,3 +198,37 @@ def test_c4_layer_shape_first_step_matches_checker(hosts, c4_batches, c4_ref, va
 @pytest.mark.parametrize("variant,tol", [("fp32", 1e-5), ("bf16", 2e-2)])
 def test_c4_layer_shape_two_steps(hosts, c4_batches, c4_ref, variant, tol):
     _check_steps(hosts, C4_LAYER, c4_batches, c4_ref, int(variant == "bf16"), tol)
+
+
+# ---- layers of the enwik profile ----------------------------------------------------------
+# nncp.c:2515-2572: d_model 1024, 8 heads of 128, gated GELU feed-forward of 3072, RMSNorm in
+# front of every block and after the last, 64 + 256 keys with one position vector per key
+# (d_pos = 320), position matrices per layer (tied_w_r = 0), position biases shared.  Two such
+# layers, 8 streams; weights and data as above.
+
+ENWIK_LAYER = dict(n_layer=2, d_model=1024, n_head=8, d_inner=3072, ff_act=2, d_pos=320, mem_len=256, seg_len=64,
+                   batch_size=8, n_symbols=256, ln_flags=2 | 4 | 16, use_bias=1, use_w_r=1, tied_w_r=0, tied_b_r=1,
+                   seed=123)
+
+
+@pytest.fixture(scope="module")
+def enwik_batches():
+    cfg = ENWIK_LAYER
+    syms = bench.markov3_dirichlet(cfg["batch_size"] * cfg["seg_len"] * 2, seed=80)
+    return M.segment_batches(syms, cfg["batch_size"], cfg["seg_len"], 2)
+
+
+@pytest.fixture(scope="module")
+def enwik_ref(hosts, enwik_batches):
+    return Reference(hosts, ENWIK_LAYER, enwik_batches)
+
+
+@pytest.mark.parametrize("variant,tol", [("fp32", 1e-5), ("bf16", 2e-2)])
+def test_enwik_layer_shape_first_step_matches_checker(hosts, enwik_batches, enwik_ref, variant, tol):
+    _check_first_step(hosts, ENWIK_LAYER, enwik_batches, enwik_ref, int(variant == "bf16"), tol)
+
+
+@pytest.mark.parametrize("variant,tol", [("fp32", 1e-5), ("bf16", 2e-2)])
+def test_enwik_layer_shape_two_steps(hosts, enwik_batches, enwik_ref, variant, tol):
+    """(the second step attends to the first step's 64 hidden states in the memory)"""
+    _check_steps(hosts, ENWIK_LAYER, enwik_batches, enwik_ref, int(variant == "bf16"), tol)

@@ -171,9 +171,15 @@ def test_c4_full_size_stream_properties(hosts, variant):
     data, st = enc.compress(syms, mode)
     w_enc = {k: enc.get_param(k) for k in ("embed", "embed_out", "w_q_0", "ff2_19", "ln_g_39", "b_r_0")}
     enc.close()
-    assert 0 < len(data) < 2 * n                       # 14 bits of alphabet: at most 2 bytes a token
+    # every 16-bit CDF keeps each symbol at a count of 1 or more: at most 16 bits a token
+    assert 0 < len(data) <= 2 * n + 64
+    # an untrained model: the first segment is coded at log2(V) + (variance of random logits),
+    # the second after one sign-like RMSProp step that overshoots - near the coder's cap
     bits = st.loss_bits / n
-    assert np.isfinite(bits) and 6.0 < bits < 14.5, bits   # untrained model on 16384 symbols: below log2(V) + slack
+    assert np.isfinite(bits) and 6.0 < bits < 17.0, bits
+    # (the summed code length of the float probabilities is an upper bound here: the CDF's
+    # floor of one count makes symbols below 2^-16 cheaper than their probability)
+    assert len(data) * 8 <= 1.02 * st.loss_bits + 1024, (len(data) * 8, st.loss_bits)
     again = _model(hosts[0], cfg, 1, bf16=bf16)
     data2, _ = again.compress(syms, mode)
     again.close()
