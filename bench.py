@@ -399,9 +399,10 @@ def decode_c3(pkg, data, n_segments, variant):
     mode = H.MODE_SEGMENT | H.MODE_STEP_DECODE | H.CODER_CDF16
 
     def model():
-        m = H.Model(H.Host(), H.make_config(**dict(C3, use_device=1, fused=1, sgd_opt=opt)))
+        m = H.Model(H.Host(), H.make_config(**dict(C3, use_device=1, fused=1, sgd_opt=opt,
+                                                   param_bf16=int(variant == "bf16_params"))))
         init_weights(m)
-        m.nc.nc_set_matmul_bf16(m.ctx, 1 if variant == "bf16" else 0)
+        m.nc.nc_set_matmul_bf16(m.ctx, 0 if variant == "fp32" else 1)
         return m
     enc = model()
     stream = np.zeros(syms.size * 4 + 4096, dtype=np.uint8)
@@ -437,9 +438,10 @@ def measure_c4(pkg, variant, warmup, steps, profile_steps):
     per_step = B * T
     data = bigram_zipf_dirichlet((warmup + steps + profile_steps) * per_step)
     opt = pkg.binding.SGDOptParams(algo=pkg.binding.SGD_OPT_RMSPROP, beta2=0.99, eps=1e-8, lr=3e-4)
-    model = H.Model(H.Host(), H.make_config(**dict(C4, use_device=1, fused=1, sgd_opt=opt)))
+    model = H.Model(H.Host(), H.make_config(**dict(C4, use_device=1, fused=1, sgd_opt=opt,
+                                                   param_bf16=int(variant == "bf16_params"))))
     init_weights(model)
-    model.nc.nc_set_matmul_bf16(model.ctx, 1 if variant == "bf16" else 0)
+    model.nc.nc_set_matmul_bf16(model.ctx, 0 if variant == "fp32" else 1)
     mode = H.MODE_SEGMENT | H.CODER_CDF16
     pos = 0
     if warmup:
@@ -457,7 +459,7 @@ def measure_c4(pkg, variant, warmup, steps, profile_steps):
         rows = gemm_profile(model, H, data[pos:pos + profile_steps * per_step], mode, pkg.binding.HIP_LIB)
         if rows:
             dom = max(rows, key=lambda r: r["seconds"])
-            peak = PEAK_TFLOPS[variant]
+            peak = PEAK_TFLOPS["fp32" if variant == "fp32" else "bf16"]
             achieved = dom["flops"] / dom["seconds"] / 1e12
             tot_f, tot_s = sum(r["flops"] for r in rows), sum(r["seconds"] for r in rows)
             roof = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 3), "peak": peak,
@@ -495,8 +497,10 @@ def main():
                          "(configs[3]); its CPU baseline is not taken (one step is about an hour of host time)")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--variant", choices=["fp32", "bf16"], default="fp32")
-    ap.add_argument("--also", default="bf16", help="further variants measured after the headline one and "
+    ap.add_argument("--variant", choices=["fp32", "bf16", "bf16_params"], default="fp32",
+                    help="fp32: the reference's arithmetic; bf16: matrix products on bf16 operands, f32 parameters; "
+                         "bf16_params: parameters stored as NC_TYPE_BF16 as well (nncp --bf16's param_type)")
+    ap.add_argument("--also", default="bf16,bf16_params", help="further variants measured after the headline one and "
                                                    "reported under `variants` (comma separated, empty for none)")
     ap.add_argument("--cpu-steps", type=int, default=4, help="0 skips the CPU baseline")
     ap.add_argument("--cpu-single-steps", type=int, default=1, help="steps of the single-thread CPU baseline (0 skips it)")
@@ -548,9 +552,10 @@ def main():
 
     def measure(variant, mode=mode, steps=args.steps, profile_steps=args.profile_steps):
         """warm-up, the timed steps and the per-launch GEMM timing of one arithmetic variant"""
-        model = H.Model(H.Host(), H.make_config(**dict(C3, use_device=1, fused=1, sgd_opt=opt)))
+        model = H.Model(H.Host(), H.make_config(**dict(C3, use_device=1, fused=1, sgd_opt=opt,
+                                                       param_bf16=int(variant == "bf16_params"))))
         init_weights(model)
-        model.nc.nc_set_matmul_bf16(model.ctx, 1 if variant == "bf16" else 0)
+        model.nc.nc_set_matmul_bf16(model.ctx, 0 if variant == "fp32" else 1)
         pos = 0
         if args.warmup:
             say("C3 %s: %d warm-up steps" % (variant, args.warmup))
@@ -569,10 +574,10 @@ def main():
             if rows:
                 dom = max(rows, key=lambda r: r["seconds"])
                 achieved = dom["flops"] / dom["seconds"] / 1e12
-                peak = PEAK_TFLOPS[variant]
+                peak = PEAK_TFLOPS["fp32" if variant == "fp32" else "bf16"]
                 tot_f = sum(r["flops"] for r in rows)
                 tot_s = sum(r["seconds"] for r in rows)
-                traffic, traffic_source = measured_traffic(dom["kernel"], variant)
+                traffic, traffic_source = measured_traffic(dom["kernel"], "fp32" if variant == "fp32" else "bf16")
                 roof = {"bound": "mfma", "kernel": dom["kernel"], "achieved": round(achieved, 3),
                         "peak": peak, "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
                         "traffic": traffic, "traffic_source": traffic_source,
@@ -583,7 +588,8 @@ def main():
                         "all_gemm_ms_per_step": round(tot_s / profile_steps * 1e3, 3)}
         model.close()
         return {"value": round(steps * per_step / sec, 1), "ms_per_step": round(sec / steps * 1e3, 3),
-                "dtype": "f32" if variant == "fp32" else "bf16-in/f32-acc",
+                "dtype": {"fp32": "f32", "bf16": "bf16-in/f32-acc",
+                          "bf16_params": "bf16 parameters (f32 master in the optimiser), bf16-in/f32-acc"}[variant],
                 "bits_per_symbol": round(nbytes * 8 / (steps * per_step), 4),
                 "kernel_launches_per_step": launches / steps,
                 "host_seconds": {"eval_and_copy": round(st.t_eval, 4), "code": round(st.t_code, 4),

@@ -219,6 +219,12 @@ NCTensor *nc_tensor_to_cpu_device(NCTensor *x);                        /* libnc.
 NCDevice *nc_get_tensor_device(const NCTensor *x);                     /* libnc.h:228 */
 
 /* ---- element-wise ops ---------------------------------------------------- */
+/* Two item types carry values: NC_TYPE_F32 and NC_TYPE_BF16 (2 bytes per element: the storage
+   type of parameters under nncp's bf16 switch, nncp.c:343-346).  F32 -> BF16 rounds to
+   nearest even, BF16 -> F32 is exact; the gradient passes through a conversion unchanged, as
+   F32.  Arithmetic is F32 throughout: an op that is handed a BF16 tensor works on its
+   widened values and returns F32 (in libnc_hip.so a bf16-operand product reads the 2-byte
+   storage directly).  The optimiser keeps an fp32 master of a BF16 parameter (nc_ext.h). */
 NCTensor *nc_convert(NCTensor *x, NCTypeEnum new_type);                /* libnc.h:231 */
 NCTensor *nc_add(NCTensor *x1, NCTensor *x2);                          /* libnc.h:232 */
 NCTensor *nc_mul(NCTensor *x1, NCTensor *x2);                          /* libnc.h:235 */

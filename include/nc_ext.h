@@ -168,7 +168,9 @@ int nc_set_deferred_weight_grad(NCContext *m, int enable);
 
 /* The optimiser's per-parameter state, for checkpoints and for tests that put two models
    into the same state: `which` 0 = first moment (Adam with beta1 != 0), 1 = second moment
-   (Adam, RMSProp).  nc_sgd_opt_get_state returns a new 1-D f32 tensor on the host device
+   (Adam, RMSProp), 2 = the fp32 master values of a parameter stored as NC_TYPE_BF16 (the
+   update works on them and leaves their rounding in the parameter; a caller that sets them
+   sets the parameter to their rounding as well).  nc_sgd_opt_get_state returns a new 1-D f32 tensor on the host device
    holding a copy (NULL when the parameter has no optimiser or the algorithm keeps no such
    moment); nc_sgd_opt_set_state copies the values of v (f32, same element count, any device)
    into it.  nc_sgd_opt_get_step / nc_sgd_opt_set_step: the count of updates applied, which

@@ -405,7 +405,10 @@ int nchip_opt_update(void *stream, int algo, float *w, float *m, float *v, const
    workgroups chunk_prefix[i] .. chunk_prefix[i+1]-1, each covering `chunk`
    consecutive elements.  m may be NULL (beta1 == 0), v may be NULL (SGD).  w16, when not
    NULL, receives the updated w rounded to bf16 (nearest even), element for element: the
-   operand copy the bf16 products read, so that no weight is cast again after its update. */
+   operand copy the bf16 products read, so that no weight is cast again after its update.
+   wide, when not NULL, receives that rounded value widened to f32 again (parameters stored
+   as bf16: w is their fp32 master, w16 the parameter itself, wide the copy that kernels
+   reading f32 use). */
 typedef struct {
     float *w, *m, *v;
     const float *g;
@@ -413,6 +416,7 @@ typedef struct {
     float lr;
     int pad_;
     uint16_t *w16;
+    float *wide;
 } NchipOptTensor;
 int nchip_opt_update_multi(void *stream, int algo, const NchipOptTensor *dev_table,
                            const int *dev_chunk_prefix, int n_tensors, int total_chunks, int chunk,
@@ -420,6 +424,8 @@ int nchip_opt_update_multi(void *stream, int algo, const NchipOptTensor *dev_tab
 
 /* dst[i] = src[i] rounded to bf16 (nearest even), i < n: one streaming pass. */
 int nchip_cast_bf16(void *stream, const float *src, uint16_t *dst, int64_t n);
+/* dst[i] = the f32 value of bf16 src[i] (exact), i < n. */
+int nchip_widen_bf16(void *stream, const uint16_t *src, float *dst, int64_t n);
 
 /* logits (v, n) f32 -> cdf (v, n) u16 as specified in nc_ext.h
    (nc_soft_max_cdf16); bit-identical to the CPU checker. */

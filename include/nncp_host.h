@@ -115,6 +115,11 @@ typedef struct { /* TransformerModelParams + the NNCPModelParams fields it needs
     int lstm_type;                                     /* NNCP_LSTM_* */
     int lstm_full_connect, lstm_use_layer_norm;
     float lstm_forget_bias;
+    /* parameters are NC_TYPE_BF16 tensors, 2 bytes per element (param_type of nncp.c:343-346
+       and 1727-1730 under nncp --bf16); matrix products then round their other operand to bf16
+       as well.  The optimiser keeps an fp32 master of every parameter; activations and the
+       memories stay f32. */
+    int param_bf16;
 } NNCPConfig;
 
 #define NNCP_MODEL_TRF 0
@@ -269,7 +274,9 @@ void nncp_decompress(NNCPModel *s, const uint8_t *in, size_t len, uint16_t *syms
 /* NNCPModelParams' file-level fields that NNCPConfig does not hold (nncp.c:142-156) */
 typedef struct {
     NNCPInterp lr, block_len; /* per training step; per file position */
-    int use_bf16;             /* matrix products round their operands to bf16 (nncp --bf16) */
+    int use_bf16;             /* nncp --bf16.  1: matrix products round their operands to bf16,
+                                 parameters stay f32; 2: parameters are stored as bf16 as well
+                                 (NNCPConfig.param_bf16).  The header byte holds the value. */
     int64_t max_size;         /* encoder: truncate the input to this many symbols; -1: no limit */
     int mode;                 /* NNCP_MODE_* | NNCP_CODER_*; 0 is the reference's stream */
 } NNCPFileParams;

@@ -16,6 +16,18 @@ HIP_LIB = os.path.join(HERE, "csrc", "libnc_hip.so")
 F32, BF16, F16, I8, I16, I32, U8, U16, U32 = range(9)
 _NP = {F32: np.float32, I8: np.int8, I32: np.int32, U16: np.uint16, U8: np.uint8}
 _NC = {np.dtype(v): k for k, v in _NP.items()}
+_NP[BF16] = np.uint16      # read as its 16 bits; numpy() widens them to float32
+
+
+def bf16_bits(a):
+    """float32 array -> the 16 bits of each value rounded to bf16 (nearest even)"""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16).reshape(np.shape(a))
+
+
+def bf16_widen(bits):
+    """the float32 value of each 16-bit bf16 pattern"""
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32).reshape(np.shape(bits))
 
 SGD_OPT_BASIC, SGD_OPT_ADAM, SGD_OPT_RMSPROP = 0, 1, 16
 NC_PAD_ZERO, NC_PAD_DUP = 0, 1
@@ -191,6 +203,8 @@ class NC:
         ptr = self.lib.nc_tensor_get_ptr(h, None)
         buf = (C.c_char * (n * np.dtype(_NP[t]).itemsize)).from_address(ptr)
         out = np.frombuffer(buf, dtype=_NP[t]).copy().reshape(tuple(reversed(dims)))
+        if t == BF16:
+            out = bf16_widen(out)
         self.lib.nc_free_tensor(h)
         if free:
             self.lib.nc_free_tensor(x)

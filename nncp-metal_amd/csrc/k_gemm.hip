@@ -1387,6 +1387,16 @@ __global__ __launch_bounds__(256) void cast_bf16_flat_kernel(const float *src, u
         for (int64_t i = units * 8 + threadIdx.x; i < n; i += 256) as_global(dst)[i] = f32_to_bf16_rne(as_global(src)[i]);
 }
 
+// dst[i] = float(bf16 src[i]) for i < n (exact): one streaming pass
+__global__ __launch_bounds__(256) void widen_bf16_flat_kernel(const uint16_t *src, float *dst, int64_t n)
+{
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const uint16_t NCHIP_GLOBAL *s = as_global(src);
+    float NCHIP_GLOBAL *d = as_global(dst);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+        d[i] = __builtin_bit_cast(float, (uint32_t)s[i] << 16);
+}
+
 // ---- optional per-launch timing (HIP events on the launch stream) ----------
 struct ProfRec {
     hipEvent_t start, stop;
@@ -1900,6 +1910,16 @@ extern "C" int nchip_cast_bf16(void *stream, const float *src, uint16_t *dst, in
     if (nb > 4096) nb = 4096;
     hipLaunchKernelGGL(cast_bf16_flat_kernel, dim3((unsigned)nb), dim3(256), 0, (hipStream_t)stream, src, dst, n);
     if (hipGetLastError() != hipSuccess) { fprintf(stderr, "nchip_cast_bf16: launch failed\n"); return -2; }
+    return 0;
+}
+
+extern "C" int nchip_widen_bf16(void *stream, const uint16_t *src, float *dst, int64_t n)
+{
+    if (n <= 0) return 0;
+    int64_t nb = (n + 255) / 256;
+    if (nb > 8192) nb = 8192;
+    hipLaunchKernelGGL(widen_bf16_flat_kernel, dim3((unsigned)nb), dim3(256), 0, (hipStream_t)stream, src, dst, n);
+    if (hipGetLastError() != hipSuccess) { fprintf(stderr, "nchip_widen_bf16: launch failed\n"); return -2; }
     return 0;
 }
 

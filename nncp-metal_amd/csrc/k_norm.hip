@@ -431,7 +431,11 @@ __global__ __launch_bounds__(TPB) void opt_update_multi_kernel(const NchipOptTen
         opt_step(algo, w, t.m ? t.m + i : nullptr, v, t.g[i], t.lr, b1, b2, eps, clip, c1, c2);
         t.w[i] = w;
         if (t.v) t.v[i] = v;
-        if (t.w16) t.w16[i] = f32_to_bf16_rne(w);
+        if (t.w16) {
+            const uint16_t r = f32_to_bf16_rne(w);
+            t.w16[i] = r;
+            if (t.wide) t.wide[i] = __builtin_bit_cast(float, (uint32_t)r << 16);
+        }
     }
 }
 

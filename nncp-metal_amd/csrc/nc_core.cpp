@@ -480,7 +480,43 @@ uint16_t *nc_shadow_for_write(NCContext *m, NCTensor *x)
 
 void nc_shadow_invalidate(NCTensor *x)
 {
-    if (x && x->buf) x->buf->sh_valid = false;
+    if (!x || !x->buf) return;
+    x->buf->sh_valid = false;
+    x->buf->wide_valid = false;
+    x->buf->version++;
+}
+
+// ---- bf16 tensors as operands --------------------------------------------------------------
+NCTensor *nc_operand(NCTensor *x)
+{
+    if (x->type != NC_TYPE_BF16) return nc_contig(x);
+    need_dev(x, "an op on a bf16 tensor");
+    NCContext *m = nc_ctx(x);
+    NCTensorBuffer *b = x->buf;
+    if (!b->wide) {
+        size_t n = b->elems ? b->elems : 1;
+        b->wide = nc_alloc(x->dev, NC_TYPE_F32, 1, &n, false);
+        NCTensorBuffer *wb = b->wide->buf;
+        wb->sh = (uint16_t *)b->ptr;
+        wb->sh_cap = 0;
+        wb->sh_alias = true;
+        wb->sh_valid = false;
+        b->wide_valid = false;
+    }
+    if (!b->wide_valid) {
+        if (nchip_widen_bf16(m->stream, (const uint16_t *)b->ptr, (float *)b->wide->buf->ptr, (int64_t)b->elems))
+            nc_fatal("bf16 widening failed");
+        m->launches++;
+        b->wide_valid = true;
+        b->wide->buf->sh_valid = true; // the bf16 buffer IS the rounding of its own widening
+    }
+    NCTensor *y = nc_view(b->wide);
+    y->off = x->off;
+    y->n_dims = x->n_dims;
+    for (int i = 0; i < x->n_dims; i++) { y->dims[i] = x->dims[i]; y->strides[i] = x->strides[i]; }
+    y->node = nc_dup_node(x->node);
+    nc_free_tensor(x);
+    return nc_contig(y);
 }
 
 float *nc_tmp_f32(NCContext *m, size_t n, size_t *cap)
@@ -523,7 +559,15 @@ extern "C" void nc_free_tensor(NCTensor *x) // libnc.h:174; NULL accepted (nncp.
     nc_free_node(x->node);
     if (--x->buf->ref == 0) {
         NCContext *m = x->buf->dev->ctx;
-        if (x->buf->sh) m->dev_pool.put(x->buf->sh, x->buf->sh_cap); // stream ordered, like the buffer itself
+        if (x->buf->sh && !x->buf->sh_alias) m->dev_pool.put(x->buf->sh, x->buf->sh_cap); // stream ordered, like the buffer itself
+        if (NCTensor *wide = x->buf->wide) {
+            // the f32 copy of a bf16 buffer borrowed this buffer as its shadow: views of the
+            // copy may outlive it, and make a shadow of their own from then on
+            wide->buf->sh = nullptr; wide->buf->sh_cap = 0;
+            wide->buf->sh_alias = false; wide->buf->sh_valid = false;
+            x->buf->wide = nullptr;
+            nc_free_tensor(wide);
+        }
         if (x->buf->in_flight && !x->buf->dev->is_hip && x->buf->in_flight > m->sync_count)
             nc_staging_retire(m, x->buf->ptr, x->buf->cap, x->buf->in_flight - 1); // a queued kernel may still use it
         else
@@ -548,7 +592,7 @@ extern "C" int nc_tensor_get_dims(const NCTensor *x, size_t *dims)
 extern "C" void *nc_tensor_get_ptr(const NCTensor *x, size_t *pstride)
 {
     if (pstride) *pstride = x->n_dims >= 2 ? x->strides[1] : (x->n_dims ? x->dims[0] : 1);
-    x->buf->sh_valid = false; // the address leaves the library: whoever holds it may write
+    nc_shadow_invalidate((NCTensor *)x); // the address leaves the library: whoever holds it may write
     return nc_data(x);
 }
 
@@ -655,9 +699,19 @@ extern "C" void nc_tensor_set_zero(NCTensor *y) // libnc.h:192
     }
 }
 
+static void upload_values(NCTensor *y, const float *host);
+
 extern "C" void nc_tensor_set_f32(NCTensor *y, float val) // libnc.h:194
 {
-    if (!nc_is_contig(y) || y->type != NC_TYPE_F32) nc_fatal("set_f32: contiguous f32 tensor expected");
+    if (y->type == NC_TYPE_BF16 && nc_is_contig(y)) { // every element the same 16 bits
+        size_t n = nc_numel(y);
+        float *tmp = (float *)nc_malloc((n ? n : 1) * sizeof(float));
+        for (size_t i = 0; i < n; i++) tmp[i] = val;
+        upload_values(y, tmp);
+        free(tmp);
+        return;
+    }
+    if (!nc_is_contig(y) || y->type != NC_TYPE_F32) nc_fatal("set_f32: contiguous f32 or bf16 tensor expected");
     nc_shadow_invalidate(y);
     if (y->dev->is_hip) { k_fill_f32(nc_stream(y), nc_f32(y), val, (int64_t)nc_numel(y)); nc_ctx(y)->launches++; }
     else for (size_t i = 0; i < nc_numel(y); i++) nc_f32(y)[i] = val;
@@ -764,6 +818,36 @@ extern "C" NCRNDState *nc_rnd_init(NCDevice *d, uint32_t seed)
 
 extern "C" void nc_rnd_end(NCRNDState *s) { nc_free(s); }
 
+static uint16_t host_bf16(float f) // nearest even; NaN stays a quiet NaN
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fff + ((u >> 16) & 1);
+    return (uint16_t)(u >> 16);
+}
+
+static void upload_f32(NCTensor *y, const float *host);
+
+// host values into contiguous f32 or bf16 tensor y (a bf16 tensor keeps their rounding)
+static void upload_values(NCTensor *y, const float *host)
+{
+    nc_shadow_invalidate(y);
+    if (y->type == NC_TYPE_F32) { upload_f32(y, host); return; }
+    NCContext *m = y->dev->ctx;
+    size_t n = nc_numel(y);
+    if (!y->dev->is_hip) {
+        for (size_t i = 0; i < n; i++) ((uint16_t *)nc_data(y))[i] = host_bf16(host[i]);
+        return;
+    }
+    size_t cap;
+    uint16_t *pin = (uint16_t *)m->host_pool.get((n ? n : 1) * sizeof(uint16_t), &cap);
+    for (size_t i = 0; i < n; i++) pin[i] = host_bf16(host[i]);
+    hip_check(hipMemcpyAsync(nc_data(y), pin, n * sizeof(uint16_t), hipMemcpyHostToDevice, m->stream), "hipMemcpyAsync h2d");
+    nc_stream_wait(m);
+    m->host_pool.put(pin, cap);
+}
+
 static void upload_f32(NCTensor *y, const float *host)
 {
     NCContext *m = y->dev->ctx;
@@ -777,15 +861,15 @@ static void upload_f32(NCTensor *y, const float *host)
 // element order and uploaded (initialisation only)
 extern "C" void nc_tensor_set_rnd_unif(NCTensor *y, float avg, float range, NCRNDState *rs)
 {
-    if (!nc_is_contig(y) || y->type != NC_TYPE_F32) nc_fatal("set_rnd_unif: contiguous f32 tensor expected");
-    nc_shadow_invalidate(y);
+    if (!nc_is_contig(y) || (y->type != NC_TYPE_F32 && y->type != NC_TYPE_BF16))
+        nc_fatal("set_rnd_unif: contiguous f32 or bf16 tensor expected");
     size_t n = nc_numel(y);
-    float *tmp = (float *)nc_malloc(n * sizeof(float));
+    float *tmp = (float *)nc_malloc((n ? n : 1) * sizeof(float));
     for (size_t i = 0; i < n; i++) {
         float u = (float)(xorwow(rs) >> 8) * (1.0f / 16777216.0f);
         tmp[i] = avg + range * (2.0f * u - 1.0f);
     }
-    upload_f32(y, tmp);
+    upload_values(y, tmp);
     free(tmp);
 }
 
@@ -856,6 +940,10 @@ struct SGDOptVarState {
     NCSGDOptState *opt;
     NCParam *param;
     NCTensor *m, *v, *g;
+    // a bf16 parameter: the fp32 values the update works on (the parameter holds their
+    // rounding), and the buffer version they were last taken from or written at
+    NCTensor *master;
+    uint64_t master_version;
     size_t n;
     bool has_grad;
 };
@@ -883,6 +971,17 @@ extern "C" void nc_sgd_opt_end(NCSGDOptState *s)
     delete s;
 }
 
+// the master copy of a bf16 parameter starts as (and, after anyone else wrote the parameter,
+// goes back to) the parameter's own value
+static void master_from_param(SGDOptVarState *vs, NCTensor *w)
+{
+    NCContext *m = nc_ctx(w);
+    if (nchip_widen_bf16(m->stream, (const uint16_t *)nc_data(w), nc_f32(vs->master), (int64_t)vs->n))
+        nc_fatal("bf16 widening failed");
+    m->launches++;
+    vs->master_version = w->buf->version;
+}
+
 extern "C" void nc_sgd_opt_set_all(NCParamList *pl, NCSGDOptState *s)
 {
     for (struct list_head *el = pl->param_list.next; el != &pl->param_list; el = el->next) {
@@ -892,16 +991,23 @@ extern "C" void nc_sgd_opt_set_all(NCParamList *pl, NCSGDOptState *s)
             auto &v = vs->opt->vars;
             for (size_t i = 0; i < v.size(); i++)
                 if (v[i] == vs) { v.erase(v.begin() + i); break; }
-            nc_free_tensor(vs->m); nc_free_tensor(vs->v); nc_free_tensor(vs->g);
+            nc_free_tensor(vs->m); nc_free_tensor(vs->v); nc_free_tensor(vs->g); nc_free_tensor(vs->master);
             delete vs;
             p->sgd_opt = nullptr;
         }
         if (s) {
             NCTensor *w = *p->pval;
-            if (w->type != NC_TYPE_F32 || !nc_is_contig(w)) nc_fatal("optimiser: contiguous f32 parameter expected");
+            if ((w->type != NC_TYPE_F32 && w->type != NC_TYPE_BF16) || !nc_is_contig(w))
+                nc_fatal("optimiser: contiguous f32 or bf16 parameter expected");
             SGDOptVarState *vs = new SGDOptVarState();
             vs->opt = s; vs->param = p; vs->n = nc_numel(w); vs->has_grad = false;
             size_t n1 = vs->n;
+            vs->master = nullptr;
+            if (w->type == NC_TYPE_BF16) {
+                need_dev(w, "optimiser on a bf16 parameter");
+                vs->master = nc_alloc(w->dev, NC_TYPE_F32, 1, &n1, false);
+                master_from_param(vs, w);
+            }
             bool need_m = s->p.algo == SGD_OPT_ADAM && s->p.u.adam.beta1 != 0.0f;
             vs->m = need_m ? nc_alloc(w->dev, NC_TYPE_F32, 1, &n1, true) : nullptr;
             vs->v = (int)s->p.algo != SGD_OPT_BASIC ? nc_alloc(w->dev, NC_TYPE_F32, 1, &n1, true) : nullptr;
@@ -918,15 +1024,17 @@ extern "C" void nc_sgd_opt_set_lr(NCSGDOptState *s, float lr) { s->p.lr = lr; }
 extern "C" NCTensor *nc_sgd_opt_get_state(NCParam *p, int which)
 {
     SGDOptVarState *vs = p->sgd_opt;
-    NCTensor *t = !vs ? nullptr : which == 0 ? vs->m : which == 1 ? vs->v : nullptr;
+    NCTensor *t = !vs ? nullptr : which == 0 ? vs->m : which == 1 ? vs->v : which == 2 ? vs->master : nullptr;
+    if (t && which == 2 && vs->master_version != (*p->pval)->buf->version) master_from_param(vs, *p->pval);
     return t ? nc_tensor_to_cpu_device(nc_dup_tensor(t)) : nullptr;
 }
 
 extern "C" void nc_sgd_opt_set_state(NCParam *p, int which, const NCTensor *v)
 {
     SGDOptVarState *vs = p->sgd_opt;
-    NCTensor *t = !vs ? nullptr : which == 0 ? vs->m : which == 1 ? vs->v : nullptr;
+    NCTensor *t = !vs ? nullptr : which == 0 ? vs->m : which == 1 ? vs->v : which == 2 ? vs->master : nullptr;
     if (!t) nc_fatal("nc_sgd_opt_set_state: '%s' keeps no moment %d", p->name, which);
+    if (which == 2) vs->master_version = (*p->pval)->buf->version; // (the caller sets the parameter to its rounding)
     if (v->type != NC_TYPE_F32 || nc_numel(v) != vs->n) nc_fatal("nc_sgd_opt_set_state: %zu f32 values expected for '%s'", vs->n, p->name);
     size_t n1 = vs->n;
     NCTensor *src = nc_reshape_view(nc_tensor_to_device(nc_dup_tensor(v), t->dev), 1, &n1);
@@ -981,6 +1089,23 @@ extern "C" void nc_sgd_opt_update(NCSGDOptState *s)
         NCTensor *w = *vs->param->pval;
         need_dev(w, "nc_sgd_opt_update");
         NchipOptTensor t;
+        t.wide = nullptr;
+        if (vs->master) {
+            // bf16 parameter: update the master, leave its rounding in the parameter and, if
+            // ops have taken the parameter as an operand before, in its f32 copy as well
+            NCTensorBuffer *b = w->buf;
+            if (vs->master_version != b->version) master_from_param(vs, w);
+            t.w = nc_f32(vs->master);
+            t.w16 = (uint16_t *)nc_data(w);
+            const bool whole = b->wide && w->off == 0 && vs->n == b->elems;
+            nc_shadow_invalidate(w);
+            vs->master_version = b->version;
+            if (whole) {
+                t.wide = nc_f32(b->wide);
+                b->wide_valid = true;
+                b->wide->buf->sh_valid = true;
+            }
+        } else
         t.w = nc_f32(w);
         t.m = vs->m ? nc_f32(vs->m) : nullptr; // with beta1 == 0 the first moment is the gradient
         t.v = vs->v ? nc_f32(vs->v) : nullptr;
@@ -990,8 +1115,10 @@ extern "C" void nc_sgd_opt_update(NCSGDOptState *s)
         t.pad_ = 0;
         // matrices are operands of the bf16 products: their shadow is written with the update
         // (vectors - biases, gains - are not, and a shadow they may have is stale from here on)
-        t.w16 = (s->ctx->matmul_bf16 && w->n_dims >= 2) ? nc_shadow_for_write(s->ctx, w) : nullptr;
-        if (!t.w16) nc_shadow_invalidate(w);
+        if (!vs->master) {
+            t.w16 = (s->ctx->matmul_bf16 && w->n_dims >= 2) ? nc_shadow_for_write(s->ctx, w) : nullptr;
+            if (!t.w16) nc_shadow_invalidate(w);
+        }
         tab.push_back(t);
         prefix.push_back(prefix.back() + (int)((vs->n + chunk - 1) / chunk));
     }

@@ -136,6 +136,16 @@ struct NCTensorBuffer {
     size_t sh_cap;
     bool sh_valid;
     size_t elems; // elements the buffer was allocated for
+    // A bf16 device buffer (NC_TYPE_BF16: 2 bytes per element are the tensor's value): `wide`
+    // is the f32 copy of all its elements that kernels reading f32 use (made by one widening
+    // pass when an op first takes the tensor as an operand, kept until the buffer goes;
+    // wide_valid: it holds what the buffer holds NOW).  The copy's own shadow is the bf16
+    // buffer itself (sh_alias: borrowed, never returned to the pool), so a bf16-operand
+    // product reads the parameter's 2 bytes directly.
+    NCTensor *wide;
+    bool wide_valid;
+    bool sh_alias;
+    uint64_t version; // counts in-place writes (nc_shadow_invalidate): lets a holder of derived data notice them
 };
 
 struct NCTensor {
@@ -192,9 +202,18 @@ NCTensor *nc_alloc(NCDevice *d, NCTypeEnum t, int nd, const size_t *dims, bool z
 NCTensor *nc_alloc_like(const NCTensor *x);
 NCTensor *nc_view(const NCTensor *x);
 NCTensor *nc_contig(NCTensor *x);                  // consumes
+// What an op does to each operand (consumes): contiguous, and a bf16 tensor replaced by the
+// same view of its buffer's f32 copy, carrying the same graph node (the gradient of a
+// conversion is the identity, and it stays f32).
+NCTensor *nc_operand(NCTensor *x);
 void nc_copy_any(NCTensor *dst, const NCTensor *src); // strided, same device
 void *nc_data(const NCTensor *x);
-static inline float *nc_f32(const NCTensor *x) { return (float *)nc_data(x); }
+static inline float *nc_f32(const NCTensor *x)
+{
+    // (a 2-byte tensor taken for floats would be read out of bounds: ops widen first)
+    if (x->type == NC_TYPE_BF16) nc_fatal("f32 access to a bf16 tensor");
+    return (float *)nc_data(x);
+}
 void need_dev(const NCTensor *x, const char *op);
 NCContext *nc_ctx(const NCTensor *x);
 static inline hipStream_t nc_stream(const NCTensor *x) { return x->dev->ctx->stream; }

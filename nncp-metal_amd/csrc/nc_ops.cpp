@@ -8,6 +8,8 @@
 #include <algorithm>
 
 #define LAUNCHED(x) (nc_ctx(x)->launches++)
+// every op takes its operands through nc_operand: contiguous, bf16 tensors as their f32 copies
+#define nc_contig(x) nc_operand(x)
 
 static NCTensor *new_f32(const NCTensor *like, int nd, const size_t *dims)
 {
@@ -167,16 +169,36 @@ static NCTensor *binary_op(NCTensor *a, NCTensor *b, int kop, int op)
 extern "C" NCTensor *nc_add(NCTensor *x1, NCTensor *x2) { return binary_op(x1, x2, KB_ADD, OP_ADD); } // libnc.h:232
 extern "C" NCTensor *nc_mul(NCTensor *x1, NCTensor *x2) { return binary_op(x1, x2, KB_MUL, OP_MUL); } // libnc.h:235
 
-// libnc.h:231: storage stays fp32 in this library (the bf16 variant rounds
-// inside the matmul), so only identity conversions exist
+// libnc.h:231.  BF16 -> F32 is what every op does to a bf16 operand anyway (nc_operand: the
+// buffer's f32 copy, same node); F32 -> BF16 is one rounding pass into a new 2-byte tensor
+// that keeps the node too (the gradient of a conversion is the identity, in f32).
 extern "C" NCTensor *nc_convert(NCTensor *x, NCTypeEnum new_type)
 {
     if (x->type == new_type) return x;
-    nc_fatal("nc_convert %d -> %d: only fp32 storage is supported; for bf16 matrix math use "
-             "nc_set_matmul_bf16() or NCHIP_MATMUL_BF16=1", (int)x->type, (int)new_type);
+    if (x->type == NC_TYPE_BF16 && new_type == NC_TYPE_F32) return nc_operand(x);
+    if (x->type == NC_TYPE_F32 && new_type == NC_TYPE_BF16) {
+        x = nc_contig(x);
+        need_dev(x, "nc_convert");
+        if (((uintptr_t)nc_data(x) & 15) != 0) { // a view at an odd offset: the cast reads 16-byte units
+            NCTensor *c = nc_alloc_like(x);
+            nc_copy_any(c, x);
+            c->node = nc_dup_node(x->node);
+            nc_free_tensor(x);
+            x = c;
+        }
+        NCTensor *y = nc_alloc(x->dev, NC_TYPE_BF16, x->n_dims, x->dims, false);
+        if (nc_numel(x)) {
+            if (nchip_cast_bf16(nc_stream(x), nc_f32(x), (uint16_t *)nc_data(y), (int64_t)nc_numel(x)))
+                nc_fatal("nc_convert: bf16 cast failed");
+            LAUNCHED(x);
+        }
+        y->node = nc_dup_node(x->node);
+        nc_free_tensor(x);
+        return y;
+    }
+    nc_fatal("nc_convert %d -> %d: f32 and bf16 are the item types that carry values here", (int)x->type, (int)new_type);
 }
 
-// libnc.h:242-244; the mask (K,T) or (K,1) is a prefix of x (K,T,H,B)
 extern "C" NCTensor *nc_masked_fill(NCTensor *x, NCTensor *mask, float c, BOOL mask_inv)
 {
     x = nc_contig(x); mask = nc_contig(mask);
@@ -551,6 +573,12 @@ const float *nc_k_major_of(const NCContext *m, const float *a, size_t rows, size
 
 extern "C" void nc_keep_k_major_weight(NCTensor *w)
 {
+    if (w->type == NC_TYPE_BF16) { // the copy is made of, and found by, the parameter's f32 copy
+        NCTensor *v = nc_operand(nc_dup_tensor(w));
+        nc_keep_k_major_weight(v);
+        nc_free_tensor(v);
+        return;
+    }
     need_f32(w, "nc_keep_k_major_weight");
     if (w->n_dims != 2 || !nc_is_contig(w)) nc_fatal("nc_keep_k_major_weight: a contiguous (m, k) matrix expected");
     NCContext *m = nc_ctx(w);
@@ -1032,6 +1060,12 @@ extern "C" NCTensor *nc_norm_linear_pair_into(NCTensor *x, NCTensor *g, NCTensor
     if (w1 && act0 != NC_ACT_NONE) nc_fatal("%s: no activation on the first product of a pair", me);
     x = nc_contig(x); w0 = nc_contig(w0);
     need_f32(x, me); need_f32(w0, me);
+    // (the other operands are taken as they are, so that the shapes this kernel does not
+    // cover fall through to the plain ops below; bf16 parameters are widened here)
+    if (g && g->type == NC_TYPE_BF16) g = nc_operand(g);
+    if (b && b->type == NC_TYPE_BF16) b = nc_operand(b);
+    if (bias0 && bias0->type == NC_TYPE_BF16) bias0 = nc_operand(bias0);
+    if (w1 && w1->type == NC_TYPE_BF16) w1 = nc_operand(w1);
     NCContext *m = nc_ctx(w0);
     int rc = 1;
     NCTensor *y0 = nullptr, *normed = nullptr;

@@ -35,7 +35,7 @@ class NNCPConfig(C.Structure):
                 ("retrain_len", C.c_int), ("has_retrain_lr", C.c_int), ("retrain_lr", NNCPInterp)] + \
                [(n, C.c_int) for n in ("model_type", "lstm_n_cells", "lstm_n_cells2", "lstm_n_embed_out",
                                        "lstm_type", "lstm_full_connect", "lstm_use_layer_norm")] + \
-               [("lstm_forget_bias", C.c_float)]
+               [("lstm_forget_bias", C.c_float), ("param_bf16", C.c_int)]
 
 
 class NNCPStats(C.Structure):
@@ -284,6 +284,8 @@ class Model:
         dt = np.dtype(B._NP[t])
         buf = (C.c_char * (cnt * dt.itemsize)).from_address(ptr)
         out = np.frombuffer(buf, dtype=dt).copy().reshape(tuple(reversed(dims)))
+        if t == B.BF16:
+            out = B.bf16_widen(out)
         self.nc.nc_free_tensor(h)
         return out
 
@@ -311,7 +313,15 @@ class Model:
 
     def set_param(self, name, arr):
         slot = self.L.nncp_model_param(self.ptr, name.encode())
-        src = self.nc.nc_tensor_to_device(self._host_tensor(arr.astype(np.float32)), self.dev)
+        arr = np.asarray(arr, dtype=np.float32)
+        if self.nc.nc_tensor_get_item_type(slot[0]) == B.BF16:     # a bf16 parameter takes the rounding
+            dims = (C.c_size_t * max(arr.ndim, 1))(*reversed(arr.shape))
+            h = self.nc.nc_new_tensor_nz(self.cpu, B.BF16, arr.ndim, dims)
+            bits = np.ascontiguousarray(B.bf16_bits(arr))
+            C.memmove(self.nc.nc_tensor_get_ptr(h, None), bits.ctypes.data, bits.nbytes)
+        else:
+            h = self._host_tensor(arr)
+        src = self.nc.nc_tensor_to_device(h, self.dev)
         self.nc.nc_tensor_copy(slot[0], src)
         self.nc.nc_free_tensor(src)
 

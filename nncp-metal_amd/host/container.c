@@ -254,7 +254,7 @@ size_t nncp_header_write(uint8_t *buf, size_t cap, const NNCPConfig *c, const NN
     put32(&k, FILE_MAGIC);
     put16(&k, FILE_VERSION);
     put8(&k, c->use_device != 0);
-    put8(&k, fp->use_bf16 != 0);
+    put8(&k, fp->use_bf16 == 2 ? 2 : fp->use_bf16 != 0);
     put16(&k, c->batch_size);
     put16(&k, c->seg_len);
     put16(&k, c->n_symbols);
@@ -432,7 +432,10 @@ static int fail(const char *what, const char *name)
 
 static NNCPModel *model_for_file(const NNCPConfig *c, const NNCPFileParams *fp)
 {
-    NNCPModel *s = nncp_model_new(c);
+    NNCPConfig cfg = *c;
+    if (fp->use_bf16 == 2)
+        cfg.param_bf16 = 1;
+    NNCPModel *s = nncp_model_new(&cfg);
     if (fp->use_bf16)
         nc_set_matmul_bf16(nncp_model_context(s), 1);
     return s;

@@ -87,28 +87,28 @@ void lstm_init(NNCPModel *s) /* nncp.c:1701-1813 */
         const int n_in = c->lstm_full_connect ? C1 * l : (l != 0 ? C1 : 0);
         lc->mat_count = c->lstm_type == NNCP_LSTM_TIED ? 3 : 4;
         const size_t rows = (size_t)C2 * lc->mat_count;
-        param(s, &lc->u, nc_new_tensor_2d(s->dev, NC_TYPE_F32, rows, C1), 1.0f / sqrtf((float)C1), "u%d", l, 0);
+        param(s, &lc->u, nc_new_tensor_2d(s->dev, s->param_type, rows, C1), 1.0f / sqrtf((float)C1), "u%d", l, 0);
         if (n_in != 0)
-            param(s, &lc->w, nc_new_tensor_2d(s->dev, NC_TYPE_F32, rows, n_in), 1.0f / sqrtf((float)n_in), "w%d", l, 0);
-        param(s, &lc->ws, nc_new_tensor_2d(s->dev, NC_TYPE_F32, rows, V), 0.75f, "ws%d", l, 0);
+            param(s, &lc->w, nc_new_tensor_2d(s->dev, s->param_type, rows, n_in), 1.0f / sqrtf((float)n_in), "w%d", l, 0);
+        param(s, &lc->ws, nc_new_tensor_2d(s->dev, s->param_type, rows, V), 0.75f, "ws%d", l, 0);
         for (int j = 0; j < lc->mat_count; j++) {
-            param(s, &lc->b[j], nc_new_tensor_1d(s->dev, NC_TYPE_F32, C2), 0, "b%d_%d", l, j);
+            param(s, &lc->b[j], nc_new_tensor_1d(s->dev, s->param_type, C2), 0, "b%d_%d", l, j);
             if (c->lstm_use_layer_norm) {
-                param(s, &lc->g[j], nc_new_scalar(s->dev, NC_TYPE_F32), 0, "g%d_%d", l, j);
+                param(s, &lc->g[j], nc_new_scalar(s->dev, s->param_type), 0, "g%d_%d", l, j);
                 nc_tensor_set_f32(lc->g[j], 1.0f);
             }
         }
         nc_tensor_set_f32(lc->b[FORGET_GATE], c->lstm_forget_bias);
         if (C2 != C1)
-            param(s, &lc->p, nc_new_tensor_2d(s->dev, NC_TYPE_F32, C1, C2), sqrtf(1.0f / (float)C2), "p%d", l, 0);
+            param(s, &lc->p, nc_new_tensor_2d(s->dev, s->param_type, C1, C2), sqrtf(1.0f / (float)C2), "p%d", l, 0);
         /* lstm_set_batch_size, nncp.c:1815-1832 */
         lc->h0 = nc_new_tensor_2d(s->dev, NC_TYPE_F32, C1, B);
         lc->c0 = nc_new_tensor_2d(s->dev, NC_TYPE_F32, C2, B);
         lc->h0_prev = nc_new_tensor_2d(s->dev, NC_TYPE_F32, C1, B);
         lc->c0_prev = nc_new_tensor_2d(s->dev, NC_TYPE_F32, C2, B);
     }
-    param(s, &ls->fc_b, nc_new_tensor_1d(s->dev, NC_TYPE_F32, V), 0, "fc_b", 0, 0);
-    param(s, &ls->fc_w, nc_new_tensor_2d(s->dev, NC_TYPE_F32, V, (size_t)C1 * c->lstm_n_embed_out),
+    param(s, &ls->fc_b, nc_new_tensor_1d(s->dev, s->param_type, V), 0, "fc_b", 0, 0);
+    param(s, &ls->fc_w, nc_new_tensor_2d(s->dev, s->param_type, V, (size_t)C1 * c->lstm_n_embed_out),
           sqrtf(12.0f / (float)(C1 * L)), "fc_w", 0, 0);
     ls->outputs = nc_mallocz(sizeof(NCTensor *) * c->seg_len);
     s->opt = nc_sgd_opt_init(s->ctx, &c->sgd_opt);

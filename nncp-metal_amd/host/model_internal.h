@@ -27,6 +27,7 @@ struct NNCPModel {
     NCContext *ctx;
     NCDevice *dev, *cpu;
     NCRNDState *rnd;
+    NCTypeEnum param_type; /* F32 or BF16 (nncp.c:255, 343-346) */
     NCParamList params;
     Layer *layers;
     NCTensor *ln_g, *ln_b, *embed, *embed_out, *out_bias;

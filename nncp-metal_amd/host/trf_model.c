@@ -55,9 +55,9 @@ static NCTensor *new_param(NNCPModel *s, NCTensor **slot, NCTensor *t, float ini
 
 static void new_layer_norm(NNCPModel *s, NCTensor **g, NCTensor **b, int idx) /* nncp.c:268-277 */
 {
-    new_param(s, g, nc_new_tensor_1d(s->dev, NC_TYPE_F32, s->cfg.d_model), 0, "ln_g_%d", idx);
+    new_param(s, g, nc_new_tensor_1d(s->dev, s->param_type, s->cfg.d_model), 0, "ln_g_%d", idx);
     nc_tensor_set_f32(*g, 1.0f);
-    new_param(s, b, nc_new_tensor_1d(s->dev, NC_TYPE_F32, s->cfg.d_model), 0, "ln_b_%d", idx);
+    new_param(s, b, nc_new_tensor_1d(s->dev, s->param_type, s->cfg.d_model), 0, "ln_b_%d", idx);
 }
 
 NNCPModel *nncp_model_new(const NNCPConfig *cfg)
@@ -72,6 +72,9 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
         s->cpu = nc_new_cpu_device(s->ctx);
         s->dev = c->use_device ? nc_new_cuda_device(s->ctx, 0) : s->cpu;
         s->rnd = nc_rnd_init(s->dev, c->seed);
+        s->param_type = c->param_bf16 ? NC_TYPE_BF16 : NC_TYPE_F32; /* nncp.c:1727-1730 */
+        if (c->param_bf16)
+            nc_set_matmul_bf16(s->ctx, 1);
         s->cls = &nncp_lstm_class;
         lstm_init(s);
         return s;
@@ -86,6 +89,9 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
     s->cpu = nc_new_cpu_device(s->ctx);
     s->dev = c->use_device ? nc_new_cuda_device(s->ctx, 0) : s->cpu;
     s->rnd = nc_rnd_init(s->dev, c->seed);
+    s->param_type = c->param_bf16 ? NC_TYPE_BF16 : NC_TYPE_F32; /* nncp.c:343-346 */
+    if (c->param_bf16)
+        nc_set_matmul_bf16(s->ctx, 1);
     s->fused_now = c->fused;
     if (c->fused)
         nc_set_deferred_weight_grad(s->ctx, 1); /* backward_cb only forwards to sgd_opt_update_var */
@@ -105,29 +111,29 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
             }
         tl->attn_mask = nc_tensor_to_device(mask, s->dev);
         if (l == 0 || !c->tied_b_r)
-            new_param(s, &tl->b_r, nc_new_tensor_2d(s->dev, NC_TYPE_F32, K, H), 0, "b_r_%d", l);
+            new_param(s, &tl->b_r, nc_new_tensor_2d(s->dev, s->param_type, K, H), 0, "b_r_%d", l);
         if (c->use_w_r && (l == 0 || !c->tied_w_r))
-            new_param(s, &tl->w_r, nc_new_tensor_3d(s->dev, NC_TYPE_F32, c->d_key, c->d_pos, H), init, "w_r_%d", l);
-        new_param(s, &tl->w_q, nc_new_tensor_2d(s->dev, NC_TYPE_F32, H * c->d_key, D), init, "w_q_%d", l);
+            new_param(s, &tl->w_r, nc_new_tensor_3d(s->dev, s->param_type, c->d_key, c->d_pos, H), init, "w_r_%d", l);
+        new_param(s, &tl->w_q, nc_new_tensor_2d(s->dev, s->param_type, H * c->d_key, D), init, "w_q_%d", l);
         if (c->query_bias)
-            new_param(s, &tl->b_q, nc_new_tensor_1d(s->dev, NC_TYPE_F32, H * c->d_key), 0, "b_q_%d", l);
-        new_param(s, &tl->w_kv, nc_new_tensor_2d(s->dev, NC_TYPE_F32, H * c->d_key + H * c->d_value, D), init, "w_kv_%d", l);
+            new_param(s, &tl->b_q, nc_new_tensor_1d(s->dev, s->param_type, H * c->d_key), 0, "b_q_%d", l);
+        new_param(s, &tl->w_kv, nc_new_tensor_2d(s->dev, s->param_type, H * c->d_key + H * c->d_value, D), init, "w_kv_%d", l);
         if (c->d_value != D)
-            new_param(s, &tl->w_o, nc_new_tensor_2d(s->dev, NC_TYPE_F32, D, H * c->d_value), init, "w_o_%d", l);
+            new_param(s, &tl->w_o, nc_new_tensor_2d(s->dev, s->param_type, D, H * c->d_value), init, "w_o_%d", l);
         int n1 = gated ? c->d_inner * 2 : c->d_inner;
-        new_param(s, &tl->ff1, nc_new_tensor_2d(s->dev, NC_TYPE_F32, n1, D), init, "ff1_%d", l);
+        new_param(s, &tl->ff1, nc_new_tensor_2d(s->dev, s->param_type, n1, D), init, "ff1_%d", l);
         if (c->use_bias)
-            new_param(s, &tl->ff_bias1, nc_new_tensor_1d(s->dev, NC_TYPE_F32, n1), 0, "ff_bias1_%d", l);
-        new_param(s, &tl->ff2, nc_new_tensor_2d(s->dev, NC_TYPE_F32, D, c->d_inner),
+            new_param(s, &tl->ff_bias1, nc_new_tensor_1d(s->dev, s->param_type, n1), 0, "ff_bias1_%d", l);
+        new_param(s, &tl->ff2, nc_new_tensor_2d(s->dev, s->param_type, D, c->d_inner),
                   init * sqrtf((float)D / (float)c->d_inner), "ff2_%d", l);
         if (c->use_bias)
-            new_param(s, &tl->ff_bias2, nc_new_tensor_1d(s->dev, NC_TYPE_F32, D), 0, "ff_bias2_%d", l);
+            new_param(s, &tl->ff_bias2, nc_new_tensor_1d(s->dev, s->param_type, D), 0, "ff_bias2_%d", l);
         if (c->ln_flags & (NNCP_LN_POST | NNCP_LN_PRE)) {
             new_layer_norm(s, &tl->ln_g1, &tl->ln_b1, l * 2);
             new_layer_norm(s, &tl->ln_g2, &tl->ln_b2, l * 2 + 1);
         }
         if (c->ln_flags & NNCP_LN_COEF)
-            new_param(s, &tl->alpha, nc_new_scalar(s->dev, NC_TYPE_F32), 0, "alpha_%d", l);
+            new_param(s, &tl->alpha, nc_new_scalar(s->dev, s->param_type), 0, "alpha_%d", l);
         /* caches and node tables of the per-timestep path, nncp.c:439-452 */
         tl->mem_key = nc_new_tensor_4d(s->dev, NC_TYPE_F32, c->d_key, K, H, B);
         tl->mem_value = nc_new_tensor_4d(s->dev, NC_TYPE_F32, c->d_value, K, H, B);
@@ -138,10 +144,10 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
     }
     if (c->ln_flags & NNCP_LN_FINAL)
         new_layer_norm(s, &s->ln_g, &s->ln_b, c->n_layer * 2);
-    new_param(s, &s->embed, nc_new_tensor_2d(s->dev, NC_TYPE_F32, D, c->n_symbols), init, "embed", 0);
-    new_param(s, &s->embed_out, nc_new_tensor_2d(s->dev, NC_TYPE_F32, c->n_symbols, D), init, "embed_out", 0);
+    new_param(s, &s->embed, nc_new_tensor_2d(s->dev, s->param_type, D, c->n_symbols), init, "embed", 0);
+    new_param(s, &s->embed_out, nc_new_tensor_2d(s->dev, s->param_type, c->n_symbols, D), init, "embed_out", 0);
     if (c->use_bias)
-        new_param(s, &s->out_bias, nc_new_tensor_1d(s->dev, NC_TYPE_F32, c->n_symbols), 0, "out_bias", 0);
+        new_param(s, &s->out_bias, nc_new_tensor_1d(s->dev, s->param_type, c->n_symbols), 0, "out_bias", 0);
     s->mem_h = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
     s->train_h = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
     for (int l = 0; l < c->n_layer; l++) {

@@ -187,6 +187,10 @@ NCTensor *nc_view(const NCTensor *x)
 
 float *nc_f32(const NCTensor *x)
 {
+    /* a 2-byte tensor read as floats would be read out of bounds: ops widen bf16 operands
+       before they come here (nc_operand) */
+    if (nc_type_size(x->type) != sizeof(float))
+        nc_fatal("f32 access to a tensor of type %d", (int)x->type);
     return (float *)x->buf->data + x->off;
 }
 

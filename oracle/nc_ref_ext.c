@@ -7,6 +7,10 @@
  */
 #include "nc_ref_internal.h"
 
+/* every op takes its operands through nc_operand (nc_ref_ops.c): contiguous, bf16 widened */
+NCTensor *nc_operand(NCTensor *x);
+#define nc_contig(x) nc_operand(x)
+
 typedef struct {
     int H, dk, dv, B, T, M, K, d_pos, attn_len;
     float b_r_scale, scale;

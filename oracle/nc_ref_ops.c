@@ -9,6 +9,10 @@
 #include <stdio.h>
 #include "nc_ref_internal.h"
 
+/* every op takes its operands through nc_operand (below): contiguous, bf16 widened */
+NCTensor *nc_operand(NCTensor *x);
+#define nc_contig(x) nc_operand(x)
+
 /* ------------------------------------------------------------------------ */
 /* graph nodes                                                              */
 
@@ -277,13 +281,50 @@ static NCTensor *binary_op(NCTensor *a, NCTensor *b, NCOpEnum op)
 NCTensor *nc_add(NCTensor *x1, NCTensor *x2) { return binary_op(x1, x2, OP_ADD); } /* libnc.h:232 */
 NCTensor *nc_mul(NCTensor *x1, NCTensor *x2) { return binary_op(x1, x2, OP_MUL); } /* libnc.h:235 */
 
-/* libnc.h:231: only F32 exists in the checker (the bf16 variant of the
-   product keeps fp32 storage and rounds inside the matmul) */
+/* libnc.h:231.  Two item types carry values here: F32 and BF16 (2 bytes, the storage type of
+   parameters under nncp's bf16 switch, nncp.c:343-346).  Arithmetic is always F32: every op
+   widens a BF16 operand first (nc_operand, exact) and gives an F32 result; F32 -> BF16 rounds
+   to nearest even.  The gradient passes through a conversion unchanged, as F32. */
+static NCTensor *convert_to(NCTensor *x, NCTypeEnum new_type)
+{
+    NCTensor *y, *args[1];
+    NCNode *n;
+    size_t cnt;
+    x = (nc_contig)(x);
+    y = nc_alloc(x->dev, new_type, x->n_dims, x->dims, 0);
+    cnt = nc_numel(x);
+    if (new_type == NC_TYPE_F32) {
+        const uint16_t *src = (const uint16_t *)x->buf->data + x->off;
+        for (size_t i = 0; i < cnt; i++)
+            nc_f32(y)[i] = nc_bf16_widen(src[i]);
+    } else {
+        uint16_t *dst = (uint16_t *)y->buf->data + y->off;
+        for (size_t i = 0; i < cnt; i++)
+            dst[i] = nc_bf16_bits(nc_f32(x)[i]);
+    }
+    args[0] = x;
+    n = nc_new_node(x->dev->ctx, OP_CONVERT, 1, args);
+    y = finish(y, n, args, 1);
+    nc_free_tensor(x);
+    return y;
+}
+
 NCTensor *nc_convert(NCTensor *x, NCTypeEnum new_type)
 {
     if (x->type == new_type)
         return x;
-    nc_fatal("convert: only identity conversions are supported (%d -> %d)", x->type, new_type);
+    if ((x->type == NC_TYPE_BF16 && new_type == NC_TYPE_F32) ||
+        (x->type == NC_TYPE_F32 && new_type == NC_TYPE_BF16))
+        return convert_to(x, new_type);
+    nc_fatal("convert: %d -> %d is not supported (f32 and bf16 only)", x->type, new_type);
+}
+
+/* what every op does to an operand: contiguous, and F32 if it was BF16 (consumes x) */
+NCTensor *nc_operand(NCTensor *x)
+{
+    if (x->type == NC_TYPE_BF16)
+        return convert_to(x, NC_TYPE_F32);
+    return (nc_contig)(x);
 }
 
 /* libnc.h:242-244: y = mask ? c : x, mask broadcast over the trailing axes */
@@ -1241,6 +1282,9 @@ static void node_backward(NCNode *nd, NCTensor *g, NCTensor **ga)
             if (nd->parents[q]) ga[q] = r[q]; else nc_free_tensor(r[q]);
         break;
     }
+    case OP_CONVERT:
+        ga[0] = nc_dup_tensor(g);
+        break;
     case OP_RESHAPE:
         ga[0] = reshape_to(nc_dup_tensor(g), nd->arg_ndims[0], nd->arg_dims[0]);
         break;

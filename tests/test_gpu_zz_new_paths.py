@@ -285,3 +285,109 @@ def test_training_100_steps_match_checker(hosts, cfg_name):
                 assert M.rel_l2(w_h[k], w_r[k]) <= 1e-5 + own, (step, k, M.rel_l2(w_h[k], w_r[k]), own)
     hip.close()
     ref.close()
+
+
+# ---- parameters stored as bf16 (NC_TYPE_BF16, nncp.c:343-346) ------------------------------
+
+def test_bf16_conversions_on_the_gpu(hip):
+    """nc_convert f32 -> bf16 -> f32 on the device against torch's conversion, bit for bit
+    (ties, neighbours of ties, subnormals, infinities; NaN stays NaN)"""
+    import test_bf16_storage as S
+    S.check_conversions(hip, M.load_pkg().binding)
+
+
+@pytest.mark.parametrize("fused", [0, 1])
+def test_bf16_parameters_follow_the_f32_route_on_the_gpu(hosts, fused):
+    """One plain-SGD step of a model whose parameters are 2-byte tensors against the same model
+    with f32 parameters that start at the same bf16-representable values and bf16-operand
+    products: the same kernels meet the same operand bits, so probabilities and loss are equal,
+    the f32 model's new weights are the bf16 model's master values, and the bf16 parameters are
+    their rounding."""
+    import test_bf16_storage as S
+    B = M.load_pkg().binding
+    (pa, la, wa, ma), (pb, lb, wb), w0 = S.check_master_and_parameters_against_the_f32_route(hosts[0], 1, fused)
+    assert np.array_equal(pa, pb) and la == lb
+    for k in w0:
+        assert np.array_equal(ma[k], wb[k]), k
+        assert np.array_equal(wa[k], B.bf16_widen(B.bf16_bits(ma[k]))), k
+
+
+@pytest.mark.parametrize("fused,tol", [(0, 2e-2), (1, 2e-2)])
+def test_bf16_parameter_model_matches_checker(hosts, fused, tol):
+    """Four RMSProp steps with bf16 parameter storage, GPU against the checker (which emulates
+    the operand rounding of the products).  Op by op both sides round the same values at the
+    same places, but a value that fp32 noise carries across a rounding boundary changes an
+    operand (or a stored parameter) by a whole bf16 unit, 2^-8 of its size: the results agree
+    to 2e-7 on the smallest model and to a few 1e-3 here - not to fp32 accuracy - and most
+    stored parameters are equal bit for bit.  The fused evaluation rounds activations at other
+    places (product epilogues, attention operands).  One bar for both: the bf16 variant's 2e-2."""
+    hp = M.load_pkg().host
+    cfg = dict(M.C1, sgd_opt=M.rmsprop(3e-4), param_bf16=1)
+    Bs, T, V = cfg["batch_size"], cfg["seg_len"], cfg["n_symbols"]
+    batches = M.segment_batches(M.markov1(Bs * T * 4, V, seed=21), Bs, T, 4)
+    gpu = hp.Model(hosts[0], hp.make_config(**dict(cfg, fused=fused, use_device=1)))
+    ref = hp.Model(hosts[1], hp.make_config(**dict(cfg, fused=0, use_device=0, nb_threads=8)))
+    ref.nc.nc_set_matmul_bf16(ref.ctx, 1)
+    try:
+        for k, v in ref.params().items():
+            assert np.array_equal(gpu.get_param(k), v), k
+        for tok, tgt in batches:
+            ph, lh = gpu.train_step(tok, tgt, 3e-4)
+            pr, lr_ = ref.train_step(tok, tgt, 3e-4)
+            assert M.relerr(ph, pr) <= tol
+            assert abs(lh - lr_) <= tol * abs(lr_)
+        wh, wr = gpu.params(), ref.params()
+    finally:
+        ref.nc.nc_set_matmul_bf16(ref.ctx, 0)
+        gpu.close()
+        ref.close()
+    for k in wr:
+        if wr[k].ndim >= 2 and not k.startswith("b_r"):
+            assert M.rel_l2(wh[k], wr[k]) <= 2e-2, (k, M.rel_l2(wh[k], wr[k]))
+            if not fused:
+                assert (wh[k] == wr[k]).mean() > 0.75, (k, (wh[k] == wr[k]).mean())  # (w_r: sign-like updates of tiny gradients)
+
+
+def test_bf16_parameter_stream_round_trips_through_the_container(hosts, tmp_path):
+    """use_bf16 = 2 in the file header: encoder and decoder both build the model with bf16
+    parameters (the decoder learns it from the header), the file decodes to the input, and the
+    size is within 2 % of the f32-parameter bf16 variant's."""
+    hp = M.load_pkg().host
+    n = 200
+    mode = hp.MODE_SEGMENT | hp.CODER_CDF16
+    syms = M.markov1(n, 40, seed=17)
+    src = str(tmp_path / "in.bin")
+    syms.astype(np.uint8).tofile(src)
+    sizes = {}
+    for use_bf16 in (1, 2):
+        cfg = hp.make_config(**dict(M.TINY, fused=1, sgd_opt=M.rmsprop(), nb_threads=4, use_device=1))
+        fp = hp.file_params(hosts[0], "3e-4,8,1e-4", "96,200,120", use_bf16=use_bf16, mode=mode)
+        packed, back = str(tmp_path / ("out%d.nncp" % use_bf16)), str(tmp_path / ("back%d.bin" % use_bf16))
+        st, _ = hp.encode_file(hosts[0], src, packed, cfg, fp)
+        hp.decode_file(hosts[0], packed, back, use_device=1, nb_threads=4)
+        assert open(back, "rb").read() == open(src, "rb").read()
+        sizes[use_bf16] = os.path.getsize(packed)
+    assert abs(sizes[2] - sizes[1]) <= max(3, 0.02 * sizes[1]), sizes
+
+
+def test_bf16_parameter_files_cross_between_the_gpu_and_the_checker(hosts, tmp_path):
+    """bf16 records (2 bytes per element) written by the product library and read by the
+    checker's reader, and back: the same bytes"""
+    hp = M.load_pkg().host
+    cfg = dict(M.TINY, fused=1, sgd_opt=M.rmsprop(3e-3), param_bf16=1)
+    Bs, T = cfg["batch_size"], cfg["seg_len"]
+    gpu = hp.Model(hosts[0], hp.make_config(**dict(cfg, use_device=1)))
+    for tok, tgt in M.segment_batches(M.markov1(Bs * T * 3, cfg["n_symbols"], seed=5), Bs, T, 3):
+        gpu.train_step(tok, tgt, 3e-3)
+    gpu.save_coefs(str(tmp_path / "from_gpu.bin"))
+    ref = hp.Model(hosts[1], hp.make_config(**dict(cfg, fused=0, seed=7, use_device=0, nb_threads=2)))
+    ref.load_coefs(str(tmp_path / "from_gpu.bin"))
+    n = 0
+    for k in gpu.param_names():
+        assert np.array_equal(gpu.get_param(k), ref.get_param(k)), k
+        n += gpu.get_param(k).size
+    ref.save_coefs(str(tmp_path / "from_checker.bin"))
+    assert (tmp_path / "from_checker.bin").read_bytes() == (tmp_path / "from_gpu.bin").read_bytes()
+    assert os.path.getsize(str(tmp_path / "from_gpu.bin")) < 2 * n + 200 * len(gpu.param_names())
+    gpu.close()
+    ref.close()
