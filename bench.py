@@ -65,7 +65,7 @@ def measured_traffic(kernel, variant):
             read_mb, write_mb = float(parts[4]), float(parts[5])
         except ValueError:
             continue
-        if name.startswith(want) and name[len(want):len(want) + 1] in (",", ">"):
+        if name.startswith(want) and name[len(want):len(want) + 1] in ("", ",", ">"):
             found.append((read_mb + write_mb) * 1e6)
     if len(found) != 1:
         return None, None

@@ -192,7 +192,15 @@ def test_gemm_bf16_from_rounded_copies(hip, ref, rng, m, n, k, ta, tb):
                                  dict(H=2, dk=64, dv=64, B=3, T=64, M=256, d_pos=320, attn_len=320),
                                  dict(H=1, dk=64, dv=64, B=2, T=40, M=160, d_pos=40, attn_len=90),
                                  dict(H=2, dk=64, dv=64, B=2, T=64, M=140, d_pos=204, attn_len=204),
-                                 dict(H=2, dk=64, dv=64, B=2, T=17, M=283, d_pos=300, attn_len=150)])
+                                 dict(H=2, dk=64, dv=64, B=2, T=17, M=283, d_pos=300, attn_len=150),
+                                 # heads of 128 features (the enwik profile: 8 x 128, 64 + 256 keys): the
+                                 # chunked kernels with the feature axis in halves; 8, 12, 16, 20 key tiles
+                                 dict(H=2, dk=128, dv=128, B=3, T=64, M=256, d_pos=320, attn_len=320),
+                                 dict(H=2, dk=128, dv=128, B=2, T=64, M=64, d_pos=128, attn_len=128),
+                                 dict(H=2, dk=128, dv=128, B=2, T=32, M=20, d_pos=29, attn_len=25),
+                                 dict(H=1, dk=128, dv=128, B=2, T=40, M=160, d_pos=40, attn_len=90),
+                                 dict(H=2, dk=128, dv=128, B=2, T=48, M=116, d_pos=164, attn_len=100),
+                                 dict(H=3, dk=128, dv=128, B=1, T=7, M=49, d_pos=56, attn_len=56)])
 def test_relpos_attention_model_shapes(hip, ref, rng, cfg):
     H, dk, dv, B, T, M, d_pos = (cfg[k] for k in ("H", "dk", "dv", "B", "T", "M", "d_pos"))
     K = M + T
@@ -211,7 +219,7 @@ def test_relpos_attention_model_shapes(hip, ref, rng, cfg):
     assert relerr(res[0][0], res[1][0]) <= TOL
     for gh, gr in zip(res[0][1], res[1][1]):
         assert relerr(gh, gr) <= 5 * TOL
-    if dk == 64 and K % 4 == 0 and K <= 320:
+    if dk in (64, 128) and K % 4 == 0 and K <= 320:
         # these shapes take one kernel each way (plus the sum of the per-stream partials)
         lib = C.CDLL(hip.lib._name)
         assert lib.nchip_relpos_attn_last_launches() <= 2
