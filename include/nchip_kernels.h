@@ -261,6 +261,13 @@ int nchip_relpos_attn_fwd_step(void *stream, const float *q, int64_t ldq,
    counterpart in the reference. */
 void nchip_relpos_attn_step_kernel(int scalar);
 
+/* Heads of 128 features (nncp's enwik profile, nncp.c:2549): the forward is one kernel up to
+   320 keys; the backward is one kernel up to 128 keys and the batched products beyond, where
+   they are faster.  always = 1 makes the backward one kernel at every key count it holds
+   (tests; shapes with many more (stream, head) pairs than CUs).  Same results to rounding.
+   No counterpart in the reference. */
+void nchip_relpos_attn_wide_backward(int always);
+
 /* Kernel launches issued by the calling thread's last successful
    nchip_relpos_attn_fwd (1 when the head fits the single-kernel path). */
 int nchip_relpos_attn_last_launches(void);

@@ -1190,6 +1190,523 @@ void relpos_attn_bwd_tiled(FusedAttnBwdArgs a)
     }
 }
 
+// ---- heads of 128 features --------------------------------------------------------------
+// The chunked kernels again with the feature axis in halves of 64 (DK = 64 NH): a staging
+// tile holds 128 rows x 64 features, every chunk of w_r, K and V passes through it once per
+// half, and only Q (forward) or dO (backward, until its fragments are in registers) is held
+// at full width.  Contractions over the features (rel, scores, dA) chain through the halves:
+// the accumulator of half 1 starts from the result of half 0, so a 128-deep sum is formed in
+// the same order as one uninterrupted MFMA chain.  Products whose OUTPUT runs over the
+// features (O, dq, dK, dV, dw_r) simply own one set of accumulators per half.  The backward
+// fetches Q and dO again, one half at a time, for the key- and position-owned phase.
+template <int NTT>
+struct WideDims {
+    static_assert(NTT % 4 == 0 && NTT >= 8 && NTT <= 20, "8, 12, 16 or 20 key tiles");
+    static constexpr int NCH = (NTT + 7) / 8;       // chunks of up to 8 tiles
+    static constexpr int KP = NTT * 16;             // padded key / position count
+    static constexpr int RST = KP + 3;              // rel strip row
+    static constexpr int NB = 1024;                 // bias row incl. every index a masked key can form
+    static constexpr int tiles_of(int c) { return NTT - 8 * c < 8 ? NTT - 8 * c : 8; }
+};
+
+template <int NH, int NTT>
+struct FwdWideLayout {
+    using D = WideDims<NTT>;
+    static constexpr int RSQ = 64 * NH + 4, RS = 68;
+    static constexpr int q = 0, st = q + FA_TMAX * RSQ, r = st + 128 * RS, b = r + 4 * 16 * D::RST,
+                         floats = b + D::NB;
+};
+
+template <int NH, int NTT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void relpos_attn_fwd_wide(FusedAttnFwdArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    using L = FwdWideLayout<NH, NTT>;
+    using D = WideDims<NTT>;
+    constexpr int DK = 64 * NH, RSQ = L::RSQ, RS = L::RS, NS = 16, ND = 4, NCH = D::NCH, RST = D::RST,
+                  NI = 3 * NCH * NH;
+    float *Qs = lds + L::q, *Ss = lds + L::st, *Rs = lds + L::r, *Bs = lds + L::b;
+
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int b = blockIdx.x % a.B, h = blockIdx.x / a.B;
+    const int il = lane & 15, g = lane >> 4;
+    const int i = 16 * w + il;
+    const bool has_w = a.w_r != nullptr;
+    const float *w_base = has_w ? a.w_r + (int64_t)h * a.d_pos * DK : a.q;
+    const int n_w = has_w ? a.d_pos : 0;
+    auto kvrow = [&](int r) {
+        return (r < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * r)
+                        : a.kv + a.ldkv * (b + (int64_t)a.B * (r - a.M))) + (int64_t)h * DK;
+    };
+    // staging items in the order they are used: position chunks, key chunks, value chunks,
+    // each chunk once per feature half
+    floatx4_t vq[FA_TMAX * (DK / 4) / 256], vs[2][128 * 16 / 256];
+    auto rows_of = [&](int item) { // valid rows of the item's chunk
+        const int kind = item / (NCH * NH), c = (item / NH) % NCH, total = kind == 0 ? n_w : a.K;
+        const int left = total - 128 * c;
+        return left < 0 ? 0 : (left > 128 ? 128 : left);
+    };
+    auto fetch = [&](int item, floatx4_t (&v)[128 * 16 / 256]) {
+        const int kind = item / (NCH * NH), c = (item / NH) % NCH, hf = item % NH, nv = rows_of(item);
+        if (kind == 0) fetch_rows<64, 128>(v, nv, [&](int r) { return w_base + (int64_t)(nv ? r + 128 * c : 0) * DK + 64 * hf; });
+        else if (kind == 1) fetch_rows<64, 128>(v, nv, [&](int r) { return kvrow(nv ? r + 128 * c : 0) + 64 * hf; });
+        else fetch_rows<64, 128>(v, nv, [&](int r) { return kvrow(nv ? r + 128 * c : 0) + (int64_t)a.H * DK + 64 * hf; });
+    };
+    for (int e = t; e < D::NB; e += 256)
+        Bs[e] = (a.b_r && e < a.K) ? as_global(a.b_r)[(int64_t)h * a.K + e] * (a.b_r_scale * a.scale) : 0.0f;
+    fetch_rows<DK, FA_TMAX>(vq, a.T, [&](int r) { return a.q + (int64_t)h * DK + a.ldq * (b + (int64_t)a.B * r); });
+    fetch(0, vs[0]);
+    fetch(1, vs[1]);
+    put_rows<DK, FA_TMAX>(Qs, vq, a.T);
+
+    float qf[NH][NS];
+    float *Rw = Rs + (w * 16 + il) * RST; // this lane's column of rel
+    float sc[NTT][4];
+    float mx = -INFINITY;
+    floatx4_t oacc[NH * ND];
+#pragma unroll
+    for (int dt = 0; dt < NH * ND; dt++) oacc[dt] = floatx4_t{ 0, 0, 0, 0 };
+    const int dbase = i + a.M - 4 * g;      // delta of key 4g of tile 0
+    const int pbase = a.d_pos - 1 - dbase;  // its rel row before clamping
+    const int pmax = a.d_pos - 1;
+    const unsigned dlim = i < a.T ? (unsigned)a.attn_len : 0u;
+
+#pragma unroll
+    for (int item = 0; item < NI; item++) {
+        const int kind = item / (NCH * NH), c = (item / NH) % NCH, hf = item % NH;
+        if (item > 0) __syncthreads(); // every wavefront has left the staging tile
+        put_rows<64, 128>(Ss, vs[item & 1], rows_of(item));
+        if (item + 2 < NI) fetch(item + 2, vs[item & 1]);
+        __syncthreads();
+        if (item == 0) {
+#pragma unroll
+            for (int hh = 0; hh < NH; hh++)
+#pragma unroll
+                for (int s = 0; s < NS; s++) qf[hh][s] = Qs[i * RSQ + 64 * hh + 4 * s + g] * a.scale; // 1/sqrt(dk) folded in
+        }
+        const int nt = D::tiles_of(c);
+        if (kind == 0) {
+            // rel = w_r^T q for the positions of this chunk -> strip (half 1 continues half 0's sums)
+            float af[2][NS];
+            load_afrag<NS>(af[0], Ss + il * RS + g);
+#pragma unroll
+            for (int pt = 0; pt < 8; pt++) {
+                if (pt >= nt) break;
+                if (pt + 1 < nt) load_afrag<NS>(af[(pt + 1) & 1], Ss + ((pt + 1) * 16 + il) * RS + g);
+                float *rw = Rw + (8 * c + pt) * 16 + 4 * g;
+                floatx4_t acc = { 0, 0, 0, 0 };
+                if (hf > 0) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[r] = rw[r]; // written by this lane in the half before
+                }
+                PIPELINE_FENCE();
+#pragma unroll
+                for (int s = 0; s < NS; s++) acc = mfma16(af[pt & 1][s], qf[hf][s], acc);
+#pragma unroll
+                for (int r = 0; r < 4; r++) rw[r] = acc[r];
+            }
+            if (c == NCH - 1 && hf == NH - 1) wave_lds_sync();
+        } else if (kind == 1) {
+            float af[2][NS];
+            load_afrag<NS>(af[0], Ss + il * RS + g);
+#pragma unroll
+            for (int jl = 0; jl < 8; jl++) {
+                if (jl >= nt) break;
+                const int jt = 8 * c + jl;
+                if (jl + 1 < nt) load_afrag<NS>(af[(jl + 1) & 1], Ss + ((jl + 1) * 16 + il) * RS + g);
+                PIPELINE_FENCE();
+                floatx4_t acc = { 0, 0, 0, 0 };
+                if (hf > 0) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[r] = sc[jt][r];
+                }
+#pragma unroll
+                for (int s = 0; s < NS; s++) acc = mfma16(af[jl & 1][s], qf[hf][s], acc);
+                if (hf < NH - 1) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) sc[jt][r] = acc[r];
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const unsigned delta = (unsigned)(dbase - (jt * 16 + r));
+                        int pi = pbase + (jt * 16 + r); // d_pos-1-delta
+                        pi = pi < 0 ? 0 : (pi > pmax ? pmax : pi);
+                        const float relv = Rw[pi];
+                        const float bv = Bs[(a.K - 1 - (int)delta) & (D::NB - 1)];
+                        float v = delta < dlim ? acc[r] + relv + bv : -INFINITY;
+                        sc[jt][r] = v;
+                        mx = fmaxf(mx, v);
+                    }
+                }
+            }
+            if (c == NCH - 1 && hf == NH - 1) {
+                // softmax over all keys of the column (lanes l, l^16, l^32, l^48 share it)
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                if (mx == -INFINITY) mx = 0.0f; // padding column
+                float sum = 0.0f;
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float e = __expf(sc[jt][r] - mx); // exp(-inf) = 0 for masked keys
+                        sc[jt][r] = e;
+                        sum += e;
+                    }
+                sum += __shfl_xor(sum, 16, 64);
+                sum += __shfl_xor(sum, 32, 64);
+                float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) sc[jt][r] *= inv;
+                if (a.probs && i < a.T) {
+                    float NCHIP_GLOBAL *pc = as_global(a.probs) + (((int64_t)b * a.H + h) * a.T + i) * a.K;
+#pragma unroll
+                    for (int jt = 0; jt < NTT; jt++) {
+                        int j0 = jt * 16 + 4 * g;
+                        if (j0 < a.K) { // K is a multiple of 4: whole quads
+                            floatx4_t v = { sc[jt][0], sc[jt][1], sc[jt][2], sc[jt][3] };
+                            *reinterpret_cast<floatx4_t NCHIP_GLOBAL *>(pc + j0) = v;
+                        }
+                    }
+                }
+            }
+        } else {
+            // O[:, half] += V[:, half] P over the keys of this chunk
+            float vf[2][ND][4];
+            load_tokfrag<ND, RS>(vf[0], Ss, 0, g, il);
+#pragma unroll
+            for (int jl = 0; jl < 8; jl++) {
+                if (jl >= nt) break;
+                const int jt = 8 * c + jl;
+                if (jl + 1 < nt) load_tokfrag<ND, RS>(vf[(jl + 1) & 1], Ss, jl + 1, g, il);
+                PIPELINE_FENCE();
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int dt = 0; dt < ND; dt++)
+                        oacc[hf * ND + dt] = mfma16(vf[jl & 1][dt][r], sc[jt][r], oacc[hf * ND + dt]);
+            }
+        }
+    }
+    if (i < a.T) {
+#pragma unroll
+        for (int dt = 0; dt < NH * ND; dt++) {
+            float NCHIP_GLOBAL *o = as_global(a.out) + (int64_t)h * DK + dt * 16 + 4 * g + a.ldo * (b + (int64_t)a.B * i);
+            *reinterpret_cast<floatx4_t NCHIP_GLOBAL *>(o) = oacc[dt];
+        }
+    }
+}
+
+template <int NH, int NTT>
+struct BwdWideLayout {
+    using D = WideDims<NTT>;
+    static constexpr int RSQ = 64 * NH + 4, RS = 68;
+    // x: dO at full width until its fragments are in registers, then one half of Q and of dO
+    static constexpr int xsz = FA_TMAX * RSQ > 2 * FA_TMAX * RS ? FA_TMAX * RSQ : 2 * FA_TMAX * RS;
+    static_assert(2 * 64 * FA_PSTRIDE <= 128 * RS, "the transposed P / dS tiles of 64 keys fit in the staging tile");
+    static constexpr int x = 0, st = x + xsz, r = st + 128 * RS, floats = r + FA_TMAX * D::RST;
+};
+
+template <int NH, int NTT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void relpos_attn_bwd_wide(FusedAttnBwdArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    using L = BwdWideLayout<NH, NTT>;
+    using D = WideDims<NTT>;
+    constexpr int DK = 64 * NH, RSQ = L::RSQ, RS = L::RS, NS = 16, ND = 4, NCH = D::NCH, RST = D::RST,
+                  NI = 3 * NCH * NH, PS = FA_PSTRIDE;
+    constexpr int NSQ = FA_TMAX / 4, KP = D::KP;
+    float *Xs = lds + L::x, *Ss = lds + L::st, *Rs = lds + L::r;
+    float *Qh = Xs, *Oh = Xs + FA_TMAX * RS; // [64 queries][RS] each, one feature half
+    float *Pt = Ss, *St = Ss + 64 * PS;      // [64 keys][PS] each
+
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int b = blockIdx.x % a.B, h = blockIdx.x / a.B;
+    const bool has_w = a.w_r != nullptr;
+    const int il = lane & 15, g = lane >> 4;
+    const int i = 16 * w + il;
+    const float *w_base = has_w ? a.w_r + (int64_t)h * a.d_pos * DK : a.q;
+    const int n_w = has_w ? a.d_pos : 0;
+    auto kvrow = [&](int r) {
+        return (r < a.M ? a.kvm + a.ldkv * (b + (int64_t)a.B * r)
+                        : a.kv + a.ldkv * (b + (int64_t)a.B * (r - a.M))) + (int64_t)h * DK;
+    };
+    // staging items: value chunks (dA), key chunks (dq), position chunks (dq), once per half
+    floatx4_t vo[FA_TMAX * (DK / 4) / 256], vs[2][128 * 16 / 256];
+    auto rows_of = [&](int item) {
+        const int kind = item / (NCH * NH), c = (item / NH) % NCH, total = kind < 2 ? a.K : n_w;
+        const int left = total - 128 * c;
+        return left < 0 ? 0 : (left > 128 ? 128 : left);
+    };
+    auto fetch = [&](int item, floatx4_t (&v)[128 * 16 / 256]) {
+        const int kind = item / (NCH * NH), c = (item / NH) % NCH, hf = item % NH, nv = rows_of(item);
+        if (kind == 0) fetch_rows<64, 128>(v, nv, [&](int r) { return kvrow(nv ? r + 128 * c : 0) + (int64_t)a.H * DK + 64 * hf; });
+        else if (kind == 1) fetch_rows<64, 128>(v, nv, [&](int r) { return kvrow(nv ? r + 128 * c : 0) + 64 * hf; });
+        else fetch_rows<64, 128>(v, nv, [&](int r) { return w_base + (int64_t)(nv ? r + 128 * c : 0) * DK + 64 * hf; });
+    };
+    float p[NTT][4], ds[NTT][4];
+    fetch_rows<DK, FA_TMAX>(vo, a.T, [&](int r) { return a.dout + (int64_t)h * DK + a.ldo * (b + (int64_t)a.B * r); });
+    fetch(0, vs[0]);
+    {
+        const float NCHIP_GLOBAL *pc = as_global(a.probs) + (((int64_t)b * a.H + h) * a.T + (i < a.T ? i : 0)) * a.K;
+#pragma unroll
+        for (int jt = 0; jt < NTT; jt++) { // unconditional loads from clamped addresses; masked at first use
+            int j0 = jt * 16 + 4 * g;
+            floatx4_t v = *reinterpret_cast<const floatx4_t NCHIP_GLOBAL *>(pc + (j0 < a.K ? j0 : 0));
+#pragma unroll
+            for (int r = 0; r < 4; r++) p[jt][r] = v[r];
+        }
+    }
+    fetch(1, vs[1]);
+    put_rows<DK, FA_TMAX>(Xs, vo, a.T);
+
+    float dof[NH][NS];
+    float dot = 0.0f;
+    float *Rw = Rs + i * RST;
+    floatx4_t dqa[NH * ND];
+#pragma unroll
+    for (int dt = 0; dt < NH * ND; dt++) dqa[dt] = floatx4_t{ 0, 0, 0, 0 };
+
+#pragma unroll
+    for (int item = 0; item < NI; item++) {
+        const int kind = item / (NCH * NH), c = (item / NH) % NCH, hf = item % NH;
+        if (item > 0) __syncthreads(); // every wavefront has left the staging tile
+        put_rows<64, 128>(Ss, vs[item & 1], rows_of(item));
+        if (item + 2 < NI) fetch(item + 2, vs[item & 1]);
+        __syncthreads();
+        const int nt = D::tiles_of(c);
+        if (kind == 0) {
+            if (item == 0) {
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        p[jt][r] = (i < a.T && jt * 16 + 4 * g + r < a.K) ? p[jt][r] : 0.0f;
+#pragma unroll
+                for (int hh = 0; hh < NH; hh++)
+#pragma unroll
+                    for (int s = 0; s < NS; s++) dof[hh][s] = Xs[i * RSQ + 64 * hh + 4 * s + g];
+            }
+            // dA = V^T dO for the keys of this chunk (half 1 continues half 0's sums)
+            float af[2][NS];
+            load_afrag<NS>(af[0], Ss + il * RS + g);
+#pragma unroll
+            for (int jl = 0; jl < 8; jl++) {
+                if (jl >= nt) break;
+                const int jt = 8 * c + jl;
+                if (jl + 1 < nt) load_afrag<NS>(af[(jl + 1) & 1], Ss + ((jl + 1) * 16 + il) * RS + g);
+                PIPELINE_FENCE();
+                floatx4_t acc = { 0, 0, 0, 0 };
+                if (hf > 0) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[r] = ds[jt][r];
+                }
+#pragma unroll
+                for (int s = 0; s < NS; s++) acc = mfma16(af[jl & 1][s], dof[hf][s], acc);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    ds[jt][r] = acc[r];
+                    if (hf == NH - 1) dot += p[jt][r] * acc[r];
+                }
+            }
+            if (c == NCH - 1 && hf == NH - 1) {
+                // dS = P (dA - colsum(P dA)) / sqrt(dk), then its rel-shift adjoint into the strip
+                dot += __shfl_xor(dot, 16, 64);
+                dot += __shfl_xor(dot, 32, 64);
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) ds[jt][r] = p[jt][r] * (ds[jt][r] - dot) * a.scale; // masked: p = 0
+                for (int pp = g; pp < KP; pp += 4) Rw[pp] = 0.0f;
+                wave_lds_sync();
+                const int dbase = i + a.M - 4 * g, pbase = a.d_pos - 1 - dbase;
+                const unsigned dlim = (i < a.T && has_w) ? (unsigned)a.attn_len : 0u;
+                float acc0 = 0.0f;
+#pragma unroll
+                for (int jt = 0; jt < NTT; jt++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        unsigned delta = (unsigned)(dbase - (jt * 16 + r));
+                        int pi = pbase + (jt * 16 + r);
+                        // rows >= 1 receive exactly one key; row 0 collects the far keys;
+                        // masked keys go to a dump slot past the strip (never read)
+                        const bool on = delta < dlim;
+                        Rw[(on && pi >= 1) ? pi : RST - 1] = ds[jt][r];
+                        acc0 += (on && pi < 1) ? ds[jt][r] : 0.0f;
+                    }
+                acc0 += __shfl_xor(acc0, 16, 64);
+                acc0 += __shfl_xor(acc0, 32, 64);
+                if (g == 0) Rw[0] = acc0;
+                wave_lds_sync();
+            }
+        } else {
+            // dq[:, half] += K[:, half] dS (kind 1) or w_r[:, half] dRel (kind 2) over the rows of this chunk
+            float kf[2][ND][4], rf[2][4];
+            load_tokfrag<ND, RS>(kf[0], Ss, 0, g, il);
+            if (kind == 2) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) rf[0][r] = Rw[(8 * c) * 16 + 4 * g + r];
+            }
+#pragma unroll
+            for (int jl = 0; jl < 8; jl++) {
+                if (jl >= nt) break;
+                const int jt = 8 * c + jl;
+                if (jl + 1 < nt) {
+                    load_tokfrag<ND, RS>(kf[(jl + 1) & 1], Ss, jl + 1, g, il);
+                    if (kind == 2) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) rf[(jl + 1) & 1][r] = Rw[(jt + 1) * 16 + 4 * g + r];
+                    }
+                }
+                PIPELINE_FENCE();
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int dt = 0; dt < ND; dt++)
+                        dqa[hf * ND + dt] = mfma16(kf[jl & 1][dt][r], kind == 1 ? ds[jt][r] : rf[jl & 1][r], dqa[hf * ND + dt]);
+            }
+        }
+    }
+    if (i < a.T) {
+#pragma unroll
+        for (int dt = 0; dt < NH * ND; dt++) {
+            float *o = a.dq + (int64_t)h * DK + dt * 16 + 4 * g + a.ldq * (b + (int64_t)a.B * i);
+            *reinterpret_cast<floatx4_t *>(o) = dqa[dt];
+        }
+    }
+
+    // the contraction now runs over the query index; k-slot g of step s is
+    // query 16*(s/4) + 4g + s%4, which keeps the Q / dO reads conflict-free
+    auto load_qd = [&](float (&f)[ND], const float *base, int s) {
+        int iq = 16 * (s >> 2) + 4 * g + (s & 3);
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++) f[dt] = base[iq * RS + dt * 16 + il];
+    };
+    float dbacc[2] = { 0.0f, 0.0f };
+#pragma unroll
+    for (int hf = 0; hf < NH; hf++) {
+        // this half of Q and dO into x (dO's full-width copy went into registers long ago; with
+        // hf > 0 every wavefront must have left the half before)
+        floatx4_t vqh[FA_TMAX * 16 / 256], voh[FA_TMAX * 16 / 256];
+        fetch_rows<64, FA_TMAX>(vqh, a.T, [&](int r) { return a.q + (int64_t)h * DK + 64 * hf + a.ldq * (b + (int64_t)a.B * r); });
+        fetch_rows<64, FA_TMAX>(voh, a.T, [&](int r) { return a.dout + (int64_t)h * DK + 64 * hf + a.ldo * (b + (int64_t)a.B * r); });
+        __syncthreads();
+        put_rows<64, FA_TMAX>(Qh, vqh, a.T);
+        put_rows<64, FA_TMAX>(Oh, voh, a.T);
+        // dK = Q dS^T, dV = dO P^T, 64 keys at a time: wavefront w owns key tile 4*hc + w;
+        // db_r (first half only): thread t sums the diagonals delta = t and t + 256 over the parked keys
+#pragma unroll
+        for (int hc = 0; hc < NTT / 4; hc++) {
+            __syncthreads(); // the staging tile (or the previous 64 keys) is dead
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int jl = e * 16 + 4 * g + r;
+                    Pt[jl * PS + i] = p[4 * hc + e][r];
+                    St[jl * PS + i] = ds[4 * hc + e][r];
+                }
+            __syncthreads();
+            {
+                float sb[NSQ], pb[NSQ];
+#pragma unroll
+                for (int s = 0; s < NSQ; s++) {
+                    int iq = 16 * (s >> 2) + 4 * g + (s & 3);
+                    sb[s] = St[(w * 16 + il) * PS + iq];
+                    pb[s] = Pt[(w * 16 + il) * PS + iq];
+                }
+                floatx4_t ak[ND], av[ND];
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++) { ak[dt] = floatx4_t{ 0, 0, 0, 0 }; av[dt] = floatx4_t{ 0, 0, 0, 0 }; }
+                float qa[2][ND], oa[2][ND];
+                load_qd(qa[0], Qh, 0);
+                load_qd(oa[0], Oh, 0);
+#pragma unroll
+                for (int s = 0; s < NSQ; s++) {
+                    if (s + 1 < NSQ) { load_qd(qa[(s + 1) & 1], Qh, s + 1); load_qd(oa[(s + 1) & 1], Oh, s + 1); }
+                    PIPELINE_FENCE();
+#pragma unroll
+                    for (int dt = 0; dt < ND; dt++) {
+                        ak[dt] = mfma16(qa[s & 1][dt], sb[s], ak[dt]);
+                        av[dt] = mfma16(oa[s & 1][dt], pb[s], av[dt]);
+                    }
+                }
+                const int j = (4 * hc + w) * 16 + il;
+                if (j < a.K) {
+                    float *dst = (j < a.M ? a.dkvm + a.ldkv * (b + (int64_t)a.B * j)
+                                          : a.dkv + a.ldkv * (b + (int64_t)a.B * (j - a.M))) + (int64_t)h * DK + 64 * hf;
+#pragma unroll
+                    for (int dt = 0; dt < ND; dt++) {
+                        *reinterpret_cast<floatx4_t *>(dst + dt * 16 + 4 * g) = ak[dt];
+                        *reinterpret_cast<floatx4_t *>(dst + (int64_t)a.H * DK + dt * 16 + 4 * g) = av[dt];
+                    }
+                }
+            }
+            if (hf == 0 && a.dbp) {
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const int delta = t + 256 * u;
+                    // keys 64*hc .. 64*hc+63 of diagonal delta belong to queries lo .. lo+63
+                    const int lo = delta - a.M + 64 * hc;
+                    float acc = 0.0f;
+#pragma unroll 8
+                    for (int q8 = 0; q8 < 64; q8++) {
+                        const int iq = lo + q8;
+                        const bool on = delta < a.K && iq >= 0 && iq < a.T && 64 * hc + q8 < a.K;
+                        float v = St[(on ? q8 : 0) * PS + (on ? iq : 0)];
+                        acc += on ? v : 0.0f;
+                    }
+                    dbacc[u] += acc;
+                }
+            }
+        }
+        // dw_r partial of this (stream, head), this half: Q dRel^T, wavefront w owns position tiles w, w+4, ...
+        if (has_w) {
+            float *dwz = a.dwp + ((int64_t)b * a.H + h) * a.d_pos * DK + 64 * hf;
+#pragma unroll
+            for (int u = 0; u < NTT / 4; u++) {
+                const int pt = w + 4 * u;
+                float rb[NSQ];
+#pragma unroll
+                for (int s = 0; s < NSQ; s++) {
+                    int iq = 16 * (s >> 2) + 4 * g + (s & 3);
+                    rb[s] = Rs[iq * RST + pt * 16 + il];
+                }
+                floatx4_t acc[ND];
+#pragma unroll
+                for (int dt = 0; dt < ND; dt++) acc[dt] = floatx4_t{ 0, 0, 0, 0 };
+                float qa[2][ND];
+                load_qd(qa[0], Qh, 0);
+#pragma unroll
+                for (int s = 0; s < NSQ; s++) {
+                    if (s + 1 < NSQ) load_qd(qa[(s + 1) & 1], Qh, s + 1);
+                    PIPELINE_FENCE();
+#pragma unroll
+                    for (int dt = 0; dt < ND; dt++) acc[dt] = mfma16(qa[s & 1][dt], rb[s], acc[dt]);
+                }
+                const int pp = pt * 16 + il;
+                if (pp < a.d_pos) {
+#pragma unroll
+                    for (int dt = 0; dt < ND; dt++)
+                        *reinterpret_cast<floatx4_t *>(dwz + (int64_t)pp * DK + dt * 16 + 4 * g) = acc[dt];
+                }
+            }
+        }
+    }
+    if (a.dbp) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int delta = t + 256 * u;
+            if (delta < a.K)
+                a.dbp[((int64_t)b * a.H + h) * a.K + (a.K - 1 - delta)] = a.b_r_scale * dbacc[u];
+        }
+    }
+}
+
 // ---- one query per (stream, head): the decoder's timestep ---------------------------------
 // The single query of a timestep through the arithmetic of relpos_attn_fwd_fused, on the
 // vector ALUs.  An fp32 MFMA accumulates its k values one after the other with fused
@@ -1334,6 +1851,7 @@ __global__ __launch_bounds__(512) void relpos_attn_step_scalar(FusedAttnFwdArgs 
 }
 
 int g_attn_step_scalar = 1; // 0: single-query calls go through the whole-segment kernel (testing aid)
+int g_attn_wide_bwd = 0;    // 1: heads of 128 take the single-kernel backward at every key count
 
 template <typename KernelT>
 bool allow_lds(KernelT kern, size_t bytes)
@@ -1406,6 +1924,37 @@ int launch_bwd_tiled(hipStream_t st, const FusedAttnBwdArgs &a)
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
+template <int NH, int NTT>
+int launch_fwd_wide(hipStream_t st, const FusedAttnFwdArgs &a)
+{
+    constexpr size_t bytes = sizeof(float) * FwdWideLayout<NH, NTT>::floats;
+    static_assert(bytes <= 160 * 1024, "forward tiles exceed LDS");
+    static const bool ok = allow_lds(relpos_attn_fwd_wide<NH, NTT>, bytes);
+    if (!ok) return -1;
+    hipLaunchKernelGGL((relpos_attn_fwd_wide<NH, NTT>), dim3(a.B * a.H), dim3(256), bytes, st, a);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <int NH, int NTT>
+int launch_bwd_wide(hipStream_t st, const FusedAttnBwdArgs &a)
+{
+    constexpr size_t bytes = sizeof(float) * BwdWideLayout<NH, NTT>::floats;
+    static_assert(bytes <= 160 * 1024, "backward tiles exceed LDS");
+    static const bool ok = allow_lds(relpos_attn_bwd_wide<NH, NTT>, bytes);
+    if (!ok) return -1;
+    hipLaunchKernelGGL((relpos_attn_bwd_wide<NH, NTT>), dim3(a.B * a.H), dim3(256), bytes, st, a);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// 16-key tiles the kernels for heads of 128 need for K keys and d_pos positions (0: not their shape)
+int wide_ntt(int K, int d_pos)
+{
+    const int need = K > d_pos ? K : d_pos;
+    int ntt = ((need + 15) / 16 + 3) / 4 * 4;
+    if (ntt < 8) ntt = 8;
+    return (ntt <= 20 && (K & 3) == 0) ? ntt : 0;
+}
+
 // 16-key tiles the chunked kernels need for K keys and d_pos positions (0: not their shape)
 int tiled_ntt(int K, int d_pos)
 {
@@ -1424,6 +1973,7 @@ bool k_attn_fused_step_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr)
 bool k_attn_fused_shape_ok(int dk, int dv, int T, int K, int d_pos, bool has_wr)
 {
     if (k_attn_fused_step_ok(dk, dv, T, K, d_pos, has_wr)) return true;
+    if (dk == 128 && dv == 128) return T <= FA_TMAX && wide_ntt(K, has_wr ? d_pos : 1) != 0;
     return dk == 64 && dv == 64 && T <= FA_TMAX && tiled_ntt(K, has_wr ? d_pos : 1) != 0;
 }
 
@@ -1434,12 +1984,26 @@ extern "C" void nchip_relpos_attn_step_kernel(int scalar)
     g_attn_step_scalar = scalar;
 }
 
+// 1: the backward of heads of 128 features runs as one kernel for every key count it holds
+// (up to 320); 0 (default): only up to 128 keys, beyond that the batched products, which
+// are faster there.  Same results to rounding either way.
+extern "C" void nchip_relpos_attn_wide_backward(int always)
+{
+    g_attn_wide_bwd = always;
+}
+
 int k_attn_fused_fwd(hipStream_t st, const FusedAttnFwdArgs &a, int dk)
 {
     if (a.q_only >= 0 && g_attn_step_scalar && a.K <= 128 && a.d_pos <= 128 && !a.probs) {
         if (dk == 64) hipLaunchKernelGGL(relpos_attn_step_scalar<64>, dim3(a.B * a.H), dim3(512), 0, st, a);
         else hipLaunchKernelGGL(relpos_attn_step_scalar<32>, dim3(a.B * a.H), dim3(512), 0, st, a);
         return hipGetLastError() == hipSuccess ? 0 : -1;
+    }
+    if (dk == 128) {
+        const int ntt = wide_ntt(a.K, a.d_pos);
+        if (!ntt || a.T > FA_TMAX || a.q_only >= 0 || !a.probs || !probs_vec(a)) return -1;
+        return ntt == 8 ? launch_fwd_wide<2, 8>(st, a) : ntt == 12 ? launch_fwd_wide<2, 12>(st, a)
+             : ntt == 16 ? launch_fwd_wide<2, 16>(st, a) : launch_fwd_wide<2, 20>(st, a);
     }
     if (const int ntt = (a.K > 128 || a.d_pos > 128) ? tiled_ntt(a.K, a.d_pos) : 0) {
         if (dk != 64 || a.q_only >= 0 || !a.probs || !probs_vec(a)) return -1;
@@ -1457,7 +2021,18 @@ int k_attn_fused_bwd(hipStream_t st, const FusedAttnBwdArgs &a, int dk, float *d
 {
     const bool small = a.K <= 64 && a.d_pos <= 64;
     int rc;
-    if (a.K > 128 || a.d_pos > 128) {
+    if (dk == 128) {
+        const int ntt = wide_ntt(a.K, a.d_pos);
+        if (!ntt || a.T > FA_TMAX || !probs_vec(a)) return -1;
+        // Measured at 8 heads x 32 streams (one workgroup per CU): up to 128 keys this kernel and
+        // the batched-product backward take the same time (123 us); at 320 keys the batched
+        // products are faster (228 us against 340-390 us: this kernel keeps one wavefront per
+        // SIMD busy with 36 staged tiles and two passes over the key-owned phase), so they
+        // take those shapes unless the caller asks for this kernel.
+        if (ntt > 8 && !g_attn_wide_bwd) return -1;
+        rc = ntt == 8 ? launch_bwd_wide<2, 8>(st, a) : ntt == 12 ? launch_bwd_wide<2, 12>(st, a)
+           : ntt == 16 ? launch_bwd_wide<2, 16>(st, a) : launch_bwd_wide<2, 20>(st, a);
+    } else if (a.K > 128 || a.d_pos > 128) {
         const int ntt = tiled_ntt(a.K, a.d_pos);
         if (!ntt || dk != 64 || !probs_vec(a)) return -1;
         rc = ntt == 12 ? launch_bwd_tiled<64, 12>(st, a) : ntt == 16 ? launch_bwd_tiled<64, 16>(st, a)

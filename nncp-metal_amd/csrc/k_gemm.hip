@@ -90,9 +90,16 @@ struct GemmArgs {
 
 __device__ __forceinline__ float gelu_tanh(float x) { return nchip_gelu(x); } // k_act.h
 
+// GELU of the products that round their operands to bf16: the launchers turn NCHIP_ACT_GELU
+// into this code when the precision argument is not fp32 (k_act.h says why there are two)
+constexpr int ACT_GELU_FAST = 3;
+static_assert(ACT_GELU_FAST != NCHIP_ACT_NONE && ACT_GELU_FAST != NCHIP_ACT_GELU && ACT_GELU_FAST != NCHIP_ACT_RELU, "");
+inline int act_for_precision(int act, int precision) { return (act == NCHIP_ACT_GELU && precision != 0) ? ACT_GELU_FAST : act; }
+
 __device__ __forceinline__ float act_grad(float x, int act)
 {
     if (act == NCHIP_ACT_GELU) return nchip_gelu_grad(x);
+    if (act == ACT_GELU_FAST) return nchip_gelu_grad_fast(x);
     if (act == NCHIP_ACT_RELU) return x > 0.0f ? 1.0f : 0.0f;
     return 1.0f;
 }
@@ -100,6 +107,7 @@ __device__ __forceinline__ float act_grad(float x, int act)
 __device__ __forceinline__ float apply_act(float v, int act)
 {
     if (act == NCHIP_ACT_GELU) return gelu_tanh(v);
+    if (act == ACT_GELU_FAST) return nchip_gelu_fast(v);
     if (act == NCHIP_ACT_RELU) return v > 0.0f ? v : 0.0f;
     return v;
 }
@@ -395,6 +403,9 @@ __device__ __forceinline__ void epilogue_tile(const GemmArgs &g, const floatx16 
     if (g.act == NCHIP_ACT_GELU) {
 #pragma unroll
         for (int r = 0; r < 16; r++) v[r] = gelu_tanh(v[r]);
+    } else if (g.act == ACT_GELU_FAST) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) v[r] = nchip_gelu_fast(v[r]);
     } else if (g.act == NCHIP_ACT_RELU) {
 #pragma unroll
         for (int r = 0; r < 16; r++) v[r] = v[r] > 0.0f ? v[r] : 0.0f;
@@ -660,8 +671,7 @@ __global__ __launch_bounds__(256) void gemm_fewcol_fma(GemmArgs g)
     }
     v = g.alpha * v + bv;
     if (P) P[(int64_t)col * g.ldc + row] = v;
-    if (g.act == NCHIP_ACT_GELU) v = gelu_tanh(v);
-    else if (g.act == NCHIP_ACT_RELU) v = v > 0.0f ? v : 0.0f;
+    v = apply_act(v, g.act);
     *Cp = v + extra;
 }
 
@@ -841,8 +851,7 @@ __global__ __launch_bounds__(256) void gemm_fewcol_mfma(GemmArgs g)
     }
     float v = g.alpha * sum + bv;
     if (P) P[(int64_t)col * g.ldc + row] = v;
-    if (g.act == NCHIP_ACT_GELU) v = gelu_tanh(v);
-    else if (g.act == NCHIP_ACT_RELU) v = v > 0.0f ? v : 0.0f;
+    v = apply_act(v, g.act);
     *Cp = v + extra;
 }
 
@@ -1583,14 +1592,14 @@ static int gemm2_impl(void *stream, int ta, int tb, int m, int n, int k, float a
     GemmArgs g;
     memset(&g, 0, sizeof(g));
     g.A = A; g.B = B; g.C = C; g.bias = bias; g.add = addend; g.pre = pre; g.ws = workspace;
-    g.dpre = dpre; g.dact = dact;
+    g.dpre = dpre; g.dact = act_for_precision(dact, precision);
     g.rowsum = nullptr;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.sa = sa_out; g.sb = sb_out; g.sc = sc_out;
     g.sa_in = sa_in; g.sb_in = sb_in; g.sc_in = sc_in; g.batch_in = batch_in;
     g.M = m; g.N = n; g.K = k; g.batch = batch; g.ksplit = ksplit;
     g.kchunk = ((k + ksplit - 1) / ksplit + KALIGN - 1) / KALIGN * KALIGN;
     if (g.kchunk < KALIGN) g.kchunk = KALIGN;
-    g.alpha = alpha; g.beta = beta; g.act = act;
+    g.alpha = alpha; g.beta = beta; g.act = act_for_precision(act, precision);
     g.grp = nullptr; g.n_grp = 0;
     hipStream_t st = (hipStream_t)stream;
     // tile choice from the shape only: large tiles when they still fill the chip
@@ -1946,10 +1955,10 @@ extern "C" int nchip_gemm_bf16_operands(void *stream, const NchipGemmBf16Args *a
     memset(&g, 0, sizeof(g));
     g.A = reinterpret_cast<const float *>(a->A16); g.B = reinterpret_cast<const float *>(a->B16);
     g.C = a->C; g.c16 = a->C16; g.bias = a->bias; g.add = a->addend; g.pre = a->pre;
-    g.dpre = a->dpre; g.dact = a->dact;
+    g.dpre = a->dpre; g.dact = act_for_precision(a->dact, 2);
     g.lda = a->lda; g.ldb = a->ldb; g.ldc = a->ldc;
     g.batch_in = 1; g.M = m; g.N = n; g.K = k; g.batch = 1; g.ksplit = 1; g.kchunk = k;
-    g.alpha = a->alpha; g.beta = 0.0f; g.act = a->act;
+    g.alpha = a->alpha; g.beta = 0.0f; g.act = act_for_precision(a->act, 2);
     hipStream_t st = (hipStream_t)stream;
     // tile class from the tile counts: the largest tile that still gives every CU a workgroup
     const int64_t t128 = (int64_t)((m + 127) / 128) * ((n + 127) / 128);

@@ -1166,7 +1166,9 @@ extern "C" NCTensor *nc_relpos_attention(NCTensor *q, NCTensor *kv, NCTensor *kv
     bool on_bf16 = false;
     NCTensor *probs = nullptr;
     static const bool bf16_attn_off = getenv("NCHIP_BF16_ATTENTION") && atoi(getenv("NCHIP_BF16_ATTENTION")) == 0;
-    if (m->matmul_bf16 && !bf16_attn_off && k_attn_bf16_shape_ok(a.dk, a.dv, a.T, a.K, a.d_pos, all[3] != nullptr) &&
+    // (not in width-invariant mode: there the per-timestep decoder must find the bits of this
+    // whole-segment evaluation, and its one-query kernel computes in fp32)
+    if (m->matmul_bf16 && !m->matmul_invariant && !bf16_attn_off && k_attn_bf16_shape_ok(a.dk, a.dv, a.T, a.K, a.d_pos, all[3] != nullptr) &&
         all[0]->dims[0] % 8 == 0 && all[1]->dims[0] % 8 == 0) {
         const uint16_t *q16 = nc_shadow_of(m, all[0]), *kv16 = nc_shadow_of(m, all[1]);
         const uint16_t *kvm16 = all[2] ? nc_shadow_of(m, all[2]) : nullptr;

@@ -199,7 +199,7 @@ def test_profile_variants_match_checker(hosts, name, fused):
             assert M.tensors_close(w_h[k], w_r[k], 1e-5), (name, k, M.rel_l2(w_h[k], w_r[k]))
 
 
-@pytest.mark.parametrize("cfg_name,bf16", [("SMALL32", 0), ("C1", 0), ("C1", 1), ("C3S", 0)])
+@pytest.mark.parametrize("cfg_name,bf16", [("SMALL32", 0), ("C1", 0), ("C1", 1), ("C3S", 0), ("C3S", 1)])
 def test_cached_timestep_logits_are_bit_identical(hosts, cfg_name, bf16):
     """With width-invariant products, the decoder's one-column evaluations
     (trf_eval_step) give exactly the logits of the encoder's whole-segment
