@@ -371,6 +371,41 @@ def cdf_c5(pkg, iters=50):
             "invariants_ok": ok}
 
 
+def copy_floor(iters=50):
+    """What a kernel that only moves bytes costs at the sizes of this workload's bandwidth kernels:
+    device-to-device copies (the runtime's own copy kernel) of 4, 8 and 64 MiB, back to back on
+    the null stream between two HIP events.  A norm kernel of the headline step reads 4 MiB and
+    writes 8 MiB; its time is to be read against the copy that moves as much, not against
+    8 TB/s, which a transfer of this size cannot reach (launch, ramp and drain are microseconds)."""
+    hip = hip_runtime()
+    out = {}
+    for mib in (4, 8, 64):
+        n = mib << 20
+        src, dst = C.c_void_p(), C.c_void_p()
+        assert hip.hipMalloc(C.byref(src), C.c_size_t(n)) == 0 and hip.hipMalloc(C.byref(dst), C.c_size_t(n)) == 0
+        hip.hipMemset(src, 1, C.c_size_t(n))
+        e0, e1 = C.c_void_p(), C.c_void_p()
+        hip.hipEventCreate(C.byref(e0))
+        hip.hipEventCreate(C.byref(e1))
+        for _ in range(3):
+            hip.hipMemcpyAsync(dst, src, C.c_size_t(n), 3, None)
+        hip.hipDeviceSynchronize()
+        hip.hipEventRecord(e0, None)
+        for _ in range(iters):
+            hip.hipMemcpyAsync(dst, src, C.c_size_t(n), 3, None)       # hipMemcpyDeviceToDevice
+        hip.hipEventRecord(e1, None)
+        hip.hipEventSynchronize(e1)
+        ms = C.c_float()
+        hip.hipEventElapsedTime(C.byref(ms), e0, e1)
+        us = ms.value * 1e3 / iters
+        out["%d_MiB" % mib] = {"us": round(us, 2), "moved_MB": round(2 * n / 1e6, 1), "GBps": round(2 * n / us / 1e3, 1)}
+        hip.hipEventDestroy(e0)
+        hip.hipEventDestroy(e1)
+        hip.hipFree(src)
+        hip.hipFree(dst)
+    return out
+
+
 def cpu_baseline(pkg, data, n_steps, threads):
     """The CPU checker driving the reference op sequence (whole-segment
     evaluation, float symbol coder: what `nncp --encode_only` does) on the
@@ -617,6 +652,7 @@ def main():
                     "mode": "NNCP_MODE_SEGMENT | NNCP_MODE_STEP_DECODE | NNCP_CODER_CDF16"}
 
     attn = cdf = dec = None
+    floor = copy_floor() if args.cdf_iters else None
     if args.attention_iters:
         say("isolated attention, B32 H8 d64 T64 K128, %d forward+backward pairs" % args.attention_iters)
         attn = attention_c2(pkg, args.attention_iters)
@@ -663,7 +699,7 @@ def main():
         "kernel_launches_per_step": head["kernel_launches_per_step"],
         "host_seconds": head["host_seconds"],
         "roofline": head["roofline"], "encode_step_decodable": step_dec, "variants": variants,
-        "c4": c4, "attention": attn, "cdf": cdf, "decode": dec,
+        "c4": c4, "attention": attn, "cdf": cdf, "copy_floor": floor, "decode": dec,
         "cpu_baseline": cpu}))
 
 
