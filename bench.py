@@ -406,6 +406,64 @@ def copy_floor(iters=50):
     return out
 
 
+def norms_isolated(pkg, iters=50):
+    """The norm kernels of the headline step (d 512, 2048 columns: LayerNorm forward reads x and
+    writes y and the normalised values, 12.6 MB; backward reads g and xhat and writes dx, 12.6 MB
+    plus the partial rows of the gain / bias gradients), through the raw entry points, back to
+    back on the null stream on resident buffers - measured the way copy_floor measures the copies
+    they are to be read against (in the step their inputs come cold from the producing kernel)."""
+    nc = pkg.binding.NC(pkg.binding.HIP_LIB)
+    lib = C.CDLL(pkg.binding.HIP_LIB)
+    hip = hip_runtime()
+    d, n = 512, 2048
+    rng = np.random.default_rng(1)
+    t = {k: nc.tensor(rng.standard_normal(shape).astype(np.float32)) for k, shape in
+         (("x", (n, d)), ("w", (d,)), ("b", (d,)), ("g", (n, d)))}
+    rows = lib.nchip_norm_bwd_partial_rows(C.c_int64(n))
+    for k, shape in (("y", (n, d)), ("xhat", (n, d)), ("rstd", (n,)), ("dx", (n, d)), ("dw", (d,)), ("db", (d,)),
+                     ("partial", (rows * 2 * d,))):
+        t[k] = nc.tensor(np.zeros(shape, np.float32))
+    P = {k: C.c_void_p(nc.lib.nc_tensor_get_ptr(v, None)) for k, v in t.items()}
+
+    def fwd():
+        return lib.nchip_norm_fwd(None, P["x"], P["w"], P["b"], P["y"], P["xhat"], P["rstd"], C.c_int(d), C.c_int64(n),
+                                  C.c_float(1e-5), C.c_int(1))
+
+    def bwd():
+        # (dw = db = NULL: the partial rows are left to the caller, as in the step, where one launch
+        # sums the rows of all norms of the backward pass)
+        return lib.nchip_norm_bwd(None, P["g"], P["xhat"], P["rstd"], P["w"], P["dx"], None, None, None, P["partial"],
+                                  C.c_int(d), C.c_int64(n), C.c_int(1))
+
+    def timed(f):
+        e0, e1 = C.c_void_p(), C.c_void_p()
+        hip.hipEventCreate(C.byref(e0))
+        hip.hipEventCreate(C.byref(e1))
+        for _ in range(3):
+            assert f() == 0
+        hip.hipDeviceSynchronize()
+        hip.hipEventRecord(e0, None)
+        for _ in range(iters):
+            f()
+        hip.hipEventRecord(e1, None)
+        hip.hipEventSynchronize(e1)
+        ms = C.c_float()
+        hip.hipEventElapsedTime(C.byref(ms), e0, e1)
+        hip.hipEventDestroy(e0)
+        hip.hipEventDestroy(e1)
+        return ms.value * 1e3 / iters
+
+    us_f, us_b = timed(fwd), timed(bwd)
+    nbytes = 3 * d * n * 4
+    for v in t.values():
+        nc.free(v)
+    nc.close()
+    return {"workload": "LayerNorm d512 x 2048 columns, isolated, back to back", "us_fwd": round(us_f, 2),
+            "us_bwd": round(us_b, 2), "algorithmic_MB": round(nbytes / 1e6, 1),
+            "fwd_GBps": round(nbytes / us_f / 1e3, 1), "bwd_GBps": round(nbytes / us_b / 1e3, 1),
+            "fwd_hbm_frac": round(nbytes / us_f / 1e3 / 8000, 4), "bwd_hbm_frac": round(nbytes / us_b / 1e3 / 8000, 4)}
+
+
 def cpu_baseline(pkg, data, n_steps, threads):
     """The CPU checker driving the reference op sequence (whole-segment
     evaluation, float symbol coder: what `nncp --encode_only` does) on the
@@ -653,6 +711,7 @@ def main():
 
     attn = cdf = dec = None
     floor = copy_floor() if args.cdf_iters else None
+    norms = norms_isolated(pkg) if args.cdf_iters else None
     if args.attention_iters:
         say("isolated attention, B32 H8 d64 T64 K128, %d forward+backward pairs" % args.attention_iters)
         attn = attention_c2(pkg, args.attention_iters)
@@ -699,7 +758,7 @@ def main():
         "kernel_launches_per_step": head["kernel_launches_per_step"],
         "host_seconds": head["host_seconds"],
         "roofline": head["roofline"], "encode_step_decodable": step_dec, "variants": variants,
-        "c4": c4, "attention": attn, "cdf": cdf, "copy_floor": floor, "decode": dec,
+        "c4": c4, "attention": attn, "cdf": cdf, "norms": norms, "copy_floor": floor, "decode": dec,
         "cpu_baseline": cpu}))
 
 
