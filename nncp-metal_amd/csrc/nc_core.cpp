@@ -670,6 +670,22 @@ extern "C" void nc_tensor_copy(NCTensor *dst, NCTensor *src) { nc_copy_any(dst, 
 extern "C" void nc_tensor_copy_slice(NCTensor *dst, NCTensor *src, int axis, size_t dst_start,
                                      size_t dst_end, size_t src_start)
 {
+    if (dst == src && src_start > dst_start && dst_start < dst_end) {
+        // A shift towards the front of the same tensor (the memory update): pieces no longer than
+        // the shift distance do not overlap their own source, and copied front to back (the
+        // stream keeps the order) each piece reads data no earlier piece has written - no
+        // temporary, and every element moves once.
+        const size_t dist = src_start - dst_start;
+        for (size_t a = dst_start; a < dst_end; a += dist) {
+            const size_t b = a + dist < dst_end ? a + dist : dst_end;
+            NCTensor *dp = nc_slice_alias(dst, axis, a, b);
+            NCTensor *sp = nc_slice_alias(src, axis, a + dist, b + dist);
+            nc_copy_any(dp, sp);
+            nc_free_tensor(dp);
+            nc_free_tensor(sp);
+        }
+        return;
+    }
     NCTensor *d = nc_slice_alias(dst, axis, dst_start, dst_end);
     NCTensor *s = nc_slice_alias(src, axis, src_start, src_start + (dst_end - dst_start));
     if (dst->buf == src->buf) {

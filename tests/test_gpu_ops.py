@@ -363,6 +363,24 @@ def test_views_and_copies_on_device(hip, rng):
     hip.free(t)
 
 
+@pytest.mark.parametrize("axis,n,dst0,dst1,src0", [(2, 7, 0, 6, 1), (2, 7, 0, 2, 5), (2, 9, 1, 7, 3), (1, 8, 0, 5, 3),
+                                                    (0, 10, 2, 9, 3), (2, 7, 2, 6, 0), (2, 6, 0, 4, 2)])
+def test_copy_slice_within_one_tensor(hip, rng, axis, n, dst0, dst1, src0):
+    """nc_tensor_copy_slice of a tensor onto itself (the memory update, nncp.c:1205-1221): shifts
+    towards the front go piece by piece without a temporary, whatever the distance and the length;
+    a shift towards the back goes through one; both equal numpy's copy of the source first."""
+    shape = [4, 5, 6]
+    shape[2 - axis] = n                                  # numpy axes are libnc's reversed
+    x = rng.standard_normal(shape).astype(np.float32)
+    t = hip.tensor(x)
+    hip.nc_tensor_copy_slice(t, t, axis, dst0, dst1, src0)
+    sl = lambda a, b: tuple(slice(a, b) if i == 2 - axis else slice(None) for i in range(3))
+    want = x.copy()
+    want[sl(dst0, dst1)] = x[sl(src0, src0 + dst1 - dst0)]
+    assert np.array_equal(hip.numpy(t), want)
+    hip.free(t)
+
+
 def _run_graph(nc, arrays, build, weight):
     hs = [nc.param(a, "p%d" % i) for i, a in enumerate(arrays)]
     y = build(nc, *[nc.dup(h.value) for h, _ in hs])
