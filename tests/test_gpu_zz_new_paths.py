@@ -391,3 +391,30 @@ def test_bf16_parameter_files_cross_between_the_gpu_and_the_checker(hosts, tmp_p
     assert os.path.getsize(str(tmp_path / "from_gpu.bin")) < 2 * n + 200 * len(gpu.param_names())
     gpu.close()
     ref.close()
+
+
+def test_enwik8_profile_round_trips_a_small_file_on_gpu(hosts, tmp_path):
+    """nncp's enwik8 profile as `nncp_profile` fills it (nncp.c:2515-2572: 20 layers of d1024, 8 heads of
+    128, gated GELU 3072, RMSNorm before every block and at the end, 64 + 256 keys with per-layer
+    position tables, Adam with clipping, bf16 products, a retrain pass with dropout after the
+    block) on a file of two one-segment blocks and a ragged tail, through the file container: the decoder
+    rebuilds the model from the header and returns the input."""
+    hp = M.load_pkg().host
+    cfg, fp = hp.profile(hosts[0], "enwik8")
+    assert (cfg.n_layer, cfg.d_model, cfg.n_head, cfg.d_key, cfg.d_inner, cfg.mem_len, cfg.d_pos) == (20, 1024, 8, 128, 3072, 256, 320)
+    cfg.use_device, cfg.fused, cfg.nb_threads = 1, 1, 4
+    fp.mode = hp.MODE_SEGMENT | hp.CODER_CDF16
+    # one training step per block instead of the profile's 100 000 symbols, so that this small
+    # file has blocks to retrain between (the pass runs after every block but the last)
+    import ctypes as C
+    assert hosts[0].lib.nncp_parse_interp(C.byref(fp.block_len), b"2048") == 0
+    n = cfg.batch_size * cfg.seg_len * 2 + 77
+    syms = M.markov1(n, 256, seed=23)
+    src, packed, back = (str(tmp_path / f) for f in ("in.bin", "out.nncp", "back.bin"))
+    syms.astype(np.uint8).tofile(src)
+    st, rst = hp.encode_file(hosts[0], src, packed, cfg, fp)
+    assert st.n_symbols == n and st.n_steps == 2
+    assert rst.n_steps >= 1                                   # the retrain pass ran (dropout on, op by op)
+    assert 0 < os.path.getsize(packed) < n * 1.1              # an untrained model: about 8 bits a byte
+    hp.decode_file(hosts[0], packed, back, use_device=1, nb_threads=4)
+    assert open(back, "rb").read() == open(src, "rb").read()
