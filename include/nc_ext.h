@@ -126,6 +126,14 @@ NCTensor *nc_get_col_host_indices(NCTensor *w, NCTensor *x, float scale);
    with cdf[s, col] <= target (cumulative-frequency search of a decoder). */
 NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets);
 
+/* cdf (V, n) U16, symbols: n contiguous I32 on the same device -> (L, n) U16, L = max(1,
+   ceil(log2 V)): the entries of each column that nncp_write_sym_cdf reads when it codes that
+   column's symbol (the split point of every level of its tree, 0 below the leaf), in the order
+   it reads them - nncp_write_sym_cdf_path codes from them.  An encoder brings these L values
+   per column to the host instead of the V of the column.  Consumes both.  No counterpart in
+   the reference. */
+NCTensor *nc_cdf_path(NCTensor *cdf, NCTensor *symbols);
+
 /* The deterministic exponential used by nc_soft_max_cdf16, for x <= 0:
    n = rint(x*log2e); r = x - n*ln2 (two fmaf steps); degree-6 polynomial in
    fmaf form; result scaled by 2^n through the exponent field.  Only IEEE

@@ -441,6 +441,12 @@ int nchip_softmax_cdf16(void *stream, const float *logits, uint16_t *cdf, int v,
    max(floor(q[i] * mult / sum q), 1) as int32, q the 24-bit integer exponentials of the CDF
    above; 0 <= mult <= 2^32; bit-identical to the CPU checker. */
 int nchip_softmax_int(void *stream, const float *logits, int32_t *out, int v, int64_t n, float mult);
+/* path[l, c], l < levels: the entries of column c of cdf (v, n) that nncp_write_sym_cdf reads
+   when it codes sym[c] - cdf[start + (len >> 1)] at each level of the balanced tree over [0, v)
+   (cp_utils.c:299-323), 0 below the leaf.  levels >= ceil(log2 v).  No index leaves the column
+   whatever sym[c] holds. */
+int nchip_cdf_path(void *stream, const uint16_t *cdf, const int32_t *sym, uint16_t *path,
+                   int v, int64_t n, int levels);
 /* sym[i, c] = largest s with cdf[s, c] <= target[i, c]; targets (m, n). */
 int nchip_cdf_lookup(void *stream, const uint16_t *cdf, const uint16_t *target,
                      uint16_t *sym, int v, int64_t m, int64_t n);

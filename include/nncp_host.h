@@ -59,6 +59,9 @@ int nncp_read_sym(NNCPGetBit *gb, const float *prob, int n_symb);
    clamped to [1, 32767]; O(log n_symb) integer work per symbol */
 void nncp_write_sym_cdf(NNCPPutBit *pb, const uint16_t *cdf, int n_symb, int sym);
 int nncp_read_sym_cdf(NNCPGetBit *gb, const uint16_t *cdf, int n_symb);
+/* nncp_write_sym_cdf given only the entries it reads for this symbol, in reading order (a column
+   of nc_cdf_path, nc_ext.h): the same bits */
+void nncp_write_sym_cdf_path(NNCPPutBit *pb, const uint16_t *path, int n_symb, int sym);
 
 /* piece-wise linear schedule with optional power decay (cp_utils.c:380-410) */
 typedef struct {

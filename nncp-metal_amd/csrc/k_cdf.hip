@@ -432,6 +432,41 @@ extern "C" int nchip_softmax_cdf16(void *stream, const float *logits, uint16_t *
     return 0;
 }
 
+// What a binary-tree coder reads of a column when it knows the symbol: at every level of the
+// balanced tree over [0, v) (cp_utils.c:299-323) the CDF entry at the split point.  One thread per
+// column walks the tree for its symbol; whatever the symbol's value, start + n0 < v.
+__global__ __launch_bounds__(TPB) void cdf_path_kernel(const uint16_t *cdf, const int32_t *sym, uint16_t *path,
+                                                        int v, int64_t ncol, int levels)
+{
+    const int64_t c = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (c >= ncol) return;
+    const uint16_t *col = cdf + c * v;
+    uint16_t *out = path + c * levels;
+    const int s = sym[c];
+    int start = 0, n = v;
+    for (int l = 0; l < levels; l++) {
+        uint16_t mid = 0;
+        if (n > 1) {
+            const int n0 = n >> 1;
+            mid = col[start + n0];
+            if (s >= start + n0) { start += n0; n -= n0; }
+            else n = n0;
+        }
+        out[l] = mid;
+    }
+}
+
+extern "C" int nchip_cdf_path(void *stream, const uint16_t *cdf, const int32_t *sym, uint16_t *path,
+                              int v, int64_t n, int levels)
+{
+    if (n <= 0 || levels <= 0) return 0;
+    if (v <= 0 || (levels < 31 && (1 << levels) < v)) { fprintf(stderr, "nchip_cdf_path: %d levels do not reach %d symbols\n", levels, v); return -1; }
+    hipLaunchKernelGGL(cdf_path_kernel, dim3((unsigned)((n + TPB - 1) / TPB)), dim3(TPB), 0, (hipStream_t)stream, cdf, sym, path, v, n, levels);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { fprintf(stderr, "nchip_cdf_path: %s\n", hipGetErrorString(e)); return -2; }
+    return 0;
+}
+
 extern "C" int nchip_cdf_lookup(void *stream, const uint16_t *cdf, const uint16_t *target,
                                 uint16_t *sym, int v, int64_t m, int64_t n)
 {

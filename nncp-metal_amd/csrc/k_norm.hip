@@ -267,6 +267,46 @@ __global__ __launch_bounds__(TPB) void softmax_fwd_kernel(const float *x, float 
     for (int i = lane; i < v; i += 64) yc[i] *= inv;
 }
 
+// Long columns (a vocabulary of thousands): one workgroup per column, the column read once
+// into registers (thread t holds the float4 at 4 (r TPB + t), r < R), written once.
+template <int R>
+__global__ __launch_bounds__(TPB) void softmax_fwd_block_kernel(const float *x, float *y, int v)
+{
+    __shared__ float red[2][WPB];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const float *xc = x + (int64_t)blockIdx.x * v;
+    float *yc = y + (int64_t)blockIdx.x * v;
+    float4 f[R];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i0 = (r * TPB + t) * 4;
+        f[r] = i0 < v ? *reinterpret_cast<const float4 *>(xc + i0) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        mx = fmaxf(fmaxf(mx, fmaxf(f[r].x, f[r].y)), fmaxf(f[r].z, f[r].w));
+    }
+    mx = wave_max(mx);
+    if (lane == 0) red[0][wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+    float s = 0.0f;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        f[r].x = expf(f[r].x - mx); f[r].y = expf(f[r].y - mx);
+        f[r].z = expf(f[r].z - mx); f[r].w = expf(f[r].w - mx);
+        s += (f[r].x + f[r].y) + (f[r].z + f[r].w);
+    }
+    s = wave_sum(s);
+    if (lane == 0) red[1][wave] = s;
+    __syncthreads();
+    const float inv = 1.0f / ((red[1][0] + red[1][1]) + (red[1][2] + red[1][3]));
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i0 = (r * TPB + t) * 4;
+        if (i0 < v)
+            *reinterpret_cast<float4 *>(yc + i0) = make_float4(f[r].x * inv, f[r].y * inv, f[r].z * inv, f[r].w * inv);
+    }
+}
+
 __global__ __launch_bounds__(TPB) void softmax_bwd_kernel(const float *y, const float *g, float *dx,
                                                           int v, int64_t n)
 {
@@ -306,6 +346,26 @@ __global__ void nll_bwd_kernel(const float *p, const int32_t *idx, const float *
     }
 }
 
+// the same for long columns: blockIdx.x the column, blockIdx.y a run of 4 TPB rows of it
+__global__ __launch_bounds__(TPB) void nll_bwd_vec_kernel(const float *p, const int32_t *idx, const float *g, float *dl,
+                                                          int v, int fused)
+{
+    const int64_t c = blockIdx.x;
+    const int i0 = ((int)blockIdx.y * TPB + (int)threadIdx.x) * 4;
+    if (i0 >= v) return;
+    const float gc = g[c];
+    const int s = idx[c];
+    const float4 pv = *reinterpret_cast<const float4 *>(p + c * v + i0);
+    const float in[4] = { pv.x, pv.y, pv.z, pv.w };
+    float r[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if (fused) r[j] = gc * ((i0 + j == s ? 1.0f : 0.0f) - in[j]);
+        else r[j] = (i0 + j == s) ? gc / in[j] : 0.0f;
+    }
+    *reinterpret_cast<float4 *>(dl + c * v + i0) = make_float4(r[0], r[1], r[2], r[3]);
+}
+
 __global__ void get_col_kernel(const float *w, const int32_t *idx, float *y, int d, int v, int64_t total, int *bad,
                                float scale)
 {
@@ -330,23 +390,41 @@ __global__ __launch_bounds__(TPB) void add_col_kernel(const float *g, const int3
                                                       int d, int64_t n)
 {
     __shared__ int list[ADD_COL_MAX_N];
-    __shared__ int cnt[TPB + 1];
-    const int sym = blockIdx.x, t = threadIdx.x;
-    const int per = (int)((n + TPB - 1) / TPB);
+    __shared__ int wave_hits[WPB];
+    const int sym = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int per = (int)((n + TPB - 1) / TPB); // <= 32: a thread's hits fit one mask
     const int c0 = t * per, c1 = (int)(c0 + per < n ? c0 + per : n);
-    int mine = 0;
-    for (int c = c0; c < c1; c++) mine += idx[c] == sym;
-    cnt[t + 1] = mine;
-    if (t == 0) cnt[0] = 0;
+    unsigned int mask = 0;
+    if ((per & 3) == 0 && c0 + per <= n && ((uintptr_t)idx & 15) == 0) {
+        for (int q = 0; q < per; q += 4) {
+            const uint4 w = *reinterpret_cast<const uint4 *>(idx + c0 + q);
+            mask |= ((unsigned int)((int)w.x == sym) | (unsigned int)((int)w.y == sym) << 1 |
+                     (unsigned int)((int)w.z == sym) << 2 | (unsigned int)((int)w.w == sym) << 3) << q;
+        }
+    } else {
+        for (int c = c0; c < c1; c++) mask |= (unsigned int)(idx[c] == sym) << (c - c0);
+    }
+    // exclusive prefix of the threads' hit counts: by shuffles inside a wave, through LDS across the four
+    const int mine = __builtin_popcount(mask);
+    int incl = mine;
+#pragma unroll
+    for (int dd = 1; dd < 64; dd <<= 1) {
+        const int o = __shfl_up(incl, dd, 64);
+        if (lane >= dd) incl += o;
+    }
+    if (lane == 63) wave_hits[wave] = incl;
     __syncthreads();
-    if (t == 0)
-        for (int k = 1; k <= TPB; k++) cnt[k] += cnt[k - 1];
+    int pos = incl - mine, total = 0;
+#pragma unroll
+    for (int w = 0; w < WPB; w++) {
+        if (w < wave) pos += wave_hits[w];
+        total += wave_hits[w];
+    }
+    while (mask) {
+        list[pos++] = c0 + __builtin_ctz(mask);
+        mask &= mask - 1;
+    }
     __syncthreads();
-    int pos = cnt[t];
-    for (int c = c0; c < c1; c++)
-        if (idx[c] == sym) list[pos++] = c;
-    __syncthreads();
-    const int total = cnt[TPB];
     for (int i = t; i < d; i += TPB) {
         float acc = 0.0f;
 #pragma unroll 4
@@ -613,7 +691,16 @@ int nchip_norm_bwd_static(void *stream, const float *g, const float *xhat, const
 int nchip_softmax_fwd(void *stream, const float *x, float *y, int v, int64_t n)
 {
     if (n <= 0 || v <= 0) return 0;
-    hipLaunchKernelGGL(softmax_fwd_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, (hipStream_t)stream, x, y, v, n);
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec = v % 4 == 0 && (((uintptr_t)x | (uintptr_t)y) & 15) == 0 && n <= 0x7fffffff;
+    if (vec && v >= 2048 && v <= 16 * 4 * TPB) { // a workgroup per column, the column in registers
+        const dim3 grid((unsigned)n);
+        if (v <= 2 * 4 * TPB) hipLaunchKernelGGL(softmax_fwd_block_kernel<2>, grid, dim3(TPB), 0, st, x, y, v);
+        else if (v <= 4 * 4 * TPB) hipLaunchKernelGGL(softmax_fwd_block_kernel<4>, grid, dim3(TPB), 0, st, x, y, v);
+        else if (v <= 8 * 4 * TPB) hipLaunchKernelGGL(softmax_fwd_block_kernel<8>, grid, dim3(TPB), 0, st, x, y, v);
+        else hipLaunchKernelGGL(softmax_fwd_block_kernel<16>, grid, dim3(TPB), 0, st, x, y, v);
+    } else
+        hipLaunchKernelGGL(softmax_fwd_kernel, dim3((unsigned)((n + WPB - 1) / WPB)), dim3(TPB), 0, st, x, y, v, n);
     return check("nchip_softmax_fwd");
 }
 
@@ -663,7 +750,11 @@ int nchip_nll_bwd(void *stream, const float *p, const int32_t *idx, const float 
                   int v, int64_t n, int fused)
 {
     if (n <= 0) return 0;
-    hipLaunchKernelGGL(nll_bwd_kernel, dim3(grid_for(n * v)), dim3(TPB), 0, (hipStream_t)stream, p, idx, g, dl, v, n * v, fused);
+    if (v >= 1024 && v % 4 == 0 && (((uintptr_t)p | (uintptr_t)dl) & 15) == 0 && n <= 0x7fffffff && v <= 65535 * 4 * TPB)
+        hipLaunchKernelGGL(nll_bwd_vec_kernel, dim3((unsigned)n, (unsigned)((v + 4 * TPB - 1) / (4 * TPB))), dim3(TPB), 0,
+                           (hipStream_t)stream, p, idx, g, dl, v, fused);
+    else
+        hipLaunchKernelGGL(nll_bwd_kernel, dim3(grid_for(n * v)), dim3(TPB), 0, (hipStream_t)stream, p, idx, g, dl, v, n * v, fused);
     return check("nchip_nll_bwd");
 }
 

@@ -1389,6 +1389,30 @@ extern "C" NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets)
     return y;
 }
 
+static int cdf_path_levels(size_t v)
+{
+    int levels = 1;
+    while (((size_t)1 << levels) < v) levels++;
+    return levels;
+}
+
+extern "C" NCTensor *nc_cdf_path(NCTensor *cdf, NCTensor *symbols)
+{
+    cdf = nc_contig(cdf); symbols = nc_contig(symbols);
+    need_dev(cdf, "nc_cdf_path"); need_dev(symbols, "nc_cdf_path");
+    if (cdf->type != NC_TYPE_U16 || symbols->type != NC_TYPE_I32) nc_fatal("nc_cdf_path: a u16 cdf and i32 symbols expected");
+    size_t v = cdf->dims[0], cols = v ? nc_numel(cdf) / v : 0;
+    if (v == 0 || nc_numel(symbols) != cols) nc_fatal("nc_cdf_path: one symbol per column of the cdf expected");
+    size_t dims[2] = { (size_t)cdf_path_levels(v), cols };
+    NCTensor *y = nc_alloc(cdf->dev, NC_TYPE_U16, 2, dims, false);
+    if (nchip_cdf_path(nc_stream(cdf), (const uint16_t *)nc_data(cdf), (const int32_t *)nc_data(symbols),
+                       (uint16_t *)nc_data(y), (int)v, (int64_t)cols, (int)dims[0]))
+        nc_fatal("nc_cdf_path failed");
+    LAUNCHED(cdf);
+    nc_free_tensor(cdf); nc_free_tensor(symbols);
+    return y;
+}
+
 // same arithmetic as the device exponential of k_cdf.hip, for host callers
 extern "C" float nc_exp_det(float x)
 {

@@ -192,6 +192,7 @@ class Host:
         L.nncp_read_sym.argtypes = [C.POINTER(NNCPGetBit), _P, C.c_int]
         L.nncp_write_sym_cdf.argtypes = [C.POINTER(NNCPPutBit), _P, C.c_int, C.c_int]
         L.nncp_read_sym_cdf.argtypes = [C.POINTER(NNCPGetBit), _P, C.c_int]
+        L.nncp_write_sym_cdf_path.argtypes = [C.POINTER(NNCPPutBit), _P, C.c_int, C.c_int]
         L.nncp_interp.restype = C.c_float
         L.nncp_interp.argtypes = [C.POINTER(NNCPInterp), C.c_int64]
         L.nncp_profile.argtypes = [C.POINTER(NNCPConfig), C.POINTER(NNCPFileParams), C.c_char_p]

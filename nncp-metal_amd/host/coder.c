@@ -200,6 +200,22 @@ void nncp_write_sym_cdf(NNCPPutBit *pb, const uint16_t *cdf, int n_symb, int sym
     }
 }
 
+/* nncp_write_sym_cdf from the entries it would read, in the order it reads them (nc_cdf_path) */
+void nncp_write_sym_cdf_path(NNCPPutBit *pb, const uint16_t *path, int n_symb, int sym)
+{
+    int start = 0, n = n_symb;
+    uint32_t lo = 0, hi = 65536;
+    while (n > 1) {
+        int n0 = n >> 1;
+        uint32_t mid = *path++;
+        int prob0 = clamp_prob((long)(((uint64_t)(mid - lo) << NNCP_PROB_BITS) / (hi - lo)));
+        int bit = sym >= start + n0;
+        nncp_put_bit(pb, prob0, bit);
+        if (bit) { start += n0; n -= n0; lo = mid; }
+        else { n = n0; hi = mid; }
+    }
+}
+
 int nncp_read_sym_cdf(NNCPGetBit *gb, const uint16_t *cdf, int n_symb)
 {
     int start = 0, n = n_symb;

@@ -72,10 +72,13 @@ typedef struct {
     NCTensor *host;
     const float *prob;
     const uint16_t *cdf;
+    const uint16_t *path; /* encoder, whole segment: per column the CDF entries its symbol's walk reads */
     size_t stride;
 } HostDist;
 
-static HostDist fetch_dist(Coder *c, NCTensor *output)
+/* `symbols` (consumed; may be NULL): the symbol of every column, known to an encoder before it
+   codes.  With them only the CDF entries that the coder will read cross to the host. */
+static HostDist fetch_dist(Coder *c, NCTensor *output, NCTensor *symbols)
 {
     HostDist d;
     memset(&d, 0, sizeof(d));
@@ -85,6 +88,14 @@ static HostDist fetch_dist(Coder *c, NCTensor *output)
         int nd = nc_tensor_get_dims(logits, dims);
         for (int i = 1; i < nd; i++) cols *= dims[i];
         nc_free_tensor(output);
+        if (symbols) {
+            NCDevice *dev = nc_get_tensor_device(logits);
+            size_t n1 = cols;
+            NCTensor *sym = nc_tensor_to_device(nc_reshape_1d(symbols, n1), dev);
+            d.host = nc_tensor_to_cpu_device(nc_cdf_path(nc_soft_max_cdf16(nc_dup_tensor(logits)), sym));
+            d.path = nc_tensor_get_ptr(d.host, &d.stride);
+            return d;
+        }
         if (cols <= 64) { /* a timestep's rows: the kernel writes them to the host itself */
             NCDevice *dev = nc_get_tensor_device(logits);
             d.host = nc_soft_max_cdf16_to_host(nc_dup_tensor(logits));
@@ -107,7 +118,8 @@ static int code_symbol(Coder *c, const HostDist *d, size_t col, int stream, int 
     prof_start(PROF_WRITE_SYM); /* nncp.c:3007, 3039 */
     if (!c->is_decode) {
         sym = get_symb(&c->view, stream, pos);
-        if (d->cdf) nncp_write_sym_cdf(c->pb, d->cdf + col * d->stride, c->n_symbols, sym);
+        if (d->path) nncp_write_sym_cdf_path(c->pb, d->path + col * d->stride, c->n_symbols, sym);
+        else if (d->cdf) nncp_write_sym_cdf(c->pb, d->cdf + col * d->stride, c->n_symbols, sym);
         else nncp_write_sym(c->pb, d->prob + col * d->stride, c->n_symbols, sym);
     } else {
         if (d->cdf) sym = nncp_read_sym_cdf(c->gb, d->cdf + col * d->stride, c->n_symbols);
@@ -133,15 +145,23 @@ static HostDist encode_segment_eval(Coder *c, int idx, int n_t, int len2, int fu
                                     NCTensor *input, NCTensor *expected)
 {
     int B = c->B;
+    NCTensor *symbols = NULL;
+    if (c->coder == NNCP_CODER_CDF16) { /* (B, T) like input: column t*B + b, zero where nothing is coded */
+        size_t dims[2];
+        nc_tensor_get_dims(input, dims);
+        symbols = nc_new_tensor_2d(nc_get_tensor_device(input), NC_TYPE_I32, dims[0], dims[1]);
+    }
     for (int t = 0; t < n_t; t++)
         for (int b = 0; b < B; b++) {
             nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
-            if (expected && symbol_is_coded(t, b, len2, c->view.rem, full))
-                nc_set1_i32_2d(expected, b, t, get_symb(&c->view, b, idx + t));
+            if (!symbol_is_coded(t, b, len2, c->view.rem, full))
+                continue;
+            if (expected) nc_set1_i32_2d(expected, b, t, get_symb(&c->view, b, idx + t));
+            if (symbols) nc_set1_i32_2d(symbols, b, t, get_symb(&c->view, b, idx + t));
         }
     double t0 = now_s();
     NCTensor *out = c->cls->eval(c->s, -1, input);
-    HostDist d = fetch_dist(c, out);
+    HostDist d = fetch_dist(c, out, symbols);
     c->st->t_eval += now_s() - t0;
     return d;
 }
@@ -182,7 +202,7 @@ static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int ful
                 nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
             t0 = now_s();
             NCTensor *out = trf_eval_step(s, t, input);
-            HostDist d = fetch_dist(c, out);
+            HostDist d = fetch_dist(c, out, NULL);
             c->st->t_eval += now_s() - t0;
             t0 = now_s();
             for (int b = 0; b < B; b++)
@@ -207,7 +227,7 @@ static void code_segment(Coder *c, int mode, int idx, int n_t, int len2, int ful
             nc_set1_i32_2d(input, b, t, get_symb(&c->view, b, idx + t - 1));
         t0 = now_s();
         NCTensor *out = c->cls->eval(s, mode == NNCP_MODE_SEGMENT ? -1 : t, input);
-        HostDist d = fetch_dist(c, out);
+        HostDist d = fetch_dist(c, out, NULL);
         c->st->t_eval += now_s() - t0;
         t0 = now_s();
         for (int b = 0; b < B; b++)

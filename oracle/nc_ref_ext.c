@@ -412,6 +412,38 @@ NCTensor *nc_soft_max_int(NCTensor *x, float mult)
     return y;
 }
 
+/* nc_ext.h: the walk of nncp_write_sym_cdf (cp_utils.c:299-323 on integer counts), keeping what it reads */
+NCTensor *nc_cdf_path(NCTensor *cdf, NCTensor *symbols)
+{
+    NCTensor *y;
+    size_t V, cols, dims[2];
+    int levels = 1;
+    cdf = nc_contig(cdf); symbols = nc_contig(symbols);
+    if (cdf->type != NC_TYPE_U16 || symbols->type != NC_TYPE_I32)
+        nc_fatal("cdf_path: a u16 cdf and i32 symbols expected");
+    V = cdf->dims[0];
+    cols = V ? nc_numel(cdf) / V : 0;
+    if (V == 0 || nc_numel(symbols) != cols)
+        nc_fatal("cdf_path: one symbol per column of the cdf expected");
+    while (((size_t)1 << levels) < V) levels++;
+    dims[0] = (size_t)levels; dims[1] = cols;
+    y = nc_alloc(cdf->dev, NC_TYPE_U16, 2, dims, 1);
+    for (size_t c = 0; c < cols; c++) {
+        const uint16_t *cp = (const uint16_t *)cdf->buf->data + cdf->off + c * V;
+        uint16_t *yp = (uint16_t *)y->buf->data + c * (size_t)levels;
+        long sym = ((const int32_t *)symbols->buf->data + symbols->off)[c];
+        size_t start = 0, n = V;
+        for (int l = 0; l < levels && n > 1; l++) {
+            size_t n0 = n >> 1;
+            yp[l] = cp[start + n0];
+            if (sym >= (long)(start + n0)) { start += n0; n -= n0; }
+            else n = n0;
+        }
+    }
+    nc_free_tensor(cdf); nc_free_tensor(symbols);
+    return y;
+}
+
 NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets)
 {
     NCTensor *y;

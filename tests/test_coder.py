@@ -162,6 +162,50 @@ def test_cdf_symbol_coder_round_trip_and_length(ref, hostc, pkg_mod, V):
     assert got.size * 8 <= ideal * 1.02 + 64
 
 
+@pytest.mark.parametrize("V", [2, 3, 256, 1000, 16384, 65535])
+def test_cdf_path_holds_what_the_coder_reads_and_codes_the_same_bytes(ref, hostc, pkg_mod, V):
+    """nc_cdf_path against a walk of the tree written here (the split point of every level,
+    zero below the leaf), and nncp_write_sym_cdf_path on its columns against nncp_write_sym_cdf
+    on the whole rows: the same bytes.  Symbols include both ends and, for the kernel's sake,
+    values outside the alphabet (they index nothing outside the column)."""
+    rng = np.random.default_rng(V + 1)
+    n = 120
+    logits = (rng.standard_normal((n, V)) * 3).astype(np.float32)
+    cdf_t = ref.nc_soft_max_cdf16(ref.tensor(logits))
+    cdf = ref.numpy(ref.dup(cdf_t))
+    syms = rng.integers(0, V, n).astype(np.int32)
+    syms[:2] = [0, V - 1]
+    wild = syms.copy()
+    wild[5:9] = [-1, V, 2 ** 31 - 1, -2 ** 31]
+    levels = max(1, int(np.ceil(np.log2(V))))
+
+    def walk(row, s):
+        out, start, m = [], 0, V
+        while m > 1:
+            m0 = m >> 1
+            out.append(int(row[start + m0]))
+            if s >= start + m0:
+                start, m = start + m0, m - m0
+            else:
+                m = m0
+        return out + [0] * (levels - len(out))
+    path = ref.numpy(ref.nc_cdf_path(ref.dup(cdf_t), ref.tensor(wild)), free=True)
+    ref.free(cdf_t)
+    assert path.shape == (n, levels) and path.dtype == np.uint16
+    for c in range(n):
+        assert path[c].tolist() == walk(cdf[c], int(wild[c])), c
+    path = np.ascontiguousarray(path)
+    a, abuf = _host_encoder(pkg_mod, hostc, n * 8 + 64)
+    b, bbuf = _host_encoder(pkg_mod, hostc, n * 8 + 64)
+    for c in range(n):
+        if wild[c] != syms[c]:
+            continue
+        hostc.lib.nncp_write_sym_cdf(C.byref(a), cdf[c].ctypes.data, V, int(syms[c]))
+        hostc.lib.nncp_write_sym_cdf_path(C.byref(b), path[c].ctypes.data, V, int(syms[c]))
+    na, nb = hostc.lib.nncp_put_bit_flush(C.byref(a)), hostc.lib.nncp_put_bit_flush(C.byref(b))
+    assert na == nb and bytes(abuf[:na]) == bytes(bbuf[:nb]) and na > 0
+
+
 def test_interp_matches_reference(refc, hostc, pkg_mod):
     class RefInterp(C.Structure):  # cp_utils.h:60-67
         _fields_ = [("n_steps", C.c_int), ("val", C.c_float * 9), ("pos", C.c_int64 * 8),

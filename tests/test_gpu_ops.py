@@ -271,6 +271,19 @@ def test_cdf_lookup_bit_exact(hip, ref, rng, V, n, m):
     assert np.array_equal(res[0], res[1])
 
 
+@pytest.mark.parametrize("V,n", [(256, 2048), (16384, 129), (2, 5), (3, 300), (1000, 257), (65535, 9)])
+def test_cdf_path_bit_exact(hip, ref, rng, V, n):
+    """The CDF entries an encoder's coder reads for known symbols (symbols outside the alphabet
+    included: they read nothing outside their column)."""
+    x = _adversarial_logits(rng, V, max(n, 5))
+    sym = rng.integers(0, V, size=x.shape[0]).astype(np.int32)
+    sym[:5] = [0, V - 1, -7, V, 2 ** 31 - 1]
+    res = []
+    for nc in (hip, ref):
+        res.append(nc.numpy(nc.nc_cdf_path(nc.nc_soft_max_cdf16(nc.tensor(x)), nc.tensor(sym)), free=True))
+    assert res[0].shape == (x.shape[0], max(1, int(np.ceil(np.log2(V))))) and np.array_equal(res[0], res[1])
+
+
 @pytest.mark.parametrize("algo", [16, 1, 0])
 def test_optimiser_step(hip, ref, rng, pkg, algo):
     B = pkg.binding
@@ -407,10 +420,12 @@ def test_norm_model_shapes(hip, ref, rng, d, n, avg):
         assert relerr(a, b) <= 5 * TOL
 
 
-@pytest.mark.parametrize("v,d,n", [(256, 512, 2048), (50, 128, 333), (16, 40, 9000)])
+@pytest.mark.parametrize("v,d,n", [(256, 512, 2048), (50, 128, 333), (16, 40, 9000), (16384, 64, 4096),
+                                   (3000, 32, 8192), (1000, 100, 4095), (700, 8, 1023)])
 def test_embedding_gradient_model_shapes(hip, ref, rng, v, d, n):
     """get_col backward (deterministic scatter-add), including a token count
-    beyond the in-LDS index list."""
+    beyond the in-LDS index list, a vocabulary of thousands (most symbols without
+    a token) and token counts that leave the threads' slices ragged."""
     w = rng.standard_normal((v, d)).astype(np.float32)
     idx = rng.integers(0, v, size=n).astype(np.int32)
     idx[: min(n, 7)] = 3  # repeated symbol
@@ -424,6 +439,30 @@ def test_embedding_gradient_model_shapes(hip, ref, rng, v, d, n):
     # same inputs, same bits
     again = _run_graph(hip, [w], lambda nc, w_: nc.nc_get_col(w_, nc.tensor(idx)), weight)
     assert np.array_equal(again[1][0], res[0][1][0])
+
+
+@pytest.mark.parametrize("v,n", [(2048, 37), (4096, 5), (5000, 9), (16384, 33), (4098, 6), (20000, 3)])
+def test_long_column_softmax_and_log_likelihood(hip, ref, rng, v, n):
+    """Vocabularies of thousands: the softmax that holds a column in one workgroup's registers
+    (2048..16384 entries in multiples of 4; other lengths take the wave-per-column kernel) and
+    the vectorised gradient of the log-likelihood, against float64 and against the checker."""
+    x = (3.0 * rng.standard_normal((n, v))).astype(np.float32)
+    tgt = rng.integers(0, v, size=n).astype(np.int32)
+    tgt[0], tgt[-1] = 0, v - 1
+    weight = rng.standard_normal(n).astype(np.float32)
+    build = lambda nc, x_: nc.nc_indexed_log(nc.nc_soft_max(x_), nc.tensor(tgt))
+    (oh, gh), (orf, gr) = (_run_graph(nc, [x], build, weight) for nc in (hip, ref))
+    x64 = x.astype(np.float64)
+    lse = np.log(np.exp(x64 - x64.max(axis=1, keepdims=True)).sum(axis=1)) + x64.max(axis=1)
+    assert np.abs(oh - (x64[np.arange(n), tgt] - lse)).max() <= 2e-5
+    assert relerr(oh, orf) <= TOL
+    p64 = np.exp(x64 - lse[:, None])
+    want = -p64 * weight[:, None].astype(np.float64)
+    want[np.arange(n), tgt] += weight
+    assert relerr(gh[0], want) <= 5 * TOL
+    assert relerr(gh[0], gr[0]) <= 5 * TOL
+    p = hip.numpy(hip.nc_soft_max(hip.tensor(x)), free=True)
+    assert relerr(p, p64) <= TOL and np.abs(p.astype(np.float64).sum(axis=1) - 1).max() <= 1e-5
 
 
 @pytest.mark.parametrize("f,n", [(2048, 2048), (512, 2048), (256, 77), (1000, 513)])
