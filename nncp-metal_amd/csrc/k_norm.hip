@@ -425,10 +425,38 @@ __global__ __launch_bounds__(TPB) void add_col_kernel(const float *g, const int3
         mask &= mask - 1;
     }
     __syncthreads();
+    // A frequent symbol's list is hundreds of tokens long and its sums (each in token order) are
+    // bound by the loads in flight: eight rows are requested before the first is added.
+    if ((d & 3) == 0 && (((uintptr_t)g | (uintptr_t)dw) & 15) == 0) {
+        for (int i0 = 4 * t; i0 < d; i0 += 4 * TPB) {
+            float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            int k = 0;
+            for (; k + 8 <= total; k += 8) {
+                float4 r[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) r[u] = *reinterpret_cast<const float4 *>(g + (int64_t)list[k + u] * d + i0);
+#pragma unroll
+                for (int u = 0; u < 8; u++) { acc.x += r[u].x; acc.y += r[u].y; acc.z += r[u].z; acc.w += r[u].w; }
+            }
+            for (; k < total; k++) {
+                const float4 r = *reinterpret_cast<const float4 *>(g + (int64_t)list[k] * d + i0);
+                acc.x += r.x; acc.y += r.y; acc.z += r.z; acc.w += r.w;
+            }
+            *reinterpret_cast<float4 *>(dw + (int64_t)sym * d + i0) = acc;
+        }
+        return;
+    }
     for (int i = t; i < d; i += TPB) {
         float acc = 0.0f;
-#pragma unroll 4
-        for (int k = 0; k < total; k++) acc += g[(int64_t)list[k] * d + i];
+        int k = 0;
+        for (; k + 8 <= total; k += 8) {
+            float r[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) r[u] = g[(int64_t)list[k + u] * d + i];
+#pragma unroll
+            for (int u = 0; u < 8; u++) acc += r[u];
+        }
+        for (; k < total; k++) acc += g[(int64_t)list[k] * d + i];
         dw[(int64_t)sym * d + i] = acc;
     }
 }

@@ -421,7 +421,7 @@ def test_norm_model_shapes(hip, ref, rng, d, n, avg):
 
 
 @pytest.mark.parametrize("v,d,n", [(256, 512, 2048), (50, 128, 333), (16, 40, 9000), (16384, 64, 4096),
-                                   (3000, 32, 8192), (1000, 100, 4095), (700, 8, 1023)])
+                                   (3000, 32, 8192), (1000, 100, 4095), (700, 9, 1023)])
 def test_embedding_gradient_model_shapes(hip, ref, rng, v, d, n):
     """get_col backward (deterministic scatter-add), including a token count
     beyond the in-LDS index list, a vocabulary of thousands (most symbols without
@@ -429,6 +429,7 @@ def test_embedding_gradient_model_shapes(hip, ref, rng, v, d, n):
     w = rng.standard_normal((v, d)).astype(np.float32)
     idx = rng.integers(0, v, size=n).astype(np.int32)
     idx[: min(n, 7)] = 3  # repeated symbol
+    idx[n // 3: n // 3 + n // 5] = 5  # and a frequent one: a list of hundreds of tokens
     weight = rng.standard_normal((n, d)).astype(np.float32)
     res = []
     for nc in (hip, ref):
