@@ -447,6 +447,10 @@ int nchip_softmax_int(void *stream, const float *logits, int32_t *out, int v, in
    whatever sym[c] holds. */
 int nchip_cdf_path(void *stream, const uint16_t *cdf, const int32_t *sym, uint16_t *path,
                    int v, int64_t n, int levels);
+/* nchip_cdf_path of the table nchip_softmax_cdf16 would write, without the table: one read of the
+   logits, `levels` entries per column out (ceil(log2 v) <= levels <= 16).  Same values. */
+int nchip_softmax_cdf16_path(void *stream, const float *logits, const int32_t *sym, uint16_t *path,
+                             int v, int64_t n, int levels);
 /* sym[i, c] = largest s with cdf[s, c] <= target[i, c]; targets (m, n). */
 int nchip_cdf_lookup(void *stream, const uint16_t *cdf, const uint16_t *target,
                      uint16_t *sym, int v, int64_t m, int64_t n);

@@ -72,9 +72,15 @@ __device__ __forceinline__ unsigned long long wave_scan_incl(unsigned long long 
 // is (chunks before) + (waves before, via LDS) + (lanes before, via shuffles)
 // + (own earlier elements).  All sums are integers, so their grouping does
 // not change the result.
-template <int NT, int NC, bool KEEP>
+//
+// PATH: the caller knows each column's symbol and wants only what a coder reads for it - the CDF
+// entry at the split point of every level of the balanced tree over [0, v) (cp_utils.c:299-323),
+// `levels` 16-bit values per column, 0 below the leaf.  Nothing else is divided or stored: the
+// kernel is then one read of the logits.  Whatever the symbol's value, the split points lie in [1, v).
+template <int NT, int NC, bool KEEP, bool PATH>
 __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(const float *logits, uint16_t *cdf,
-                                                                        int v, int64_t ncol, int vec)
+                                                                        int v, int64_t ncol, int vec,
+                                                                        const int32_t *sym, uint16_t *path, int levels)
 {
     constexpr int NW = NT / 64;
     constexpr int UNR = KEEP ? NC : 1; // chunk loops stay rolled when chunks are re-read
@@ -87,7 +93,22 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(cons
     const int64_t col = NT == 64 ? (int64_t)blockIdx.x * 4 + ((int)threadIdx.x >> 6) : (int64_t)blockIdx.x;
     if (NT == 64 && col >= ncol) return; // whole wave; this shape uses no workgroup barrier
     const float *x = logits + col * v;
-    uint16_t *out = cdf + col * v;
+    uint16_t *out = PATH ? nullptr : cdf + col * v;
+    int split[PATH ? 16 : 1]; // the same for every thread of the column
+    if (PATH) {
+        const int s = sym[col];
+        int start = 0, len = v;
+#pragma unroll
+        for (int l = 0; l < 16; l++) {
+            split[l] = -1;
+            if (l < levels && len > 1) {
+                const int n0 = len >> 1;
+                split[l] = start + n0;
+                if (s >= start + n0) { start += n0; len -= n0; }
+                else len = n0;
+            }
+        }
+    }
 
     // KEEP: the logits stay in registers from the first read on; otherwise
     // (columns too long for that) each pass reads its chunk again, from L2
@@ -191,6 +212,22 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(cons
             chunk_base += wave_tot[c];
         }
         if (i0 >= v) continue;
+        if (PATH) {
+            uint16_t *po = path + col * levels;
+#pragma unroll
+            for (int l = 0; l < 16; l++) {
+                const int dj = split[l] - i0;
+                if (dj >= 0 && dj < 4) { // this thread owns the split point of level l
+                    unsigned long long r = run;
+#pragma unroll
+                    for (int j = 0; j < 3; j++) r += j < dj ? q[j] : 0u;
+                    po[l] = (uint16_t)(div_floor(r * scale, tot, inv) + (unsigned int)split[l]);
+                } else if (split[l] < 0 && l < levels && i0 == 0) {
+                    po[l] = 0; // below the leaf
+                }
+            }
+            continue;
+        }
         unsigned int o[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -410,25 +447,44 @@ extern "C" int nchip_softmax_int(void *stream, const float *logits, int32_t *out
     return 0;
 }
 
+template <bool PATH>
+static void launch_softmax_cdf16(hipStream_t st, const float *logits, uint16_t *cdf, int v, int64_t n, int vec,
+                                 const int32_t *sym, uint16_t *path, int levels)
+{
+    if (v <= 256)
+        hipLaunchKernelGGL((softmax_cdf16_kernel<64, 1, true, PATH>), dim3((unsigned)((n + 3) / 4)), dim3(256), 0, st, logits, cdf, v, n, vec, sym, path, levels);
+    else if (v <= 1024)
+        hipLaunchKernelGGL((softmax_cdf16_kernel<256, 1, true, PATH>), dim3((unsigned)n), dim3(256), 0, st, logits, cdf, v, n, vec, sym, path, levels);
+    else if (v <= 4096)
+        hipLaunchKernelGGL((softmax_cdf16_kernel<256, 4, true, PATH>), dim3((unsigned)n), dim3(256), 0, st, logits, cdf, v, n, vec, sym, path, levels);
+    else if (v <= 16384)
+        hipLaunchKernelGGL((softmax_cdf16_kernel<1024, 4, true, PATH>), dim3((unsigned)n), dim3(1024), 0, st, logits, cdf, v, n, vec, sym, path, levels);
+    else
+        hipLaunchKernelGGL((softmax_cdf16_kernel<1024, 16, false, PATH>), dim3((unsigned)n), dim3(1024), 0, st, logits, cdf, v, n, vec, sym, path, levels);
+}
+
 extern "C" int nchip_softmax_cdf16(void *stream, const float *logits, uint16_t *cdf, int v, int64_t n)
 {
     if (n <= 0) return 0;
     if (v < 1 || v > 65535) { fprintf(stderr, "nchip_softmax_cdf16: vocabulary %d outside [1, 65535]\n", v); return -1; }
-    hipStream_t st = (hipStream_t)stream;
     // 16-byte loads and 8-byte stores need every column to start aligned
     int vec = (v & 3) == 0 && ((uintptr_t)logits & 15) == 0 && ((uintptr_t)cdf & 7) == 0;
-    if (v <= 256)
-        hipLaunchKernelGGL((softmax_cdf16_kernel<64, 1, true>), dim3((unsigned)((n + 3) / 4)), dim3(256), 0, st, logits, cdf, v, n, vec);
-    else if (v <= 1024)
-        hipLaunchKernelGGL((softmax_cdf16_kernel<256, 1, true>), dim3((unsigned)n), dim3(256), 0, st, logits, cdf, v, n, vec);
-    else if (v <= 4096)
-        hipLaunchKernelGGL((softmax_cdf16_kernel<256, 4, true>), dim3((unsigned)n), dim3(256), 0, st, logits, cdf, v, n, vec);
-    else if (v <= 16384)
-        hipLaunchKernelGGL((softmax_cdf16_kernel<1024, 4, true>), dim3((unsigned)n), dim3(1024), 0, st, logits, cdf, v, n, vec);
-    else
-        hipLaunchKernelGGL((softmax_cdf16_kernel<1024, 16, false>), dim3((unsigned)n), dim3(1024), 0, st, logits, cdf, v, n, vec);
+    launch_softmax_cdf16<false>((hipStream_t)stream, logits, cdf, v, n, vec, nullptr, nullptr, 0);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { fprintf(stderr, "nchip_softmax_cdf16: %s\n", hipGetErrorString(e)); return -2; }
+    return 0;
+}
+
+extern "C" int nchip_softmax_cdf16_path(void *stream, const float *logits, const int32_t *sym, uint16_t *path,
+                                        int v, int64_t n, int levels)
+{
+    if (n <= 0 || levels <= 0) return 0;
+    if (v < 1 || v > 65535) { fprintf(stderr, "nchip_softmax_cdf16_path: vocabulary %d outside [1, 65535]\n", v); return -1; }
+    if (levels > 16 || (1 << levels) < v) { fprintf(stderr, "nchip_softmax_cdf16_path: %d levels for %d symbols\n", levels, v); return -1; }
+    int vec = (v & 3) == 0 && ((uintptr_t)logits & 15) == 0;
+    launch_softmax_cdf16<true>((hipStream_t)stream, logits, nullptr, v, n, vec, sym, path, levels);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { fprintf(stderr, "nchip_softmax_cdf16_path: %s\n", hipGetErrorString(e)); return -2; }
     return 0;
 }
 

@@ -1413,6 +1413,24 @@ extern "C" NCTensor *nc_cdf_path(NCTensor *cdf, NCTensor *symbols)
     return y;
 }
 
+extern "C" NCTensor *nc_soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols)
+{
+    logits = nc_contig(logits); symbols = nc_contig(symbols);
+    need_dev(logits, "nc_soft_max_cdf16_path"); need_dev(symbols, "nc_soft_max_cdf16_path");
+    if (logits->type != NC_TYPE_F32 || symbols->type != NC_TYPE_I32) nc_fatal("nc_soft_max_cdf16_path: f32 logits and i32 symbols expected");
+    size_t v = logits->dims[0], cols = v ? nc_numel(logits) / v : 0;
+    if (v == 0 || v > 65535) nc_fatal("nc_soft_max_cdf16_path: 1..65535 symbols expected");
+    if (nc_numel(symbols) != cols) nc_fatal("nc_soft_max_cdf16_path: one symbol per column of the logits expected");
+    size_t dims[2] = { (size_t)cdf_path_levels(v), cols };
+    NCTensor *y = nc_alloc(logits->dev, NC_TYPE_U16, 2, dims, false);
+    if (nchip_softmax_cdf16_path(nc_stream(logits), nc_f32(logits), (const int32_t *)nc_data(symbols),
+                                 (uint16_t *)nc_data(y), (int)v, (int64_t)cols, (int)dims[0]))
+        nc_fatal("nc_soft_max_cdf16_path failed");
+    LAUNCHED(logits);
+    nc_free_tensor(logits); nc_free_tensor(symbols);
+    return y;
+}
+
 // same arithmetic as the device exponential of k_cdf.hip, for host callers
 extern "C" float nc_exp_det(float x)
 {

@@ -76,8 +76,9 @@ typedef struct {
     size_t stride;
 } HostDist;
 
-/* `symbols` (consumed; may be NULL): the symbol of every column, known to an encoder before it
-   codes.  With them only the CDF entries that the coder will read cross to the host. */
+/* `symbols` (consumed; may be NULL): the symbol of every column, one I32 each on the model's
+   device, known to an encoder before it codes.  With them only the CDF entries that the coder
+   will read cross to the host. */
 static HostDist fetch_dist(Coder *c, NCTensor *output, NCTensor *symbols)
 {
     HostDist d;
@@ -88,11 +89,8 @@ static HostDist fetch_dist(Coder *c, NCTensor *output, NCTensor *symbols)
         int nd = nc_tensor_get_dims(logits, dims);
         for (int i = 1; i < nd; i++) cols *= dims[i];
         nc_free_tensor(output);
-        if (symbols) {
-            NCDevice *dev = nc_get_tensor_device(logits);
-            size_t n1 = cols;
-            NCTensor *sym = nc_tensor_to_device(nc_reshape_1d(symbols, n1), dev);
-            d.host = nc_tensor_to_cpu_device(nc_cdf_path(nc_soft_max_cdf16(nc_dup_tensor(logits)), sym));
+        if (symbols) { /* already on the model's device */
+            d.host = nc_tensor_to_cpu_device(nc_soft_max_cdf16_path(nc_dup_tensor(logits), symbols));
             d.path = nc_tensor_get_ptr(d.host, &d.stride);
             return d;
         }
@@ -160,6 +158,11 @@ static HostDist encode_segment_eval(Coder *c, int idx, int n_t, int len2, int fu
             if (symbols) nc_set1_i32_2d(symbols, b, t, get_symb(&c->view, b, idx + t));
         }
     double t0 = now_s();
+    if (symbols) { /* up before the evaluation is queued: an upload waits for the stream */
+        size_t dims[2];
+        nc_tensor_get_dims(symbols, dims);
+        symbols = nc_tensor_to_device(nc_reshape_1d(symbols, dims[0] * dims[1]), nncp_model_device(c->s));
+    }
     NCTensor *out = c->cls->eval(c->s, -1, input);
     HostDist d = fetch_dist(c, out, symbols);
     c->st->t_eval += now_s() - t0;

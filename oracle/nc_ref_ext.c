@@ -444,6 +444,11 @@ NCTensor *nc_cdf_path(NCTensor *cdf, NCTensor *symbols)
     return y;
 }
 
+NCTensor *nc_soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols) /* nc_ext.h: by its definition */
+{
+    return nc_cdf_path(nc_soft_max_cdf16(logits), symbols);
+}
+
 NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets)
 {
     NCTensor *y;

@@ -271,7 +271,8 @@ def test_cdf_lookup_bit_exact(hip, ref, rng, V, n, m):
     assert np.array_equal(res[0], res[1])
 
 
-@pytest.mark.parametrize("V,n", [(256, 2048), (16384, 129), (2, 5), (3, 300), (1000, 257), (65535, 9)])
+@pytest.mark.parametrize("V,n", [(256, 2048), (16384, 129), (2, 5), (3, 300), (1000, 257), (65535, 9), (4096, 40), (1, 7),
+                                 (255, 33), (4097, 12)])
 def test_cdf_path_bit_exact(hip, ref, rng, V, n):
     """The CDF entries an encoder's coder reads for known symbols (symbols outside the alphabet
     included: they read nothing outside their column)."""
@@ -282,6 +283,10 @@ def test_cdf_path_bit_exact(hip, ref, rng, V, n):
     for nc in (hip, ref):
         res.append(nc.numpy(nc.nc_cdf_path(nc.nc_soft_max_cdf16(nc.tensor(x)), nc.tensor(sym)), free=True))
     assert res[0].shape == (x.shape[0], max(1, int(np.ceil(np.log2(V))))) and np.array_equal(res[0], res[1])
+    # and in one pass over the logits, the table never written (every kernel shape of the CDF build)
+    for nc in (hip, ref):
+        one = nc.numpy(nc.nc_soft_max_cdf16_path(nc.tensor(x), nc.tensor(sym)), free=True)
+        assert np.array_equal(one, res[0])
 
 
 @pytest.mark.parametrize("algo", [16, 1, 0])
