@@ -625,12 +625,32 @@ void nc_copy_any(NCTensor *dst, const NCTensor *src)
     if (dst->dev != src->dev)
         nc_fatal("copy: tensors live on different devices");
     if (nc_numel(dst) == 0) return;
+    // A contiguous range written into a buffer whose bf16 copy is in use (the memory of a layer,
+    // which takes a new segment per step): the copy is brought up to date over that range - from
+    // the source's own copy when it has one, else by a cast of the range - instead of being
+    // dropped and rebuilt over the whole buffer at its next use.
+    const bool keep_shadow = dst->dev->is_hip && dst->dev->ctx->matmul_bf16 && dst->buf->sh && dst->buf->sh_valid &&
+                             shadow_capable(dst) && nc_is_contig(src) && nc_numel(dst) < dst->buf->elems;
     nc_shadow_invalidate(dst);
     if (!dst->dev->is_hip) { host_copy_strided(dst, src); return; }
     NCContext *m = dst->dev->ctx;
     if (nc_is_contig(dst) && nc_is_contig(src)) {
-        hip_check(hipMemcpyAsync(nc_data(dst), nc_data(src), nc_numel(dst) * nc_type_size(dst->type),
+        const size_t n = nc_numel(dst);
+        hip_check(hipMemcpyAsync(nc_data(dst), nc_data(src), n * nc_type_size(dst->type),
                                  hipMemcpyDeviceToDevice, m->stream), "hipMemcpyAsync d2d");
+        if (keep_shadow) {
+            uint16_t *range = dst->buf->sh + dst->off;
+            // (within one buffer the flag was just cleared: a cast of the range then)
+            if (src->buf != dst->buf && src->buf->sh && src->buf->sh_valid && shadow_capable(src))
+                hip_check(hipMemcpyAsync(range, src->buf->sh + src->off, n * sizeof(uint16_t), hipMemcpyDeviceToDevice, m->stream),
+                          "hipMemcpyAsync d2d (bf16 copy)");
+            else {
+                if (nchip_cast_bf16(m->stream, nc_f32(dst), range, (int64_t)n)) nc_fatal("bf16 cast failed");
+                m->launches++;
+                m->shadow_casts++;
+            }
+            dst->buf->sh_valid = true;
+        }
         return;
     }
     NdDesc d;

@@ -32,6 +32,10 @@ struct NNCPModel {
     Layer *layers;
     NCTensor *ln_g, *ln_b, *embed, *embed_out, *out_bias;
     NCTensor **mem_h, **train_h, **outputs;
+    /* on the GPU with mem_len > seg_len: mem_h[l] is a window of mem_len steps in mem_store[l]
+       (mem_cap steps), which an update moves by one segment instead of shifting the rows */
+    NCTensor **mem_store;
+    int *mem_pos, mem_cap;
     NCTensor **step_kv, **step_kvm; /* per-timestep decoding: K/V of the segment so far, K/V of the memory */
     NCTensor *step_embed_mult; /* the embedding scale as a device scalar, kept for the timesteps of a segment */
     int step_logits_only;      /* trf_eval_step returns the logits: the caller builds integer CDFs from them */

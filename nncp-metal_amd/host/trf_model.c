@@ -150,8 +150,25 @@ NNCPModel *nncp_model_new(const NNCPConfig *cfg)
         new_param(s, &s->out_bias, nc_new_tensor_1d(s->dev, s->param_type, c->n_symbols), 0, "out_bias", 0);
     s->mem_h = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
     s->train_h = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
+    s->mem_store = nc_mallocz(sizeof(NCTensor *) * c->n_layer);
+    s->mem_pos = nc_mallocz(sizeof(int) * c->n_layer);
+    s->mem_cap = 0;
+    if (c->use_device && M > T) {
+        /* room for the window to move: up to 8 segments, at most 256 MiB, behind the memory */
+        size_t seg_bytes = (size_t)D * B * T * sizeof(float);
+        size_t slack = ((size_t)256 << 20) / seg_bytes;
+        slack = slack < 1 ? 1 : (slack > 8 ? 8 : slack);
+        const char *e = getenv("NNCP_MEM_SLACK_SEGMENTS"); /* tests: 1 makes the window start over at every other update */
+        if (e && atoi(e) >= 1 && atoi(e) <= 64) slack = (size_t)atoi(e);
+        s->mem_cap = M + (int)slack * T;
+    }
     for (int l = 0; l < c->n_layer; l++) {
-        s->mem_h[l] = nc_new_tensor_3d(s->dev, NC_TYPE_F32, D, B, M);
+        if (s->mem_cap) {
+            s->mem_store[l] = nc_new_tensor_3d(s->dev, NC_TYPE_F32, D, B, s->mem_cap);
+            s->mem_h[l] = nc_slice_alias(s->mem_store[l], 2, 0, M);
+        } else {
+            s->mem_h[l] = nc_new_tensor_3d(s->dev, NC_TYPE_F32, D, B, M);
+        }
         s->train_h[l] = nc_new_tensor_3d(s->dev, NC_TYPE_F32, D, B, T);
     }
     s->outputs = nc_mallocz(sizeof(NCTensor *) * T);
@@ -173,13 +190,13 @@ void nncp_model_free(NNCPModel *s) /* trf_end nncp.c:522-550, nncp_end nncp.c:28
     trf_eval_end(s);
     for (int l = 0; l < s->cfg.n_layer; l++) {
         Layer *tl = &s->layers[l];
-        nc_free_tensor(s->mem_h[l]); nc_free_tensor(s->train_h[l]);
+        nc_free_tensor(s->mem_h[l]); nc_free_tensor(s->mem_store[l]); nc_free_tensor(s->train_h[l]);
         nc_free_tensor(tl->mem_key); nc_free_tensor(tl->mem_value); nc_free_tensor(tl->attn_mask);
         nc_free(tl->key_nodes); nc_free(tl->kq_nodes); nc_free(tl->value_nodes); nc_free(tl->va_nodes);
     }
     trf_step_end(s);
     nc_free(s->step_kv); nc_free(s->step_kvm);
-    nc_free(s->mem_h); nc_free(s->train_h); nc_free(s->outputs);
+    nc_free(s->mem_h); nc_free(s->mem_store); nc_free(s->mem_pos); nc_free(s->train_h); nc_free(s->outputs);
     nc_sgd_opt_set_all(&s->params, NULL);
     nc_sgd_opt_end(s->opt);
     nc_param_list_end(&s->params);
@@ -907,7 +924,24 @@ void trf_update(NNCPModel *s) /* nncp.c:1224-1235 with mem_update nncp.c:1205-12
     prof_start(PROF_UPDATE); /* nncp.c:1227 */
     nc_sgd_opt_update(s->opt);
     for (int l = 0; l < s->cfg.n_layer && M > 0; l++) {
-        if (M > T) {
+        if (M > T && s->mem_cap) {
+            /* the same memory as below, at a new place: the segment goes behind the window
+               and the window moves on by T; at the end of the store the rows that stay go
+               back to its start (once in mem_cap / T - M / T + 1 updates) */
+            NCTensor *store = s->mem_store[l];
+            int pos = s->mem_pos[l];
+            if (pos + M + T <= s->mem_cap) {
+                nc_tensor_copy_slice(store, s->train_h[l], 2, pos + M, pos + M + T, 0);
+                pos += T;
+            } else {
+                nc_tensor_copy_slice(store, store, 2, 0, M - T, pos + T);
+                nc_tensor_copy_slice(store, s->train_h[l], 2, M - T, M, 0);
+                pos = 0;
+            }
+            s->mem_pos[l] = pos;
+            nc_free_tensor(s->mem_h[l]);
+            s->mem_h[l] = nc_slice_alias(store, 2, pos, pos + M);
+        } else if (M > T) {
             nc_tensor_copy_slice(s->mem_h[l], s->mem_h[l], 2, 0, M - T, T);
             nc_tensor_copy_slice(s->mem_h[l], s->train_h[l], 2, M - T, M, 0);
         } else if (M == T) {

@@ -418,3 +418,47 @@ def test_enwik8_profile_round_trips_a_small_file_on_gpu(hosts, tmp_path):
     assert 0 < os.path.getsize(packed) < n * 1.1              # an untrained model: about 8 bits a byte
     hp.decode_file(hosts[0], packed, back, use_device=1, nb_threads=4)
     assert open(back, "rb").read() == open(src, "rb").read()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bf16", [0, 1])
+def test_memory_window_moves_and_starts_over_without_changing_a_bit(monkeypatch, bf16):
+    """A memory longer than the segment lives, on the GPU, in a store with room behind it: an
+    update writes the new segment behind the window and moves the window instead of shifting the
+    rows, and at the end of the store the rows that stay go back to its start.  Seven steps with
+    room for one segment (the window starts over at every other update), with the default room
+    (it does not) and on the checker (which shifts, nncp.c:1205-1221): the two GPU runs agree
+    bit for bit in probabilities, loss and memories, and with the checker at the variant's bar.
+    With bf16 products the consistency checker of the operand copies is on: the copy of the
+    store is kept up to date over each written range, and a stale one ends the process."""
+    hp = M.load_pkg().host
+    cfg = dict(n_layer=2, d_model=128, n_head=2, d_inner=256, d_pos=48, mem_len=40, seg_len=16,
+               batch_size=8, n_symbols=64, seed=5)
+    n_steps = 7
+    syms = M.markov1(cfg["batch_size"] * cfg["seg_len"] * n_steps, cfg["n_symbols"], seed=6)
+    batches = M.segment_batches(syms, cfg["batch_size"], cfg["seg_len"], n_steps)
+    runs = []
+    for host, dev, room in ((M.hip_host(), 1, "1"), (M.hip_host(), 1, None), (M.ref_host(), 0, None)):
+        if room:
+            monkeypatch.setenv("NNCP_MEM_SLACK_SEGMENTS", room)
+        else:
+            monkeypatch.delenv("NNCP_MEM_SLACK_SEGMENTS", raising=False)
+        m = hp.Model(host, hp.make_config(**dict(cfg, use_device=dev, fused=1, nb_threads=4, sgd_opt=M.rmsprop(3e-4))))
+        m.nc.nc_set_matmul_bf16(m.ctx, bf16)
+        old = m.nc.nc_set_bf16_shadow_check(bf16)
+        out = []
+        for tok, tgt in batches:
+            p, loss = m.train_step(tok, tgt, 3e-4)
+            out.append((p, loss, m.state()["mem"]))
+        m.nc.nc_set_bf16_shadow_check(old)
+        m.nc.nc_set_matmul_bf16(m.ctx, 0)
+        m.close()
+        runs.append(out)
+    tol = 2e-2 if bf16 else 1e-5
+    for (pa, la, ma), (pb, lb, mb), (pr, lr_, mr) in zip(*runs):
+        assert np.array_equal(pa, pb) and la == lb
+        for x, y, z in zip(ma, mb, mr):
+            assert x.shape == z.shape
+            assert np.array_equal(x, y)
+            assert M.rel_l2(x, z) <= tol     # (hidden states: in the norm the variant's bar is stated in)
+        assert M.relerr(pa, pr) <= tol and abs(la - lr_) <= tol * abs(lr_)

@@ -64,7 +64,8 @@ def test_gpu_parity_tests_pass_on_the_cpu_build(emulated):
     # (and the full-size round trip is hours of fibers: it waits for the GPU)
     new = _pytest(emulated, ["-n", "6", "tests/test_gpu_zz_new_paths.py", "-k",
                              "not (file_container and (reference or bf16)) and not full_size and "
-                             "not (properties_small and bf16) and not 100_steps and not enwik8_profile"])
+                             "not (properties_small and bf16) and not 100_steps and not enwik8_profile and "
+                             "not (memory_window and 0)"])
     out_ops, out_model = ops.communicate(timeout=1500)[0], model.communicate(timeout=1500)[0]
     out_new = new.communicate(timeout=1500)[0]
     assert ops.returncode == 0, out_ops[-3000:]
