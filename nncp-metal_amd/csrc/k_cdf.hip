@@ -192,9 +192,23 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(cons
     const unsigned long long scale = (unsigned long long)(65536 - v);
     const double inv = 1.0 / (double)tot;
     unsigned long long chunk_base = 0;
+    if (PATH && t == 0) {
+#pragma unroll
+        for (int l = 0; l < 16; l++)
+            if (split[l] < 0 && l < levels) path[col * levels + l] = 0; // below the leaf
+    }
 #pragma unroll UNR
     for (int c = 0; c < NC; c++) {
         int i0 = (c * NT + t) * 4;
+        if (PATH) {
+            // the 256 elements of this wave in this chunk hold a split point, or nothing here is needed
+            // (NT == 64 adds the chunks up as it goes, so it passes through all of them)
+            const int w0 = (c * NT + wave * 64) * 4;
+            bool hit = NT == 64;
+#pragma unroll
+            for (int l = 0; l < 16; l++) hit = hit || (split[l] >= w0 && split[l] < w0 + 256);
+            if (!hit) continue; // the same for the whole wave
+        }
         unsigned int q[4];
         unsigned long long s = 0;
         float f[4];
@@ -214,17 +228,26 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(cons
         if (i0 >= v) continue;
         if (PATH) {
             uint16_t *po = path + col * levels;
+            unsigned int own = 0; // the levels whose split point is one of this thread's four elements
 #pragma unroll
             for (int l = 0; l < 16; l++) {
                 const int dj = split[l] - i0;
-                if (dj >= 0 && dj < 4) { // this thread owns the split point of level l
-                    unsigned long long r = run;
+                own |= (unsigned int)(dj >= 0 && dj < 4) << l;
+            }
+            if (own) { // rare: at most 16 threads of a column divide at all
+                unsigned int o[4];
+                unsigned long long r = run;
 #pragma unroll
-                    for (int j = 0; j < 3; j++) r += j < dj ? q[j] : 0u;
-                    po[l] = (uint16_t)(div_floor(r * scale, tot, inv) + (unsigned int)split[l]);
-                } else if (split[l] < 0 && l < levels && i0 == 0) {
-                    po[l] = 0; // below the leaf
+                for (int j = 0; j < 4; j++) {
+                    o[j] = div_floor(r * scale, tot, inv) + (unsigned int)(i0 + j);
+                    r += q[j];
                 }
+#pragma unroll
+                for (int l = 0; l < 16; l++)
+                    if (own >> l & 1) {
+                        const int dj = split[l] - i0;
+                        po[l] = (uint16_t)(dj == 0 ? o[0] : dj == 1 ? o[1] : dj == 2 ? o[2] : o[3]);
+                    }
             }
             continue;
         }

@@ -283,10 +283,21 @@ def test_cdf_path_bit_exact(hip, ref, rng, V, n):
     for nc in (hip, ref):
         res.append(nc.numpy(nc.nc_cdf_path(nc.nc_soft_max_cdf16(nc.tensor(x)), nc.tensor(sym)), free=True))
     assert res[0].shape == (x.shape[0], max(1, int(np.ceil(np.log2(V))))) and np.array_equal(res[0], res[1])
-    # and in one pass over the logits, the table never written (every kernel shape of the CDF build)
+    # and as one op (which builds no table for columns up to 1024 entries)
     for nc in (hip, ref):
         one = nc.numpy(nc.nc_soft_max_cdf16_path(nc.tensor(x), nc.tensor(sym)), free=True)
         assert np.array_equal(one, res[0])
+    # the build kernel's own path form through its entry point, for every kernel shape of the build
+    lib = C.CDLL(hip.lib._name)
+    lib.nchip_softmax_cdf16_path.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int]
+    st = C.c_void_p(hip.nc_context_stream(hip.ctx))
+    ptr = lambda t: C.c_void_p(hip.lib.nc_tensor_get_ptr(t, None))
+    levels = res[0].shape[1]
+    tx, ts, tp = hip.tensor(x), hip.tensor(sym), hip.tensor(np.full(res[0].shape, 0xABCD, np.uint16))
+    assert lib.nchip_softmax_cdf16_path(st, ptr(tx), ptr(ts), ptr(tp), V, x.shape[0], levels) == 0
+    got = hip.numpy(tp)
+    hip.free(tx, ts, tp)
+    assert np.array_equal(got, res[0])
 
 
 @pytest.mark.parametrize("algo", [16, 1, 0])
