@@ -158,8 +158,9 @@ int64_t nncp_model_train_step(NNCPModel *s);
    for tests that put two models into the same state: the optimiser's moment `which` of the
    named parameter (nc_sgd_opt_get_state / nc_sgd_opt_set_state of nc_ext.h; get returns an
    owned host tensor or NULL, set copies v in) and the memory of layer l, the (d_model, B,
-   mem_len) tensor mem_h[l] of nncp.c:1205-1221 (borrowed; Transformer models only, NULL for
-   an LSTM or without memory). */
+   mem_len) tensor mem_h[l] of nncp.c:1205-1221 (borrowed until the model's next update, which
+   may replace it: on the GPU a memory longer than a segment is a window that moves through a
+   larger store; Transformer models only, NULL for an LSTM or without memory). */
 NCTensor *nncp_model_opt_state(NNCPModel *s, const char *name, int which);
 void nncp_model_set_opt_state(NNCPModel *s, const char *name, int which, const NCTensor *v);
 NCTensor *nncp_model_memory(NNCPModel *s, int l);
