@@ -133,9 +133,8 @@ NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets);
    per column to the host instead of the V of the column.  Consumes both.  No counterpart in
    the reference. */
 NCTensor *nc_cdf_path(NCTensor *cdf, NCTensor *symbols);
-/* nc_cdf_path(nc_soft_max_cdf16(logits), symbols) as one op: for columns of up to 1024 entries one
-   pass over the logits that writes no table, for longer ones the composition itself (a temporary
-   table on the device).  Same values.  Consumes both. */
+/* nc_cdf_path(nc_soft_max_cdf16(logits), symbols) in one pass over the logits: the table itself is
+   never written.  Same values.  Consumes both. */
 NCTensor *nc_soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols);
 
 /* The deterministic exponential used by nc_soft_max_cdf16, for x <= 0:

@@ -77,8 +77,10 @@ __device__ __forceinline__ unsigned long long wave_scan_incl(unsigned long long 
 // entry at the split point of every level of the balanced tree over [0, v) (cp_utils.c:299-323),
 // `levels` 16-bit values per column, 0 below the leaf.  Nothing else is divided or stored: the
 // kernel is then one read of the logits.  Whatever the symbol's value, the split points lie in [1, v).
+// (eight waves per SIMD asked of the compiler: two 1024-thread workgroups share a CU only when the
+// scalar registers allow all 32 waves, and with one the phases of a column have nothing to overlap)
 template <int NT, int NC, bool KEEP, bool PATH>
-__global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(const float *logits, uint16_t *cdf,
+__global__ __launch_bounds__(NT == 64 ? 256 : NT) __attribute__((amdgpu_waves_per_eu(NT >= 1024 ? 8 : 4))) void softmax_cdf16_kernel(const float *logits, uint16_t *cdf,
                                                                         int v, int64_t ncol, int vec,
                                                                         const int32_t *sym, uint16_t *path, int levels)
 {
@@ -94,19 +96,26 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(cons
     if (NT == 64 && col >= ncol) return; // whole wave; this shape uses no workgroup barrier
     const float *x = logits + col * v;
     uint16_t *out = PATH ? nullptr : cdf + col * v;
-    int split[PATH ? 16 : 1]; // the same for every thread of the column
+    // the split points of the symbol's walk, the same for every thread of the column: two 16-bit
+    // values per register (a split point is below v <= 65535; 0xffff = the walk ended above this level)
+    unsigned int split2[PATH ? 8 : 1];
+    auto split_at = [&](int l) -> int {
+        const unsigned int s16 = (split2[l >> 1] >> ((l & 1) * 16)) & 0xffffu;
+        return s16 == 0xffffu ? -1 : (int)s16;
+    };
     if (PATH) {
         const int s = sym[col];
         int start = 0, len = v;
 #pragma unroll
         for (int l = 0; l < 16; l++) {
-            split[l] = -1;
+            unsigned int here = 0xffffu;
             if (l < levels && len > 1) {
                 const int n0 = len >> 1;
-                split[l] = start + n0;
+                here = (unsigned int)(start + n0);
                 if (s >= start + n0) { start += n0; len -= n0; }
                 else len = n0;
             }
+            split2[l >> 1] = (l & 1) ? (split2[l >> 1] | here << 16) : here;
         }
     }
 
@@ -195,7 +204,7 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(cons
     if (PATH && t == 0) {
 #pragma unroll
         for (int l = 0; l < 16; l++)
-            if (split[l] < 0 && l < levels) path[col * levels + l] = 0; // below the leaf
+            if (split_at(l) < 0 && l < levels) path[col * levels + l] = 0; // below the leaf
     }
 #pragma unroll UNR
     for (int c = 0; c < NC; c++) {
@@ -206,7 +215,7 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(cons
             const int w0 = (c * NT + wave * 64) * 4;
             bool hit = NT == 64;
 #pragma unroll
-            for (int l = 0; l < 16; l++) hit = hit || (split[l] >= w0 && split[l] < w0 + 256);
+            for (int l = 0; l < 16; l++) hit = hit || (split_at(l) >= w0 && split_at(l) < w0 + 256);
             if (!hit) continue; // the same for the whole wave
         }
         unsigned int q[4];
@@ -231,8 +240,8 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(cons
             unsigned int own = 0; // the levels whose split point is one of this thread's four elements
 #pragma unroll
             for (int l = 0; l < 16; l++) {
-                const int dj = split[l] - i0;
-                own |= (unsigned int)(dj >= 0 && dj < 4) << l;
+                const int dj = split_at(l) - i0;
+                own |= (unsigned int)(split_at(l) >= 0 && dj >= 0 && dj < 4) << l;
             }
             if (own) { // rare: at most 16 threads of a column divide at all
                 unsigned int o[4];
@@ -245,7 +254,7 @@ __global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_cdf16_kernel(cons
 #pragma unroll
                 for (int l = 0; l < 16; l++)
                     if (own >> l & 1) {
-                        const int dj = split[l] - i0;
+                        const int dj = split_at(l) - i0;
                         po[l] = (uint16_t)(dj == 0 ? o[0] : dj == 1 ? o[1] : dj == 2 ? o[2] : o[3]);
                     }
             }

@@ -1421,10 +1421,6 @@ extern "C" NCTensor *nc_soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols)
     size_t v = logits->dims[0], cols = v ? nc_numel(logits) / v : 0;
     if (v == 0 || v > 65535) nc_fatal("nc_soft_max_cdf16_path: 1..65535 symbols expected");
     if (nc_numel(symbols) != cols) nc_fatal("nc_soft_max_cdf16_path: one symbol per column of the logits expected");
-    // Long columns: the build kernel is bound by its own arithmetic, not by the table it writes, and
-    // its path form costs more than the thread-per-column gather after it (measured at 16384 entries x
-    // 4096 columns: 203 us against 176 + 9 us), so the table goes to a temporary there.  Same values.
-    if (v > 1024) return nc_cdf_path(nc_soft_max_cdf16(logits), symbols);
     size_t dims[2] = { (size_t)cdf_path_levels(v), cols };
     NCTensor *y = nc_alloc(logits->dev, NC_TYPE_U16, 2, dims, false);
     if (nchip_softmax_cdf16_path(nc_stream(logits), nc_f32(logits), (const int32_t *)nc_data(symbols),

@@ -283,7 +283,7 @@ def test_cdf_path_bit_exact(hip, ref, rng, V, n):
     for nc in (hip, ref):
         res.append(nc.numpy(nc.nc_cdf_path(nc.nc_soft_max_cdf16(nc.tensor(x)), nc.tensor(sym)), free=True))
     assert res[0].shape == (x.shape[0], max(1, int(np.ceil(np.log2(V))))) and np.array_equal(res[0], res[1])
-    # and as one op (which builds no table for columns up to 1024 entries)
+    # and as one op (no table is built)
     for nc in (hip, ref):
         one = nc.numpy(nc.nc_soft_max_cdf16_path(nc.tensor(x), nc.tensor(sym)), free=True)
         assert np.array_equal(one, res[0])
