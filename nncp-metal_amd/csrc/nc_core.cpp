@@ -784,7 +784,11 @@ extern "C" NCTensor *nc_tensor_to_device(NCTensor *x, NCDevice *d)
         hip_check(hipMemcpyAsync(nc_data(y), nc_data(x), bytes,
                                  d->is_hip ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost, m->stream),
                   "hipMemcpyAsync");
-        nc_stream_wait(m);
+        // An upload from a pinned host tensor that ends here (this was its last reference, so no
+        // caller can write it again): the copy stays queued and the buffer is recycled after the
+        // next wait.  Any other transfer is complete on return.
+        if (d->is_hip && x->ref == 1 && x->buf->ref == 1) nc_mark_in_flight(x);
+        else nc_stream_wait(m);
     }
     nc_free_tensor(x);
     return y;
