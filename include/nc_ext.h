@@ -136,6 +136,13 @@ NCTensor *nc_cdf_path(NCTensor *cdf, NCTensor *symbols);
 /* nc_cdf_path(nc_soft_max_cdf16(logits), symbols) in one pass over the logits: the table itself is
    never written.  Same values.  Consumes both. */
 NCTensor *nc_soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols);
+/* nc_soft_max_cdf16_path with the result on the host device, written there by the kernel itself
+   (pinned memory), and nc_tensor_to_cpu_device without its wait: in both cases the contents are
+   valid after the next nc_synchronize of the source's device.  An encoder queues everything it
+   wants from an evaluation - these entries, the loss - and waits once.  No counterpart in the
+   reference (libnc_ref.so: the plain forms). */
+NCTensor *nc_soft_max_cdf16_path_to_host(NCTensor *logits, NCTensor *symbols);
+NCTensor *nc_tensor_to_cpu_device_queued(NCTensor *x);
 
 /* The deterministic exponential used by nc_soft_max_cdf16, for x <= 0:
    n = rint(x*log2e); r = x - n*ln2 (two fmaf steps); degree-6 polynomial in

@@ -206,6 +206,12 @@ typedef struct {
     /* eval_end for an evaluation that is to leave no trace (the replaying decoder of
        NNCP_MODE_SEGMENT): also takes back the recurrent state it handed on */
     void (*eval_discard)(NNCPModel *s);
+    /* optional (NULL: not offered).  After a whole-segment eval, with the expected symbols
+       already on the model's device ((B, T) i32, consumed): queues the loss of that evaluation
+       and its transfer to the host, without waiting.  The eval_gradient that follows - after
+       the caller has synchronised the device for its own purposes - takes the loss from there
+       instead of uploading `expected_output`, computing it and waiting for it. */
+    void (*queue_loss)(NNCPModel *s, NCTensor *expected_on_device);
 } NNCPModelClass;
 const NNCPModelClass *nncp_model_class(NNCPModel *s);
 /* logits of the last evaluation of either class (V, B, T|1), borrowed */

@@ -133,7 +133,8 @@ _PROTOS = {
     "nc_set_matmul_width_invariant": (_I, [_P, _I]),
     "nc_relpos_attention": (_P, [_P, _P, _P, _P, _P, _I, _I, _I, _F]),
     "nc_soft_max_int": (_P, [_P, C.c_float]),
-    "nc_soft_max_cdf16": (_P, [_P]), "nc_cdf_lookup": (_P, [_P, _P]), "nc_cdf_path": (_P, [_P, _P]), "nc_soft_max_cdf16_path": (_P, [_P, _P]),
+    "nc_soft_max_cdf16": (_P, [_P]), "nc_cdf_lookup": (_P, [_P, _P]), "nc_cdf_path": (_P, [_P, _P]), "nc_soft_max_cdf16_path": (_P, [_P, _P]), "nc_soft_max_cdf16_path_to_host": (_P, [_P, _P]),
+    "nc_tensor_to_cpu_device_queued": (_P, [_P]),
     "nc_soft_max_cdf16_to_host": (_P, [_P]), "nc_get_col_host_indices": (_P, [_P, _P, C.c_float]),
     "nc_exp_det": (_F, [_F]),
     "nc_set_matmul_bf16": (_I, [_P, _I]),

@@ -810,6 +810,21 @@ extern "C" NCTensor *nc_tensor_to_cpu_device(NCTensor *x)
     return y;
 }
 
+extern "C" NCTensor *nc_tensor_to_cpu_device_queued(NCTensor *x) // nc_ext.h: valid after the next wait
+{
+    NCContext *m = x->dev->ctx;
+    if (!x->dev->is_hip) return nc_contig(x);
+    NCTensor *c = nc_contig(x);
+    NCTensor *y = nc_alloc(&m->cpu, c->type, c->n_dims, c->dims, false);
+    size_t bytes = nc_numel(c) * nc_type_size(c->type);
+    if (bytes) {
+        hip_check(hipMemcpyAsync(nc_data(y), nc_data(c), bytes, hipMemcpyDeviceToHost, m->stream), "hipMemcpyAsync d2h");
+        nc_mark_in_flight(y);
+    }
+    nc_free_tensor(c);
+    return y;
+}
+
 extern "C" float nc_get_scalar_f32(const NCTensor *x) // libnc.h:214 (synchronises)
 {
     if (nc_numel(x) != 1 || x->type != NC_TYPE_F32) nc_fatal("get_scalar_f32: f32 scalar expected");

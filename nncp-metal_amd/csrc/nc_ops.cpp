@@ -1413,7 +1413,11 @@ extern "C" NCTensor *nc_cdf_path(NCTensor *cdf, NCTensor *symbols)
     return y;
 }
 
-extern "C" NCTensor *nc_soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols)
+static NCTensor *soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols, bool to_host);
+extern "C" NCTensor *nc_soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols) { return soft_max_cdf16_path(logits, symbols, false); }
+extern "C" NCTensor *nc_soft_max_cdf16_path_to_host(NCTensor *logits, NCTensor *symbols) { return soft_max_cdf16_path(logits, symbols, true); }
+
+static NCTensor *soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols, bool to_host)
 {
     logits = nc_contig(logits); symbols = nc_contig(symbols);
     need_dev(logits, "nc_soft_max_cdf16_path"); need_dev(symbols, "nc_soft_max_cdf16_path");
@@ -1422,11 +1426,12 @@ extern "C" NCTensor *nc_soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols)
     if (v == 0 || v > 65535) nc_fatal("nc_soft_max_cdf16_path: 1..65535 symbols expected");
     if (nc_numel(symbols) != cols) nc_fatal("nc_soft_max_cdf16_path: one symbol per column of the logits expected");
     size_t dims[2] = { (size_t)cdf_path_levels(v), cols };
-    NCTensor *y = nc_alloc(logits->dev, NC_TYPE_U16, 2, dims, false);
+    NCTensor *y = nc_alloc(to_host ? &nc_ctx(logits)->cpu : logits->dev, NC_TYPE_U16, 2, dims, false);
     if (nchip_softmax_cdf16_path(nc_stream(logits), nc_f32(logits), (const int32_t *)nc_data(symbols),
                                  (uint16_t *)nc_data(y), (int)v, (int64_t)cols, (int)dims[0]))
         nc_fatal("nc_soft_max_cdf16_path failed");
     LAUNCHED(logits);
+    if (to_host) nc_mark_in_flight(y); // freed before the next wait, the buffer must not serve another tensor yet
     nc_free_tensor(logits); nc_free_tensor(symbols);
     return y;
 }

@@ -340,5 +340,5 @@ static NCTensor *lstm_last_logits(NNCPModel *s) { return s->lstm->logits; }
 
 const NNCPModelClass nncp_lstm_class = { /* nncp.c:2312-2330 */
     lstm_eval, lstm_eval_end, lstm_eval_gradient, lstm_reset, lstm_update, lstm_set_lr, lstm_set_retrain,
-    lstm_last_logits, lstm_eval_discard,
+    lstm_last_logits, lstm_eval_discard, NULL,
 };

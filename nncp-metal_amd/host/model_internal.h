@@ -40,6 +40,7 @@ struct NNCPModel {
     NCTensor *step_embed_mult; /* the embedding scale as a device scalar, kept for the timesteps of a segment */
     int step_logits_only;      /* trf_eval_step returns the logits: the caller builds integer CDFs from them */
     NCTensor *logits;
+    NCTensor *pending_loss, *pending_loss_host; /* queue_loss: the summed log-likelihood with its graph, and its copy on the way to the host */
     NCSGDOptState *opt;
     int seq_eval;
     float embed_mult;

@@ -90,7 +90,9 @@ static HostDist fetch_dist(Coder *c, NCTensor *output, NCTensor *symbols)
         for (int i = 1; i < nd; i++) cols *= dims[i];
         nc_free_tensor(output);
         if (symbols) { /* already on the model's device */
-            d.host = nc_tensor_to_cpu_device(nc_soft_max_cdf16_path(nc_dup_tensor(logits), symbols));
+            NCDevice *dev = nc_get_tensor_device(logits);
+            d.host = nc_soft_max_cdf16_path_to_host(nc_dup_tensor(logits), symbols);
+            nc_synchronize(dev); /* the one wait of the evaluation: these entries, and the loss if it was queued */
             d.path = nc_tensor_get_ptr(d.host, &d.stride);
             return d;
         }
@@ -158,12 +160,13 @@ static HostDist encode_segment_eval(Coder *c, int idx, int n_t, int len2, int fu
             if (symbols) nc_set1_i32_2d(symbols, b, t, get_symb(&c->view, b, idx + t));
         }
     double t0 = now_s();
-    if (symbols) { /* up before the evaluation is queued: an upload waits for the stream */
-        size_t dims[2];
-        nc_tensor_get_dims(symbols, dims);
-        symbols = nc_tensor_to_device(nc_reshape_1d(symbols, dims[0] * dims[1]), nncp_model_device(c->s));
-    }
+    if (symbols)
+        symbols = nc_tensor_to_device(symbols, nncp_model_device(c->s));
     NCTensor *out = c->cls->eval(c->s, -1, input);
+    /* a full segment that training follows: its expected symbols are these, so the loss is queued
+       behind the evaluation now and arrives with the CDF entries */
+    if (symbols && expected && full && c->cls->queue_loss)
+        c->cls->queue_loss(c->s, nc_dup_tensor(symbols));
     HostDist d = fetch_dist(c, out, symbols);
     c->st->t_eval += now_s() - t0;
     return d;

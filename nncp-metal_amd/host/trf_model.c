@@ -584,7 +584,10 @@ NCTensor *trf_eval(NNCPModel *s, int output_index, const NCTensor *input)
     if (fused && output_index >= 0)
         die("the fused path evaluates whole segments only (output_index < 0)");
     if (output_index < 0) { /* nncp.c:612-623 */
-        t0 = nc_dup_tensor(input);
+        /* a copy of the caller's tokens that ends with its upload: the library can leave
+           that transfer queued instead of waiting for it (the caller may rewrite `input`) */
+        t0 = nc_new_tensor_from_tensor_nz(input);
+        nc_tensor_copy(t0, (NCTensor *)input);
         s->seq_eval = 0;
         seg_len = c->seg_len;
     } else {
@@ -843,6 +846,8 @@ void trf_eval_end(NNCPModel *s) /* nncp.c:1032-1060 */
     }
     nc_free_tensor(s->logits);
     s->logits = NULL;
+    nc_free_tensor(s->pending_loss); nc_free_tensor(s->pending_loss_host);
+    s->pending_loss = s->pending_loss_host = NULL;
 }
 
 void nncp_backward_cb(void *opaque, NCTensor *yg, NCTensor *get_col_index) /* nncp.c:1078-1096 */
@@ -874,12 +879,36 @@ static NCNode *merge_timestep_nodes(NNCPModel *s, NCNode **src, NCNode **consume
     return n;
 }
 
+/* NNCPModelClass.queue_loss: the first half of trf_eval_gradient for a whole-segment
+   evaluation, queued behind it without a wait */
+static void trf_queue_loss(NNCPModel *s, NCTensor *expected)
+{
+    if (s->seq_eval || !s->outputs[0] || s->pending_loss) {
+        nc_free_tensor(expected);
+        return;
+    }
+    NCTensor *output = s->outputs[0];
+    s->outputs[0] = NULL;
+    NCTensor *loss = nc_sum(nc_indexed_log(output, expected));
+    s->pending_loss_host = nc_tensor_to_cpu_device_queued(nc_dup_tensor(loss));
+    s->pending_loss = loss;
+}
+
 float trf_eval_gradient(NNCPModel *s, const NCTensor *expected_output1) /* nncp.c:1099-1193 */
 {
     const NNCPConfig *c = &s->cfg;
-    NCTensor *expected = nc_tensor_to_device(nc_dup_tensor(expected_output1), s->dev);
-    NCTensor *output, *loss;
+    NCTensor *expected, *output, *loss;
     float ret;
+    if (s->pending_loss) { /* queued by trf_queue_loss; the caller has waited since */
+        prof_start(PROF_GRAD);
+        nc_synchronize(s->dev); /* (no cost on a drained stream; a guard for a caller that has not) */
+        loss = s->pending_loss;
+        ret = ((const float *)nc_tensor_get_ptr(s->pending_loss_host, NULL))[0];
+        nc_free_tensor(s->pending_loss_host);
+        s->pending_loss = s->pending_loss_host = NULL;
+        goto backward;
+    }
+    expected = nc_tensor_to_device(nc_dup_tensor(expected_output1), s->dev);
     prof_start(PROF_GRAD); /* nncp.c:1108 */
     if (s->seq_eval) {
         NCNode **tab = nc_malloc(sizeof(NCNode *) * (c->n_layer * 2 + 1));
@@ -903,6 +932,7 @@ float trf_eval_gradient(NNCPModel *s, const NCTensor *expected_output1) /* nncp.
     nc_free_tensor(expected);
     loss = nc_sum(loss);
     ret = nc_get_scalar_f32(loss);
+backward:
     loss = nc_mul(loss, nc_new_f32(nc_get_tensor_device(loss), -1.0f / (float)(c->seg_len * c->batch_size)));
     nc_backward(loss, nc_new_f32(s->dev, 1.0f), nncp_backward_cb, 0);
     nc_free_tensor(loss);
@@ -971,6 +1001,7 @@ void nncp_model_set_train_step(NNCPModel *s, int64_t step) { s->train_step = ste
 const NNCPModelClass nncp_trf_class = { /* nncp.c:1544-1562 */
     trf_eval, trf_eval_end, trf_eval_gradient, trf_reset, trf_update, trf_set_lr, trf_set_retrain, trf_last_logits,
     trf_eval_end, /* no state is handed on before trf_update */
+    trf_queue_loss,
 };
 
 const NNCPModelClass *nncp_model_class(NNCPModel *s) { return s->cls; }

@@ -449,6 +449,9 @@ NCTensor *nc_soft_max_cdf16_path(NCTensor *logits, NCTensor *symbols) /* nc_ext.
     return nc_cdf_path(nc_soft_max_cdf16(logits), symbols);
 }
 
+NCTensor *nc_soft_max_cdf16_path_to_host(NCTensor *logits, NCTensor *symbols) { return nc_soft_max_cdf16_path(logits, symbols); }
+NCTensor *nc_tensor_to_cpu_device_queued(NCTensor *x) { return nc_tensor_to_cpu_device(x); }
+
 NCTensor *nc_cdf_lookup(NCTensor *cdf, NCTensor *targets)
 {
     NCTensor *y;
